@@ -1,0 +1,190 @@
+"""``HipLinear``: the autograd function that occupies the accelerated-operator slot of
+``AnalogLinear.forward`` (the place of ``TritonLinear`` in the reference,
+``nn/modules/linear.py:120-135`` / ``triton_utils/triton_linear.py:446-764``), with the
+semantics of the reference's torch-mode (``torch_utils/torch_linear.py:116-314``).
+"""
+import os
+from typing import List, Optional
+
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from . import library as L
+from .ops import OPS
+from ....exceptions import ConfigError, HipBackendError
+from ....simulator.configs import (
+    TorchInferenceRPUConfig,
+    WeightClipType,
+    WeightNoiseInjectionType,
+    WeightQuantizationType,
+)
+
+NOISE_IDS = {
+    WeightNoiseInjectionType.NONE: L.AHL_NOISE_NONE,
+    WeightNoiseInjectionType.ADD_NORMAL: L.AHL_NOISE_ADD_NORMAL,
+    WeightNoiseInjectionType.ADD_NORMAL_PER_CHANNEL: L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL,
+}
+QUANT_IDS = {
+    WeightQuantizationType.NONE: L.AHL_QUANT_NONE,
+    WeightQuantizationType.DISCRETIZE: L.AHL_QUANT_DISCRETIZE,
+    WeightQuantizationType.DISCRETIZE_PER_CHANNEL: L.AHL_QUANT_DISCRETIZE_PER_CHANNEL,
+}
+
+
+def draw_seed() -> int:
+    """One Philox key per call from torch's CPU generator, so ``torch.manual_seed`` makes runs
+    reproducible (the reference seeds its kernels the same way, ``triton_linear.py:541,617``)."""
+    return int(torch.randint(0, 2**62, (1,)).item())
+
+
+def check_supported(rpu_config: TorchInferenceRPUConfig) -> None:
+    """Reject configuration branches that the HIP backend does not implement."""
+    if rpu_config.clip.type == WeightClipType.LEARNABLE_PER_CHANNEL:
+        raise ConfigError("WeightClipType.LEARNABLE_PER_CHANNEL is not implemented by the HIP backend")
+    ir_params = rpu_config.pre_post.input_range
+    if ir_params.enable and ir_params.fast_mode:
+        raise ConfigError("input_range.fast_mode is not implemented by the HIP backend")
+
+
+class HipLinear(Function):
+    """y = analog_mvm(x, W) + b with DAC/ADC, noise and tiling, on MI355X."""
+
+    # pylint: disable=abstract-method, arguments-differ, too-many-locals, too-many-arguments
+
+    @staticmethod
+    def forward(
+        ctx,
+        inp: Tensor,
+        weights: Tensor,
+        bias: Optional[Tensor],
+        input_range: Optional[Tensor],
+        input_range_update_idx: Optional[Tensor],
+        in_sizes: List[int],
+        rpu_config: TorchInferenceRPUConfig,
+        training: bool,
+        init_active: bool,
+    ) -> Tensor:
+        if not inp.is_cuda:
+            raise HipBackendError(
+                "AnalogLinear runs only on a ROCm device (got a CPU tensor); there is no CPU path"
+            )
+        check_supported(rpu_config)
+        fwd, modifier = rpu_config.forward, rpu_config.modifier
+        ir_params = rpu_config.pre_post.input_range
+        k_in, n_out = weights.size(1), weights.size(0)
+        out_shape = inp.shape[:-1] + (n_out,)
+        x2 = inp.reshape(-1, k_in)
+        if x2.stride(-1) != 1:
+            x2 = x2.contiguous()
+        weights_c = weights if weights.stride(1) == 1 else weights.contiguous()
+        if weights.dtype != inp.dtype:
+            raise HipBackendError("input and weight dtypes differ")
+        m_rows = x2.size(0)
+
+        apply_out_quantization = fwd.out_res > 0
+        if apply_out_quantization:
+            assert fwd.out_bound > 0, "Out quant. without a bound."
+            assert ir_params.enable, "Out quant. without IR."
+        if ir_params.enable and not ir_params.dynamic:
+            assert input_range is not None, "Input range must be provided"
+            assert input_range_update_idx is not None, "Input range update index must be provided"
+            ir_mode = L.AHL_IR_STATIC
+        elif ir_params.enable:
+            ir_mode = L.AHL_IR_DYNAMIC
+        else:
+            ir_mode = L.AHL_IR_NONE
+            assert fwd.inp_res <= 0, "Input range must be provided"
+        noise_on = training and fwd.out_noise > 0
+        if noise_on:
+            assert ir_params.enable, "Input range must be enabled"
+        bound_on = fwd.out_bound > 0 or apply_out_quantization
+        if bound_on:
+            assert ir_params.enable, (
+                "Input range must be provided when using an out_bound or out quantization"
+            )
+        w_noise = training and modifier.noise_type != WeightNoiseInjectionType.NONE
+        w_quant = modifier.quantization_type != WeightQuantizationType.NONE
+        need_wmax = bound_on or noise_on or w_noise or w_quant
+        ir_needs_grad = ir_mode == L.AHL_IR_STATIC and input_range.requires_grad
+        need_dx = ctx.needs_input_grad[0] or (ctx.needs_input_grad[3] and ir_needs_grad)
+        need_dw = ctx.needs_input_grad[1]
+
+        seed = draw_seed() if (noise_on or w_noise) else 0
+        wmax = tile_max = None
+        w_eff, w_eff_t = weights_c, None
+        if m_rows > 0 and (need_wmax or need_dx):
+            res = float(modifier.res) if w_quant else 1.0
+            wmax, tile_max, _, eff, eff_t = OPS.weight_prep(
+                weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
+                NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE, res,
+                float(modifier.std_dev), seed, 1, w_noise or w_quant, need_dx,
+            )
+            if w_noise or w_quant:
+                w_eff = eff
+            w_eff_t = eff_t if need_dx else None
+
+        ir_dev = None
+        if ir_mode == L.AHL_IR_STATIC:
+            if training and init_active and m_rows > 0:
+                std = OPS.sliced_std(x2, in_sizes)
+                OPS.ir_init_update(
+                    input_range.data, input_range_update_idx, std, float(ir_params.init_from_data),
+                    float(ir_params.init_std_alpha),
+                )
+            ir_dev = input_range.detach()
+            if not ir_dev.is_contiguous():
+                ir_dev = ir_dev.contiguous()
+        elif ir_mode == L.AHL_IR_DYNAMIC and m_rows > 0:
+            ir_dev = OPS.sliced_absmax(x2, in_sizes, False)[0]
+
+        skip_rounding = 1 if os.environ.get("_AIHWKIT_NO_ROUNDING", False) else 0
+        icfg = [
+            ir_mode, int(fwd.out_noise_per_channel),
+            int(rpu_config.clip.type in (WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL,
+                                         WeightClipType.LEARNABLE_PER_CHANNEL)),
+            int(training), skip_rounding, seed, 0,
+        ]
+        fcfg = [
+            float(fwd.inp_res), float(fwd.out_res), float(fwd.out_bound),
+            float(fwd.out_noise) if noise_on else 0.0, float(ir_params.decay),
+            float(ir_params.input_min_percentage),
+        ]
+        want_keep = fwd.out_bound > 0 and (need_dx or need_dw)
+        if m_rows == 0:
+            return inp.new_zeros(out_shape)
+        y, keep = OPS.linear_fwd(
+            x2, w_eff, bias, ir_dev, wmax, tile_max, in_sizes, icfg, fcfg, want_keep
+        )
+
+        ctx.in_sizes, ctx.icfg, ctx.fcfg = in_sizes, icfg, fcfg
+        ctx.inp_shape, ctx.ir_mode, ctx.has_bias = inp.shape, ir_mode, bias is not None
+        ctx.need_dx, ctx.need_dw, ctx.ir_needs_grad = need_dx, need_dw, ir_needs_grad
+        ctx.save_for_backward(
+            x2, w_eff_t, keep if want_keep else None,
+            ir_dev.clone() if ir_mode == L.AHL_IR_STATIC else ir_dev,
+        )
+        return y.view(out_shape)
+
+    @staticmethod
+    def backward(ctx, grad_out: Tensor):
+        x2, w_eff_t, keep, ir_dev = ctx.saved_tensors
+        n_out = grad_out.size(-1)
+        g2 = grad_out.reshape(-1, n_out)
+        if g2.stride(-1) != 1 or (g2.size(0) > 1 and g2.stride(0) != n_out):
+            g2 = g2.contiguous()
+        grad_inp = grad_w = grad_b = grad_ir = None
+        if ctx.need_dx:
+            dx, ir_grad = OPS.linear_bwd_dx(
+                g2, keep, w_eff_t, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
+                ctx.in_sizes, ctx.icfg, ctx.fcfg,
+            )
+            if ctx.needs_input_grad[0]:
+                grad_inp = dx.view(ctx.inp_shape)
+            if ctx.ir_needs_grad and ctx.needs_input_grad[3]:
+                grad_ir = ir_grad
+        if ctx.need_dw:
+            grad_w = OPS.linear_bwd_dw(g2, keep, x2, ir_dev, ctx.in_sizes, ctx.icfg, ctx.fcfg)
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            grad_b = OPS.col_sum(g2)
+        return grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None

@@ -1,0 +1,181 @@
+"""ctypes binding of ``libanalog_hip.so`` (the C ABI declared in ``include/analog_hip.h``).
+
+The library is built in-tree by ``aihwkit-lightning_amd/build.py`` into ``aihwkit_lightning/_lib``.
+Loading is lazy and failure is loud: there is no software fallback for any entry point.
+"""
+import ctypes
+import os
+from ctypes import c_void_p, c_int32, c_int64, c_float, c_uint64, c_char_p, POINTER, Structure
+
+from ....exceptions import HipBackendError
+
+LIB_NAME = "libanalog_hip.so"
+LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
+ABI_VERSION = 1
+
+AHL_F32, AHL_BF16 = 0, 1
+AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
+AHL_NOISE_NONE, AHL_NOISE_ADD_NORMAL, AHL_NOISE_ADD_NORMAL_PER_CHANNEL = 0, 1, 2
+AHL_QUANT_NONE, AHL_QUANT_DISCRETIZE, AHL_QUANT_DISCRETIZE_PER_CHANNEL = 0, 1, 2
+AHL_CLIP_LAYER, AHL_CLIP_PER_CHANNEL = 0, 1
+
+STATUS_TEXT = {
+    1: "invalid argument",
+    2: "tile ends do not follow the K-tile split rule",
+    3: "not supported by the HIP backend",
+    4: "HIP launch failed",
+    5: "workspace too small or misaligned",
+}
+
+
+class AhlLinearCfg(Structure):
+    """Mirror of ``struct AhlLinearCfg``."""
+
+    _fields_ = [
+        ("dtype", c_int32),
+        ("ir_mode", c_int32),
+        ("inp_res", c_float),
+        ("out_res", c_float),
+        ("out_bound", c_float),
+        ("out_noise", c_float),
+        ("out_noise_per_channel", c_int32),
+        ("bound_per_channel", c_int32),
+        ("training", c_int32),
+        ("skip_rounding", c_int32),
+        ("ir_decay", c_float),
+        ("ir_input_min_percentage", c_float),
+        ("seed", c_uint64),
+        ("offset", c_uint64),
+    ]
+
+
+class AhlModifierCfg(Structure):
+    """Mirror of ``struct AhlModifierCfg``."""
+
+    _fields_ = [
+        ("dtype", c_int32),
+        ("quant_type", c_int32),
+        ("noise_type", c_int32),
+        ("res", c_float),
+        ("std_dev", c_float),
+        ("seed", c_uint64),
+        ("offset", c_uint64),
+    ]
+
+
+_I32P = POINTER(c_int32)
+
+# name -> (restype, argtypes); every exported symbol of include/analog_hip.h
+SIGNATURES = {
+    "ahl_abi_version": (c_int32, []),
+    "ahl_last_hip_error": (c_char_p, []),
+    "ahl_sliced_absmax": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int64, c_int64, _I32P, c_int32, c_void_p, c_void_p,
+         c_void_p, c_void_p],
+    ),
+    "ahl_sliced_std": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int64, c_int64, _I32P, c_int32, c_void_p, c_void_p, c_void_p],
+    ),
+    "ahl_sliced_std_ws_bytes": (c_int64, [c_int64, c_int32]),
+    "ahl_ir_init_update": (
+        c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_float, c_float, c_void_p]
+    ),
+    "ahl_running_absmax": (
+        c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, _I32P, c_int32, c_void_p, c_void_p]
+    ),
+    "ahl_clip_weights": (
+        c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_float, c_int32, c_void_p, c_void_p]
+    ),
+    "ahl_clip_weights_ws_bytes": (c_int64, [c_int64]),
+    "ahl_col_sum": (
+        c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p]
+    ),
+    "ahl_col_sum_ws_bytes": (c_int64, [c_int64]),
+    "ahl_weight_prep": (
+        c_int32,
+        [c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32, POINTER(AhlModifierCfg), c_void_p,
+         c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p],
+    ),
+    "ahl_quantize_weights": (
+        c_int32,
+        [c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32, POINTER(AhlModifierCfg), c_void_p,
+         c_void_p, c_void_p],
+    ),
+    "ahl_linear_fwd": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32, POINTER(AhlLinearCfg),
+         c_void_p],
+    ),
+    "ahl_linear_bwd_dx": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+         c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32, POINTER(AhlLinearCfg), c_void_p,
+         c_void_p],
+    ),
+    "ahl_linear_bwd_dx_ws_bytes": (c_int64, [c_int64, c_int64, c_int32]),
+    "ahl_linear_bwd_dw": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64,
+         c_int64, c_int64, _I32P, c_int32, POINTER(AhlLinearCfg), c_void_p, c_void_p],
+    ),
+    "ahl_linear_bwd_dw_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32]),
+}
+
+_LIB = None
+
+
+def lib_path() -> str:
+    """Absolute path where the built library is expected."""
+    return os.path.join(LIB_DIR, LIB_NAME)
+
+
+def load() -> ctypes.CDLL:
+    """Load the library once and bind every symbol; raises HipBackendError if anything is missing."""
+    global _LIB  # pylint: disable=global-statement
+    if _LIB is not None:
+        return _LIB
+    path = lib_path()
+    if not os.path.exists(path):
+        raise HipBackendError(
+            f"{path} not found: build it with `python aihwkit-lightning_amd/build.py` "
+            "(hipcc --offload-arch=gfx950). There is no fallback implementation."
+        )
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as exc:
+        raise HipBackendError(f"could not load {path}: {exc}") from exc
+    for name, (restype, argtypes) in SIGNATURES.items():
+        try:
+            func = getattr(lib, name)
+        except AttributeError as exc:
+            raise HipBackendError(f"{path} does not export {name}") from exc
+        func.restype = restype
+        func.argtypes = argtypes
+    if lib.ahl_abi_version() != ABI_VERSION:
+        raise HipBackendError(
+            f"{path} has ABI version {lib.ahl_abi_version()}, expected {ABI_VERSION}; rebuild it"
+        )
+    _LIB = lib
+    return lib
+
+
+def check(status: int, where: str) -> None:
+    """Turn a non-zero status into an exception."""
+    if status == 0:
+        return
+    text = STATUS_TEXT.get(status, f"status {status}")
+    if status == 4:
+        text += ": " + load().ahl_last_hip_error().decode()
+    raise HipBackendError(f"{where}: {text}")
+
+
+def tile_ends_array(in_sizes):
+    """Cumulative tile ends as a host int32 array (the reference's ``upper_end_of_slices``)."""
+    ends, acc = [], 0
+    for size in in_sizes:
+        acc += int(size)
+        ends.append(acc)
+    return (c_int32 * len(ends))(*ends)

@@ -1,0 +1,334 @@
+"""Torch custom ops (namespace ``aihwkit_hip``) over the C ABI of ``libanalog_hip.so``.
+
+Each op allocates its outputs and scratch with torch (device memory plumbing only), passes raw
+device pointers, sizes and the current HIP stream to one C entry point, and returns. The ops are
+registered for the CUDA (= ROCm/HIP) dispatch key only: calling them on CPU tensors raises.
+"""
+from ctypes import byref, c_void_p
+from typing import List, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import library as L
+from ....exceptions import HipBackendError
+
+_DTYPES = {torch.float32: L.AHL_F32, torch.bfloat16: L.AHL_BF16}
+
+
+def dtype_id(dtype: torch.dtype) -> int:
+    """Map a torch dtype onto the ABI's dtype enum."""
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise HipBackendError(
+            f"dtype {dtype} is not supported by the HIP backend (float32 and bfloat16 are)"
+        ) from None
+
+
+def _ptr(tensor: Optional[Tensor]):
+    return None if tensor is None else c_void_p(tensor.data_ptr())
+
+
+def _stream():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _rows2d(tensor: Tensor, name: str) -> Tensor:
+    if tensor.dim() != 2:
+        raise HipBackendError(f"{name} must be 2-D, got shape {tuple(tensor.shape)}")
+    if tensor.stride(1) != 1 and tensor.size(1) != 1:
+        tensor = tensor.contiguous()
+    if tensor.size(0) > 1 and tensor.stride(0) < tensor.size(1):
+        tensor = tensor.contiguous()
+    return tensor
+
+
+def _ld(tensor: Tensor) -> int:
+    return tensor.stride(0) if tensor.size(0) > 1 else max(tensor.size(1), tensor.stride(0))
+
+
+def _linear_cfg(dtype: torch.dtype, icfg: List[int], fcfg: List[float]) -> L.AhlLinearCfg:
+    cfg = L.AhlLinearCfg()
+    cfg.dtype = dtype_id(dtype)
+    (cfg.ir_mode, cfg.out_noise_per_channel, cfg.bound_per_channel, cfg.training,
+     cfg.skip_rounding, seed, offset) = icfg
+    (cfg.inp_res, cfg.out_res, cfg.out_bound, cfg.out_noise, cfg.ir_decay,
+     cfg.ir_input_min_percentage) = fcfg
+    cfg.seed, cfg.offset = seed, offset
+    return cfg
+
+
+LIB = torch.library.Library("aihwkit_hip", "DEF")
+
+LIB.define("sliced_absmax(Tensor x, int[] in_sizes, bool tile_stats) -> (Tensor, Tensor, Tensor)")
+LIB.define("sliced_std(Tensor x, int[] in_sizes) -> Tensor")
+LIB.define(
+    "ir_init_update(Tensor(a!) ir, Tensor(b!) idx, Tensor std, float init_from_data, "
+    "float alpha) -> ()"
+)
+LIB.define("running_absmax(Tensor x, int[] in_sizes, Tensor(a!) cache) -> ()")
+LIB.define("clip_weights(Tensor(a!) w, float sigma, int kind) -> ()")
+LIB.define("col_sum(Tensor x) -> Tensor")
+LIB.define(
+    "weight_prep(Tensor w, int[] in_sizes, int quant_type, int noise_type, float res, "
+    "float std_dev, int seed, int offset, bool want_eff, bool want_eff_t) "
+    "-> (Tensor, Tensor, Tensor, Tensor, Tensor)"
+)
+LIB.define("quantize_weights(Tensor(a!) w, int[] in_sizes, int quant_type, float res) -> ()")
+LIB.define(
+    "linear_fwd(Tensor x, Tensor w_eff, Tensor? bias, Tensor? ir, Tensor? wmax, Tensor? tile_max, "
+    "int[] in_sizes, int[] icfg, float[] fcfg, bool want_keep) -> (Tensor, Tensor)"
+)
+LIB.define(
+    "linear_bwd_dx(Tensor g, Tensor? keep, Tensor w_eff_t, Tensor? x, Tensor? ir, int[] in_sizes, "
+    "int[] icfg, float[] fcfg) -> (Tensor, Tensor)"
+)
+LIB.define(
+    "linear_bwd_dw(Tensor g, Tensor? keep, Tensor x, Tensor? ir, int[] in_sizes, int[] icfg, "
+    "float[] fcfg) -> Tensor"
+)
+
+
+def sliced_absmax(x: Tensor, in_sizes: List[int], tile_stats: bool) -> Tuple[Tensor, Tensor, Tensor]:
+    """``out[t, r] = max |x[r, tile t]|`` (+ per-tile max/min over rows)."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    n_tiles, rows = len(in_sizes), x.size(0)
+    out = torch.empty((n_tiles, rows), dtype=x.dtype, device=x.device)
+    n_stats = n_tiles if tile_stats else 0
+    tile_max = torch.empty((n_stats,), dtype=torch.float32, device=x.device)
+    tile_min = torch.empty((n_stats,), dtype=torch.float32, device=x.device)
+    L.check(
+        lib.ahl_sliced_absmax(
+            _ptr(x), dtype_id(x.dtype), rows, x.size(1), _ld(x), L.tile_ends_array(in_sizes), n_tiles,
+            _ptr(out), _ptr(tile_max) if tile_stats else None,
+            _ptr(tile_min) if tile_stats else None, _stream(),
+        ),
+        "ahl_sliced_absmax",
+    )
+    return out, tile_max, tile_min
+
+
+def sliced_std(x: Tensor, in_sizes: List[int]) -> Tensor:
+    """Unbiased std of every K-tile over all rows, float32 ``[T]``."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    n_tiles = len(in_sizes)
+    out = torch.empty((n_tiles,), dtype=torch.float32, device=x.device)
+    ws = torch.empty((lib.ahl_sliced_std_ws_bytes(x.size(0), n_tiles),), dtype=torch.uint8,
+                     device=x.device)
+    L.check(
+        lib.ahl_sliced_std(
+            _ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), L.tile_ends_array(in_sizes),
+            n_tiles, _ptr(out), _ptr(ws), _stream(),
+        ),
+        "ahl_sliced_std",
+    )
+    return out
+
+
+def ir_init_update(ir: Tensor, idx: Tensor, std: Tensor, init_from_data: float, alpha: float) -> None:
+    """In-place input-range initialisation step from the per-tile std."""
+    lib = L.load()
+    if not (ir.is_contiguous() and idx.is_contiguous() and ir.dtype == idx.dtype):
+        raise HipBackendError("input_range and input_range_update_idx must be contiguous, same dtype")
+    L.check(
+        lib.ahl_ir_init_update(
+            _ptr(ir), _ptr(idx), _ptr(std), dtype_id(ir.dtype), ir.numel(), init_from_data, alpha,
+            _stream(),
+        ),
+        "ahl_ir_init_update",
+    )
+
+
+def running_absmax(x: Tensor, in_sizes: List[int], cache: Tensor) -> None:
+    """``cache[t] = max(cache[t], max |x[:, tile t]|)``; cache is float32 ``[T]`` on the device."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    if cache.dtype != torch.float32 or not cache.is_contiguous() or cache.numel() != len(in_sizes):
+        raise HipBackendError("cache must be a contiguous float32 tensor with one entry per tile")
+    L.check(
+        lib.ahl_running_absmax(
+            _ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), L.tile_ends_array(in_sizes),
+            len(in_sizes), _ptr(cache), _stream(),
+        ),
+        "ahl_running_absmax",
+    )
+
+
+def clip_weights(w: Tensor, sigma: float, kind: int) -> None:
+    """In-place clamp of ``w`` at ``sigma`` standard deviations (per matrix or per row)."""
+    lib = L.load()
+    if w.dim() != 2 or w.stride(1) != 1:
+        raise HipBackendError("weight must be a row-major 2-D tensor")
+    ws = torch.empty((lib.ahl_clip_weights_ws_bytes(w.size(0)),), dtype=torch.uint8, device=w.device)
+    L.check(
+        lib.ahl_clip_weights(
+            _ptr(w), dtype_id(w.dtype), w.size(0), w.size(1), _ld(w), sigma, kind, _ptr(ws), _stream()
+        ),
+        "ahl_clip_weights",
+    )
+
+
+def col_sum(x: Tensor) -> Tensor:
+    """Column sums of a 2-D tensor in its dtype (float accumulation)."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    out = torch.empty((x.size(1),), dtype=x.dtype, device=x.device)
+    ws = torch.empty((lib.ahl_col_sum_ws_bytes(x.size(1)),), dtype=torch.uint8, device=x.device)
+    L.check(
+        lib.ahl_col_sum(
+            _ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), _ptr(out), _ptr(ws), _stream()
+        ),
+        "ahl_col_sum",
+    )
+    return out
+
+
+def _modifier_cfg(dtype, quant_type, noise_type, res, std_dev, seed, offset) -> L.AhlModifierCfg:
+    cfg = L.AhlModifierCfg()
+    cfg.dtype = dtype_id(dtype)
+    cfg.quant_type, cfg.noise_type = quant_type, noise_type
+    cfg.res, cfg.std_dev = res, std_dev
+    cfg.seed, cfg.offset = seed, offset
+    return cfg
+
+
+def weight_prep(
+    w: Tensor, in_sizes: List[int], quant_type: int, noise_type: int, res: float, std_dev: float,
+    seed: int, offset: int, want_eff: bool, want_eff_t: bool,
+) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
+    """wmax ``[T, N]``, tile max/min ``[T]``, optional modified copy ``[N, K]`` and its transpose."""
+    lib = L.load()
+    if w.dim() != 2 or w.stride(1) != 1:
+        raise HipBackendError("weight must be a row-major 2-D tensor")
+    n_out, n_in = w.shape
+    n_tiles = len(in_sizes)
+    dev = w.device
+    wmax = torch.empty((n_tiles, n_out), dtype=w.dtype, device=dev)
+    tile_max = torch.empty((n_tiles,), dtype=torch.float32, device=dev)
+    tile_min = torch.empty((n_tiles,), dtype=torch.float32, device=dev)
+    w_eff = torch.empty((n_out, n_in) if want_eff else (0,), dtype=w.dtype, device=dev)
+    w_eff_t = torch.empty((n_in, n_out) if want_eff_t else (0,), dtype=w.dtype, device=dev)
+    cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset)
+    L.check(
+        lib.ahl_weight_prep(
+            _ptr(w), n_out, n_in, _ld(w), L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(wmax),
+            _ptr(tile_max), _ptr(tile_min), _ptr(w_eff) if want_eff else None, n_in,
+            _ptr(w_eff_t) if want_eff_t else None, _stream(),
+        ),
+        "ahl_weight_prep",
+    )
+    return wmax, tile_max, tile_min, w_eff, w_eff_t
+
+
+def quantize_weights(w: Tensor, in_sizes: List[int], quant_type: int, res: float) -> None:
+    """In-place per-tile weight quantisation with scales from each slice's own abs-max."""
+    lib = L.load()
+    if w.dim() != 2 or w.stride(1) != 1:
+        raise HipBackendError("weight must be a row-major 2-D tensor")
+    n_tiles = len(in_sizes)
+    ws_wmax = torch.empty((n_tiles, w.size(0)), dtype=w.dtype, device=w.device)
+    ws_tile = torch.empty((2 * n_tiles,), dtype=torch.float32, device=w.device)
+    cfg = _modifier_cfg(w.dtype, quant_type, L.AHL_NOISE_NONE, res, 0.0, 0, 0)
+    L.check(
+        lib.ahl_quantize_weights(
+            _ptr(w), w.size(0), w.size(1), _ld(w), L.tile_ends_array(in_sizes), n_tiles, byref(cfg),
+            _ptr(ws_wmax), _ptr(ws_tile), _stream(),
+        ),
+        "ahl_quantize_weights",
+    )
+
+
+def linear_fwd(
+    x: Tensor, w_eff: Tensor, bias: Optional[Tensor], ir: Optional[Tensor], wmax: Optional[Tensor],
+    tile_max: Optional[Tensor], in_sizes: List[int], icfg: List[int], fcfg: List[float],
+    want_keep: bool,
+) -> Tuple[Tensor, Tensor]:
+    """The fused analog forward; returns ``y [M, N]`` and the clamp mask (empty if not wanted)."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    m_rows, k_in = x.shape
+    n_out = w_eff.size(0)
+    n_tiles = len(in_sizes)
+    cfg = _linear_cfg(x.dtype, icfg, fcfg)
+    y = torch.empty((m_rows, n_out), dtype=x.dtype, device=x.device)
+    planes = (n_tiles + 7) // 8
+    keep = torch.empty((planes, m_rows, n_out) if want_keep else (0,), dtype=torch.uint8,
+                       device=x.device)
+    L.check(
+        lib.ahl_linear_fwd(
+            _ptr(x), _ld(x), _ptr(w_eff), _ld(w_eff), _ptr(bias), _ptr(y), n_out,
+            _ptr(keep) if want_keep else None, _ptr(ir), _ptr(wmax), _ptr(tile_max), m_rows, k_in,
+            n_out, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _stream(),
+        ),
+        "ahl_linear_fwd",
+    )
+    return y, keep
+
+
+def linear_bwd_dx(
+    g: Tensor, keep: Optional[Tensor], w_eff_t: Tensor, x: Optional[Tensor], ir: Optional[Tensor],
+    in_sizes: List[int], icfg: List[int], fcfg: List[float],
+) -> Tuple[Tensor, Tensor]:
+    """Input gradient ``[M, K]`` and input-range gradient ``[T]`` (empty unless static range)."""
+    lib = L.load()
+    g = _rows2d(g, "g")
+    m_rows, n_out = g.shape
+    k_in = w_eff_t.size(0)
+    n_tiles = len(in_sizes)
+    cfg = _linear_cfg(g.dtype, icfg, fcfg)
+    static = cfg.ir_mode == L.AHL_IR_STATIC
+    dx = torch.empty((m_rows, k_in), dtype=g.dtype, device=g.device)
+    ir_grad = torch.empty((n_tiles,) if static else (0,), dtype=g.dtype, device=g.device)
+    ws = torch.empty((max(lib.ahl_linear_bwd_dx_ws_bytes(m_rows, k_in, n_tiles), 16),),
+                     dtype=torch.uint8, device=g.device)
+    if x is not None:
+        x = _rows2d(x, "x")
+    L.check(
+        lib.ahl_linear_bwd_dx(
+            _ptr(g), _ld(g), _ptr(keep), _ptr(w_eff_t), _ptr(x), _ld(x) if x is not None else 0,
+            _ptr(ir), _ptr(dx), k_in, _ptr(ir_grad) if static else None, m_rows, k_in, n_out,
+            L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(ws), _stream(),
+        ),
+        "ahl_linear_bwd_dx",
+    )
+    return dx, ir_grad
+
+
+def linear_bwd_dw(
+    g: Tensor, keep: Optional[Tensor], x: Tensor, ir: Optional[Tensor], in_sizes: List[int],
+    icfg: List[int], fcfg: List[float],
+) -> Tensor:
+    """Weight gradient ``[N, K]``."""
+    lib = L.load()
+    g = _rows2d(g, "g")
+    x = _rows2d(x, "x")
+    m_rows, n_out = g.shape
+    k_in = x.size(1)
+    n_tiles = len(in_sizes)
+    cfg = _linear_cfg(g.dtype, icfg, fcfg)
+    dw = torch.empty((n_out, k_in), dtype=g.dtype, device=g.device)
+    ws_bytes = lib.ahl_linear_bwd_dw_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype,
+                                              0 if keep is None else 1)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=g.device)
+    L.check(
+        lib.ahl_linear_bwd_dw(
+            _ptr(g), _ld(g), _ptr(keep), _ptr(x), _ld(x), _ptr(ir), _ptr(dw), k_in, m_rows, k_in,
+            n_out, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(ws), _stream(),
+        ),
+        "ahl_linear_bwd_dw",
+    )
+    return dw
+
+
+for _name, _fn in [
+    ("sliced_absmax", sliced_absmax), ("sliced_std", sliced_std), ("ir_init_update", ir_init_update),
+    ("running_absmax", running_absmax), ("clip_weights", clip_weights), ("col_sum", col_sum),
+    ("weight_prep", weight_prep), ("quantize_weights", quantize_weights),
+    ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
+]:
+    LIB.impl(_name, _fn, "CUDA")
+
+OPS = torch.ops.aihwkit_hip

@@ -1,0 +1,246 @@
+// Device-side building blocks shared by every kernel of libanalog_hip.so (gfx950 only).
+//
+//  * dtype traits: F32 / BF16 with rd() = "round the fp32 result of one elementwise op to the
+//    tensor dtype", which is where torch rounds when it evaluates an op on bf16 tensors.
+//  * Tiling: the reference's K-tile split rule in closed form.
+//  * Philox4x32-10 counter-based RNG + Box-Muller.
+//  * wave64 reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define AHL_DEV __device__ __forceinline__
+
+namespace ahl {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// ---------------------------------------------------------------------------------------------
+// K-tile split (reference nn/modules/linear.py:155-170): n_tiles = ceil(K / max_input_size),
+// base, extra = divmod(K, n_tiles); the first `extra` tiles have base+1 columns, the rest base.
+struct Tiling {
+  int32_t n_tiles;
+  int32_t base;
+  int32_t extra;
+  AHL_DEV int32_t start(int32_t t) const { return t * base + (t < extra ? t : extra); }
+  AHL_DEV int32_t size(int32_t t) const { return base + (t < extra ? 1 : 0); }
+  AHL_DEV int32_t tile_of(int32_t k) const {
+    const int32_t big = extra * (base + 1);
+    return k < big ? k / (base + 1) : extra + (k - big) / base;
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// bf16 <-> f32
+AHL_DEV float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
+AHL_DEV uint32_t f32_to_bf16_bits(float x) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x);
+}
+AHL_DEV uint32_t pack_bf16x2(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  bf16x2 b = __builtin_convertvector(v, bf16x2);  // one v_cvt_pk_bf16_f32 (RNE)
+  return __builtin_bit_cast(uint32_t, b);
+}
+AHL_DEV float unpack_lo(uint32_t w) { return __uint_as_float(w << 16); }
+AHL_DEV float unpack_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// ---------------------------------------------------------------------------------------------
+// dtype traits. `vec` is one 16-byte global/LDS transaction holding EPV elements.
+struct F32 {
+  typedef float elem;
+  static constexpr int kId = 0;
+  static constexpr int EPV = 4;
+  static constexpr bool kIsBf16 = false;
+  static AHL_DEV float rd(float x) { return x; }
+  static AHL_DEV elem to_elem(float x) { return x; }
+  static AHL_DEV float load(const void* p, int64_t i) { return ((const float*)p)[i]; }
+  static AHL_DEV void store(void* p, int64_t i, float v) { ((float*)p)[i] = v; }
+  static AHL_DEV void unpack(const u32x4& v, float* f) {
+    f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+    f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+  }
+  static AHL_DEV u32x4 pack(const float* f) {
+    u32x4 v = {__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]),
+               __float_as_uint(f[3])};
+    return v;
+  }
+  // x / d, where rcp_d is 1/d: fp32 tensors use the IEEE quotient like torch on the CPU.
+  static AHL_DEV float div(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
+};
+
+struct BF16 {
+  typedef uint16_t elem;
+  static constexpr int kId = 1;
+  static constexpr int EPV = 8;
+  static constexpr bool kIsBf16 = true;
+  static AHL_DEV float rd(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
+  static AHL_DEV elem to_elem(float x) { return (elem)f32_to_bf16_bits(x); }
+  static AHL_DEV float load(const void* p, int64_t i) {
+    return bf16_bits_to_f32(((const uint16_t*)p)[i]);
+  }
+  static AHL_DEV void store(void* p, int64_t i, float v) {
+    ((uint16_t*)p)[i] = (uint16_t)f32_to_bf16_bits(v);
+  }
+  static AHL_DEV void unpack(const u32x4& v, float* f) {
+    f[0] = unpack_lo(v.x); f[1] = unpack_hi(v.x); f[2] = unpack_lo(v.y); f[3] = unpack_hi(v.y);
+    f[4] = unpack_lo(v.z); f[5] = unpack_hi(v.z); f[6] = unpack_lo(v.w); f[7] = unpack_hi(v.w);
+  }
+  static AHL_DEV u32x4 pack(const float* f) {
+    u32x4 v = {pack_bf16x2(f[0], f[1]), pack_bf16x2(f[2], f[3]), pack_bf16x2(f[4], f[5]),
+               pack_bf16x2(f[6], f[7])};
+    return v;
+  }
+  // For bf16 operands x and d (8-bit significands) the exact quotient is never closer than
+  // 2^-17 (relative) to a bf16 rounding boundary unless it is representable, so rounding
+  // x * fl32(1/d) to bf16 gives bit-identical results to rounding fl32(x / d). The caller
+  // rounds the returned value with rd().
+  static AHL_DEV float div(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
+};
+
+static constexpr float kTinyF32 = 1.17549435e-38f;  // finfo(float32).tiny == finfo(bfloat16).tiny
+
+// ---------------------------------------------------------------------------------------------
+// Resolution convention of the reference's UniformQuantize (torch_utils/quant_utils.py:63-76):
+// res > 1 is a number of states (step = 2*bound / res), otherwise the step is 2*bound * res.
+template <class D>
+AHL_DEV float quant_step(float bound, float res) {
+  const float alpha = D::rd(2.0f * bound);
+  return res > 1.0f ? D::rd(__fdiv_rn(alpha, res)) : D::rd(alpha * res);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11).
+AHL_DEV u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c.x;
+    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c.z;
+    u32x4 n;
+    n.x = (uint32_t)(p1 >> 32) ^ c.y ^ k0;
+    n.y = (uint32_t)p1;
+    n.z = (uint32_t)(p0 >> 32) ^ c.w ^ k1;
+    n.w = (uint32_t)p0;
+    c = n;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return c;
+}
+
+// Two standard normals from two 32-bit words (Box-Muller, 24-bit uniforms in (0,1)).
+AHL_DEV void box_muller(uint32_t a, uint32_t b, float& n0, float& n1) {
+  const float u1 = ((float)(a >> 8) + 0.5f) * 5.9604644775390625e-08f;  // 2^-24
+  const float u2 = ((float)(b >> 8) + 0.5f) * 5.9604644775390625e-08f;
+  const float r = __fsqrt_rn(-2.0f * __logf(u1));
+  float s, c;
+  __sincosf(6.283185307179586f * u2, &s, &c);
+  n0 = r * c;
+  n1 = r * s;
+}
+
+// Four standard normals for one counter value. Streams: 0 = output noise, 1 = weight noise.
+AHL_DEV void normal4(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, uint64_t group,
+                     float* out4) {
+  u32x4 c = {(uint32_t)group, (uint32_t)(group >> 32), stream_and_tile, (uint32_t)offset};
+  const u32x4 r = philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
+  box_muller(r.x, r.y, out4[0], out4[1]);
+  box_muller(r.z, r.w, out4[2], out4[3]);
+}
+
+// ---------------------------------------------------------------------------------------------
+// wave64 reductions (all lanes end up with the result)
+AHL_DEV float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+AHL_DEV float wave_min(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+AHL_DEV float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+AHL_DEV double wave_sum(double v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+AHL_DEV int64_t cdiv_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// 16-byte global load / store of one `vec`
+AHL_DEV u32x4 ld16(const void* p) { return *(const u32x4*)p; }
+AHL_DEV void st16(void* p, const u32x4& v) { *(u32x4*)p = v; }
+
+}  // namespace ahl
+
+namespace ahl {
+
+// ---------------------------------------------------------------------------------------------
+// DAC: clamp to the input range and quantise (Appendix of the torch-mode arithmetic):
+//   r = step(ir, inp_res); q = rd(xc / max(r, tiny)); q = rne(q); xq = rd(q * r)
+// (reference torch_utils/quant_utils.py:63-99 called from torch_utils/torch_linear.py:182-192).
+struct Dac {
+  float ir;    // clamp bound (ignored when clamp is off)
+  float r;     // quantisation step (unclamped; the product uses this one)
+  float rc;    // max(r, tiny): the divisor
+  float rcp;   // 1 / rc
+};
+
+template <class D>
+AHL_DEV Dac make_dac(float ir, float inp_res) {
+  Dac d;
+  d.ir = ir;
+  d.r = inp_res > 0.0f ? quant_step<D>(ir, inp_res) : 1.0f;
+  d.rc = fmaxf(d.r, kTinyF32);
+  d.rcp = __fdiv_rn(1.0f, d.rc);
+  return d;
+}
+
+template <class D, bool CLAMP, bool QUANT>
+AHL_DEV float dac_apply(float x, const Dac& d, bool skip_rounding) {
+  float v = x;
+  if (CLAMP) v = fminf(fmaxf(v, -d.ir), d.ir);
+  if (QUANT) {
+    float q = D::rd(D::div(v, d.rc, d.rcp));
+    if (!skip_rounding) q = rintf(q);  // v_rndne_f32: round half to even like torch.round
+    v = D::rd(q * d.r);
+  }
+  return v;
+}
+
+// Iterates one wave over the columns [c0, c1) of a row; f(value) is called once per element.
+// VEC: the row base (p + row*ld) is 16-byte aligned, so whole `vec`s can be loaded for the
+// aligned middle part; head and tail are done element-wise.
+template <class D, bool VEC, class F>
+AHL_DEV void wave_row_foreach(const void* row, int32_t c0, int32_t c1, int lane, F f) {
+  if (VEC) {
+    constexpr int E = D::EPV;
+    int32_t a0 = (c0 + E - 1) / E * E;
+    int32_t a1 = c1 / E * E;
+    if (a0 > a1) { a0 = c1; a1 = c1; }
+    for (int32_t c = c0 + lane; c < a0; c += 64) f(D::load(row, c));
+    const typename D::elem* base = (const typename D::elem*)row;
+    for (int32_t v = a0 / E + lane; v < a1 / E; v += 64) {
+      float e[E];
+      D::unpack(ld16(base + (int64_t)v * E), e);
+#pragma unroll
+      for (int i = 0; i < E; ++i) f(e[i]);
+    }
+    for (int32_t c = a1 + lane; c < c1; c += 64) f(D::load(row, c));
+  } else {
+    for (int32_t c = c0 + lane; c < c1; c += 64) f(D::load(row, c));
+  }
+}
+
+}  // namespace ahl

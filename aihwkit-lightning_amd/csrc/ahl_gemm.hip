@@ -1,0 +1,850 @@
+// The analog matrix product on CDNA4 MFMA: forward with fused DAC prologue and per-K-tile
+// noise/ADC/clamp epilogue, input gradient with fused input-range gradient, weight gradient.
+//
+// All three products are "row x row" contractions C[i, j] = sum_k A[i, k] * B[j, k] with both
+// operands contiguous along k, staged global -> registers -> LDS in 128-byte-wide row chunks
+// and consumed by v_mfma_f32_32x32x16_bf16 (bf16) or v_mfma_f32_32x32x2_f32 (fp32).
+//
+// Block: 256 threads = 4 waves in a 2x2 grid; block tile 128 x 128; wave tile 64 x 64 =
+// 2 x 2 MFMA blocks of 32 x 32 (16 fp32 accumulators per lane per block).
+//
+// LDS layout: one chunk = 128 rows x 128 data bytes, row stride 144 bytes; with this stride
+// the 16 lanes that the LDS services together for a 16-byte read hit 16 distinct 4-bank groups.
+//
+// MFMA operand convention: lane l supplies, for row/column (l % 32), the 16 bytes at byte
+// offset 32 * s + 16 * (l / 32) of the chunk row (s = k-step). A and B use the same rule, so
+// the contraction pairs identical k positions whatever the hardware's internal k order is.
+// MFMA 32x32 result convention: register v of lane l holds
+//   C[8 * (v / 4) + 4 * (l / 32) + (v % 4)][l % 32].
+#include "ahl_host.h"
+#include <math.h>
+
+namespace ahl {
+
+static constexpr int kBM = 128;
+static constexpr int kBN = 128;
+static constexpr int kRowBytes = 128;
+static constexpr int kLdsStride = 144;
+static constexpr int kChunkLds = 128 * kLdsStride;  // bytes per operand chunk in LDS
+
+template <class D>
+struct ChunkK {  // elements along k per chunk
+  static constexpr int value = kRowBytes / (int)sizeof(typename D::elem);
+};
+
+// ---- MFMA wrappers ---------------------------------------------------------------------------
+template <class D>
+struct Mma;
+template <>
+struct Mma<BF16> {
+  static AHL_DEV void run(const u32x4& a, const u32x4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<F32> {
+  static AHL_DEV void run(const u32x4& a, const u32x4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+};
+
+// One chunk of MFMAs for a wave: acc[bi][bj] += A(rows wm*64+bi*32..) x B(rows wn*64+bj*32..)
+template <class D>
+AHL_DEV void mfma_chunk(const char* ldsA, const char* ldsB, int wm, int wn, int lane,
+                        f32x16 (&acc)[2][2]) {
+  const int r = lane & 31, h = lane >> 5;
+  const char* pa = ldsA + (wm * 64 + r) * kLdsStride + h * 16;
+  const char* pb = ldsB + (wn * 64 + r) * kLdsStride + h * 16;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    u32x4 a0 = *(const u32x4*)(pa + s * 32);
+    u32x4 a1 = *(const u32x4*)(pa + 32 * kLdsStride + s * 32);
+    u32x4 b0 = *(const u32x4*)(pb + s * 32);
+    u32x4 b1 = *(const u32x4*)(pb + 32 * kLdsStride + s * 32);
+    Mma<D>::run(a0, b0, acc[0][0]);
+    Mma<D>::run(a0, b1, acc[0][1]);
+    Mma<D>::run(a1, b0, acc[1][0]);
+    Mma<D>::run(a1, b1, acc[1][1]);
+  }
+}
+
+// ---- chunk staging ---------------------------------------------------------------------------
+// A thread owns 4 of the 1024 16-byte vectors of a 128 x 128-byte chunk: vector j lives in
+// chunk row (tid / 8 + 32 * j), byte column 16 * (tid % 8).
+struct VecPos {
+  int row0;  // tid / 8
+  int cv;    // tid % 8
+};
+AHL_DEV VecPos vec_pos(int tid) { return VecPos{tid >> 3, tid & 7}; }
+
+// Loads the raw vectors of one chunk: rows [row_base, row_base+128) of `p` (ld elements),
+// columns [kc, kc + chunkK) clipped to k_end; rows >= n_rows and columns >= k_end read as 0.
+template <class D, bool VEC>
+AHL_DEV void load_chunk(const void* p, int64_t ld, int64_t row_base, int64_t n_rows, int32_t kc,
+                        int32_t k_end, const VecPos& vp, u32x4 (&raw)[4]) {
+  constexpr int E = D::EPV;
+  const typename D::elem* base = (const typename D::elem*)p;
+  const int32_t k = kc + vp.cv * E;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t row = row_base + vp.row0 + 32 * j;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (row < n_rows) {
+      const typename D::elem* q = base + row * ld + k;
+      if (VEC) {
+        if (k < k_end) v = ld16(q);
+      } else {
+        float e[E];
+#pragma unroll
+        for (int i = 0; i < E; ++i) e[i] = (k + i < k_end) ? D::load(q, i) : 0.0f;
+        v = D::pack(e);
+      }
+    }
+    raw[j] = v;
+  }
+}
+
+AHL_DEV void store_chunk(char* lds, const VecPos& vp, const u32x4 (&v)[4]) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    *(u32x4*)(lds + (vp.row0 + 32 * j) * kLdsStride + vp.cv * 16) = v[j];
+}
+
+// XCD-aware block order: the hardware deals consecutive workgroup ids round-robin to the 8
+// XCDs; this maps them back so that each XCD (own L2) works on a contiguous range of tiles.
+AHL_DEV int64_t xcd_remap(int64_t bid, int64_t nb) {
+  if ((nb & 7) != 0) return bid;
+  return (bid & 7) * (nb >> 3) + (bid >> 3);
+}
+
+// =============================================================================================
+// Forward
+// =============================================================================================
+struct FwdArgs {
+  const void* x; int64_t ldx;
+  const void* w; int64_t ldw;
+  const void* bias;
+  void* y; int64_t ldy;
+  uint8_t* keep;
+  const void* ir;
+  const void* wmax;
+  const float* tile_max;
+  int64_t M, N;
+  Tiling tl;
+  float inp_res, out_res, out_bound;
+  float noise_scale;  // out_noise / sqrt(n_tiles) as float, 0 when the noise is off
+  int32_t noise_per_channel, bound_per_channel, skip_rounding;
+  int32_t dac_on, adc_on, bound_on, clamp_on, noise_on;
+  uint64_t seed, offset;
+};
+
+template <class D, bool VEC, int IRMODE>
+__global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* ldsA = lds;
+  char* ldsB = lds + kChunkLds;
+  float* rowir = (float*)(lds + 2 * kChunkLds);  // [2][128] per-row input range (dynamic mode)
+
+  constexpr int CK = ChunkK<D>::value;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const VecPos vp = vec_pos(tid);
+
+  const int64_t nbn = cdiv_dev(a.N, kBN);
+  const int64_t logical = xcd_remap(blockIdx.x, gridDim.x);
+  const int64_t m0 = (logical / nbn) * kBM, n0 = (logical % nbn) * kBN;
+  const int T = a.tl.n_tiles;
+
+  f32x16 total[2][2], acc[2][2];
+  uint32_t keepbits[2][2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) { total[i][j][v] = 0.0f; acc[i][j][v] = 0.0f; }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) keepbits[i][j][v] = 0u;
+    }
+
+  // --- state of the chunk being loaded ---
+  int ld_t = 0;
+  int32_t ld_kc = a.tl.start(0), ld_kend = a.tl.start(1);
+  u32x4 rawA[4], rawB[4];
+  load_chunk<D, VEC>(a.x, a.ldx, m0, a.M, ld_kc, ld_kend, vp, rawA);
+  load_chunk<D, VEC>(a.w, a.ldw, n0, a.N, ld_kc, ld_kend, vp, rawB);
+  bool have = true;
+
+  while (have) {
+    const int cur_t = ld_t;
+    const bool cur_last = (ld_kc + CK >= ld_kend);  // last chunk of its K-tile
+    const bool cur_first = (ld_kc == a.tl.start(cur_t));
+
+    // ---- A prologue: clamp + DAC in registers, then stage to LDS ----
+    u32x4 qa[4];
+    if (IRMODE == AHL_IR_NONE) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) qa[j] = rawA[j];
+    } else {
+      Dac dac;
+      if (IRMODE == AHL_IR_STATIC) dac = make_dac<D>(D::load(a.ir, cur_t), a.inp_res);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (IRMODE == AHL_IR_DYNAMIC) {
+          const int64_t m = m0 + vp.row0 + 32 * j;
+          const float irm = m < a.M ? D::load(a.ir, (int64_t)cur_t * a.M + m) : 0.0f;
+          dac = make_dac<D>(irm, a.inp_res);
+        }
+        float e[D::EPV];
+        D::unpack(rawA[j], e);
+        if (a.dac_on) {
+#pragma unroll
+          for (int i = 0; i < D::EPV; ++i)
+            e[i] = dac_apply<D, IRMODE == AHL_IR_STATIC, true>(e[i], dac, a.skip_rounding != 0);
+        } else if (IRMODE == AHL_IR_STATIC) {
+#pragma unroll
+          for (int i = 0; i < D::EPV; ++i)
+            e[i] = dac_apply<D, true, false>(e[i], dac, false);
+        }
+        qa[j] = D::pack(e);
+      }
+    }
+    __syncthreads();
+    store_chunk(ldsA, vp, qa);
+    store_chunk(ldsB, vp, rawB);
+    if (IRMODE == AHL_IR_DYNAMIC && cur_first && tid < 128) {
+      const int64_t m = m0 + tid;
+      rowir[(cur_t & 1) * 128 + tid] = m < a.M ? D::load(a.ir, (int64_t)cur_t * a.M + m) : 0.0f;
+    }
+    __syncthreads();
+
+    // ---- issue the next chunk's global loads ----
+    ld_kc += CK;
+    if (ld_kc >= ld_kend) {
+      ld_t += 1;
+      if (ld_t < T) { ld_kc = a.tl.start(ld_t); ld_kend = a.tl.start(ld_t + 1); }
+    }
+    have = ld_t < T;
+    if (have) {
+      load_chunk<D, VEC>(a.x, a.ldx, m0, a.M, ld_kc, ld_kend, vp, rawA);
+      load_chunk<D, VEC>(a.w, a.ldw, n0, a.N, ld_kc, ld_kend, vp, rawB);
+    }
+
+    mfma_chunk<D>(ldsA, ldsB, wm, wn, lane, acc);
+
+    // ---- per-K-tile epilogue: noise, ADC, clamp, accumulate in dtype ----
+    if (cur_last) {
+      const int t = cur_t;
+      const float ir_t = IRMODE == AHL_IR_STATIC ? D::load(a.ir, t) : 0.0f;
+      const float tmax = (a.noise_on || a.bound_on) ? a.tile_max[t] : 0.0f;
+      const int h = lane >> 5;
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) {
+        const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
+        const bool nvalid = n < a.N;
+        float wch = 0.0f;
+        if ((a.noise_on || a.bound_on) && nvalid) wch = D::load(a.wmax, (int64_t)t * a.N + n);
+        const float wr = a.noise_per_channel ? wch : tmax;
+        const float wb = a.bound_per_channel ? wch : tmax;
+        // per-column constants of the static mode
+        float nscale = 0.0f, B = 0.0f, r = 1.0f, rc = 1.0f, rcp = 1.0f;
+        if (IRMODE == AHL_IR_STATIC) {
+          if (a.noise_on) nscale = D::rd(wr * D::rd(a.noise_scale * ir_t));
+          if (a.bound_on) {
+            B = D::rd(D::rd(ir_t * a.out_bound) * wb);
+            if (a.adc_on) {
+              r = quant_step<D>(B, a.out_res);
+              rc = fmaxf(r, kTinyF32);
+              rcp = __fdiv_rn(1.0f, rc);
+            }
+          }
+        }
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi) {
+          const int rbase = wm * 64 + bi * 32 + 4 * h;  // block-local row of v = 0
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            float xi[4] = {0.f, 0.f, 0.f, 0.f};
+            if (a.noise_on) {
+              const uint64_t mg = (uint64_t)(m0 + rbase + 8 * g) >> 2;
+              normal4(a.seed, a.offset, (uint32_t)t, mg * (uint64_t)a.N + (uint64_t)n, xi);
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              const int v = 4 * g + c;
+              const int rl = rbase + 8 * g + c;
+              float y = D::rd(acc[bi][bj][v]);
+              acc[bi][bj][v] = 0.0f;
+              if (IRMODE == AHL_IR_DYNAMIC && (a.noise_on || a.bound_on)) {
+                const float irm = rowir[(t & 1) * 128 + rl];
+                if (a.noise_on) nscale = D::rd(wr * D::rd(a.noise_scale * irm));
+                if (a.bound_on) {
+                  B = D::rd(D::rd(irm * a.out_bound) * wb);
+                  if (a.adc_on) {
+                    r = quant_step<D>(B, a.out_res);
+                    rc = fmaxf(r, kTinyF32);
+                    rcp = __fdiv_rn(1.0f, rc);
+                  }
+                }
+              }
+              if (a.noise_on) y = D::rd(y + D::rd(nscale * D::rd(xi[c])));
+              if (a.bound_on) {
+                if (a.adc_on) {
+                  float q = D::rd(D::div(y, rc, rcp));
+                  if (!a.skip_rounding) q = rintf(q);
+                  y = D::rd(q * r);
+                }
+                if (a.clamp_on) {
+                  const bool kp = (y >= -B) && (y <= B);
+                  keepbits[bi][bj][g] |= (kp ? 1u : 0u) << (8 * c + (t & 7));
+                  y = fminf(fmaxf(y, -B), B);
+                }
+              }
+              total[bi][bj][v] = D::rd(total[bi][bj][v] + y);
+            }
+          }
+          // flush one plane of the clamp mask every 8 tiles
+          if (a.keep != nullptr && a.clamp_on && ((t & 7) == 7 || t == T - 1)) {
+            uint8_t* plane = a.keep + (int64_t)(t >> 3) * a.M * a.N;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+#pragma unroll
+              for (int c = 0; c < 4; ++c) {
+                const int64_t m = m0 + rbase + 8 * g + c;
+                if (m < a.M && nvalid) plane[m * a.N + n] = (uint8_t)(keepbits[bi][bj][g] >> (8 * c));
+              }
+              keepbits[bi][bj][g] = 0u;
+            }
+          }
+        }
+      }
+    }
+  }
+
+  // ---- store: y = total (+ bias) ----
+  {
+    const int h = lane >> 5;
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+      const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
+      if (n >= a.N) continue;
+      const float b = a.bias ? D::load(a.bias, n) : 0.0f;
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int64_t m = m0 + wm * 64 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+          if (m < a.M) {
+            float o = total[bi][bj][v];
+            if (a.bias) o = D::rd(o + b);
+            D::store(a.y, m * a.ldy + n, o);
+          }
+        }
+    }
+  }
+}
+
+// =============================================================================================
+// Input gradient (+ input-range gradient partials)
+// =============================================================================================
+struct DxArgs {
+  const void* g; int64_t ldg;
+  const uint8_t* keep;
+  const void* wt;  // w_eff_t [K, N]
+  const void* x; int64_t ldx;
+  const void* ir;
+  void* dx; int64_t lddx;
+  float* partial;  // [m_blocks * k_blocks][4]
+  int64_t M, N, K;
+  Tiling tl;
+  int32_t kb_big, kb_small;  // 128-wide column blocks per tile of size base+1 / base
+};
+
+// Decodes a column-block index into (tile, first column, end column).
+AHL_DEV void decode_kblock(const Tiling& tl, int32_t kb_big, int32_t kb_small, int32_t idx, int& t,
+                           int32_t& c0, int32_t& c1) {
+  const int32_t big_total = tl.extra * kb_big;
+  int32_t within;
+  if (idx < big_total) { t = idx / kb_big; within = idx % kb_big; }
+  else { t = tl.extra + (idx - big_total) / kb_small; within = (idx - big_total) % kb_small; }
+  c0 = tl.start(t) + within * kBN;
+  c1 = tl.start(t + 1);
+}
+
+// Applies the clamp mask of tile t to a vector of gradient values.
+template <class D, bool VEC>
+AHL_DEV u32x4 mask_vec(const u32x4& raw, const uint8_t* keep_plane, int64_t ld, int64_t row,
+                       int64_t n_rows, int32_t k, int32_t k_end, int bit) {
+  constexpr int E = D::EPV;
+  if (row >= n_rows || k >= k_end) return raw;
+  float e[E];
+  D::unpack(raw, e);
+  const uint8_t* q = keep_plane + row * ld + k;
+  if (VEC) {
+    uint32_t w[2];
+    w[0] = *(const uint32_t*)q;
+    w[1] = E == 8 ? *(const uint32_t*)(q + 4) : 0u;
+#pragma unroll
+    for (int i = 0; i < E; ++i) if (!((w[i >> 2] >> (8 * (i & 3) + bit)) & 1u)) e[i] = 0.0f;
+  } else {
+#pragma unroll
+    for (int i = 0; i < E; ++i) if (k + i < k_end && !((q[i] >> bit) & 1)) e[i] = 0.0f;
+  }
+  return D::pack(e);
+}
+
+template <class D, bool VEC, int IRMODE>
+__global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* ldsA = lds;
+  char* ldsB = lds + kChunkLds;
+  __shared__ float red[4][3];
+
+  constexpr int CK = ChunkK<D>::value;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const VecPos vp = vec_pos(tid);
+
+  const int32_t nkb = a.tl.extra * a.kb_big + (a.tl.n_tiles - a.tl.extra) * a.kb_small;
+  const int64_t logical = xcd_remap(blockIdx.x, gridDim.x);
+  const int64_t m0 = (logical / nkb) * kBM;
+  int t; int32_t c0, c1;
+  decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
+  const uint8_t* plane = a.keep ? a.keep + (int64_t)(t >> 3) * a.M * a.N : nullptr;
+  const int bit = t & 7;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  u32x4 rawA[4], rawB[4];
+  int32_t kc = 0;
+  const int32_t kend = (int32_t)a.N;
+  load_chunk<D, VEC>(a.g, a.ldg, m0, a.M, kc, kend, vp, rawA);
+  load_chunk<D, VEC>(a.wt, a.N, c0, c1, kc, kend, vp, rawB);
+  while (true) {
+    u32x4 qa[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      qa[j] = plane ? mask_vec<D, VEC>(rawA[j], plane, a.N, m0 + vp.row0 + 32 * j, a.M,
+                                       kc + vp.cv * D::EPV, kend, bit)
+                    : rawA[j];
+    __syncthreads();
+    store_chunk(ldsA, vp, qa);
+    store_chunk(ldsB, vp, rawB);
+    __syncthreads();
+    kc += CK;
+    const bool more = kc < kend;
+    if (more) {
+      load_chunk<D, VEC>(a.g, a.ldg, m0, a.M, kc, kend, vp, rawA);
+      load_chunk<D, VEC>(a.wt, a.N, c0, c1, kc, kend, vp, rawB);
+    }
+    mfma_chunk<D>(ldsA, ldsB, wm, wn, lane, acc);
+    if (!more) break;
+  }
+
+  // ---- epilogue: round, input-range gradient partial sums, straight-through clamp mask ----
+  const float ir_t = IRMODE == AHL_IR_STATIC ? D::load(a.ir, t) : 0.0f;
+  float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
+  const int h = lane >> 5;
+#pragma unroll
+  for (int bj = 0; bj < 2; ++bj) {
+    const int64_t k = (int64_t)c0 + wn * 64 + bj * 32 + (lane & 31);
+    if (k >= c1) continue;
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t m = m0 + wm * 64 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (m >= a.M) continue;
+        float d = D::rd(acc[bi][bj][v]);
+        if (IRMODE == AHL_IR_STATIC) {
+          const float xv = D::load(a.x, m * a.ldx + k);
+          const bool up = xv >= ir_t, lo = xv <= -ir_t;
+          if (up) s_up += fminf(d, 0.0f);
+          if (lo) s_lo += fmaxf(d, 0.0f);
+          if (up || lo) cnt += 1.0f;
+          if (fabsf(xv) > ir_t) d = 0.0f;
+        }
+        D::store(a.dx, m * a.lddx + k, d);
+      }
+  }
+  if (IRMODE == AHL_IR_STATIC) {
+    s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
+    if (lane == 0) { red[wave][0] = s_up; red[wave][1] = s_lo; red[wave][2] = cnt; }
+    __syncthreads();
+    if (tid == 0) {
+      float* p = a.partial + logical * 4;
+      p[0] = (red[0][0] + red[1][0]) + (red[2][0] + red[3][0]);
+      p[1] = (red[0][1] + red[1][1]) + (red[2][1] + red[3][1]);
+      p[2] = (red[0][2] + red[1][2]) + (red[2][2] + red[3][2]);
+      p[3] = 0.0f;
+    }
+  }
+}
+
+// ir_grad[t] from the per-block partials (reference torch_utils/torch_linear.py:92-106).
+template <class D>
+__global__ __launch_bounds__(64) void k_ir_grad_finalize(const float* __restrict__ partial,
+                                                         int64_t m_blocks, int32_t nkb,
+                                                         int32_t kb_big, int32_t kb_small,
+                                                         Tiling tl, int64_t M, const void* ir,
+                                                         void* ir_grad, float decay, float min_pct) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const int32_t first = t < tl.extra ? t * kb_big : tl.extra * kb_big + (t - tl.extra) * kb_small;
+  const int32_t count = t < tl.extra ? kb_big : kb_small;
+  double s_up = 0.0, s_lo = 0.0, cnt = 0.0;
+  const int64_t total = m_blocks * count;
+  for (int64_t i = lane; i < total; i += 64) {
+    const int64_t mb = i / count, kb = first + i % count;
+    const float* p = partial + (mb * nkb + kb) * 4;
+    s_up += (double)p[0]; s_lo += (double)p[1]; cnt += (double)p[2];
+  }
+  s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
+  if (lane == 0) {
+    const float irv = D::load(ir, t);
+    float gr = D::rd(0.0f + D::rd((float)s_up));
+    gr = D::rd(gr - D::rd((float)s_lo));
+    gr = D::rd(gr * irv);
+    if (decay > 0.0f) {
+      const float numel = (float)((double)M * (double)tl.size(t));
+      const float pct = 1.0f - __fdiv_rn((float)cnt, numel);
+      const float add = pct > min_pct ? D::rd(decay * irv) : 0.0f;
+      gr = D::rd(gr + add);
+    }
+    D::store(ir_grad, t, gr);
+  }
+}
+
+// =============================================================================================
+// Weight gradient: dw[n, k] = sum_m gT[n, m] * xqT[k, m], gT masked by keepT bit t
+// =============================================================================================
+struct DwArgs {
+  const void* gt;       // [N, M]
+  const uint8_t* keept; // [P, N, M] or null
+  const void* xqt;      // [K, M]
+  void* dw; int64_t lddw;
+  int64_t M, N, K;
+  Tiling tl;
+  int32_t kb_big, kb_small;
+};
+
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_linear_bwd_dw(DwArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* ldsA = lds;
+  char* ldsB = lds + kChunkLds;
+  constexpr int CK = ChunkK<D>::value;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const VecPos vp = vec_pos(tid);
+
+  const int32_t nkb = a.tl.extra * a.kb_big + (a.tl.n_tiles - a.tl.extra) * a.kb_small;
+  const int64_t logical = xcd_remap(blockIdx.x, gridDim.x);
+  const int64_t n0 = (logical / nkb) * kBM;
+  int t; int32_t c0, c1;
+  decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
+  const uint8_t* plane = a.keept ? a.keept + (int64_t)(t >> 3) * a.N * a.M : nullptr;
+  const int bit = t & 7;
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  u32x4 rawA[4], rawB[4];
+  int32_t kc = 0;
+  const int32_t kend = (int32_t)a.M;
+  load_chunk<D, VEC>(a.gt, a.M, n0, a.N, kc, kend, vp, rawA);
+  load_chunk<D, VEC>(a.xqt, a.M, c0, c1, kc, kend, vp, rawB);
+  while (true) {
+    u32x4 qa[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      qa[j] = plane ? mask_vec<D, VEC>(rawA[j], plane, a.M, n0 + vp.row0 + 32 * j, a.N,
+                                       kc + vp.cv * D::EPV, kend, bit)
+                    : rawA[j];
+    __syncthreads();
+    store_chunk(ldsA, vp, qa);
+    store_chunk(ldsB, vp, rawB);
+    __syncthreads();
+    kc += CK;
+    const bool more = kc < kend;
+    if (more) {
+      load_chunk<D, VEC>(a.gt, a.M, n0, a.N, kc, kend, vp, rawA);
+      load_chunk<D, VEC>(a.xqt, a.M, c0, c1, kc, kend, vp, rawB);
+    }
+    mfma_chunk<D>(ldsA, ldsB, wm, wn, lane, acc);
+    if (!more) break;
+  }
+  const int h = lane >> 5;
+#pragma unroll
+  for (int bj = 0; bj < 2; ++bj) {
+    const int64_t k = (int64_t)c0 + wn * 64 + bj * 32 + (lane & 31);
+    if (k >= c1) continue;
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t n = n0 + wm * 64 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (n < a.N) D::store(a.dw, n * a.lddw + k, D::rd(acc[bi][bj][v]));
+      }
+  }
+}
+
+// =============================================================================================
+// Transposes feeding the weight gradient
+// =============================================================================================
+// out[c, r] = f(in[r, c]); 64 x 64 tiles through LDS; E = element type.
+template <class E>
+__global__ __launch_bounds__(256) void k_transpose(const E* __restrict__ in, int64_t R, int64_t C,
+                                                   int64_t ld_in, E* __restrict__ out,
+                                                   int64_t ld_out) {
+  __shared__ E tile[64][64 + 4 / sizeof(E) + 1];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const E* inp = in + (int64_t)blockIdx.z * R * ld_in;
+  E* outp = out + (int64_t)blockIdx.z * C * ld_out;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t r = r0 + i, c = c0 + tx;
+    if (r < R && c < C) tile[i][tx] = inp[r * ld_in + c];
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t c = c0 + i, r = r0 + tx;
+    if (r < R && c < C) outp[c * ld_out + r] = tile[tx][i];
+  }
+}
+
+// xqt[k, m] = DAC(clamp(x[m, k])) with the input range of k's tile.
+template <class D, int IRMODE>
+__global__ __launch_bounds__(256) void k_dac_transpose(const void* __restrict__ x, int64_t M,
+                                                       int64_t K, int64_t ldx, const void* ir,
+                                                       Tiling tl, float inp_res, int32_t dac_on,
+                                                       int32_t skip_rounding,
+                                                       void* __restrict__ out) {
+  __shared__ typename D::elem tile[64][64 + 4];
+  const int64_t r0 = (int64_t)blockIdx.y * 64, c0 = (int64_t)blockIdx.x * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int64_t k = c0 + tx;
+  const int t = k < K ? tl.tile_of((int32_t)k) : 0;
+  Dac dac;
+  if (IRMODE == AHL_IR_STATIC) dac = make_dac<D>(D::load(ir, t), inp_res);
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t m = r0 + i;
+    if (m < M && k < K) {
+      float v = D::load(x, m * ldx + k);
+      if (IRMODE == AHL_IR_DYNAMIC) dac = make_dac<D>(D::load(ir, (int64_t)t * M + m), inp_res);
+      if (IRMODE != AHL_IR_NONE) {
+        if (dac_on) v = dac_apply<D, IRMODE == AHL_IR_STATIC, true>(v, dac, skip_rounding != 0);
+        else if (IRMODE == AHL_IR_STATIC) v = dac_apply<D, true, false>(v, dac, false);
+      }
+      tile[i][tx] = D::to_elem(v);
+    }
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t kk = c0 + i, m = r0 + tx;
+    if (m < M && kk < K) ((typename D::elem*)out)[kk * M + m] = tile[tx][i];
+  }
+}
+
+}  // namespace ahl
+
+using namespace ahl;
+
+static constexpr int kGemmLds = 2 * kChunkLds + 2 * 128 * (int)sizeof(float);
+
+static bool cfg_ok(const AhlLinearCfg* c) {
+  if (!c) return false;
+  if (c->dtype != AHL_F32 && c->dtype != AHL_BF16) return false;
+  if (c->ir_mode < 0 || c->ir_mode > 2) return false;
+  return true;
+}
+
+template <class D>
+static bool tiles_vec_ok(const Tiling& tl) {
+  return tl.extra == 0 ? (tl.base % D::EPV == 0) : false;
+}
+
+template <class D>
+static void launch_fwd(const FwdArgs& a, int ir_mode, dim3 grid, hipStream_t s) {
+  const bool vec = aligned16(a.x) && aligned16(a.w) && a.ldx % D::EPV == 0 && a.ldw % D::EPV == 0 &&
+                   tiles_vec_ok<D>(a.tl);
+  const dim3 block(256);
+  if (vec) {
+    if (ir_mode == AHL_IR_NONE) hipLaunchKernelGGL((k_linear_fwd<D, true, 0>), grid, block, kGemmLds, s, a);
+    else if (ir_mode == AHL_IR_STATIC) hipLaunchKernelGGL((k_linear_fwd<D, true, 1>), grid, block, kGemmLds, s, a);
+    else hipLaunchKernelGGL((k_linear_fwd<D, true, 2>), grid, block, kGemmLds, s, a);
+  } else {
+    if (ir_mode == AHL_IR_NONE) hipLaunchKernelGGL((k_linear_fwd<D, false, 0>), grid, block, kGemmLds, s, a);
+    else if (ir_mode == AHL_IR_STATIC) hipLaunchKernelGGL((k_linear_fwd<D, false, 1>), grid, block, kGemmLds, s, a);
+    else hipLaunchKernelGGL((k_linear_fwd<D, false, 2>), grid, block, kGemmLds, s, a);
+  }
+}
+
+template <class D>
+static void launch_dx(const DxArgs& a, bool is_static, dim3 grid, hipStream_t s) {
+  const bool vec = aligned16(a.g) && aligned16(a.wt) && a.ldg % D::EPV == 0 && a.N % D::EPV == 0 &&
+                   (!a.keep || (((uintptr_t)a.keep) & 7u) == 0);
+  const dim3 block(256);
+  if (vec) {
+    if (is_static) hipLaunchKernelGGL((k_linear_bwd_dx<D, true, 1>), grid, block, kGemmLds, s, a);
+    else hipLaunchKernelGGL((k_linear_bwd_dx<D, true, 0>), grid, block, kGemmLds, s, a);
+  } else {
+    if (is_static) hipLaunchKernelGGL((k_linear_bwd_dx<D, false, 1>), grid, block, kGemmLds, s, a);
+    else hipLaunchKernelGGL((k_linear_bwd_dx<D, false, 0>), grid, block, kGemmLds, s, a);
+  }
+}
+
+extern "C" {
+
+int ahl_linear_fwd(const void* x, int64_t ldx, const void* w_eff, int64_t ldw, const void* bias,
+                   void* y, int64_t ldy, uint8_t* keep, const void* ir, const void* wmax,
+                   const float* tile_max, int64_t M, int64_t K, int64_t N,
+                   const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
+                   void* stream) {
+  if (!cfg_ok(cfg) || !x || !w_eff || !y || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
+  if (ldx < K || ldw < K || ldy < N) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  FwdArgs a;
+  a.x = x; a.ldx = ldx; a.w = w_eff; a.ldw = ldw; a.bias = bias; a.y = y; a.ldy = ldy;
+  a.keep = keep; a.ir = ir; a.wmax = wmax; a.tile_max = tile_max; a.M = M; a.N = N; a.tl = tl;
+  a.inp_res = cfg->inp_res; a.out_res = cfg->out_res; a.out_bound = cfg->out_bound;
+  a.noise_on = (cfg->training && cfg->out_noise > 0.0f) ? 1 : 0;
+  a.noise_scale = a.noise_on ? (float)((double)cfg->out_noise / sqrt((double)n_tiles)) : 0.0f;
+  a.noise_per_channel = cfg->out_noise_per_channel; a.bound_per_channel = cfg->bound_per_channel;
+  a.skip_rounding = cfg->skip_rounding;
+  a.dac_on = cfg->inp_res > 0.0f ? 1 : 0;
+  a.adc_on = cfg->out_res > 0.0f ? 1 : 0;
+  a.clamp_on = cfg->out_bound > 0.0f ? 1 : 0;
+  a.bound_on = (a.adc_on || a.clamp_on) ? 1 : 0;
+  a.seed = cfg->seed; a.offset = cfg->offset;
+  if (cfg->ir_mode == AHL_IR_NONE && (a.dac_on || a.bound_on || a.noise_on)) return AHL_ERR_ARG;
+  if (cfg->ir_mode != AHL_IR_NONE && !ir) return AHL_ERR_ARG;
+  if ((a.noise_on || a.bound_on) && (!wmax || !tile_max)) return AHL_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t nb = cdiv(M, kBM) * cdiv(N, kBN);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
+  const dim3 grid((unsigned)nb);
+  if (cfg->dtype == AHL_F32) launch_fwd<F32>(a, cfg->ir_mode, grid, s);
+  else launch_fwd<BF16>(a, cfg->ir_mode, grid, s);
+  return check_launch("ahl_linear_fwd");
+}
+
+static void kblocks(const Tiling& tl, int32_t* kb_big, int32_t* kb_small) {
+  *kb_big = (int32_t)cdiv(tl.base + 1, kBN);
+  *kb_small = (int32_t)cdiv(tl.base, kBN);
+}
+
+int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int32_t n_tiles) {
+  if (n_tiles <= 0 || K <= 0 || M <= 0) return 0;
+  Tiling tl{n_tiles, (int32_t)(K / n_tiles), (int32_t)(K % n_tiles)};
+  int32_t kb, ks;
+  kblocks(tl, &kb, &ks);
+  const int64_t nkb = (int64_t)tl.extra * kb + (int64_t)(n_tiles - tl.extra) * ks;
+  return cdiv(M, kBM) * nkb * 4 * (int64_t)sizeof(float);
+}
+
+int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const void* w_eff_t,
+                      const void* x, int64_t ldx, const void* ir, void* dx, int64_t lddx,
+                      void* ir_grad, int64_t M, int64_t K, int64_t N,
+                      const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
+                      void* ws, void* stream) {
+  if (!cfg_ok(cfg) || !g || !w_eff_t || !dx || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
+  if (ldg < N || lddx < K) return AHL_ERR_ARG;
+  const bool is_static = cfg->ir_mode == AHL_IR_STATIC;
+  if (is_static && (!x || !ir || !ir_grad || !ws || ldx < K)) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  DxArgs a;
+  a.g = g; a.ldg = ldg; a.keep = keep; a.wt = w_eff_t; a.x = x; a.ldx = ldx; a.ir = ir;
+  a.dx = dx; a.lddx = lddx; a.partial = (float*)ws; a.M = M; a.N = N; a.K = K; a.tl = tl;
+  kblocks(tl, &a.kb_big, &a.kb_small);
+  const int64_t nkb = (int64_t)tl.extra * a.kb_big + (int64_t)(n_tiles - tl.extra) * a.kb_small;
+  const int64_t mb = cdiv(M, kBM);
+  if (mb * nkb > 0x7fffffff) return AHL_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)(mb * nkb));
+  if (cfg->dtype == AHL_F32) launch_dx<F32>(a, is_static, grid, s);
+  else launch_dx<BF16>(a, is_static, grid, s);
+  if (is_static) {
+    AHL_DISPATCH_DTYPE(cfg->dtype, {
+      hipLaunchKernelGGL((k_ir_grad_finalize<D>), dim3(n_tiles), dim3(64), 0, s, (const float*)ws, mb,
+                         (int32_t)nkb, a.kb_big, a.kb_small, tl, M, ir, ir_grad, cfg->ir_decay,
+                         cfg->ir_input_min_percentage);
+    });
+  }
+  return check_launch("ahl_linear_bwd_dx");
+}
+
+static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
+                                   int32_t has_keep) {
+  const int64_t es = dtype == AHL_BF16 ? 2 : 4;
+  int64_t b = align256(N * M * es) + align256(K * M * es);
+  if (has_keep) b += align256((int64_t)((n_tiles + 7) / 8) * N * M);
+  return b;
+}
+
+int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const void* x, int64_t ldx,
+                      const void* ir, void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
+                      const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
+                      void* ws, void* stream) {
+  if (!cfg_ok(cfg) || !g || !x || !dw || !ws || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
+  if (ldg < N || ldx < K || lddw < K) return AHL_ERR_ARG;
+  if (cfg->ir_mode != AHL_IR_NONE && !ir) return AHL_ERR_ARG;
+  if (!aligned16(ws)) return AHL_ERR_WORKSPACE;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
+  const int planes = (n_tiles + 7) / 8;
+  DwArgs a;
+  a.M = M; a.N = N; a.K = K; a.tl = tl; a.dw = dw; a.lddw = lddw;
+  kblocks(tl, &a.kb_big, &a.kb_small);
+  const int64_t nkb = (int64_t)tl.extra * a.kb_big + (int64_t)(n_tiles - tl.extra) * a.kb_small;
+  const int64_t nbn = cdiv(N, kBM);
+  if (nbn * nkb > 0x7fffffff) return AHL_ERR_ARG;
+  const dim3 tgrid_g((unsigned)cdiv(N, 64), (unsigned)cdiv(M, 64), 1);
+  const dim3 tgrid_x((unsigned)cdiv(K, 64), (unsigned)cdiv(M, 64), 1);
+  AHL_DISPATCH_DTYPE(cfg->dtype, {
+    typedef typename D::elem E;
+    char* p = (char*)ws;
+    E* gt = (E*)p; p += align256(N * M * (int64_t)sizeof(E));
+    E* xqt = (E*)p; p += align256(K * M * (int64_t)sizeof(E));
+    uint8_t* keept = keep ? (uint8_t*)p : nullptr;
+    hipLaunchKernelGGL((k_transpose<E>), tgrid_g, dim3(256), 0, s, (const E*)g, M, N, ldg, gt, M);
+    if (keep) {
+      const dim3 tgrid_k((unsigned)cdiv(N, 64), (unsigned)cdiv(M, 64), (unsigned)planes);
+      hipLaunchKernelGGL((k_transpose<uint8_t>), tgrid_k, dim3(256), 0, s, keep, M, N, N, keept, M);
+    }
+    if (cfg->ir_mode == AHL_IR_NONE)
+      hipLaunchKernelGGL((k_dac_transpose<D, 0>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
+    else if (cfg->ir_mode == AHL_IR_STATIC)
+      hipLaunchKernelGGL((k_dac_transpose<D, 1>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
+    else
+      hipLaunchKernelGGL((k_dac_transpose<D, 2>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
+    a.gt = gt; a.keept = keept; a.xqt = xqt;
+    const bool vec = M % D::EPV == 0;
+    const dim3 grid((unsigned)(nbn * nkb)), block(256);
+    if (vec) hipLaunchKernelGGL((k_linear_bwd_dw<D, true>), grid, block, kGemmLds, s, a);
+    else hipLaunchKernelGGL((k_linear_bwd_dw<D, false>), grid, block, kGemmLds, s, a);
+  });
+  return check_launch("ahl_linear_bwd_dw");
+}
+
+}  // extern "C"

@@ -1,0 +1,393 @@
+// Memory-bound kernels of the AnalogLinear path: per-tile abs-max and std reductions, running
+// abs-max (calibration), input-range initialisation, weight clipping, column sums, transposes.
+// All are wave64 shuffle reductions over coalesced 16-byte row reads; none uses LDS for data
+// except the transposes. Reductions are two-stage and deterministic (no float atomics).
+#include "ahl_host.h"
+#include "ahl_reduce_kernels.h"
+
+namespace ahl {
+
+static thread_local char g_err[256] = {0};
+int record_hip_error(hipError_t e, const char* where) {
+  snprintf(g_err, sizeof(g_err), "%s: %s", where, hipGetErrorString(e));
+  return AHL_ERR_LAUNCH;
+}
+
+// ------------------------------------------------------------------------------------------
+// Per-tile sum and sum of squares over a block of kStdRows rows, in double.
+static constexpr int kStdRows = 16;
+
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_sliced_sums(const void* __restrict__ x, int64_t rows,
+                                                     int64_t ld, Tiling tl,
+                                                     double* __restrict__ partial) {
+  __shared__ double sh[4][2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r0 = (int64_t)blockIdx.x * kStdRows;
+  for (int32_t t = 0; t < tl.n_tiles; ++t) {
+    double s = 0.0, s2 = 0.0;
+    for (int i = wave; i < kStdRows; i += 4) {
+      const int64_t r = r0 + i;
+      if (r >= rows) break;
+      const typename D::elem* row = (const typename D::elem*)x + r * ld;
+      wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
+        s += (double)v;
+        s2 += (double)v * (double)v;
+      });
+    }
+    s = wave_sum(s);
+    s2 = wave_sum(s2);
+    __syncthreads();
+    if (lane == 0) { sh[wave][0] = s; sh[wave][1] = s2; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double* p = partial + ((int64_t)blockIdx.x * tl.n_tiles + t) * 2;
+      p[0] = (sh[0][0] + sh[1][0]) + (sh[2][0] + sh[3][0]);
+      p[1] = (sh[0][1] + sh[1][1]) + (sh[2][1] + sh[3][1]);
+    }
+  }
+}
+
+// out[t] = sqrt((S2 - S^2/n) / (n - 1)); one wave per tile, fixed summation order.
+__global__ __launch_bounds__(64) void k_std_finalize(const double* __restrict__ partial,
+                                                     int64_t n_blocks, int64_t rows, Tiling tl,
+                                                     float* __restrict__ out) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  double s = 0.0, s2 = 0.0;
+  for (int64_t b = lane; b < n_blocks; b += 64) {
+    s += partial[(b * tl.n_tiles + t) * 2];
+    s2 += partial[(b * tl.n_tiles + t) * 2 + 1];
+  }
+  s = wave_sum(s);
+  s2 = wave_sum(s2);
+  if (lane == 0) {
+    const double n = (double)rows * (double)tl.size(t);
+    double var = (s2 - s * s / n) / (n - 1.0);  // n == 1 gives 0/0 = nan like torch
+    if (var < 0.0) var = 0.0;
+    out[t] = (float)sqrt(var);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Input-range initialisation from data (reference torch_utils/torch_linear.py:338-352).
+template <class D>
+__global__ void k_ir_init_update(void* ir, void* idx, const float* __restrict__ stdv, int32_t T,
+                                 float init_from_data, float alpha) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= T) return;
+  const float i = D::load(idx, t);
+  if (!(i < init_from_data)) return;
+  float r = D::load(ir, t);
+  const float s = D::rd(stdv[t]);  // std() is returned in the tensor dtype
+  if (s > 0.0f) {
+    // float(ir) * idx + alpha * float(std), divided by (idx + 1) evaluated in the tensor dtype
+    const float num = r * i + alpha * s;
+    r = D::rd(__fdiv_rn(num, D::rd(i + 1.0f)));
+    D::store(idx, t, D::rd(i + 1.0f));
+  }
+  D::store(ir, t, fabsf(r));
+}
+
+// ------------------------------------------------------------------------------------------
+// cache[t] = max(cache[t], max over the block's rows and the tile's columns of |x|).
+// Non-negative floats order like their int32 bit patterns, and -inf (the initial value) is a
+// negative int, so a signed integer atomicMax implements the float max exactly.
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_running_absmax(const void* __restrict__ x, int64_t rows,
+                                                        int64_t ld, Tiling tl, float* cache) {
+  __shared__ float sh[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r0 = (int64_t)blockIdx.x * kStdRows;
+  for (int32_t t = 0; t < tl.n_tiles; ++t) {
+    float m = 0.0f;
+    for (int i = wave; i < kStdRows; i += 4) {
+      const int64_t r = r0 + i;
+      if (r >= rows) break;
+      const typename D::elem* row = (const typename D::elem*)x + r * ld;
+      wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane,
+                               [&](float v) { m = fmaxf(m, fabsf(v)); });
+    }
+    m = wave_max(m);
+    __syncthreads();
+    if (lane == 0) sh[wave] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const float b = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
+      atomicMax((int*)cache + t, __float_as_int(b));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Weight clipping. Per channel: one wave per row computes the unbiased std of the row in
+// double, then re-reads the row (L2 resident) and stores only the 16-byte vectors in which
+// at least one element changed.
+template <class D, bool VEC>
+AHL_DEV void clamp_row(void* rowp, int32_t cols, int lane, float bound) {
+  typename D::elem* row = (typename D::elem*)rowp;
+  if (VEC) {
+    constexpr int E = D::EPV;
+    const int32_t nv = cols / E;
+    for (int32_t v = lane; v < nv; v += 64) {
+      float e[E];
+      D::unpack(ld16(row + (int64_t)v * E), e);
+      bool changed = false;
+#pragma unroll
+      for (int i = 0; i < E; ++i) {
+        const float c = fminf(fmaxf(e[i], -bound), bound);
+        changed |= (c != e[i]);
+        e[i] = c;
+      }
+      if (changed) st16(row + (int64_t)v * E, D::pack(e));
+    }
+    for (int32_t c = nv * E + lane; c < cols; c += 64) {
+      const float a = D::load(row, c);
+      const float b = fminf(fmaxf(a, -bound), bound);
+      if (a != b) D::store(row, c, b);
+    }
+  } else {
+    for (int32_t c = lane; c < cols; c += 64) {
+      const float a = D::load(row, c);
+      const float b = fminf(fmaxf(a, -bound), bound);
+      if (a != b) D::store(row, c, b);
+    }
+  }
+}
+
+template <class D>
+AHL_DEV float clip_bound(double s, double s2, double n, float sigma) {
+  double var = (s2 - s * s / n) / (n - 1.0);
+  if (var < 0.0) var = 0.0;
+  const float sd = D::rd((float)sqrt(var));  // std() result in the tensor dtype
+  return D::rd(sigma * sd);                 // python float * tensor
+}
+
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_clip_rows(void* w, int64_t rows, int32_t cols, int64_t ld,
+                                                   float sigma) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  typename D::elem* row = (typename D::elem*)w + r * ld;
+  double s = 0.0, s2 = 0.0;
+  wave_row_foreach<D, VEC>(row, 0, cols, lane, [&](float v) {
+    s += (double)v;
+    s2 += (double)v * (double)v;
+  });
+  s = wave_sum(s);
+  s2 = wave_sum(s2);
+  const float bound = clip_bound<D>(s, s2, (double)cols, sigma);
+  if (bound != bound) return;  // a one-element row has no unbiased std; leave it untouched
+  clamp_row<D, VEC>(row, cols, lane, bound);
+}
+
+// Whole-matrix variant, stage 1: per-block (sum, sum of squares) over kStdRows rows.
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_matrix_sums(const void* __restrict__ w, int64_t rows,
+                                                     int32_t cols, int64_t ld,
+                                                     double* __restrict__ partial) {
+  __shared__ double sh[4][2];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r0 = (int64_t)blockIdx.x * kStdRows;
+  double s = 0.0, s2 = 0.0;
+  for (int i = wave; i < kStdRows; i += 4) {
+    const int64_t r = r0 + i;
+    if (r >= rows) break;
+    const typename D::elem* row = (const typename D::elem*)w + r * ld;
+    wave_row_foreach<D, VEC>(row, 0, cols, lane, [&](float v) {
+      s += (double)v;
+      s2 += (double)v * (double)v;
+    });
+  }
+  s = wave_sum(s);
+  s2 = wave_sum(s2);
+  if (lane == 0) { sh[wave][0] = s; sh[wave][1] = s2; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    partial[(int64_t)blockIdx.x * 2] = (sh[0][0] + sh[1][0]) + (sh[2][0] + sh[3][0]);
+    partial[(int64_t)blockIdx.x * 2 + 1] = (sh[0][1] + sh[1][1]) + (sh[2][1] + sh[3][1]);
+  }
+}
+
+// Stage 2: every block re-reduces the partials in the same fixed order, then clamps its rows.
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_clip_matrix(void* w, int64_t rows, int32_t cols,
+                                                     int64_t ld, float sigma,
+                                                     const double* __restrict__ partial,
+                                                     int64_t n_partials) {
+  __shared__ double sh[4][2];
+  __shared__ float sbound;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  double s = 0.0, s2 = 0.0;
+  for (int64_t b = threadIdx.x; b < n_partials; b += 256) {
+    s += partial[b * 2];
+    s2 += partial[b * 2 + 1];
+  }
+  s = wave_sum(s);
+  s2 = wave_sum(s2);
+  if (lane == 0) { sh[wave][0] = s; sh[wave][1] = s2; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const double S = (sh[0][0] + sh[1][0]) + (sh[2][0] + sh[3][0]);
+    const double S2 = (sh[0][1] + sh[1][1]) + (sh[2][1] + sh[3][1]);
+    sbound = clip_bound<D>(S, S2, (double)rows * (double)cols, sigma);
+  }
+  __syncthreads();
+  const float bound = sbound;
+  if (bound != bound) return;
+  const int64_t r0 = (int64_t)blockIdx.x * kStdRows;
+  for (int i = wave; i < kStdRows; i += 4) {
+    const int64_t r = r0 + i;
+    if (r >= rows) break;
+    clamp_row<D, VEC>((typename D::elem*)w + r * ld, cols, lane, bound);
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Column sums, stage 1: partial[s, c] = sum over rows r = s (mod kColSplits) ... of x[r, c].
+static constexpr int kColSplits = 64;
+
+template <class D>
+__global__ __launch_bounds__(256) void k_col_partial(const void* __restrict__ x, int64_t rows,
+                                                     int64_t cols, int64_t ld,
+                                                     float* __restrict__ partial) {
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  const int64_t per = cdiv_dev(rows, kColSplits);
+  const int64_t r0 = (int64_t)blockIdx.y * per;
+  const int64_t r1 = r0 + per < rows ? r0 + per : rows;
+  float s = 0.0f;
+  for (int64_t r = r0; r < r1; ++r) s += D::load(x, r * ld + c);
+  partial[(int64_t)blockIdx.y * cols + c] = s;
+}
+
+template <class D>
+__global__ __launch_bounds__(256) void k_col_final(const float* __restrict__ partial, int64_t cols,
+                                                   void* __restrict__ out) {
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  float s = 0.0f;
+  for (int i = 0; i < kColSplits; ++i) s += partial[(int64_t)i * cols + c];
+  D::store(out, c, D::rd(s));
+}
+
+}  // namespace ahl
+
+using namespace ahl;
+
+// ============================================================================================
+extern "C" {
+
+int ahl_abi_version(void) { return 1; }
+const char* ahl_last_hip_error(void) { return ahl::g_err; }
+
+int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                      const int32_t* tile_ends_host, int32_t n_tiles, void* out, float* tile_max,
+                      float* tile_min, void* stream) {
+  if (!x || !out || rows <= 0 || cols <= 0 || ld < cols) return AHL_ERR_ARG;
+  if ((tile_max == nullptr) != (tile_min == nullptr)) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)cdiv(rows, 4));
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(x) && (ld % D::EPV == 0);
+    if (vec) hipLaunchKernelGGL((k_sliced_absmax<D, true>), grid, dim3(256), 0, s, x, rows, ld, tl, out);
+    else hipLaunchKernelGGL((k_sliced_absmax<D, false>), grid, dim3(256), 0, s, x, rows, ld, tl, out);
+    if (tile_max)
+      hipLaunchKernelGGL((k_tile_minmax<D>), dim3(n_tiles), dim3(256), 0, s, out, rows, tile_max, tile_min);
+  });
+  return check_launch("ahl_sliced_absmax");
+}
+
+int64_t ahl_sliced_std_ws_bytes(int64_t rows, int32_t n_tiles) {
+  return cdiv(rows, kStdRows) * (int64_t)n_tiles * 2 * (int64_t)sizeof(double);
+}
+
+int ahl_sliced_std(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                   const int32_t* tile_ends_host, int32_t n_tiles, float* out, void* ws_partials,
+                   void* stream) {
+  if (!x || !out || !ws_partials || rows <= 0 || cols <= 0 || ld < cols) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t nb = cdiv(rows, kStdRows);
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(x) && (ld % D::EPV == 0);
+    if (vec) hipLaunchKernelGGL((k_sliced_sums<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, (double*)ws_partials);
+    else hipLaunchKernelGGL((k_sliced_sums<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, (double*)ws_partials);
+  });
+  hipLaunchKernelGGL(k_std_finalize, dim3(n_tiles), dim3(64), 0, s, (const double*)ws_partials, nb, rows, tl, out);
+  return check_launch("ahl_sliced_std");
+}
+
+int ahl_ir_init_update(void* ir, void* idx, const float* std, int32_t dtype, int32_t n_tiles,
+                       float init_from_data, float init_std_alpha, void* stream) {
+  if (!ir || !idx || !std || n_tiles <= 0) return AHL_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  AHL_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((k_ir_init_update<D>), dim3((unsigned)cdiv(n_tiles, 64)), dim3(64), 0, s, ir, idx, std, n_tiles, init_from_data, init_std_alpha);
+  });
+  return check_launch("ahl_ir_init_update");
+}
+
+int ahl_running_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                       const int32_t* tile_ends_host, int32_t n_tiles, float* cache, void* stream) {
+  if (!x || !cache || rows <= 0 || cols <= 0 || ld < cols) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t nb = cdiv(rows, kStdRows);
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(x) && (ld % D::EPV == 0);
+    if (vec) hipLaunchKernelGGL((k_running_absmax<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, cache);
+    else hipLaunchKernelGGL((k_running_absmax<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, cache);
+  });
+  return check_launch("ahl_running_absmax");
+}
+
+int64_t ahl_clip_weights_ws_bytes(int64_t rows) {
+  return cdiv(rows, kStdRows) * 2 * (int64_t)sizeof(double);
+}
+
+int ahl_clip_weights(void* w, int32_t dtype, int64_t rows, int64_t cols, int64_t ld, float sigma,
+                     int32_t clip_kind, void* ws, void* stream) {
+  if (!w || rows <= 0 || cols <= 0 || cols > 0x7fffffff || ld < cols) return AHL_ERR_ARG;
+  if (clip_kind != AHL_CLIP_LAYER && clip_kind != AHL_CLIP_PER_CHANNEL) return AHL_ERR_ARG;
+  if (clip_kind == AHL_CLIP_LAYER && !ws) return AHL_ERR_WORKSPACE;
+  hipStream_t s = (hipStream_t)stream;
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(w) && (ld % D::EPV == 0);
+    if (clip_kind == AHL_CLIP_PER_CHANNEL) {
+      const dim3 grid((unsigned)cdiv(rows, 4));
+      if (vec) hipLaunchKernelGGL((k_clip_rows<D, true>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
+      else hipLaunchKernelGGL((k_clip_rows<D, false>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
+    } else {
+      const int64_t nb = cdiv(rows, kStdRows);
+      const dim3 grid((unsigned)nb);
+      if (vec) {
+        hipLaunchKernelGGL((k_matrix_sums<D, true>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, (double*)ws);
+        hipLaunchKernelGGL((k_clip_matrix<D, true>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma, (const double*)ws, nb);
+      } else {
+        hipLaunchKernelGGL((k_matrix_sums<D, false>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, (double*)ws);
+        hipLaunchKernelGGL((k_clip_matrix<D, false>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma, (const double*)ws, nb);
+      }
+    }
+  });
+  return check_launch("ahl_clip_weights");
+}
+
+int64_t ahl_col_sum_ws_bytes(int64_t cols) { return (int64_t)kColSplits * cols * (int64_t)sizeof(float); }
+
+int ahl_col_sum(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld, void* out,
+                void* ws, void* stream) {
+  if (!x || !out || !ws || rows <= 0 || cols <= 0 || ld < cols) return AHL_ERR_ARG;
+  hipStream_t s = (hipStream_t)stream;
+  AHL_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((k_col_partial<D>), dim3((unsigned)cdiv(cols, 256), kColSplits), dim3(256), 0, s, x, rows, cols, ld, (float*)ws);
+    hipLaunchKernelGGL((k_col_final<D>), dim3((unsigned)cdiv(cols, 256)), dim3(256), 0, s, (const float*)ws, cols, out);
+  });
+  return check_launch("ahl_col_sum");
+}
+
+}  // extern "C"

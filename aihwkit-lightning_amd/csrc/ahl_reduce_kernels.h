@@ -1,0 +1,49 @@
+// Reduction kernels used by more than one translation unit.
+#pragma once
+#include "ahl_device.h"
+
+namespace ahl {
+
+// ------------------------------------------------------------------------------------------
+// out[t, r] = max_{c in tile t} |x[r, c]|. One wave per row, 4 rows per block.
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_sliced_absmax(const void* __restrict__ x, int64_t rows,
+                                                       int64_t ld, Tiling tl,
+                                                       void* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const typename D::elem* row = (const typename D::elem*)x + r * ld;
+  for (int32_t t = 0; t < tl.n_tiles; ++t) {
+    float m = 0.0f;
+    wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane,
+                             [&](float v) { m = fmaxf(m, fabsf(v)); });
+    m = wave_max(m);
+    if (lane == 0) D::store(out, (int64_t)t * rows + r, m);
+  }
+}
+
+// tile_max[t] = max_r v[t, r], tile_min[t] = min_r v[t, r]; one block per tile.
+template <class D>
+__global__ __launch_bounds__(256) void k_tile_minmax(const void* __restrict__ v, int64_t rows,
+                                                     float* __restrict__ tile_max,
+                                                     float* __restrict__ tile_min) {
+  __shared__ float smax[4], smin[4];
+  const int t = blockIdx.x;
+  float mx = 0.0f, mn = __builtin_inff();
+  for (int64_t r = threadIdx.x; r < rows; r += 256) {
+    const float a = D::load(v, (int64_t)t * rows + r);
+    mx = fmaxf(mx, a);
+    mn = fminf(mn, a);
+  }
+  mx = wave_max(mx);
+  mn = wave_min(mn);
+  if ((threadIdx.x & 63) == 0) { smax[threadIdx.x >> 6] = mx; smin[threadIdx.x >> 6] = mn; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    tile_max[t] = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+    tile_min[t] = fminf(fminf(smin[0], smin[1]), fminf(smin[2], smin[3]));
+  }
+}
+
+}  // namespace ahl

@@ -1,0 +1,217 @@
+/*
+ * analog_hip.h -- C ABI of libanalog_hip.so: the AnalogLinear hot path on MI355X (gfx950).
+ *
+ * Conventions
+ *   - Every entry point returns an int status (AHL_OK == 0). Nothing throws, nothing allocates,
+ *     nothing synchronises: work is enqueued on the hipStream_t passed as `stream` (a void*;
+ *     NULL is the default stream). All data pointers are DEVICE pointers unless a parameter is
+ *     named *_host. The caller owns every buffer, including scratch ("ws_*" parameters).
+ *   - Matrices are row-major with an explicit leading dimension in ELEMENTS.
+ *   - dtype is AHL_F32 or AHL_BF16 and applies to every pointer documented as "dtype".
+ *     In AHL_BF16 every elementwise result is rounded to bfloat16 (round-to-nearest-even)
+ *     exactly where the reference's torch-mode rounds when it runs on bfloat16 tensors.
+ *   - K-tiles ("analog tiles" along the input dimension) are described by `tile_ends_host`,
+ *     the reference's `upper_end_of_slices` (nn/modules/linear.py:76-80) as a HOST int32 array
+ *     of n_tiles cumulative end offsets. It must follow the reference's split rule
+ *     (nn/modules/linear.py:155-170); anything else returns AHL_ERR_TILING.
+ *
+ * Each entry point cites the reference code it replaces (paths relative to the reference's
+ * src/aihwkit_lightning/).
+ */
+#ifndef ANALOG_HIP_H_
+#define ANALOG_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes ------------------------------------------------------------------------- */
+#define AHL_OK 0
+#define AHL_ERR_ARG 1          /* null pointer, negative size, bad enum                          */
+#define AHL_ERR_TILING 2       /* tile_ends_host does not follow the reference split rule        */
+#define AHL_ERR_UNSUPPORTED 3  /* valid in the reference but not implemented here                 */
+#define AHL_ERR_LAUNCH 4       /* hipLaunchKernel reported an error (see ahl_last_hip_error)      */
+#define AHL_ERR_WORKSPACE 5    /* a ws_* buffer is too small                                      */
+
+/* ---- enums -------------------------------------------------------------------------------- */
+#define AHL_F32 0
+#define AHL_BF16 1
+
+#define AHL_IR_NONE 0     /* input range disabled: no clamp, no DAC                               */
+#define AHL_IR_STATIC 1   /* one scalar per tile, ir[n_tiles] (learned or calibrated)             */
+#define AHL_IR_DYNAMIC 2  /* per token and tile abs-max, ir[n_tiles, M]                           */
+
+#define AHL_NOISE_NONE 0
+#define AHL_NOISE_ADD_NORMAL 1              /* std = std_dev * max|W_tile|          */
+#define AHL_NOISE_ADD_NORMAL_PER_CHANNEL 2  /* std = std_dev * max|W_tile[n, :]|    */
+
+#define AHL_QUANT_NONE 0
+#define AHL_QUANT_DISCRETIZE 1              /* scale from max|W_tile|               */
+#define AHL_QUANT_DISCRETIZE_PER_CHANNEL 2  /* scale from max|W_tile[n, :]|         */
+
+#define AHL_CLIP_LAYER 0        /* one std over the whole matrix   */
+#define AHL_CLIP_PER_CHANNEL 1  /* one std per output channel (row) */
+
+/* Forward/backward behaviour of one AnalogLinear call; a flattened
+ * TorchInferenceRPUConfig (simulator/configs/configs.py:27-88) plus call state.          */
+typedef struct AhlLinearCfg {
+  int32_t dtype;                 /* AHL_F32 | AHL_BF16                                          */
+  int32_t ir_mode;               /* AHL_IR_*                                                    */
+  float inp_res;                 /* forward.inp_res; <= 0 switches the DAC off                  */
+  float out_res;                 /* forward.out_res; <= 0 switches ADC quantisation off         */
+  float out_bound;               /* forward.out_bound; <= 0 switches the output clamp off       */
+  float out_noise;               /* forward.out_noise; used only when training != 0             */
+  int32_t out_noise_per_channel; /* forward.out_noise_per_channel                               */
+  int32_t bound_per_channel;     /* clip.type is one of the *_PER_CHANNEL kinds                 */
+  int32_t training;              /* module.training                                             */
+  int32_t skip_rounding;         /* the reference's test switch _AIHWKIT_NO_ROUNDING            */
+  float ir_decay;                /* pre_post.input_range.decay                                  */
+  float ir_input_min_percentage; /* pre_post.input_range.input_min_percentage                   */
+  uint64_t seed;                 /* Philox key for this call                                    */
+  uint64_t offset;               /* Philox counter offset for this call                         */
+} AhlLinearCfg;
+
+/* Weight modifier of the training forward / post-training quantisation; a flattened
+ * WeightModifierParameter (simulator/parameters/inference.py:29-71).                     */
+typedef struct AhlModifierCfg {
+  int32_t dtype;
+  int32_t quant_type; /* AHL_QUANT_*                                                            */
+  int32_t noise_type; /* AHL_NOISE_* (ignored by ahl_quantize_weights)                          */
+  float res;          /* modifier.res (number of states, or its inverse)                        */
+  float std_dev;      /* modifier.std_dev                                                       */
+  uint64_t seed;
+  uint64_t offset;
+} AhlModifierCfg;
+
+/* ---- library ------------------------------------------------------------------------------ */
+
+/* ABI version of this header; bumped when a signature changes. */
+int ahl_abi_version(void);
+/* Text of the last HIP error seen by a launcher on this thread ("" if none). */
+const char* ahl_last_hip_error(void);
+
+/* ---- reductions (memory-bound) ------------------------------------------------------------ */
+
+/* Per-tile, per-row abs-max of x[rows, cols]: out[t, r] = max_{c in tile t} |x[r, c]|.
+ * out is dtype [n_tiles, rows]. Optionally also tile_max[t] = max_r out[t, r] and
+ * tile_min[t] = min_r out[t, r] as float (pass NULL to skip both).
+ * Replaces nn/modules/torch_utils/torch_abs_max.py:17-39 (weights [N,K] -> [T,N]),
+ * the per-forward amax at torch_utils/torch_linear.py:220, and the dynamic input range
+ * at torch_linear.py:155-157 (x [M,K] -> [T,M]); Triton counterpart
+ * triton_utils/triton_abs_max.py:232-327.                                                */
+int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                      const int32_t* tile_ends_host, int32_t n_tiles, void* out, float* tile_max,
+                      float* tile_min, void* stream);
+
+/* Per-tile unbiased standard deviation over ALL rows: out[t] = std(x[:, tile t]) as float.
+ * ws_partials needs ahl_sliced_std_ws_bytes(rows, n_tiles) bytes.
+ * Replaces `values.std()` at torch_utils/torch_linear.py:342; Triton counterpart
+ * triton_utils/triton_std.py:184-245.                                                    */
+int ahl_sliced_std(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                   const int32_t* tile_ends_host, int32_t n_tiles, float* out, void* ws_partials,
+                   void* stream);
+int64_t ahl_sliced_std_ws_bytes(int64_t rows, int32_t n_tiles);
+
+/* Input-range initialisation from data, all tiles, no host sync:
+ *   if idx[t] < init_from_data: if std[t] > 0 { ir[t] = (ir[t]*idx[t] + alpha*std[t])/(idx[t]+1);
+ *   idx[t] += 1 }  ir[t] = |ir[t]|.   ir and idx are dtype [n_tiles], updated in place.
+ * Replaces torch_utils/torch_linear.py:338-352.                                          */
+int ahl_ir_init_update(void* ir, void* idx, const float* std, int32_t dtype, int32_t n_tiles,
+                       float init_from_data, float init_std_alpha, void* stream);
+
+/* Running per-tile abs-max for input-range calibration:
+ *   cache[t] = max(cache[t], max_{r, c in tile t} |x[r, c]|), cache is float [n_tiles]
+ *   (initialise to -inf). Replaces inference/calibration/calibration.py:110-124.         */
+int ahl_running_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                       const int32_t* tile_ends_host, int32_t n_tiles, float* cache, void* stream);
+
+/* Weight clipping after an optimizer step, in place on w[rows, cols]:
+ *   bound = sigma * std_unbiased(w[r, :]) (AHL_CLIP_PER_CHANNEL) or sigma * std_unbiased(w);
+ *   w = clamp(w, -bound, bound).  ws needs ahl_clip_weights_ws_bytes(rows) bytes.
+ * Replaces AnalogLinear.clip_weights, nn/modules/linear.py:269-283.                      */
+int ahl_clip_weights(void* w, int32_t dtype, int64_t rows, int64_t cols, int64_t ld, float sigma,
+                     int32_t clip_kind, void* ws, void* stream);
+int64_t ahl_clip_weights_ws_bytes(int64_t rows);
+
+/* Column sums: out[c] = sum_r x[r, c] (float accumulate, rounded once to dtype).
+ * ws needs ahl_col_sum_ws_bytes(cols) bytes.
+ * The bias gradient of `out + bias`, torch_utils/torch_linear.py:314.                    */
+int ahl_col_sum(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld, void* out,
+                void* ws, void* stream);
+int64_t ahl_col_sum_ws_bytes(int64_t cols);
+
+/* ---- weights ------------------------------------------------------------------------------ */
+
+/* Everything the forward needs from the weights, one read of w[N, K]:
+ *   wmax[t, n]  = max_{k in tile t} |w[n, k]|                       (dtype [T, N])
+ *   tile_max[t] = max_n wmax[t, n], tile_min[t] = min_n wmax[t, n]  (float [T])
+ *   w_eff       = noise(quantize(w))  (dtype [N, K], ld_eff)   -- only if w_eff != NULL
+ *   w_eff_t     = transpose of w_eff  (dtype [K, N], ld N)     -- only if w_eff_t != NULL
+ * With quant_type/noise_type NONE, w_eff/w_eff_t receive plain copies of w.
+ * Never writes to w (the Triton path's in-place store, triton_utils/triton_linear.py:152-156,
+ * is deliberately not reproduced).
+ * Replaces torch_utils/torch_linear.py:217-251 (amax, clip_and_quantize without learnable
+ * clipping, modify_weight) and torch_utils/quant_utils.py:204-233.                       */
+int ahl_weight_prep(const void* w, int64_t N, int64_t K, int64_t ld, const int32_t* tile_ends_host,
+                    int32_t n_tiles, const AhlModifierCfg* cfg, void* wmax, float* tile_max,
+                    float* tile_min, void* w_eff, int64_t ld_eff, void* w_eff_t, void* stream);
+
+/* Post-training quantisation in place, per tile, scale from the slice's own abs-max:
+ * Replaces AnalogLinear.quantize_weights, nn/modules/linear.py:285-303.
+ * ws_wmax: dtype [T, N]; ws_tile: float [2*T].                                            */
+int ahl_quantize_weights(void* w, int64_t N, int64_t K, int64_t ld, const int32_t* tile_ends_host,
+                         int32_t n_tiles, const AhlModifierCfg* cfg, void* ws_wmax, float* ws_tile,
+                         void* stream);
+
+/* ---- the analog matrix product ------------------------------------------------------------ */
+
+/* Forward of TorchLinear.linear (torch_utils/torch_linear.py:116-314) for x[M, K]:
+ *   for every K-tile: clamp to the input range + DAC quantise (fused into the A-tile staging),
+ *   MFMA product with w_eff[N, K], output noise, ADC quantise, clamp to the output bound;
+ *   per-tile results summed in dtype; bias added last.
+ *   ir       dtype [T] (AHL_IR_STATIC) or [T, M] (AHL_IR_DYNAMIC) or NULL (AHL_IR_NONE)
+ *   wmax     dtype [T, N] from ahl_weight_prep, or NULL when neither noise nor bound is on
+ *   tile_max float [T]    from ahl_weight_prep, or NULL likewise
+ *   bias     dtype [N] or NULL
+ *   y        dtype [M, N]
+ *   keep     uint8 [ceil(T/8), M, N] or NULL: bit (t%8) of plane t/8 is set where the tile-t
+ *            output was inside [-bound, bound] (the clamp's gradient mask). Written only when
+ *            out_bound > 0 and keep != NULL.
+ * Slot of TritonLinear.forward, triton_utils/triton_linear.py:446-690.                   */
+int ahl_linear_fwd(const void* x, int64_t ldx, const void* w_eff, int64_t ldw, const void* bias,
+                   void* y, int64_t ldy, uint8_t* keep, const void* ir, const void* wmax,
+                   const float* tile_max, int64_t M, int64_t K, int64_t N,
+                   const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
+                   void* stream);
+
+/* Input gradient and input-range gradient (torch_utils/torch_linear.py:29-108 backward):
+ *   d[:, tile t] = (g * keep_t) @ w_eff[:, tile t]      w_eff_t is the [K, N] transpose
+ *   AHL_IR_STATIC: ir_grad[t] per reference InputRangeForward.backward (incl. decay switch),
+ *                  dx zeroed where |x| > ir[t]; x[M, K] is the forward input.
+ *   otherwise dx = d, ir_grad untouched.
+ *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, n_tiles) bytes.
+ * Slot of TritonLinear.backward, triton_utils/triton_linear.py:695-764.                  */
+int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const void* w_eff_t,
+                      const void* x, int64_t ldx, const void* ir, void* dx, int64_t lddx,
+                      void* ir_grad, int64_t M, int64_t K, int64_t N,
+                      const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
+                      void* ws, void* stream);
+int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int32_t n_tiles);
+
+/* Weight gradient: dw[:, tile t] = (g * keep_t)^T @ DAC(clamp(x[:, tile t])).
+ *   ws needs ahl_linear_bwd_dw_ws_bytes(M, K, N, n_tiles, dtype, keep != NULL) bytes
+ *   (transposed staging copies of g, keep and the re-quantised x).
+ * Same reference slot as ahl_linear_bwd_dx.                                               */
+int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const void* x, int64_t ldx,
+                      const void* ir, void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
+                      const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
+                      void* ws, void* stream);
+int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
+                                   int32_t has_keep);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ANALOG_HIP_H_ */

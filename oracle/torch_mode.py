@@ -1,0 +1,307 @@
+"""CPU oracle for the AnalogLinear hot path -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+
+A from-scratch restatement, in plain CPU torch tensor ops, of what the reference's torch-mode
+computes for one AnalogLinear layer: forward, the explicit (hand-derived) backward that its
+autograd graph implies, and the memory-bound helpers around it. Only ``tests/``,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` may import this module,
+and only as a checker or a timed baseline; nothing in ``aihwkit-lightning_amd/`` does.
+
+Every function cites the reference lines it follows (paths relative to the reference's
+``src/aihwkit_lightning/``). Tensors stay in the layer dtype throughout, so each elementwise
+op rounds to that dtype exactly as torch does for the reference.
+
+How the oracle itself is pinned (see ``tests/test_oracle_*.py``): golden vectors written by the
+real reference (``tests/golden/make_golden.py``), the closed forms in the reference's own tests
+(clipping, weight modifier, calibration max, quantisation idempotence), reductions to
+``F.linear`` / brute force, and Philox known-answer vectors.
+"""
+from dataclasses import dataclass
+from math import sqrt
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+from torch import Tensor
+
+# quantisation / noise / clip selectors (plain strings: the oracle does not depend on the package)
+NONE = "none"
+DISCRETIZE = "discretize"
+DISCRETIZE_PER_CHANNEL = "discretize_per_channel"
+ADD_NORMAL = "add_normal"
+ADD_NORMAL_PER_CHANNEL = "add_normal_per_channel"
+IR_NONE, IR_STATIC, IR_DYNAMIC = "none", "static", "dynamic"
+
+
+@dataclass
+class OracleCfg:
+    """Flat view of the settings that influence one layer call."""
+
+    max_input_size: int = -1
+    inp_res: float = -1.0
+    out_res: float = -1.0
+    out_bound: float = 0.0
+    out_noise: float = 0.0
+    out_noise_per_channel: bool = False
+    bound_per_channel: bool = False  # clip type is one of the per-channel kinds
+    ir_mode: str = IR_NONE
+    ir_decay: float = 0.001
+    ir_input_min_percentage: float = 0.95
+    weight_quant: str = NONE
+    weight_noise: str = NONE
+    modifier_res: float = 0.0
+    modifier_std: float = 0.0
+    skip_rounding: bool = False
+
+
+# --------------------------------------------------------------------------------------------
+def split_sizes(size: int, max_size: int) -> List[int]:
+    """K-tile sizes (nn/modules/linear.py:155-170)."""
+    if max_size <= 0:
+        return [size]
+    n_tiles = -(-size // max_size)
+    base, extra = divmod(size, n_tiles)
+    return [base + 1 if i < extra else base for i in range(n_tiles)]
+
+
+def tile_bounds(in_sizes: Sequence[int]) -> List[Tuple[int, int]]:
+    """[(lo, hi)] column ranges of the tiles."""
+    out, lo = [], 0
+    for size in in_sizes:
+        out.append((lo, lo + size))
+        lo += size
+    return out
+
+
+def _tiny(dtype: torch.dtype) -> float:
+    return torch.finfo(dtype).tiny
+
+
+def quant_step(bound: Tensor, res: float) -> Tensor:
+    """Step of a quantiser given as #states (res > 1) or 1/#states, for a tensor bound
+    (torch_utils/quant_utils.py:63-66)."""
+    alpha = 2 * bound
+    return alpha / res if res > 1.0 else alpha * res
+
+
+def quantize(values: Tensor, step: Tensor, skip_rounding: bool = False,
+             max_state: Optional[float] = None) -> Tensor:
+    """round(clamp(values / max(step, tiny))) * step (torch_utils/quant_utils.py:78-99)."""
+    out = values / step.clamp_min(_tiny(values.dtype))
+    if max_state is not None:
+        out = torch.clamp(out, min=-max_state, max=max_state)
+    if not skip_rounding:
+        out = out.round()
+    return out * step
+
+
+def sliced_abs_max(weights: Tensor, in_sizes: Sequence[int]) -> Tensor:
+    """[T, N] per-tile per-row abs-max (torch_utils/torch_abs_max.py:17-39)."""
+    return torch.stack([weights[:, lo:hi].abs().amax(dim=1) for lo, hi in tile_bounds(in_sizes)])
+
+
+def sliced_std(x: Tensor, in_sizes: Sequence[int]) -> Tensor:
+    """[T] unbiased std of each tile over all rows (torch_utils/torch_linear.py:342)."""
+    return torch.stack([x[:, lo:hi].std() for lo, hi in tile_bounds(in_sizes)])
+
+
+def quantize_weight_tile(w_t: Tensor, wmax_t: Tensor, kind: str, res: float) -> Tensor:
+    """On-the-fly weight quantiser of one tile without learnable clipping
+    (torch_utils/quant_utils.py:204-233): scale = wmax / n_states (per tile or per channel),
+    UniformQuantize(w, scale, bound=1.0, max_quant_state=n_states/2)."""
+    if kind == NONE:
+        return w_t
+    n_states = max(res, 1 / res)
+    scale = wmax_t.max() / n_states if kind == DISCRETIZE else wmax_t / n_states
+    step = 2.0 / scale if bool((scale > 1.0).all()) else 2.0 * scale
+    step = step.clone()
+    step[step == 0.0] = 1.0
+    return quantize(w_t, step, False, n_states / 2)
+
+
+def noisy_weight_tile(w_t: Tensor, wmax_t: Tensor, kind: str, std_dev: float,
+                      xi: Optional[Tensor] = None) -> Tensor:
+    """w + std_dev * wmax * N(0,1) per tile (ADD_NORMAL) or per tile and channel
+    (torch_utils/torch_linear.py:444-462). ``xi`` overrides the normal draw."""
+    if kind == NONE:
+        return w_t
+    if xi is None:
+        xi = torch.randn_like(w_t)
+    ref = wmax_t.max() if kind == ADD_NORMAL else wmax_t
+    return w_t + std_dev * ref * xi
+
+
+# --------------------------------------------------------------------------------------------
+def ir_init_update(x_t: Tensor, ir: Tensor, idx: Tensor, t: int, init_from_data: float,
+                   alpha: float) -> None:
+    """One data-initialisation step of tile t's input range, in place
+    (torch_utils/torch_linear.py:338-352)."""
+    i = idx[t]
+    if i < init_from_data:
+        std = x_t.std()
+        if std > 0.0:
+            ir[t] = ((ir[t].float() * i + alpha * std.float()) / (i + 1)).to(ir.dtype)
+            idx[t] += 1
+        ir[t] = ir[t].abs()
+
+
+def linear_forward(
+    x: Tensor,
+    weights: Tensor,
+    bias: Optional[Tensor],
+    cfg: OracleCfg,
+    input_range: Optional[Tensor],
+    training: bool,
+    out_xi: Optional[Sequence[Tensor]] = None,
+    w_xi: Optional[Sequence[Tensor]] = None,
+) -> Tuple[Tensor, Dict]:
+    """Forward of one layer call on x[M, K] (torch_utils/torch_linear.py:116-314), tile by tile:
+    input range -> DAC -> weight quantiser/noise -> product -> output noise -> ADC -> clamp ->
+    sum in dtype -> bias. Returns the output and what the explicit backward needs.
+
+    Normal draws come from torch's global generator in the reference's order (per tile: weight
+    noise, then output noise) unless ``w_xi`` / ``out_xi`` (lists per tile) are given.
+    """
+    assert x.dim() == 2
+    in_sizes = split_sizes(x.size(1), cfg.max_input_size)
+    n_tiles = len(in_sizes)
+    adc_on = cfg.out_res > 0
+    bound_on = adc_on or cfg.out_bound > 0
+    noise_on = training and cfg.out_noise > 0
+    w_noise_on = training and cfg.weight_noise != NONE
+    need_wmax = bound_on or noise_on or w_noise_on or cfg.weight_quant != NONE
+    out = 0.0
+    saved: Dict = {"cfg": cfg, "in_sizes": in_sizes, "x": x, "tiles": []}
+    for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
+        x_t = x[:, lo:hi]
+        rec: Dict = {}
+        ir_t = None
+        if cfg.ir_mode == IR_STATIC:
+            ir_t = input_range[t]
+            rec["up"] = x_t >= ir_t
+            rec["lo"] = x_t <= -ir_t
+            xc = torch.clamp(x_t, min=-ir_t, max=ir_t)
+        elif cfg.ir_mode == IR_DYNAMIC:
+            ir_t = x_t.abs().max(dim=-1, keepdim=True)[0]
+            xc = x_t
+        else:
+            xc = x_t
+        rec["ir"] = ir_t
+        if cfg.inp_res > 0:
+            xq = quantize(xc, quant_step(ir_t, cfg.inp_res), cfg.skip_rounding)
+        else:
+            xq = xc
+        w_t = weights[:, lo:hi]
+        wmax_t = w_t.abs().amax(dim=-1, keepdim=True) if need_wmax else None
+        w_eff = quantize_weight_tile(w_t, wmax_t, cfg.weight_quant, cfg.modifier_res)
+        if w_noise_on:
+            w_eff = noisy_weight_tile(w_eff, wmax_t, cfg.weight_noise, cfg.modifier_std,
+                                      None if w_xi is None else w_xi[t])
+        # one fp32-accumulated product, rounded once to the tensor dtype
+        y = (xq.float() @ w_eff.float().T).to(x.dtype)
+        if noise_on:
+            wr = wmax_t.view(1, -1) if cfg.out_noise_per_channel else wmax_t.max()
+            xi = torch.randn_like(y) if out_xi is None else out_xi[t]
+            y = y + wr * (cfg.out_noise / sqrt(n_tiles) * ir_t) * xi
+        keep = None
+        if bound_on:
+            wb = wmax_t.view(1, -1) if cfg.bound_per_channel else wmax_t.max()
+            bound = (ir_t * cfg.out_bound) * wb
+            if adc_on:
+                y = quantize(y, quant_step(bound, cfg.out_res), cfg.skip_rounding)
+            if cfg.out_bound > 0:
+                keep = (y >= -bound) & (y <= bound)
+                y = torch.clamp(y, min=-bound, max=bound)
+        out = out + y
+        rec.update(xq=xq, w_eff=w_eff, keep=keep)
+        saved["tiles"].append(rec)
+    if bias is not None:
+        out = out + bias
+    return out, saved
+
+
+def linear_backward(grad_out: Tensor, saved: Dict) -> Tuple[Tensor, Tensor, Tensor, Optional[Tensor]]:
+    """Explicit backward of :func:`linear_forward` = what autograd computes for the reference
+    graph: clamp mask (torch.clamp), straight-through ADC/DAC (quant_utils.py:152-156), product,
+    input-range gradient (torch_linear.py:92-106) and straight-through input clamp
+    (torch_linear.py:44-54). Returns (dx, dw, dbias, ir_grad or None)."""
+    cfg: OracleCfg = saved["cfg"]
+    x = saved["x"]
+    dtype = x.dtype
+    n_tiles = len(saved["in_sizes"])
+    dx = torch.zeros_like(x)
+    dw_parts = []
+    ir_grad = torch.zeros(n_tiles, dtype=dtype) if cfg.ir_mode == IR_STATIC else None
+    for t, (lo, hi) in enumerate(tile_bounds(saved["in_sizes"])):
+        rec = saved["tiles"][t]
+        gy = grad_out if rec["keep"] is None else grad_out * rec["keep"]
+        dw_parts.append((gy.float().T @ rec["xq"].float()).to(dtype))
+        d = (gy.float() @ rec["w_eff"].float()).to(dtype)
+        if cfg.ir_mode == IR_STATIC:
+            ir_t, up, low = rec["ir"], rec["up"], rec["lo"]
+            grad = torch.zeros_like(ir_t)
+            grad += torch.clamp(d[up], min=None, max=0.0).sum()
+            grad -= torch.clamp(d[low], min=0.0, max=None).sum()
+            grad *= ir_t
+            if cfg.ir_decay > 0:
+                pct = 1.0 - (up | low).sum().div(up.numel())
+                grad += cfg.ir_decay * ir_t * (pct > cfg.ir_input_min_percentage)
+            ir_grad[t] = grad
+            x_t = x[:, lo:hi]
+            d = d.clone()
+            d[(up | low) & (x_t.abs() != ir_t)] = 0.0
+        dx[:, lo:hi] = d
+    dw = torch.cat(dw_parts, dim=1)
+    dbias = grad_out.sum(dim=0)
+    return dx, dw, dbias, ir_grad
+
+
+# --------------------------------------------------------------------------------------------
+def clip_weights(weights: Tensor, sigma: float, per_channel: bool) -> Tensor:
+    """clamp(W, +-sigma * std) with the std of each row or of the whole matrix
+    (nn/modules/linear.py:269-283). Returns a new tensor."""
+    bound = sigma * (weights.std(1, keepdim=True) if per_channel else weights.std())
+    return torch.clamp(weights, -bound, bound)
+
+
+def quantize_weights(weights: Tensor, in_sizes: Sequence[int], kind: str, res: float) -> Tensor:
+    """Post-training per-tile quantisation with the slice's own abs-max
+    (nn/modules/linear.py:285-303). Returns a new tensor."""
+    out = weights.clone()
+    for lo, hi in tile_bounds(in_sizes):
+        w_t = weights[:, lo:hi]
+        out[:, lo:hi] = quantize_weight_tile(w_t, w_t.abs().amax(dim=1, keepdim=True), kind, res)
+    return out
+
+
+def calibrate_max(batches: Sequence[Tensor], in_sizes: Sequence[int]) -> Tensor:
+    """Running per-tile abs-max over batches (inference/calibration/calibration.py:110-124)."""
+    cache = torch.full((len(in_sizes),), float("-inf"), dtype=batches[0].dtype)
+    for x in batches:
+        x = x.reshape(-1, x.size(-1))
+        for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
+            cache[t] = max(cache[t], x[:, lo:hi].abs().max())
+    return cache
+
+
+# --------------------------------------------------------------------------------------------
+# Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3",
+# SC'11) in pure Python ints, to pin the device generator bit for bit.
+_M0, _M1, _W0, _W1 = 0xD2511F53, 0xCD9E8D57, 0x9E3779B9, 0xBB67AE85
+_MASK = 0xFFFFFFFF
+
+
+def philox4x32_10(ctr: Sequence[int], key: Sequence[int]) -> Tuple[int, int, int, int]:
+    """Ten Philox rounds on a 4x32-bit counter with a 2x32-bit key."""
+    c0, c1, c2, c3 = ctr
+    k0, k1 = key
+    for _ in range(10):
+        p0, p1 = _M0 * c0, _M1 * c2
+        c0, c1, c2, c3 = ((p1 >> 32) ^ c1 ^ k0) & _MASK, p1 & _MASK, ((p0 >> 32) ^ c3 ^ k1) & _MASK, p0 & _MASK
+        k0, k1 = (k0 + _W0) & _MASK, (k1 + _W1) & _MASK
+    return c0, c1, c2, c3
+
+
+def philox_counter(stream_and_tile: int, group: int, offset: int) -> Tuple[int, int, int, int]:
+    """Counter layout of the device generator: (group lo, group hi, stream<<24 | tile, offset lo).
+    Output noise: stream 0, group = (m // 4) * N + n, the 4 normals are rows 4*(m//4)+0..3.
+    Weight noise: stream 1, tile field 0, group = n * ceil(K/4) + k // 4, normals k%4 = 0..3."""
+    return group & _MASK, (group >> 32) & _MASK, stream_and_tile & _MASK, offset & _MASK
