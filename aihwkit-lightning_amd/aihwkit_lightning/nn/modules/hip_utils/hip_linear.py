@@ -124,20 +124,6 @@ class HipLinear(Function):
                 w_eff = eff
             w_eff_t = eff_t if need_dx else None
 
-        ir_dev = None
-        if ir_mode == L.AHL_IR_STATIC:
-            if training and init_active and m_rows > 0:
-                std = OPS.sliced_std(x2, in_sizes)
-                OPS.ir_init_update(
-                    input_range.data, input_range_update_idx, std, float(ir_params.init_from_data),
-                    float(ir_params.init_std_alpha),
-                )
-            ir_dev = input_range.detach()
-            if not ir_dev.is_contiguous():
-                ir_dev = ir_dev.contiguous()
-        elif ir_mode == L.AHL_IR_DYNAMIC and m_rows > 0:
-            ir_dev = OPS.sliced_absmax(x2, in_sizes, False)[0]
-
         skip_rounding = 1 if os.environ.get("_AIHWKIT_NO_ROUNDING", False) else 0
         icfg = [
             ir_mode, int(fwd.out_noise_per_channel),
@@ -150,25 +136,53 @@ class HipLinear(Function):
             float(fwd.out_noise) if noise_on else 0.0, float(ir_params.decay),
             float(ir_params.input_min_percentage),
         ]
-        want_keep = fwd.out_bound > 0 and (need_dx or need_dw)
         if m_rows == 0:
             return inp.new_zeros(out_shape)
-        y, keep = OPS.linear_fwd(
-            x2, w_eff, bias, ir_dev, wmax, tile_max, in_sizes, icfg, fcfg, want_keep
+
+        # bf16 with equal tiles of a multiple of 64 inputs: clamp + DAC (+ dynamic abs-max) run as
+        # one memory-bound pass and the matrix kernel streams the quantised input; otherwise the
+        # clamp + DAC are fused into the matrix kernel's A-tile staging.
+        split_dac = (
+            inp.dtype == torch.bfloat16 and len(set(in_sizes)) == 1 and in_sizes[0] % 64 == 0
+        )
+        ir_dev = xq = None
+        if ir_mode == L.AHL_IR_STATIC:
+            if training and init_active:
+                std = OPS.sliced_std(x2, in_sizes)
+                OPS.ir_init_update(
+                    input_range.data, input_range_update_idx, std, float(ir_params.init_from_data),
+                    float(ir_params.init_std_alpha),
+                )
+            ir_dev = input_range.detach()
+            if not ir_dev.is_contiguous():
+                ir_dev = ir_dev.contiguous()
+        if split_dac:
+            xq, ir_dyn = OPS.dac(x2, ir_dev, in_sizes, icfg, fcfg)
+            if ir_mode == L.AHL_IR_DYNAMIC:
+                ir_dev = ir_dyn
+        elif ir_mode == L.AHL_IR_DYNAMIC:
+            ir_dev = OPS.sliced_absmax(x2, in_sizes, False)[0]
+
+        want_keep = fwd.out_bound > 0 and (need_dx or need_dw)
+        y, keep, flag = OPS.linear_fwd(
+            None if split_dac else x2, xq, w_eff, bias, ir_dev, wmax, tile_max, in_sizes, icfg, fcfg,
+            want_keep,
         )
 
         ctx.in_sizes, ctx.icfg, ctx.fcfg = in_sizes, icfg, fcfg
         ctx.inp_shape, ctx.ir_mode, ctx.has_bias = inp.shape, ir_mode, bias is not None
         ctx.need_dx, ctx.need_dw, ctx.ir_needs_grad = need_dx, need_dw, ir_needs_grad
+        need_x = (need_dx and ir_mode == L.AHL_IR_STATIC) or (need_dw and xq is None)
         ctx.save_for_backward(
-            x2, w_eff_t, keep if want_keep else None,
+            x2 if need_x else None, xq if need_dw else None, w_eff_t,
+            keep if want_keep else None, flag if want_keep else None,
             ir_dev.clone() if ir_mode == L.AHL_IR_STATIC else ir_dev,
         )
         return y.view(out_shape)
 
     @staticmethod
     def backward(ctx, grad_out: Tensor):
-        x2, w_eff_t, keep, ir_dev = ctx.saved_tensors
+        x2, xq, w_eff_t, keep, flag, ir_dev = ctx.saved_tensors
         n_out = grad_out.size(-1)
         g2 = grad_out.reshape(-1, n_out)
         if g2.stride(-1) != 1 or (g2.size(0) > 1 and g2.stride(0) != n_out):
@@ -176,7 +190,7 @@ class HipLinear(Function):
         grad_inp = grad_w = grad_b = grad_ir = None
         if ctx.need_dx:
             dx, ir_grad = OPS.linear_bwd_dx(
-                g2, keep, w_eff_t, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
+                g2, keep, flag, w_eff_t, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
                 ctx.in_sizes, ctx.icfg, ctx.fcfg,
             )
             if ctx.needs_input_grad[0]:
@@ -184,7 +198,10 @@ class HipLinear(Function):
             if ctx.ir_needs_grad and ctx.needs_input_grad[3]:
                 grad_ir = ir_grad
         if ctx.need_dw:
-            grad_w = OPS.linear_bwd_dw(g2, keep, x2, ir_dev, ctx.in_sizes, ctx.icfg, ctx.fcfg)
+            grad_w = OPS.linear_bwd_dw(
+                g2, keep, flag, x2 if xq is None else None, xq, ir_dev, ctx.in_sizes, ctx.icfg,
+                ctx.fcfg,
+            )
         if ctx.has_bias and ctx.needs_input_grad[2]:
             grad_b = OPS.col_sum(g2)
         return grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None

@@ -77,16 +77,20 @@ LIB.define(
 )
 LIB.define("quantize_weights(Tensor(a!) w, int[] in_sizes, int quant_type, float res) -> ()")
 LIB.define(
-    "linear_fwd(Tensor x, Tensor w_eff, Tensor? bias, Tensor? ir, Tensor? wmax, Tensor? tile_max, "
-    "int[] in_sizes, int[] icfg, float[] fcfg, bool want_keep) -> (Tensor, Tensor)"
+    "dac(Tensor x, Tensor? ir, int[] in_sizes, int[] icfg, float[] fcfg) -> (Tensor, Tensor)"
 )
 LIB.define(
-    "linear_bwd_dx(Tensor g, Tensor? keep, Tensor w_eff_t, Tensor? x, Tensor? ir, int[] in_sizes, "
-    "int[] icfg, float[] fcfg) -> (Tensor, Tensor)"
+    "linear_fwd(Tensor? x, Tensor? xq, Tensor w_eff, Tensor? bias, Tensor? ir, Tensor? wmax, "
+    "Tensor? tile_max, int[] in_sizes, int[] icfg, float[] fcfg, bool want_keep) "
+    "-> (Tensor, Tensor, Tensor)"
 )
 LIB.define(
-    "linear_bwd_dw(Tensor g, Tensor? keep, Tensor x, Tensor? ir, int[] in_sizes, int[] icfg, "
-    "float[] fcfg) -> Tensor"
+    "linear_bwd_dx(Tensor g, Tensor? keep, Tensor? clamp_flag, Tensor w_eff_t, Tensor? x, "
+    "Tensor? ir, int[] in_sizes, int[] icfg, float[] fcfg) -> (Tensor, Tensor)"
+)
+LIB.define(
+    "linear_bwd_dw(Tensor g, Tensor? keep, Tensor? clamp_flag, Tensor? x, Tensor? xq, Tensor? ir, "
+    "int[] in_sizes, int[] icfg, float[] fcfg) -> Tensor"
 )
 
 
@@ -241,36 +245,65 @@ def quantize_weights(w: Tensor, in_sizes: List[int], quant_type: int, res: float
     )
 
 
-def linear_fwd(
-    x: Tensor, w_eff: Tensor, bias: Optional[Tensor], ir: Optional[Tensor], wmax: Optional[Tensor],
-    tile_max: Optional[Tensor], in_sizes: List[int], icfg: List[int], fcfg: List[float],
-    want_keep: bool,
-) -> Tuple[Tensor, Tensor]:
-    """The fused analog forward; returns ``y [M, N]`` and the clamp mask (empty if not wanted)."""
+def dac(x: Tensor, ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
+        fcfg: List[float]) -> Tuple[Tensor, Tensor]:
+    """Clamp + DAC pre-pass: returns ``xq [M, K]`` and, in dynamic mode, the ranges ``[T, M]``."""
     lib = L.load()
     x = _rows2d(x, "x")
     m_rows, k_in = x.shape
-    n_out = w_eff.size(0)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(x.dtype, icfg, fcfg)
-    y = torch.empty((m_rows, n_out), dtype=x.dtype, device=x.device)
+    xq = torch.empty((m_rows, k_in), dtype=x.dtype, device=x.device)
+    dynamic = cfg.ir_mode == L.AHL_IR_DYNAMIC
+    ir_dyn = torch.empty((n_tiles, m_rows) if dynamic else (0,), dtype=x.dtype, device=x.device)
+    L.check(
+        lib.ahl_dac(
+            _ptr(x), _ld(x), _ptr(xq), k_in, _ptr(ir), _ptr(ir_dyn) if dynamic else None, m_rows,
+            k_in, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _stream(),
+        ),
+        "ahl_dac",
+    )
+    return xq, ir_dyn
+
+
+def linear_fwd(
+    x: Optional[Tensor], xq: Optional[Tensor], w_eff: Tensor, bias: Optional[Tensor],
+    ir: Optional[Tensor], wmax: Optional[Tensor], tile_max: Optional[Tensor], in_sizes: List[int],
+    icfg: List[int], fcfg: List[float], want_keep: bool,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """The analog forward; returns ``y [M, N]``, the clamp mask (empty if not wanted) and the
+    one-word "anything clamped" flag."""
+    lib = L.load()
+    ref = x if x is not None else xq
+    if x is not None:
+        x = _rows2d(x, "x")
+    if xq is not None:
+        xq = _rows2d(xq, "xq")
+    m_rows, k_in = ref.shape
+    n_out = w_eff.size(0)
+    n_tiles = len(in_sizes)
+    cfg = _linear_cfg(ref.dtype, icfg, fcfg)
+    y = torch.empty((m_rows, n_out), dtype=ref.dtype, device=ref.device)
     planes = (n_tiles + 7) // 8
     keep = torch.empty((planes, m_rows, n_out) if want_keep else (0,), dtype=torch.uint8,
-                       device=x.device)
+                       device=ref.device)
+    flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
     L.check(
         lib.ahl_linear_fwd(
-            _ptr(x), _ld(x), _ptr(w_eff), _ld(w_eff), _ptr(bias), _ptr(y), n_out,
-            _ptr(keep) if want_keep else None, _ptr(ir), _ptr(wmax), _ptr(tile_max), m_rows, k_in,
+            _ptr(x), _ld(x) if x is not None else 0, _ptr(xq), _ld(xq) if xq is not None else 0,
+            _ptr(w_eff), _ld(w_eff), _ptr(bias), _ptr(y), n_out, _ptr(keep) if want_keep else None,
+            _ptr(flag) if want_keep else None, _ptr(ir), _ptr(wmax), _ptr(tile_max), m_rows, k_in,
             n_out, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _stream(),
         ),
         "ahl_linear_fwd",
     )
-    return y, keep
+    return y, keep, flag
 
 
 def linear_bwd_dx(
-    g: Tensor, keep: Optional[Tensor], w_eff_t: Tensor, x: Optional[Tensor], ir: Optional[Tensor],
-    in_sizes: List[int], icfg: List[int], fcfg: List[float],
+    g: Tensor, keep: Optional[Tensor], clamp_flag: Optional[Tensor], w_eff_t: Tensor,
+    x: Optional[Tensor], ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
+    fcfg: List[float],
 ) -> Tuple[Tensor, Tensor]:
     """Input gradient ``[M, K]`` and input-range gradient ``[T]`` (empty unless static range)."""
     lib = L.load()
@@ -288,9 +321,10 @@ def linear_bwd_dx(
         x = _rows2d(x, "x")
     L.check(
         lib.ahl_linear_bwd_dx(
-            _ptr(g), _ld(g), _ptr(keep), _ptr(w_eff_t), _ptr(x), _ld(x) if x is not None else 0,
-            _ptr(ir), _ptr(dx), k_in, _ptr(ir_grad) if static else None, m_rows, k_in, n_out,
-            L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(ws), _stream(),
+            _ptr(g), _ld(g), _ptr(keep), _ptr(clamp_flag), _ptr(w_eff_t), _ptr(x),
+            _ld(x) if x is not None else 0, _ptr(ir), _ptr(dx), k_in,
+            _ptr(ir_grad) if static else None, m_rows, k_in, n_out, L.tile_ends_array(in_sizes),
+            n_tiles, byref(cfg), _ptr(ws), _stream(),
         ),
         "ahl_linear_bwd_dx",
     )
@@ -298,15 +332,20 @@ def linear_bwd_dx(
 
 
 def linear_bwd_dw(
-    g: Tensor, keep: Optional[Tensor], x: Tensor, ir: Optional[Tensor], in_sizes: List[int],
-    icfg: List[int], fcfg: List[float],
+    g: Tensor, keep: Optional[Tensor], clamp_flag: Optional[Tensor], x: Optional[Tensor],
+    xq: Optional[Tensor], ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
+    fcfg: List[float],
 ) -> Tensor:
-    """Weight gradient ``[N, K]``."""
+    """Weight gradient ``[N, K]`` from the raw input ``x`` or the saved quantised input ``xq``."""
     lib = L.load()
     g = _rows2d(g, "g")
-    x = _rows2d(x, "x")
+    ref = xq if xq is not None else x
+    if x is not None:
+        x = _rows2d(x, "x")
+    if xq is not None:
+        xq = _rows2d(xq, "xq")
     m_rows, n_out = g.shape
-    k_in = x.size(1)
+    k_in = ref.size(1)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(g.dtype, icfg, fcfg)
     dw = torch.empty((n_out, k_in), dtype=g.dtype, device=g.device)
@@ -315,7 +354,8 @@ def linear_bwd_dw(
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=g.device)
     L.check(
         lib.ahl_linear_bwd_dw(
-            _ptr(g), _ld(g), _ptr(keep), _ptr(x), _ld(x), _ptr(ir), _ptr(dw), k_in, m_rows, k_in,
+            _ptr(g), _ld(g), _ptr(keep), _ptr(clamp_flag), _ptr(x), _ld(x) if x is not None else 0,
+            _ptr(xq), _ld(xq) if xq is not None else 0, _ptr(ir), _ptr(dw), k_in, m_rows, k_in,
             n_out, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(ws), _stream(),
         ),
         "ahl_linear_bwd_dw",
@@ -327,7 +367,7 @@ for _name, _fn in [
     ("sliced_absmax", sliced_absmax), ("sliced_std", sliced_std), ("ir_init_update", ir_init_update),
     ("running_absmax", running_absmax), ("clip_weights", clip_weights), ("col_sum", col_sum),
     ("weight_prep", weight_prep), ("quantize_weights", quantize_weights),
-    ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
+    ("dac", dac), ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
 ]:
     LIB.impl(_name, _fn, "CUDA")
 

@@ -133,24 +133,34 @@ AHL_DEV u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
   return c;
 }
 
-// Two standard normals from two 32-bit words (Box-Muller, 24-bit uniforms in (0,1)).
-AHL_DEV void box_muller(uint32_t a, uint32_t b, float& n0, float& n1) {
-  const float u1 = ((float)(a >> 8) + 0.5f) * 5.9604644775390625e-08f;  // 2^-24
-  const float u2 = ((float)(b >> 8) + 0.5f) * 5.9604644775390625e-08f;
-  const float r = __fsqrt_rn(-2.0f * __logf(u1));
-  float s, c;
-  __sincosf(6.283185307179586f * u2, &s, &c);
-  n0 = r * c;
-  n1 = r * s;
+// Two standard normals from one 32-bit word (Box-Muller with two 16-bit uniforms):
+//   u1 = (lo16 + 0.5) / 65536, u2 = (hi16 + 0.5) / 65536,
+//   r = sqrt(-2 ln u1), (n0, n1) = r * (cos 2 pi u2, sin 2 pi u2).
+// The radius is limited to 4.85 sigma (u1 >= 2^-17); the variance deficit is < 1e-4.
+// v_log_f32 is log2, v_sin_f32 / v_cos_f32 take their argument in revolutions.
+AHL_DEV void box_muller16(uint32_t w, float& n0, float& n1) {
+  const float a = (float)(w & 0xffffu) + 0.5f;
+  const float b = (float)(w >> 16) + 0.5f;
+  const float r2 = (16.0f - __builtin_amdgcn_logf(a)) * 1.3862943611198906f;  // -2 ln(a / 65536)
+  const float r = __builtin_amdgcn_sqrtf(r2);
+  const float rev = b * 1.52587890625e-05f;  // / 65536
+  n0 = r * __builtin_amdgcn_cosf(rev);
+  n1 = r * __builtin_amdgcn_sinf(rev);
 }
 
-// Four standard normals for one counter value. Streams: 0 = output noise, 1 = weight noise.
-AHL_DEV void normal4(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, uint64_t group,
-                     float* out4) {
+// Eight standard normals for one counter value.
+//   output noise: stream 0; group = ((m >> 4) * 2 + ((m >> 2) & 1)) * N + n; normal j belongs to
+//                 row 16 * (m >> 4) + 4 * ((m >> 2) & 1) + (j & 3) + 8 * (j >> 2)  -- the 8 rows one
+//                 lane of a 32x32 MFMA result holds in two consecutive register groups
+//   weight noise: stream 1, tile field 0; group = n * ceil(K / 8) + (k >> 3); normal j is k % 8
+AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, uint64_t group,
+                     float* out8) {
   u32x4 c = {(uint32_t)group, (uint32_t)(group >> 32), stream_and_tile, (uint32_t)offset};
   const u32x4 r = philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
-  box_muller(r.x, r.y, out4[0], out4[1]);
-  box_muller(r.z, r.w, out4[2], out4[3]);
+  box_muller16(r.x, out8[0], out8[1]);
+  box_muller16(r.y, out8[2], out8[3]);
+  box_muller16(r.z, out8[4], out8[5]);
+  box_muller16(r.w, out8[6], out8[7]);
 }
 
 // ---------------------------------------------------------------------------------------------

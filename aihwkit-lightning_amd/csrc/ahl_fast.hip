@@ -1,0 +1,475 @@
+// bf16 fast path of the analog forward.
+//
+// Why the DAC is a separate pass here: quantising an A element costs ~7 VALU instructions
+// (clamp, scale, two bf16 roundings, round-to-even, rescale) and a block that owns BN output
+// columns repeats that work for every one of the N/BN column blocks. At BN = 128 this is ~1.75x
+// the MFMA time of the block, on top of a per-tile epilogue that is already VALU-bound. One
+// memory-bound pass (k_dac_rows: read x once, write xq once, dynamic abs-max fused in) removes
+// that redundancy; the GEMM then streams xq through LDS untouched. The fused-prologue kernel
+// (ahl_gemm.hip) stays for fp32 and for shapes this path does not take.
+//
+// k_fwd_fast: block 256 threads = 2x2 waves, block tile 128 x 128, wave tile 64 x 64, chunks of 64
+// k; accumulator of the running K-tile in fp32 (64 registers), running total packed as bf16
+// pairs (32 registers) -- the total is a bf16 quantity by the semantics of the path -- so two to
+// three blocks fit on a CU and the VALU epilogue of one overlaps the MFMA phase of another.
+#include "ahl_host.h"
+#include <math.h>
+
+namespace ahl {
+
+static constexpr int kLdsStrideF = 144;            // bytes; 128 data + 16 pad
+static constexpr int kChunkLdsF = 128 * kLdsStrideF;
+
+// round two fp32 values to bf16 precision, keeping them in fp32 registers (3 instructions)
+AHL_DEV void rd2(float& a, float& b) {
+  const uint32_t p = pack_bf16x2(a, b);
+  a = unpack_lo(p);
+  b = unpack_hi(p);
+}
+
+// -------------------------------------------------------------------------------------------
+// DAC pre-pass, one wave per row: xq[m, k] = DAC(clamp(x[m, k])) with the input range of k's
+// tile. Dynamic mode: the range is the row's abs-max inside the tile and is written to
+// ir_out[t, m]. Generic in dtype and alignment.
+template <class D, bool VEC, int IRMODE>
+__global__ __launch_bounds__(256) void k_dac_rows(const void* __restrict__ x, int64_t ldx,
+                                                  void* __restrict__ xq, int64_t ldq,
+                                                  const void* __restrict__ ir_in,
+                                                  void* __restrict__ ir_out, int64_t M, Tiling tl,
+                                                  float inp_res, int32_t dac_on,
+                                                  int32_t skip_rounding) {
+  const int lane = threadIdx.x & 63;
+  const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= M) return;
+  constexpr int E = D::EPV;
+  const typename D::elem* row = (const typename D::elem*)x + m * ldx;
+  typename D::elem* qrow = (typename D::elem*)xq + m * ldq;
+  for (int32_t t = 0; t < tl.n_tiles; ++t) {
+    const int32_t c0 = tl.start(t), c1 = tl.start(t + 1);
+    float irv;
+    if (IRMODE == AHL_IR_DYNAMIC) {
+      float mx = 0.0f;
+      wave_row_foreach<D, VEC>(row, c0, c1, lane, [&](float v) { mx = fmaxf(mx, fabsf(v)); });
+      irv = wave_max(mx);
+      if (lane == 0) D::store(ir_out, (int64_t)t * M + m, irv);
+    } else {
+      irv = D::load(ir_in, t);
+    }
+    const Dac dac = make_dac<D>(irv, inp_res);
+    auto f = [&](float v) -> float {
+      if (dac_on) return dac_apply<D, IRMODE == AHL_IR_STATIC, true>(v, dac, skip_rounding != 0);
+      return dac_apply<D, IRMODE == AHL_IR_STATIC, false>(v, dac, false);
+    };
+    if (VEC) {  // tile bounds are multiples of E on this path
+      for (int32_t v = c0 / E + lane; v < c1 / E; v += 64) {
+        float e[E];
+        D::unpack(ld16(row + (int64_t)v * E), e);
+#pragma unroll
+        for (int i = 0; i < E; ++i) e[i] = f(e[i]);
+        st16(qrow + (int64_t)v * E, D::pack(e));
+      }
+    } else {
+      for (int32_t c = c0 + lane; c < c1; c += 64) D::store(qrow, c, f(D::load(row, c)));
+    }
+  }
+}
+
+// -------------------------------------------------------------------------------------------
+struct FastFwdArgs {
+  const void* xq; int64_t ldx;   // pre-quantised input, bf16 [M, K]
+  const void* w; int64_t ldw;    // effective weights, bf16 [N, K]
+  const void* bias;
+  void* y; int64_t ldy;
+  uint8_t* keep;                 // [planes, M, N] or null
+  uint32_t* clamp_flag;          // set to non-zero if any tile output was clamped; may be null
+  const void* ir;                // [T] static, [T, M] dynamic
+  const void* wmax;              // [T, N]
+  const float* tile_max;         // [T]
+  int64_t M, N;
+  int32_t K, tile;               // all tiles have `tile` columns (multiple of 64)
+  int32_t n_tiles;
+  float out_bound, out_res, two_inv_res;
+  float noise_scale;
+  int32_t noise_per_channel, bound_per_channel, skip_rounding, clamp_on, res_is_states, res_mul_exact;
+  uint64_t seed, offset;
+};
+
+AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                              __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// step of an ADC with bound B (bf16 value held in fp32)
+AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
+  if (a.res_is_states) {
+    // rd(rd(2B) / n): 2B is exact; for n with <= 8 significant bits the product with fl(2/n)
+    // rounds to the same bf16 as the quotient (see BF16::div), otherwise divide
+    return a.res_mul_exact ? BF16::rd(B * a.two_inv_res) : BF16::rd(__fdiv_rn(B + B, a.out_res));
+  }
+  return BF16::rd((B + B) * a.out_res);
+}
+
+template <int IRMODE, bool NOISE, bool ADC>
+__global__ __launch_bounds__(256, 2) void k_fwd_fast(FastFwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  char* ldsA = lds;
+  char* ldsB = lds + kChunkLdsF;
+  float* rowc = (float*)(lds + 2 * kChunkLdsF);  // dynamic mode: [2][3][128] per-row constants
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int row0 = tid >> 3, cv = tid & 7;
+  const int h = lane >> 5;
+
+  const int64_t nbn = cdiv_dev(a.N, 128);
+  const int64_t nb = gridDim.x;
+  int64_t logical = blockIdx.x;
+  if ((nb & 7) == 0) logical = (logical & 7) * (nb >> 3) + (logical >> 3);
+  const int64_t m0 = (logical / nbn) * 128, n0 = (logical % nbn) * 128;
+  const bool bound_on = ADC || a.clamp_on;
+  const bool full = (m0 + 128 <= a.M) && (n0 + 128 <= a.N);  // no edge predicates needed
+
+  f32x16 acc[2][2];
+  uint32_t totp[2][2][8];   // running total, bf16 pairs: [g*2 + (c>>1)] = rows c, c+1 of group g
+  uint32_t clampbits[2][2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+#pragma unroll
+      for (int v = 0; v < 8; ++v) totp[i][j][v] = 0u;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) clampbits[i][j][v] = 0u;
+    }
+  uint32_t any_clamp = 0u;
+
+  const uint16_t* A = (const uint16_t*)a.xq;
+  const uint16_t* Bw = (const uint16_t*)a.w;
+  u32x4 rawA[4], rawB[4];
+  auto load = [&](int32_t kc) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t ra = m0 + row0 + 32 * j, rb = n0 + row0 + 32 * j;
+      u32x4 z = {0u, 0u, 0u, 0u};
+      rawA[j] = ra < a.M ? ld16(A + ra * a.ldx + kc + cv * 8) : z;
+      rawB[j] = rb < a.N ? ld16(Bw + rb * a.ldw + kc + cv * 8) : z;
+    }
+  };
+  load(0);
+  const int nchunks = a.K / 64, cpt = a.tile / 64;
+  int t = 0, cin = 0;
+  for (int ch = 0; ch < nchunks; ++ch) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      *(u32x4*)(ldsA + (row0 + 32 * j) * kLdsStrideF + cv * 16) = rawA[j];
+      *(u32x4*)(ldsB + (row0 + 32 * j) * kLdsStrideF + cv * 16) = rawB[j];
+    }
+    if (IRMODE == AHL_IR_DYNAMIC && cin == 0 && tid < 128) {
+      const int64_t m = m0 + tid;
+      const float irm = m < a.M ? BF16::load(a.ir, (int64_t)t * a.M + m) : 0.0f;
+      float* rc = rowc + (t & 1) * 384;
+      rc[tid] = BF16::rd(a.noise_scale * irm);
+      rc[128 + tid] = BF16::rd(irm * a.out_bound);
+    }
+    __syncthreads();
+    if (ch + 1 < nchunks) load((ch + 1) * 64);
+
+    {
+      const int r = lane & 31;
+      const char* pa = ldsA + (wm * 64 + r) * kLdsStrideF + h * 16;
+      const char* pb = ldsB + (wn * 64 + r) * kLdsStrideF + h * 16;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const u32x4 a0 = *(const u32x4*)(pa + s * 32);
+        const u32x4 a1 = *(const u32x4*)(pa + 32 * kLdsStrideF + s * 32);
+        const u32x4 b0 = *(const u32x4*)(pb + s * 32);
+        const u32x4 b1 = *(const u32x4*)(pb + 32 * kLdsStrideF + s * 32);
+        mma_bf16(a0, b0, acc[0][0]);
+        mma_bf16(a0, b1, acc[0][1]);
+        mma_bf16(a1, b0, acc[1][0]);
+        mma_bf16(a1, b1, acc[1][1]);
+      }
+    }
+
+    if (++cin < cpt) continue;
+    cin = 0;
+    // ---------------- per-K-tile epilogue ----------------
+    const float ir_t = IRMODE == AHL_IR_STATIC ? BF16::load(a.ir, t) : 0.0f;
+    const float tmax = (NOISE || bound_on) ? a.tile_max[t] : 0.0f;
+    const float* rc_t = rowc + (t & 1) * 384;
+    const bool flush = a.keep != nullptr && a.clamp_on && ((t & 7) == 7 || t == a.n_tiles - 1);
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+      const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
+      const bool nvalid = n < a.N;
+      float wch = 0.0f;
+      if ((NOISE || bound_on) && nvalid) wch = BF16::load(a.wmax, (int64_t)t * a.N + n);
+      const float wr = a.noise_per_channel ? wch : tmax;
+      const float wb = a.bound_per_channel ? wch : tmax;
+      float nscale = 0.0f, B = 0.0f, r = 1.0f, rcp = 1.0f;
+      if (IRMODE == AHL_IR_STATIC) {
+        if (NOISE) nscale = BF16::rd(wr * BF16::rd(a.noise_scale * ir_t));
+        if (bound_on) {
+          B = BF16::rd(BF16::rd(ir_t * a.out_bound) * wb);
+          if (ADC) {
+            r = adc_step(B, a);
+            rcp = __fdiv_rn(1.0f, fmaxf(r, kTinyF32));
+          }
+        }
+      }
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi) {
+        const int rbase = wm * 64 + bi * 32 + 4 * h;
+#pragma unroll
+        for (int gp = 0; gp < 2; ++gp) {
+          float xi[8];
+          if (NOISE) {
+            const uint64_t mrow = (uint64_t)(m0 + rbase + 16 * gp);
+            const uint64_t grp = ((mrow >> 4) * 2 + ((mrow >> 2) & 1)) * (uint64_t)a.N + (uint64_t)n;
+            normal8(a.seed, a.offset, (uint32_t)t, grp, xi);
+          }
+#pragma unroll
+          for (int gg = 0; gg < 2; ++gg) {
+            const int g = 2 * gp + gg;
+            float y[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) { y[c] = acc[bi][bj][4 * g + c]; acc[bi][bj][4 * g + c] = 0.0f; }
+            rd2(y[0], y[1]); rd2(y[2], y[3]);
+            float ns[4], Bv[4], rv[4], rcpv[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) { ns[c] = nscale; Bv[c] = B; rv[c] = r; rcpv[c] = rcp; }
+            if (IRMODE == AHL_IR_DYNAMIC && (NOISE || bound_on)) {
+#pragma unroll
+              for (int c = 0; c < 4; ++c) {
+                const int rl = rbase + 8 * g + c;
+                if (NOISE) ns[c] = wr * rc_t[rl];
+                if (bound_on) Bv[c] = rc_t[128 + rl] * wb;
+              }
+              if (NOISE) { rd2(ns[0], ns[1]); rd2(ns[2], ns[3]); }
+              if (bound_on) {
+                rd2(Bv[0], Bv[1]); rd2(Bv[2], Bv[3]);
+                if (ADC) {
+#pragma unroll
+                  for (int c = 0; c < 4; ++c) {
+                    rv[c] = adc_step(Bv[c], a);
+                    rcpv[c] = __builtin_amdgcn_rcpf(fmaxf(rv[c], kTinyF32));
+                  }
+                }
+              }
+            }
+            if (NOISE) {
+              float nz[4];
+#pragma unroll
+              for (int c = 0; c < 4; ++c) nz[c] = ns[c] * xi[4 * gg + c];
+              rd2(nz[0], nz[1]); rd2(nz[2], nz[3]);
+#pragma unroll
+              for (int c = 0; c < 4; ++c) y[c] += nz[c];
+              rd2(y[0], y[1]); rd2(y[2], y[3]);
+            }
+            if (ADC) {
+#pragma unroll
+              for (int c = 0; c < 4; ++c) y[c] *= rcpv[c];
+              rd2(y[0], y[1]); rd2(y[2], y[3]);
+              if (!a.skip_rounding) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) y[c] = rintf(y[c]);
+              }
+#pragma unroll
+              for (int c = 0; c < 4; ++c) y[c] *= rv[c];
+              rd2(y[0], y[1]); rd2(y[2], y[3]);
+            }
+            if (a.clamp_on) {
+              bool over = false;
+#pragma unroll
+              for (int c = 0; c < 4; ++c) over |= !(fabsf(y[c]) <= Bv[c]);
+              if (__any(over)) {  // rare: some output of this group left the ADC range
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                  const bool cl = !(fabsf(y[c]) <= Bv[c]);
+                  clampbits[bi][bj][g] |= (cl ? 1u : 0u) << (8 * c + (t & 7));
+                  y[c] = fminf(fmaxf(y[c], -Bv[c]), Bv[c]);
+                }
+                any_clamp |= over ? 1u : 0u;
+              }
+            }
+            // total = rd(total + y), bf16 pairs
+#pragma unroll
+            for (int pr = 0; pr < 2; ++pr) {
+              const uint32_t tp = totp[bi][bj][2 * g + pr];
+              totp[bi][bj][2 * g + pr] =
+                  pack_bf16x2(unpack_lo(tp) + y[2 * pr], unpack_hi(tp) + y[2 * pr + 1]);
+            }
+          }
+          // keep the scheduler from interleaving the 8 Philox/Box-Muller chains of a block:
+          // that only lengthens live ranges (the chains of different waves overlap anyway)
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
+    if (flush) {
+      // one byte plane of the clamp mask for the last (up to) 8 tiles; addresses are a 64-bit
+      // base per lane plus 32-bit row offsets
+      const uint32_t valid = (2u << (t & 7)) - 1u;
+      const int64_t mrow0 = m0 + wm * 64 + 4 * h;
+      const int32_t mlim = (int32_t)((a.M - mrow0) < 64 ? (a.M - mrow0) : 64);
+      const int32_t ldn = (int32_t)a.N;
+#pragma unroll
+      for (int bj = 0; bj < 2; ++bj) {
+        const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
+        uint8_t* base = a.keep + ((int64_t)(t >> 3) * a.M + mrow0) * a.N + n;
+        const bool nvalid = n < a.N;
+#pragma unroll
+        for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              const int32_t ro = bi * 32 + 8 * g + c;
+              if (full || (nvalid && ro < mlim))
+                base[ro * ldn] = (uint8_t)(~(clampbits[bi][bj][g] >> (8 * c)) & valid);
+            }
+            clampbits[bi][bj][g] = 0u;
+          }
+      }
+    }
+    t += 1;
+  }
+
+  if (a.clamp_flag != nullptr && __any(any_clamp != 0u) && lane == 0) atomicOr(a.clamp_flag, 1u);
+
+  // ---- store y = total (+ bias) ----
+  {
+    const int64_t mrow0 = m0 + wm * 64 + 4 * h;
+    const int32_t mlim = (int32_t)((a.M - mrow0) < 64 ? (a.M - mrow0) : 64);
+    const int32_t ldy = (int32_t)a.ldy;
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj) {
+      const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
+      if (!full && n >= a.N) continue;
+      const float b = a.bias ? BF16::load(a.bias, n) : 0.0f;
+      uint16_t* base = (uint16_t*)a.y + mrow0 * a.ldy + n;
+#pragma unroll
+      for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int32_t ro = bi * 32 + 8 * (v >> 2) + (v & 3);
+          if (full || ro < mlim) {
+            const uint32_t tp = totp[bi][bj][v >> 1];
+            float o = (v & 1) ? unpack_hi(tp) : unpack_lo(tp);
+            if (a.bias) o = BF16::rd(o + b);
+            base[ro * ldy] = (uint16_t)f32_to_bf16_bits(o);
+          }
+        }
+    }
+  }
+}
+
+__global__ void k_zero_u32(uint32_t* p) { *p = 0u; }
+
+}  // namespace ahl
+
+using namespace ahl;
+
+static constexpr int kFastLds = 2 * kChunkLdsF + 2 * 384 * (int)sizeof(float);
+
+// number of significant bits of a positive float's significand
+static int significant_bits(float v) {
+  uint32_t u;
+  memcpy(&u, &v, 4);
+  uint32_t man = (u & 0x7fffffu) | 0x800000u;
+  int bits = 24;
+  while (bits > 1 && (man & 1u) == 0u) { man >>= 1; --bits; }
+  return bits;
+}
+
+template <int IRMODE>
+static void launch_fast(const FastFwdArgs& a, bool noise, bool adc, dim3 grid, hipStream_t s) {
+  const dim3 block(256);
+  if (noise) {
+    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, true>), grid, block, kFastLds, s, a);
+    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, false>), grid, block, kFastLds, s, a);
+  } else {
+    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, true>), grid, block, kFastLds, s, a);
+    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, false>), grid, block, kFastLds, s, a);
+  }
+}
+
+namespace ahl {
+
+// Whether ahl_linear_fwd can take the bf16 fast path for these arguments.
+bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, const void* w,
+                       int64_t ldw, int64_t K, const Tiling& tl) {
+  if (cfg->dtype != AHL_BF16 || xq == nullptr) return false;
+  if (tl.extra != 0 || tl.base % 64 != 0) return false;
+  if (!aligned16(xq) || !aligned16(w) || ldxq % 8 != 0 || ldw % 8 != 0) return false;
+  return K % 64 == 0;
+}
+
+int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
+                    void* y, int64_t ldy, uint8_t* keep, uint32_t* clamp_flag, const void* ir,
+                    const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
+                    const Tiling& tl, const AhlLinearCfg* cfg, hipStream_t s) {
+  FastFwdArgs a;
+  a.xq = xq; a.ldx = ldxq; a.w = w_eff; a.ldw = ldw; a.bias = bias; a.y = y; a.ldy = ldy;
+  a.keep = keep; a.clamp_flag = clamp_flag; a.ir = ir; a.wmax = wmax; a.tile_max = tile_max;
+  a.M = M; a.N = N; a.K = (int32_t)K; a.tile = tl.base; a.n_tiles = tl.n_tiles;
+  a.out_bound = cfg->out_bound; a.out_res = cfg->out_res;
+  const bool noise = cfg->training && cfg->out_noise > 0.0f;
+  const bool adc = cfg->out_res > 0.0f;
+  a.noise_scale = noise ? (float)((double)cfg->out_noise / sqrt((double)tl.n_tiles)) : 0.0f;
+  a.noise_per_channel = cfg->out_noise_per_channel; a.bound_per_channel = cfg->bound_per_channel;
+  a.skip_rounding = cfg->skip_rounding; a.clamp_on = cfg->out_bound > 0.0f ? 1 : 0;
+  a.res_is_states = cfg->out_res > 1.0f ? 1 : 0;
+  a.res_mul_exact = (adc && a.res_is_states && significant_bits(cfg->out_res) <= 8) ? 1 : 0;
+  a.two_inv_res = adc ? 2.0f / cfg->out_res : 0.0f;
+  a.seed = cfg->seed; a.offset = cfg->offset;
+  const int64_t nb = cdiv(M, 128) * cdiv(N, 128);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
+  const dim3 grid((unsigned)nb);
+  if (clamp_flag) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);
+  if (cfg->ir_mode == AHL_IR_NONE) launch_fast<0>(a, noise, adc, grid, s);
+  else if (cfg->ir_mode == AHL_IR_STATIC) launch_fast<1>(a, noise, adc, grid, s);
+  else launch_fast<2>(a, noise, adc, grid, s);
+  return check_launch("ahl_linear_fwd(fast)");
+}
+
+}  // namespace ahl
+
+#define AHL_DAC(V, I)                                                                          \
+  hipLaunchKernelGGL((k_dac_rows<D, V, I>), grid, block, 0, s, x, ldx, xq, ldxq, ir_in, ir_out, M, \
+                     tl, cfg->inp_res, dac_on, cfg->skip_rounding)
+
+extern "C" {
+
+int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_in, void* ir_out,
+            int64_t M, int64_t K, const int32_t* tile_ends_host, int32_t n_tiles,
+            const AhlLinearCfg* cfg, void* stream) {
+  if (!cfg || !x || !xq || M <= 0 || K <= 0 || ldx < K || ldxq < K) return AHL_ERR_ARG;
+  if (cfg->ir_mode == AHL_IR_STATIC && !ir_in) return AHL_ERR_ARG;
+  if (cfg->ir_mode == AHL_IR_DYNAMIC && !ir_out) return AHL_ERR_ARG;
+  if (cfg->ir_mode == AHL_IR_NONE && cfg->inp_res > 0.0f) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)cdiv(M, 4)), block(256);
+  const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
+  AHL_DISPATCH_DTYPE(cfg->dtype, {
+    const bool vec = aligned16(x) && aligned16(xq) && ldx % D::EPV == 0 && ldxq % D::EPV == 0 &&
+                     tl.extra == 0 && tl.base % D::EPV == 0;
+    if (vec) {
+      if (cfg->ir_mode == AHL_IR_NONE) { AHL_DAC(true, 0); }
+      else if (cfg->ir_mode == AHL_IR_STATIC) { AHL_DAC(true, 1); }
+      else { AHL_DAC(true, 2); }
+    } else {
+      if (cfg->ir_mode == AHL_IR_NONE) { AHL_DAC(false, 0); }
+      else if (cfg->ir_mode == AHL_IR_STATIC) { AHL_DAC(false, 1); }
+      else { AHL_DAC(false, 2); }
+    }
+  });
+  return check_launch("ahl_dac");
+}
+
+}  // extern "C"

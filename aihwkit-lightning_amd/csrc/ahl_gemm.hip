@@ -267,44 +267,50 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
         for (int bi = 0; bi < 2; ++bi) {
           const int rbase = wm * 64 + bi * 32 + 4 * h;  // block-local row of v = 0
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            float xi[4] = {0.f, 0.f, 0.f, 0.f};
+          for (int gp = 0; gp < 2; ++gp) {
+            float xi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             if (a.noise_on) {
-              const uint64_t mg = (uint64_t)(m0 + rbase + 8 * g) >> 2;
-              normal4(a.seed, a.offset, (uint32_t)t, mg * (uint64_t)a.N + (uint64_t)n, xi);
+              // rows m0 + rbase + 16 * gp + {0..3, 8..11}: one Philox call per lane and pair of groups
+              const uint64_t mrow = (uint64_t)(m0 + rbase + 16 * gp);
+              const uint64_t grp = ((mrow >> 4) * 2 + ((mrow >> 2) & 1)) * (uint64_t)a.N + (uint64_t)n;
+              normal8(a.seed, a.offset, (uint32_t)t, grp, xi);
             }
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-              const int v = 4 * g + c;
-              const int rl = rbase + 8 * g + c;
-              float y = D::rd(acc[bi][bj][v]);
-              acc[bi][bj][v] = 0.0f;
-              if (IRMODE == AHL_IR_DYNAMIC && (a.noise_on || a.bound_on)) {
-                const float irm = rowir[(t & 1) * 128 + rl];
-                if (a.noise_on) nscale = D::rd(wr * D::rd(a.noise_scale * irm));
-                if (a.bound_on) {
-                  B = D::rd(D::rd(irm * a.out_bound) * wb);
-                  if (a.adc_on) {
-                    r = quant_step<D>(B, a.out_res);
-                    rc = fmaxf(r, kTinyF32);
-                    rcp = __fdiv_rn(1.0f, rc);
+            for (int gg = 0; gg < 2; ++gg) {
+              const int g = 2 * gp + gg;
+#pragma unroll
+              for (int c = 0; c < 4; ++c) {
+                const int v = 4 * g + c;
+                const int rl = rbase + 8 * g + c;
+                float y = D::rd(acc[bi][bj][v]);
+                acc[bi][bj][v] = 0.0f;
+                if (IRMODE == AHL_IR_DYNAMIC && (a.noise_on || a.bound_on)) {
+                  const float irm = rowir[(t & 1) * 128 + rl];
+                  if (a.noise_on) nscale = D::rd(wr * D::rd(a.noise_scale * irm));
+                  if (a.bound_on) {
+                    B = D::rd(D::rd(irm * a.out_bound) * wb);
+                    if (a.adc_on) {
+                      r = quant_step<D>(B, a.out_res);
+                      rc = fmaxf(r, kTinyF32);
+                      rcp = __fdiv_rn(1.0f, rc);
+                    }
                   }
                 }
-              }
-              if (a.noise_on) y = D::rd(y + D::rd(nscale * D::rd(xi[c])));
-              if (a.bound_on) {
-                if (a.adc_on) {
-                  float q = D::rd(D::div(y, rc, rcp));
-                  if (!a.skip_rounding) q = rintf(q);
-                  y = D::rd(q * r);
+                if (a.noise_on) y = D::rd(y + D::rd(nscale * xi[4 * gg + c]));
+                if (a.bound_on) {
+                  if (a.adc_on) {
+                    float q = D::rd(D::div(y, rc, rcp));
+                    if (!a.skip_rounding) q = rintf(q);
+                    y = D::rd(q * r);
+                  }
+                  if (a.clamp_on) {
+                    const bool kp = (y >= -B) && (y <= B);
+                    keepbits[bi][bj][g] |= (kp ? 1u : 0u) << (8 * c + (t & 7));
+                    y = fminf(fmaxf(y, -B), B);
+                  }
                 }
-                if (a.clamp_on) {
-                  const bool kp = (y >= -B) && (y <= B);
-                  keepbits[bi][bj][g] |= (kp ? 1u : 0u) << (8 * c + (t & 7));
-                  y = fminf(fmaxf(y, -B), B);
-                }
+                total[bi][bj][v] = D::rd(total[bi][bj][v] + y);
               }
-              total[bi][bj][v] = D::rd(total[bi][bj][v] + y);
             }
           }
           // flush one plane of the clamp mask every 8 tiles
@@ -354,6 +360,7 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
 struct DxArgs {
   const void* g; int64_t ldg;
   const uint8_t* keep;
+  const uint32_t* clamp_flag;
   const void* wt;  // w_eff_t [K, N]
   const void* x; int64_t ldx;
   const void* ir;
@@ -414,7 +421,8 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
   const int64_t m0 = (logical / nkb) * kBM;
   int t; int32_t c0, c1;
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
-  const uint8_t* plane = a.keep ? a.keep + (int64_t)(t >> 3) * a.M * a.N : nullptr;
+  const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
+  const uint8_t* plane = use_keep ? a.keep + (int64_t)(t >> 3) * a.M * a.N : nullptr;
   const int bit = t & 7;
 
   f32x16 acc[2][2];
@@ -530,6 +538,7 @@ __global__ __launch_bounds__(64) void k_ir_grad_finalize(const float* __restrict
 struct DwArgs {
   const void* gt;       // [N, M]
   const uint8_t* keept; // [P, N, M] or null
+  const uint32_t* clamp_flag;
   const void* xqt;      // [K, M]
   void* dw; int64_t lddw;
   int64_t M, N, K;
@@ -552,7 +561,8 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dw(DwArgs a) {
   const int64_t n0 = (logical / nkb) * kBM;
   int t; int32_t c0, c1;
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
-  const uint8_t* plane = a.keept ? a.keept + (int64_t)(t >> 3) * a.N * a.M : nullptr;
+  const bool use_keep = a.keept != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
+  const uint8_t* plane = use_keep ? a.keept + (int64_t)(t >> 3) * a.N * a.M : nullptr;
   const int bit = t & 7;
 
   f32x16 acc[2][2];
@@ -673,6 +683,16 @@ static bool cfg_ok(const AhlLinearCfg* c) {
   return true;
 }
 
+namespace ahl {
+bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, const void* w,
+                       int64_t ldw, int64_t K, const Tiling& tl);
+int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
+                    void* y, int64_t ldy, uint8_t* keep, uint32_t* clamp_flag, const void* ir,
+                    const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
+                    const Tiling& tl, const AhlLinearCfg* cfg, hipStream_t s);
+__global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
+}  // namespace ahl
+
 template <class D>
 static bool tiles_vec_ok(const Tiling& tl) {
   return tl.extra == 0 ? (tl.base % D::EPV == 0) : false;
@@ -710,15 +730,26 @@ static void launch_dx(const DxArgs& a, bool is_static, dim3 grid, hipStream_t s)
 
 extern "C" {
 
-int ahl_linear_fwd(const void* x, int64_t ldx, const void* w_eff, int64_t ldw, const void* bias,
-                   void* y, int64_t ldy, uint8_t* keep, const void* ir, const void* wmax,
-                   const float* tile_max, int64_t M, int64_t K, int64_t N,
-                   const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
-                   void* stream) {
-  if (!cfg_ok(cfg) || !x || !w_eff || !y || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
-  if (ldx < K || ldw < K || ldy < N) return AHL_ERR_ARG;
+int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* w_eff,
+                   int64_t ldw, const void* bias, void* y, int64_t ldy, uint8_t* keep,
+                   uint32_t* clamp_flag, const void* ir, const void* wmax, const float* tile_max,
+                   int64_t M, int64_t K, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
+                   const AhlLinearCfg* cfg, void* stream) {
+  if (!cfg_ok(cfg) || (!x && !xq) || !w_eff || !y || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
+  if ((x && ldx < K) || (xq && ldxq < K) || ldw < K || ldy < N) return AHL_ERR_ARG;
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  {
+    const bool noise_on = cfg->training && cfg->out_noise > 0.0f;
+    const bool bound_on = cfg->out_res > 0.0f || cfg->out_bound > 0.0f;
+    if (cfg->ir_mode == AHL_IR_NONE && (cfg->inp_res > 0.0f || bound_on || noise_on)) return AHL_ERR_ARG;
+    if (cfg->ir_mode != AHL_IR_NONE && !ir) return AHL_ERR_ARG;
+    if ((noise_on || bound_on) && (!wmax || !tile_max)) return AHL_ERR_ARG;
+  }
+  if (fast_fwd_eligible(cfg, xq, ldxq, w_eff, ldw, K, tl))
+    return launch_fast_fwd(xq, ldxq, w_eff, ldw, bias, y, ldy, keep, clamp_flag, ir, wmax, tile_max,
+                           M, K, N, tl, cfg, (hipStream_t)stream);
+  if (!x) return AHL_ERR_UNSUPPORTED;  // only the fast path can start from xq alone
   FwdArgs a;
   a.x = x; a.ldx = ldx; a.w = w_eff; a.ldw = ldw; a.bias = bias; a.y = y; a.ldy = ldy;
   a.keep = keep; a.ir = ir; a.wmax = wmax; a.tile_max = tile_max; a.M = M; a.N = N; a.tl = tl;
@@ -739,6 +770,8 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* w_eff, int64_t ldw, c
   const int64_t nb = cdiv(M, kBM) * cdiv(N, kBN);
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   const dim3 grid((unsigned)nb);
+  // this kernel does not track clamping: tell the backward to honour the mask
+  if (clamp_flag) hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, s, clamp_flag, 1u);
   if (cfg->dtype == AHL_F32) launch_fwd<F32>(a, cfg->ir_mode, grid, s);
   else launch_fwd<BF16>(a, cfg->ir_mode, grid, s);
   return check_launch("ahl_linear_fwd");
@@ -758,9 +791,9 @@ int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int32_t n_tiles) {
   return cdiv(M, kBM) * nkb * 4 * (int64_t)sizeof(float);
 }
 
-int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const void* w_eff_t,
-                      const void* x, int64_t ldx, const void* ir, void* dx, int64_t lddx,
-                      void* ir_grad, int64_t M, int64_t K, int64_t N,
+int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                      const void* w_eff_t, const void* x, int64_t ldx, const void* ir, void* dx,
+                      int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream) {
   if (!cfg_ok(cfg) || !g || !w_eff_t || !dx || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
@@ -770,7 +803,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const voi
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   DxArgs a;
-  a.g = g; a.ldg = ldg; a.keep = keep; a.wt = w_eff_t; a.x = x; a.ldx = ldx; a.ir = ir;
+  a.g = g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.wt = w_eff_t; a.x = x; a.ldx = ldx; a.ir = ir;
   a.dx = dx; a.lddx = lddx; a.partial = (float*)ws; a.M = M; a.N = N; a.K = K; a.tl = tl;
   kblocks(tl, &a.kb_big, &a.kb_small);
   const int64_t nkb = (int64_t)tl.extra * a.kb_big + (int64_t)(n_tiles - tl.extra) * a.kb_small;
@@ -800,13 +833,14 @@ int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
   return b;
 }
 
-int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const void* x, int64_t ldx,
-                      const void* ir, void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
+int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                      const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* ir,
+                      void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream) {
-  if (!cfg_ok(cfg) || !g || !x || !dw || !ws || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
-  if (ldg < N || ldx < K || lddw < K) return AHL_ERR_ARG;
-  if (cfg->ir_mode != AHL_IR_NONE && !ir) return AHL_ERR_ARG;
+  if (!cfg_ok(cfg) || !g || (!x && !xq) || !dw || !ws || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
+  if (ldg < N || (x && ldx < K) || (xq && ldxq < K) || lddw < K) return AHL_ERR_ARG;
+  if (!xq && cfg->ir_mode != AHL_IR_NONE && !ir) return AHL_ERR_ARG;
   if (!aligned16(ws)) return AHL_ERR_WORKSPACE;
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
@@ -832,13 +866,15 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const voi
       const dim3 tgrid_k((unsigned)cdiv(N, 64), (unsigned)cdiv(M, 64), (unsigned)planes);
       hipLaunchKernelGGL((k_transpose<uint8_t>), tgrid_k, dim3(256), 0, s, keep, M, N, N, keept, M);
     }
-    if (cfg->ir_mode == AHL_IR_NONE)
+    if (xq)
+      hipLaunchKernelGGL((k_transpose<E>), tgrid_x, dim3(256), 0, s, (const E*)xq, M, K, ldxq, xqt, M);
+    else if (cfg->ir_mode == AHL_IR_NONE)
       hipLaunchKernelGGL((k_dac_transpose<D, 0>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
     else if (cfg->ir_mode == AHL_IR_STATIC)
       hipLaunchKernelGGL((k_dac_transpose<D, 1>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
     else
       hipLaunchKernelGGL((k_dac_transpose<D, 2>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
-    a.gt = gt; a.keept = keept; a.xqt = xqt;
+    a.gt = gt; a.keept = keept; a.xqt = xqt; a.clamp_flag = clamp_flag;
     const bool vec = M % D::EPV == 0;
     const dim3 grid((unsigned)(nbn * nkb)), block(256);
     if (vec) hipLaunchKernelGGL((k_linear_bwd_dw<D, true>), grid, block, kGemmLds, s, a);

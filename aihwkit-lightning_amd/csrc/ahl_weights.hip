@@ -49,22 +49,22 @@ struct ModArgs {
   uint64_t seed, offset;
 };
 
-// 64 (channels) x 64 (inputs) tile per block; thread = 4 consecutive inputs x 4 channels.
+// 64 (channels) x 64 (inputs) tile per block; thread = 8 consecutive inputs x 2 channels.
 template <class D>
 __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a) {
   __shared__ typename D::elem tileT[64][64 + 4];
   const int k0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
-  const int kq = threadIdx.x & 15, nr = threadIdx.x >> 4;
-  const int64_t kgroups = (a.K + 3) >> 2;
+  const int kq = threadIdx.x & 7, nr = threadIdx.x >> 3;
+  const int64_t kgroups = (a.K + 7) >> 3;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t n = n0 + nr + 16 * j;
-    const int kb = k0 + 4 * kq;
-    float xi[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < 2; ++j) {
+    const int64_t n = n0 + nr + 32 * j;
+    const int kb = k0 + 8 * kq;
+    float xi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (a.noise_type != AHL_NOISE_NONE && n < a.N && kb < a.K)
-      normal4(a.seed, a.offset, 1u << 24, (uint64_t)n * (uint64_t)kgroups + (uint64_t)(kb >> 2), xi);
+      normal8(a.seed, a.offset, 1u << 24, (uint64_t)n * (uint64_t)kgroups + (uint64_t)(kb >> 3), xi);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < 8; ++e) {
       const int k = kb + e;
       float v = 0.0f;
       if (n < a.N && k < a.K) {
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a) {
         }
         if (a.w_eff) D::store(a.w_eff, n * a.ld_eff + k, v);
       }
-      tileT[4 * kq + e][nr + 16 * j] = D::to_elem(v);
+      tileT[8 * kq + e][nr + 32 * j] = D::to_elem(v);
     }
   }
   if (!a.w_eff_t) return;

@@ -1,0 +1,202 @@
+"""Benchmark of the AnalogLinear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
+
+Workload (the configuration the headline metric is quoted on): one AnalogLinear 4096 -> 4096,
+bf16, 8192 tokens, 8 analog tiles of 512 inputs, learned input range (decay 0.01), 8-bit DAC and
+ADC (out_bound 10), output noise 0.04, additive per-channel Gaussian weight noise 0.02, training
+mode; one step = forward + straight-through backward (dX, dW, dBias, d input_range) on
+synthetic N(0,1) inputs and N(0, 0.02^2) weights resident in HBM.
+
+Prints ONE JSON line: whole-step throughput in algorithmic TFLOP/s (3 GEMMs x 2*M*N*K), the
+roofline of the dominant kernel measured with HIP events on the launch stream, and the CPU
+baseline (the torch-mode oracle on the host cores, on a token subsample).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "aihwkit-lightning_amd"))
+sys.path.insert(0, ROOT)
+
+import torch  # noqa: E402
+
+M_TOKENS, K_IN, N_OUT, TILE = 8192, 4096, 4096, 512
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+
+
+def build_layer():
+    from aihwkit_lightning.nn import AnalogLinear
+    from aihwkit_lightning.simulator.configs import (
+        TorchInferenceRPUConfig, WeightClipType, WeightNoiseInjectionType,
+    )
+
+    cfg = TorchInferenceRPUConfig()
+    cfg.mapping.max_input_size = TILE
+    cfg.forward.inp_res = 254
+    cfg.forward.out_res = 254
+    cfg.forward.out_bound = 10.0
+    cfg.forward.out_noise = 0.04
+    cfg.clip.type = WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL
+    cfg.clip.sigma = 2.5
+    cfg.modifier.noise_type = WeightNoiseInjectionType.ADD_NORMAL_PER_CHANNEL
+    cfg.modifier.std_dev = 0.02
+    ir = cfg.pre_post.input_range
+    ir.enable, ir.dynamic, ir.learn_input_range = True, False, True
+    ir.init_value, ir.init_from_data, ir.decay, ir.input_min_percentage = 3.0, 0, 0.01, 0.95
+    gen = torch.Generator().manual_seed(2)
+    layer = AnalogLinear(K_IN, N_OUT, bias=True, dtype=torch.bfloat16, rpu_config=cfg)
+    layer.set_weights_and_biases(
+        (0.02 * torch.randn(N_OUT, K_IN, generator=gen)).to(torch.bfloat16),
+        torch.zeros(N_OUT, dtype=torch.bfloat16),
+    )
+    x = torch.randn(M_TOKENS, K_IN, generator=gen).to(torch.bfloat16)
+    g = torch.randn(M_TOKENS, N_OUT, generator=gen).to(torch.bfloat16)
+    return layer, x, g
+
+
+def event_time_ms(fn, reps):
+    """Average duration of fn() over `reps` back-to-back calls, HIP events on the current stream."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    fn()
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def kernel_rooflines(layer, x, g, reps):
+    """Per-kernel timings of the three MFMA kernels through the same custom ops the layer uses."""
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+    from aihwkit_lightning.nn.modules.hip_utils import library as L
+
+    in_sizes = layer.in_sizes
+    wmax, tile_max, _, w_eff, w_eff_t = OPS.weight_prep(
+        layer.weight.data, in_sizes, L.AHL_QUANT_NONE, L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02,
+        11, 1, True, True)
+    ir = layer.input_range.detach()
+    icfg = [L.AHL_IR_STATIC, 0, 1, 1, 0, 12345, 0]
+    fcfg = [254.0, 254.0, 10.0, 0.04, 0.01, 0.95]
+    xq, _ = OPS.dac(x, ir, in_sizes, icfg, fcfg)
+    y, keep, flag = OPS.linear_fwd(None, xq, w_eff, layer.bias.data, ir, wmax, tile_max, in_sizes, icfg,
+                                   fcfg, True)
+    flops = 2.0 * M_TOKENS * K_IN * N_OUT
+    out = {}
+    t = event_time_ms(lambda: OPS.linear_fwd(None, xq, w_eff, layer.bias.data, ir, wmax, tile_max,
+                                             in_sizes, icfg, fcfg, True), reps)
+    out["linear_fwd"] = t
+    t = event_time_ms(lambda: OPS.linear_bwd_dx(g, keep, flag, w_eff_t, x, ir, in_sizes, icfg, fcfg), reps)
+    out["linear_bwd_dx(+ir_grad)"] = t
+    t = event_time_ms(lambda: OPS.linear_bwd_dw(g, keep, flag, None, xq, ir, in_sizes, icfg, fcfg), reps)
+    out["linear_bwd_dw(+transposes)"] = t
+    out["dac"] = event_time_ms(lambda: OPS.dac(x, ir, in_sizes, icfg, fcfg), reps)
+    t = event_time_ms(lambda: OPS.weight_prep(layer.weight.data, in_sizes, L.AHL_QUANT_NONE,
+                                              L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02, 11, 1,
+                                              True, True), reps)
+    out["weight_prep"] = t
+    return out, flops
+
+
+def cpu_baseline(sample_tokens=1024):
+    """The torch-mode oracle (CPU restatement of the reference) on a token subsample."""
+    from oracle import torch_mode as om
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    gen = torch.Generator().manual_seed(2)
+    w = (0.02 * torch.randn(N_OUT, K_IN, generator=gen)).to(torch.bfloat16)
+    x = torch.randn(sample_tokens, K_IN, generator=gen).to(torch.bfloat16)
+    g = torch.randn(sample_tokens, N_OUT, generator=gen).to(torch.bfloat16)
+    b = torch.zeros(N_OUT, dtype=torch.bfloat16)
+    cfg = om.OracleCfg(max_input_size=TILE, inp_res=254, out_res=254, out_bound=10.0, out_noise=0.04,
+                       bound_per_channel=True, ir_mode=om.IR_STATIC, ir_decay=0.01,
+                       weight_noise=om.ADD_NORMAL_PER_CHANNEL, modifier_std=0.02)
+    ir = torch.full((K_IN // TILE,), 3.0, dtype=torch.bfloat16)
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        out, saved = om.linear_forward(x, w, b, cfg, ir, True)
+        om.linear_backward(g, saved)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    flops = 3 * 2.0 * sample_tokens * K_IN * N_OUT
+    return {
+        "value": flops / best / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"{sample_tokens} of {M_TOKENS} tokens, same layer, fwd+bwd, best of 2 "
+                  f"({best:.2f} s)",
+    }
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ns = parser.parse_args()
+    if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        sys.exit(2)
+
+    layer, x, g = build_layer()
+    layer = layer.cuda().train()
+    x = x.cuda().requires_grad_(True)
+    g = g.cuda()
+    torch.manual_seed(0)
+
+    def step():
+        x.grad = None
+        layer.zero_grad(set_to_none=True)
+        out = layer(x)
+        out.backward(g)
+
+    for _ in range(ns.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(ns.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / ns.steps * 1e3
+    step_flops = 3 * 2.0 * M_TOKENS * K_IN * N_OUT
+    value = step_flops / (ms_per_step * 1e-3) / 1e12
+
+    kernels, gemm_flops = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 5))
+    dom = max(("linear_fwd", "linear_bwd_dx(+ir_grad)", "linear_bwd_dw(+transposes)"),
+              key=lambda k: kernels[k])
+    achieved = gemm_flops / (kernels[dom] * 1e-3) / 1e12
+    result = {
+        "metric": "AnalogLinear fwd+bwd TFLOP/s (4096^2, 8192 tok, bf16) + % MFMA peak",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": ns.steps,
+        "warmup": ns.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": "AnalogLinear 4096->4096 bf16, 8192 tokens, 8 tiles x 512, learned input "
+                        "range (decay 0.01), 8-bit DAC/ADC, out_noise 0.04, weight noise 0.02 per "
+                        "channel, fwd+bwd",
+            "frac_of_bf16_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
+        },
+        "roofline": {
+            "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+            "ms_per_launch": {k: round(v, 4) for k, v in kernels.items()},
+        },
+    }
+    if not ns.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -167,10 +167,23 @@ int ahl_quantize_weights(void* w, int64_t N, int64_t K, int64_t ld, const int32_
 
 /* ---- the analog matrix product ------------------------------------------------------------ */
 
+/* Input-range clamp + DAC quantisation as one memory-bound pass over x[M, K]:
+ *   AHL_IR_STATIC : xq = DAC(clamp(x, -ir_in[t], ir_in[t]))            ir_in dtype [T]
+ *   AHL_IR_DYNAMIC: ir_out[t, m] = max_k |x[m, tile t]| (dtype [T, M]), xq = DAC(x) with it
+ *   AHL_IR_NONE   : xq = x
+ * Replaces torch_utils/torch_linear.py:155-192 (apply_input_range forward, dynamic abs-max,
+ * UniformQuantize of the input). ahl_linear_fwd accepts the result as `xq`.               */
+int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_in, void* ir_out,
+            int64_t M, int64_t K, const int32_t* tile_ends_host, int32_t n_tiles,
+            const AhlLinearCfg* cfg, void* stream);
+
 /* Forward of TorchLinear.linear (torch_utils/torch_linear.py:116-314) for x[M, K]:
- *   for every K-tile: clamp to the input range + DAC quantise (fused into the A-tile staging),
- *   MFMA product with w_eff[N, K], output noise, ADC quantise, clamp to the output bound;
- *   per-tile results summed in dtype; bias added last.
+ *   for every K-tile: clamp to the input range + DAC quantise, MFMA product with w_eff[N, K],
+ *   output noise, ADC quantise, clamp to the output bound; per-tile results summed in dtype;
+ *   bias added last.
+ *   x        dtype [M, K] raw input; the clamp + DAC then run fused in the A-tile staging.
+ *   xq       dtype [M, K] from ahl_dac, or NULL. bf16 calls whose tiles are equal multiples of
+ *            64 take a faster kernel when xq is given (x may then be NULL).
  *   ir       dtype [T] (AHL_IR_STATIC) or [T, M] (AHL_IR_DYNAMIC) or NULL (AHL_IR_NONE)
  *   wmax     dtype [T, N] from ahl_weight_prep, or NULL when neither noise nor bound is on
  *   tile_max float [T]    from ahl_weight_prep, or NULL likewise
@@ -179,33 +192,38 @@ int ahl_quantize_weights(void* w, int64_t N, int64_t K, int64_t ld, const int32_
  *   keep     uint8 [ceil(T/8), M, N] or NULL: bit (t%8) of plane t/8 is set where the tile-t
  *            output was inside [-bound, bound] (the clamp's gradient mask). Written only when
  *            out_bound > 0 and keep != NULL.
+ *   clamp_flag  uint32 [1] or NULL: receives non-zero if any tile output was clamped (or if the
+ *            kernel does not track it); the backward entry points skip `keep` when it is zero.
  * Slot of TritonLinear.forward, triton_utils/triton_linear.py:446-690.                   */
-int ahl_linear_fwd(const void* x, int64_t ldx, const void* w_eff, int64_t ldw, const void* bias,
-                   void* y, int64_t ldy, uint8_t* keep, const void* ir, const void* wmax,
-                   const float* tile_max, int64_t M, int64_t K, int64_t N,
-                   const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
-                   void* stream);
+int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* w_eff,
+                   int64_t ldw, const void* bias, void* y, int64_t ldy, uint8_t* keep,
+                   uint32_t* clamp_flag, const void* ir, const void* wmax, const float* tile_max,
+                   int64_t M, int64_t K, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
+                   const AhlLinearCfg* cfg, void* stream);
 
 /* Input gradient and input-range gradient (torch_utils/torch_linear.py:29-108 backward):
  *   d[:, tile t] = (g * keep_t) @ w_eff[:, tile t]      w_eff_t is the [K, N] transpose
  *   AHL_IR_STATIC: ir_grad[t] per reference InputRangeForward.backward (incl. decay switch),
  *                  dx zeroed where |x| > ir[t]; x[M, K] is the forward input.
  *   otherwise dx = d, ir_grad untouched.
+ *   clamp_flag: NULL, or the flag written by ahl_linear_fwd (keep is ignored when it reads 0).
  *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, n_tiles) bytes.
  * Slot of TritonLinear.backward, triton_utils/triton_linear.py:695-764.                  */
-int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const void* w_eff_t,
-                      const void* x, int64_t ldx, const void* ir, void* dx, int64_t lddx,
-                      void* ir_grad, int64_t M, int64_t K, int64_t N,
+int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                      const void* w_eff_t, const void* x, int64_t ldx, const void* ir, void* dx,
+                      int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
 int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int32_t n_tiles);
 
 /* Weight gradient: dw[:, tile t] = (g * keep_t)^T @ DAC(clamp(x[:, tile t])).
+ *   xq: the quantised input saved from the forward (ahl_dac), or NULL to re-quantise x here.
  *   ws needs ahl_linear_bwd_dw_ws_bytes(M, K, N, n_tiles, dtype, keep != NULL) bytes
- *   (transposed staging copies of g, keep and the re-quantised x).
+ *   (transposed staging copies of g, keep and the quantised input).
  * Same reference slot as ahl_linear_bwd_dx.                                               */
-int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const void* x, int64_t ldx,
-                      const void* ir, void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
+int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                      const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* ir,
+                      void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
