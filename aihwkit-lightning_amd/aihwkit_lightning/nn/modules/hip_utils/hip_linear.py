@@ -112,17 +112,16 @@ class HipLinear(Function):
 
         seed = draw_seed() if (noise_on or w_noise) else 0
         wmax = tile_max = None
-        w_eff, w_eff_t = weights_c, None
-        if m_rows > 0 and (need_wmax or need_dx):
+        w_eff = weights_c
+        if m_rows > 0 and need_wmax:
             res = float(modifier.res) if w_quant else 1.0
-            wmax, tile_max, _, eff, eff_t = OPS.weight_prep(
+            wmax, tile_max, _, eff = OPS.weight_prep(
                 weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
                 NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE, res,
-                float(modifier.std_dev), seed, 1, w_noise or w_quant, need_dx,
+                float(modifier.std_dev), seed, 1, w_noise or w_quant,
             )
             if w_noise or w_quant:
                 w_eff = eff
-            w_eff_t = eff_t if need_dx else None
 
         skip_rounding = 1 if os.environ.get("_AIHWKIT_NO_ROUNDING", False) else 0
         icfg = [
@@ -174,7 +173,8 @@ class HipLinear(Function):
         ctx.need_dx, ctx.need_dw, ctx.ir_needs_grad = need_dx, need_dw, ir_needs_grad
         need_x = (need_dx and ir_mode == L.AHL_IR_STATIC) or (need_dw and xq is None)
         ctx.save_for_backward(
-            x2 if need_x else None, xq if need_dw else None, w_eff_t,
+            x2 if need_x else None, xq if need_dw else None,
+            (w_eff if w_eff is not weights else weights.detach()) if need_dx else None,
             keep if want_keep else None, flag if want_keep else None,
             ir_dev.clone() if ir_mode == L.AHL_IR_STATIC else ir_dev,
         )
@@ -182,7 +182,7 @@ class HipLinear(Function):
 
     @staticmethod
     def backward(ctx, grad_out: Tensor):
-        x2, xq, w_eff_t, keep, flag, ir_dev = ctx.saved_tensors
+        x2, xq, w_eff, keep, flag, ir_dev = ctx.saved_tensors
         n_out = grad_out.size(-1)
         g2 = grad_out.reshape(-1, n_out)
         if g2.stride(-1) != 1 or (g2.size(0) > 1 and g2.stride(0) != n_out):
@@ -190,7 +190,7 @@ class HipLinear(Function):
         grad_inp = grad_w = grad_b = grad_ir = None
         if ctx.need_dx:
             dx, ir_grad = OPS.linear_bwd_dx(
-                g2, keep, flag, w_eff_t, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
+                g2, keep, flag, w_eff, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
                 ctx.in_sizes, ctx.icfg, ctx.fcfg,
             )
             if ctx.needs_input_grad[0]:

@@ -72,8 +72,7 @@ LIB.define("clip_weights(Tensor(a!) w, float sigma, int kind) -> ()")
 LIB.define("col_sum(Tensor x) -> Tensor")
 LIB.define(
     "weight_prep(Tensor w, int[] in_sizes, int quant_type, int noise_type, float res, "
-    "float std_dev, int seed, int offset, bool want_eff, bool want_eff_t) "
-    "-> (Tensor, Tensor, Tensor, Tensor, Tensor)"
+    "float std_dev, int seed, int offset, bool want_eff) -> (Tensor, Tensor, Tensor, Tensor)"
 )
 LIB.define("quantize_weights(Tensor(a!) w, int[] in_sizes, int quant_type, float res) -> ()")
 LIB.define(
@@ -85,7 +84,7 @@ LIB.define(
     "-> (Tensor, Tensor, Tensor)"
 )
 LIB.define(
-    "linear_bwd_dx(Tensor g, Tensor? keep, Tensor? clamp_flag, Tensor w_eff_t, Tensor? x, "
+    "linear_bwd_dx(Tensor g, Tensor? keep, Tensor? clamp_flag, Tensor w_eff, Tensor? x, "
     "Tensor? ir, int[] in_sizes, int[] icfg, float[] fcfg) -> (Tensor, Tensor)"
 )
 LIB.define(
@@ -201,9 +200,9 @@ def _modifier_cfg(dtype, quant_type, noise_type, res, std_dev, seed, offset) -> 
 
 def weight_prep(
     w: Tensor, in_sizes: List[int], quant_type: int, noise_type: int, res: float, std_dev: float,
-    seed: int, offset: int, want_eff: bool, want_eff_t: bool,
-) -> Tuple[Tensor, Tensor, Tensor, Tensor, Tensor]:
-    """wmax ``[T, N]``, tile max/min ``[T]``, optional modified copy ``[N, K]`` and its transpose."""
+    seed: int, offset: int, want_eff: bool,
+) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
+    """wmax ``[T, N]``, tile max/min ``[T]`` and, if wanted, the modified copy ``[N, K]``."""
     lib = L.load()
     if w.dim() != 2 or w.stride(1) != 1:
         raise HipBackendError("weight must be a row-major 2-D tensor")
@@ -214,17 +213,15 @@ def weight_prep(
     tile_max = torch.empty((n_tiles,), dtype=torch.float32, device=dev)
     tile_min = torch.empty((n_tiles,), dtype=torch.float32, device=dev)
     w_eff = torch.empty((n_out, n_in) if want_eff else (0,), dtype=w.dtype, device=dev)
-    w_eff_t = torch.empty((n_in, n_out) if want_eff_t else (0,), dtype=w.dtype, device=dev)
     cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset)
     L.check(
         lib.ahl_weight_prep(
             _ptr(w), n_out, n_in, _ld(w), L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(wmax),
-            _ptr(tile_max), _ptr(tile_min), _ptr(w_eff) if want_eff else None, n_in,
-            _ptr(w_eff_t) if want_eff_t else None, _stream(),
+            _ptr(tile_max), _ptr(tile_min), _ptr(w_eff) if want_eff else None, n_in, _stream(),
         ),
         "ahl_weight_prep",
     )
-    return wmax, tile_max, tile_min, w_eff, w_eff_t
+    return wmax, tile_max, tile_min, w_eff
 
 
 def quantize_weights(w: Tensor, in_sizes: List[int], quant_type: int, res: float) -> None:
@@ -301,7 +298,7 @@ def linear_fwd(
 
 
 def linear_bwd_dx(
-    g: Tensor, keep: Optional[Tensor], clamp_flag: Optional[Tensor], w_eff_t: Tensor,
+    g: Tensor, keep: Optional[Tensor], clamp_flag: Optional[Tensor], w_eff: Tensor,
     x: Optional[Tensor], ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
     fcfg: List[float],
 ) -> Tuple[Tensor, Tensor]:
@@ -309,19 +306,19 @@ def linear_bwd_dx(
     lib = L.load()
     g = _rows2d(g, "g")
     m_rows, n_out = g.shape
-    k_in = w_eff_t.size(0)
+    k_in = w_eff.size(1)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(g.dtype, icfg, fcfg)
     static = cfg.ir_mode == L.AHL_IR_STATIC
     dx = torch.empty((m_rows, k_in), dtype=g.dtype, device=g.device)
     ir_grad = torch.empty((n_tiles,) if static else (0,), dtype=g.dtype, device=g.device)
-    ws = torch.empty((max(lib.ahl_linear_bwd_dx_ws_bytes(m_rows, k_in, n_tiles), 16),),
+    ws = torch.empty((lib.ahl_linear_bwd_dx_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype),),
                      dtype=torch.uint8, device=g.device)
     if x is not None:
         x = _rows2d(x, "x")
     L.check(
         lib.ahl_linear_bwd_dx(
-            _ptr(g), _ld(g), _ptr(keep), _ptr(clamp_flag), _ptr(w_eff_t), _ptr(x),
+            _ptr(g), _ld(g), _ptr(keep), _ptr(clamp_flag), _ptr(w_eff), _ld(w_eff), _ptr(x),
             _ld(x) if x is not None else 0, _ptr(ir), _ptr(dx), k_in,
             _ptr(ir_grad) if static else None, m_rows, k_in, n_out, L.tile_ends_array(in_sizes),
             n_tiles, byref(cfg), _ptr(ws), _stream(),

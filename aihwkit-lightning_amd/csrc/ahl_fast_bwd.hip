@@ -1,0 +1,280 @@
+// bf16 fast path of the backward products.
+//
+//   dX[m, k] = sum_n gy[m, n] * W_eff[n, k]        (MODE_DX)   gy = g, masked by keep bit t(k)
+//   dW[n, k] = sum_m gy[m, n] * xq[m, k]           (MODE_DW)
+//
+// Neither product has both operands contiguous along the contraction index in memory: W_eff
+// and xq (and g for dW) are stored with the contraction index as the ROW. Instead of
+// materialising transposed copies, those operands are staged in LDS as they are ("k-major":
+// [64 contraction rows][256 output columns]) and read with ds_read_b64_tr_b16, the CDNA4
+// transposing LDS read: within each group of 16 lanes, lane r supplies the address of 4
+// consecutive b16 of contraction row (r / 4), columns 4 * (r % 4) ..; lane i receives, for
+// column i of the 16-column block, the 4 values of the 4 contraction rows -- exactly the
+// "one column, consecutive k" shape of an MFMA operand register pair. Two such reads give the 8
+// bf16 of one v_mfma_f32_32x32x16_bf16 operand.
+//
+// Block: 512 threads = 8 waves as 2 (rows) x 4 (columns); block tile 256 x 256, wave tile
+// 128 x 64 (4 x 2 MFMA blocks, 128 fp32 accumulators), 64 contraction steps per chunk,
+// double-buffered LDS (2 x 72 KB), one barrier per chunk, next chunk's global loads in flight
+// during the MFMAs of the current one.
+#include "ahl_host.h"
+#include <type_traits>
+
+namespace ahl {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
+
+static constexpr int kRowkStride = 144;               // k-contiguous operand: 128 B + 16 B pad
+static constexpr int kKmajStride = 576;               // k-major operand: 512 B + 64 B pad
+static constexpr int kOperandLds = 256 * kRowkStride; // == 64 * kKmajStride == 36864
+static constexpr int kBwdLds = 4 * kOperandLds;       // 2 operands x 2 stages
+
+static constexpr int MODE_DX = 0;
+static constexpr int MODE_DW = 1;
+
+struct BwdArgs {
+  const uint16_t* g; int64_t ldg;      // [M, N]
+  const uint8_t* keep;                 // [planes, M, N] or null
+  const uint32_t* clamp_flag;          // null or the forward's flag
+  const uint16_t* b; int64_t ldb;      // DX: W_eff [N, K]; DW: xq [M, K]
+  const uint16_t* x; int64_t ldx;      // DX static range: the forward input [M, K]
+  const uint16_t* ir;                  // DX static range: [T]
+  uint16_t* out; int64_t ldo;          // DX: dx [M, K]; DW: dw [N, K]
+  float* partial;                      // DX static range: [blocks][4]
+  int64_t M, N, K;
+  int32_t tile;                        // K-tile width (multiple of 256)
+  int32_t ir_static;
+};
+
+AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                              __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// zero the elements of a vector of 8 bf16 whose mask byte has bit `bit` clear
+AHL_DEV u32x4 apply_keep(const u32x4& v, const uint8_t* q, int bit) {
+  const uint32_t w0 = *(const uint32_t*)q, w1 = *(const uint32_t*)(q + 4);
+  u32x4 o = v;
+  uint32_t m;
+  m = (((w0 >> bit) & 1u) ? 0xffffu : 0u) | (((w0 >> (8 + bit)) & 1u) ? 0xffff0000u : 0u); o.x &= m;
+  m = (((w0 >> (16 + bit)) & 1u) ? 0xffffu : 0u) | (((w0 >> (24 + bit)) & 1u) ? 0xffff0000u : 0u); o.y &= m;
+  m = (((w1 >> bit) & 1u) ? 0xffffu : 0u) | (((w1 >> (8 + bit)) & 1u) ? 0xffff0000u : 0u); o.z &= m;
+  m = (((w1 >> (16 + bit)) & 1u) ? 0xffffu : 0u) | (((w1 >> (24 + bit)) & 1u) ? 0xffff0000u : 0u); o.w &= m;
+  return o;
+}
+
+template <int MODE>
+__global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  __shared__ float red[8][3];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves
+  const int h = lane >> 5;
+
+  // ---- block -> output tile. columns of the output are k (both modes), 256 per block ----
+  const int64_t nkb = a.K / 256;
+  const int64_t nb = gridDim.x;
+  int64_t logical = blockIdx.x;
+  if ((nb & 7) == 0) logical = (logical & 7) * (nb >> 3) + (logical >> 3);
+  const int64_t r0 = (logical / nkb) * 256;          // DX: m0; DW: n0
+  const int64_t c0 = (logical % nkb) * 256;          // k0
+  const int t = (int)(c0 / a.tile);
+  const int64_t R = MODE == MODE_DX ? a.M : a.N;      // output rows
+  const int64_t L = MODE == MODE_DX ? a.N : a.M;      // contraction length
+  const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
+  const uint8_t* plane = use_keep ? a.keep + (int64_t)(t >> 3) * a.M * a.N : nullptr;
+  const int bit = t & 7;
+
+  f32x16 acc[4][2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  // ---- staging maps ----
+  // k-contiguous operand (DX: g rows m): vector j -> row tid/8 + 64 j, 16-byte column tid%8
+  // k-major operand: vector j -> contraction row tid/32 + 16 j, 16-byte column tid%32
+  const int rk_row = tid >> 3, rk_cv = tid & 7;
+  const int km_row = tid >> 5, km_cv = tid & 31;
+  u32x4 rawA[4], rawB[4];
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+  // Rows of the output tile that lie beyond the matrix are redirected to the last valid row:
+  // they only feed accumulators that are never stored. No predicates in the hot loop.
+  const uint16_t* pa[4];
+  const uint8_t* pk[4];
+  const uint16_t* pb[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (MODE == MODE_DX) {
+      int64_t m = r0 + rk_row + 64 * j;
+      m = m < a.M ? m : a.M - 1;
+      pa[j] = a.g + m * a.ldg + rk_cv * 8;              // + l0 (contraction n)
+      pk[j] = plane ? plane + m * a.N + rk_cv * 8 : nullptr;
+    } else {
+      int64_t n = r0 + km_cv * 8;
+      n = n < a.N ? n : a.N - 8;
+      pa[j] = a.g + (int64_t)(km_row + 16 * j) * a.ldg + n;  // + l0 * ldg (contraction m)
+      pk[j] = plane ? plane + (int64_t)(km_row + 16 * j) * a.N + n : nullptr;
+    }
+    pb[j] = a.b + (int64_t)(km_row + 16 * j) * a.ldb + c0 + km_cv * 8;  // + l0 * ldb
+  }
+  const int64_t a_step = MODE == MODE_DX ? 64 : 64 * a.ldg;
+  const int64_t k_step = MODE == MODE_DX ? 64 : 64 * a.N;
+  const int64_t b_step = 64 * a.ldb;
+  auto load = [&](bool masked) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      u32x4 v = ld16(pa[j]);
+      if (masked) { v = apply_keep(v, pk[j], bit); pk[j] += k_step; }
+      rawA[j] = v;
+      rawB[j] = ld16(pb[j]);
+      pa[j] += a_step;
+      pb[j] += b_step;
+    }
+  };
+  auto stage = [&](char* sa, char* sb) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if (MODE == MODE_DX) *(u32x4*)(sa + (rk_row + 64 * j) * kRowkStride + rk_cv * 16) = rawA[j];
+      else *(u32x4*)(sa + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawA[j];
+      *(u32x4*)(sb + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawB[j];
+    }
+  };
+
+  // transposing read of one MFMA operand (8 bf16 of column `col` at contraction rows
+  // 16 s + 8 h + 0..7) from a k-major LDS tile
+  const int tr_r = lane & 15, tr_g = (lane >> 4) & 1;
+  auto read_kmaj = [&](const char* base, int col0, int s) -> u32x4 {
+    const char* p = base + (16 * s + 8 * h + (tr_r >> 2)) * kKmajStride +
+                    (col0 + 16 * tr_g + 4 * (tr_r & 3)) * 2;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * kKmajStride));
+    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 o = {l2.x, l2.y, h2.x, h2.y};
+    return o;
+  };
+
+  const int nchunks = (int)(L / 64);
+  auto main_loop = [&](auto masked_tag) {
+    constexpr bool kMasked = decltype(masked_tag)::value;
+    load(kMasked);
+    stage(lds, lds + kOperandLds);
+    __syncthreads();
+    for (int ch = 0; ch < nchunks; ++ch) {
+      const char* sa = lds + (ch & 1) * 2 * kOperandLds;
+      const char* sb = sa + kOperandLds;
+      if (ch + 1 < nchunks) load(kMasked);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        u32x4 fa[4], fb[2];
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi) {
+          if (MODE == MODE_DX)
+            fa[bi] = *(const u32x4*)(sa + (wm * 128 + bi * 32 + (lane & 31)) * kRowkStride + s * 32 + h * 16);
+          else
+            fa[bi] = read_kmaj(sa, wm * 128 + bi * 32, s);
+        }
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj) fb[bj] = read_kmaj(sb, wn * 64 + bj * 32, s);
+#pragma unroll
+        for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+          for (int bj = 0; bj < 2; ++bj) mma16(fa[bi], fb[bj], acc[bi][bj]);
+      }
+      if (ch + 1 < nchunks) {
+        char* na = lds + ((ch + 1) & 1) * 2 * kOperandLds;
+        stage(na, na + kOperandLds);
+      }
+      __syncthreads();
+    }
+  };
+  if (plane) main_loop(std::true_type{});
+  else main_loop(std::false_type{});
+
+  // ---- epilogue ----
+  float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
+  const bool do_ir = MODE == MODE_DX && a.ir_static != 0;
+  const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
+  const int64_t row_w = r0 + wm * 128 + 4 * h;
+#pragma unroll
+  for (int bj = 0; bj < 2; ++bj) {
+    const int64_t k = c0 + wn * 64 + bj * 32 + (lane & 31);
+    uint16_t* obase = a.out + row_w * a.ldo + k;
+    const uint16_t* xbase = do_ir ? a.x + row_w * a.ldx + k : nullptr;
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
+        if (row_w + ro >= R) continue;
+        float d = BF16::rd(acc[bi][bj][v]);
+        if (do_ir) {
+          const float xv = bf16_bits_to_f32(xbase[(int64_t)ro * a.ldx]);
+          const bool up = xv >= ir_t, lo = xv <= -ir_t;
+          if (up) s_up += fminf(d, 0.0f);
+          if (lo) s_lo += fmaxf(d, 0.0f);
+          if (up || lo) cnt += 1.0f;
+          if (fabsf(xv) > ir_t) d = 0.0f;
+        }
+        obase[(int64_t)ro * a.ldo] = (uint16_t)f32_to_bf16_bits(d);
+      }
+  }
+  if (do_ir) {
+    s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
+    if (lane == 0) { red[wave][0] = s_up; red[wave][1] = s_lo; red[wave][2] = cnt; }
+    __syncthreads();
+    if (tid == 0) {
+      float u = 0.f, l = 0.f, c = 0.f;
+      for (int w = 0; w < 8; ++w) { u += red[w][0]; l += red[w][1]; c += red[w][2]; }
+      float* p = a.partial + logical * 4;
+      p[0] = u; p[1] = l; p[2] = c; p[3] = 0.0f;
+    }
+  }
+}
+
+// Whether the fast backward kernels can be used: bf16, equal K-tiles of a multiple of 256,
+// 16-byte aligned rows everywhere.
+bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N) {
+  if (dtype != AHL_BF16) return false;
+  if (tl.extra != 0 || tl.base % 256 != 0) return false;
+  // the contraction length (N for dX, M for dW) must be a multiple of 64 so that the hot loop
+  // needs no predicates; output rows beyond the matrix are handled by clamping the row index
+  return K % 256 == 0 && N % 64 == 0 && M % 64 == 0;
+}
+
+int launch_fast_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                   const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
+                   void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
+                   const Tiling& tl, bool ir_static, hipStream_t s) {
+  BwdArgs a;
+  a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
+  a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
+  a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial;
+  a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = ir_static ? 1 : 0;
+  const int64_t nb = cdiv(M, 256) * (K / 256);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
+  hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+  hipLaunchKernelGGL((k_bwd_fast<MODE_DX>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  return check_launch("ahl_linear_bwd_dx(fast)");
+}
+
+int launch_fast_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, int64_t M, int64_t K,
+                   int64_t N, const Tiling& tl, hipStream_t s) {
+  BwdArgs a;
+  a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
+  a.b = (const uint16_t*)xq; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;
+  a.out = (uint16_t*)dw; a.ldo = lddw; a.partial = nullptr;
+  a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = 0;
+  const int64_t nb = cdiv(N, 256) * (K / 256);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
+  hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+  hipLaunchKernelGGL((k_bwd_fast<MODE_DW>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  return check_launch("ahl_linear_bwd_dw(fast)");
+}
+
+}  // namespace ahl

@@ -691,6 +691,14 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
                     const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
                     const Tiling& tl, const AhlLinearCfg* cfg, hipStream_t s);
 __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
+bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N);
+int launch_fast_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                   const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
+                   void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
+                   const Tiling& tl, bool ir_static, hipStream_t s);
+int launch_fast_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, int64_t M, int64_t K,
+                   int64_t N, const Tiling& tl, hipStream_t s);
 }  // namespace ahl
 
 template <class D>
@@ -782,40 +790,71 @@ static void kblocks(const Tiling& tl, int32_t* kb_big, int32_t* kb_small) {
   *kb_small = (int32_t)cdiv(tl.base, kBN);
 }
 
-int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int32_t n_tiles) {
-  if (n_tiles <= 0 || K <= 0 || M <= 0) return 0;
+static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+static int64_t dx_partial_bytes(int64_t M, int64_t K, int32_t n_tiles) {
   Tiling tl{n_tiles, (int32_t)(K / n_tiles), (int32_t)(K % n_tiles)};
   int32_t kb, ks;
   kblocks(tl, &kb, &ks);
   const int64_t nkb = (int64_t)tl.extra * kb + (int64_t)(n_tiles - tl.extra) * ks;
-  return cdiv(M, kBM) * nkb * 4 * (int64_t)sizeof(float);
+  return align256(cdiv(M, kBM) * nkb * 4 * (int64_t)sizeof(float));
+}
+
+int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype) {
+  if (n_tiles <= 0 || K <= 0 || M <= 0 || N <= 0) return 0;
+  const int64_t es = dtype == AHL_BF16 ? 2 : 4;
+  return dx_partial_bytes(M, K, n_tiles) + align256(K * N * es);  // partials + transposed weights
 }
 
 int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
-                      const void* w_eff_t, const void* x, int64_t ldx, const void* ir, void* dx,
-                      int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
+                      const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
+                      void* dx, int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream) {
-  if (!cfg_ok(cfg) || !g || !w_eff_t || !dx || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
-  if (ldg < N || lddx < K) return AHL_ERR_ARG;
+  if (!cfg_ok(cfg) || !g || !w_eff || !dx || !ws || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
+  if (ldg < N || lddx < K || ldw < K) return AHL_ERR_ARG;
   const bool is_static = cfg->ir_mode == AHL_IR_STATIC;
-  if (is_static && (!x || !ir || !ir_grad || !ws || ldx < K)) return AHL_ERR_ARG;
+  if (is_static && (!x || !ir || !ir_grad || ldx < K)) return AHL_ERR_ARG;
+  if (!aligned16(ws)) return AHL_ERR_WORKSPACE;
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  float* partial = (float*)ws;
+  void* wt = (char*)ws + dx_partial_bytes(M, K, n_tiles);
+  const bool fast = fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(w_eff) &&
+                    ldg % 8 == 0 && ldw % 8 == 0 && lddx % 8 == 0 &&
+                    (!keep || (((uintptr_t)keep) & 7u) == 0) &&
+                    (!is_static || (ldx % 8 == 0 && aligned16(x)));
+  if (fast) {
+    int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
+                            N, tl, is_static, s);
+    if (rc != AHL_OK) return rc;
+    if (is_static) {
+      const int32_t per_tile = tl.base / 256;
+      hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
+                         (const float*)partial, cdiv(M, 256), (int32_t)(K / 256), per_tile, per_tile,
+                         tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
+    }
+    return check_launch("ahl_linear_bwd_dx(fast)");
+  }
   DxArgs a;
-  a.g = g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.wt = w_eff_t; a.x = x; a.ldx = ldx; a.ir = ir;
-  a.dx = dx; a.lddx = lddx; a.partial = (float*)ws; a.M = M; a.N = N; a.K = K; a.tl = tl;
+  a.g = g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.wt = wt; a.x = x; a.ldx = ldx;
+  a.ir = ir; a.dx = dx; a.lddx = lddx; a.partial = partial; a.M = M; a.N = N; a.K = K; a.tl = tl;
   kblocks(tl, &a.kb_big, &a.kb_small);
   const int64_t nkb = (int64_t)tl.extra * a.kb_big + (int64_t)(n_tiles - tl.extra) * a.kb_small;
   const int64_t mb = cdiv(M, kBM);
   if (mb * nkb > 0x7fffffff) return AHL_ERR_ARG;
-  hipStream_t s = (hipStream_t)stream;
+  const dim3 tgrid((unsigned)cdiv(K, 64), (unsigned)cdiv(N, 64), 1);
+  if (cfg->dtype == AHL_F32)
+    hipLaunchKernelGGL((k_transpose<float>), tgrid, dim3(256), 0, s, (const float*)w_eff, N, K, ldw, (float*)wt, N);
+  else
+    hipLaunchKernelGGL((k_transpose<uint16_t>), tgrid, dim3(256), 0, s, (const uint16_t*)w_eff, N, K, ldw, (uint16_t*)wt, N);
   const dim3 grid((unsigned)(mb * nkb));
   if (cfg->dtype == AHL_F32) launch_dx<F32>(a, is_static, grid, s);
   else launch_dx<BF16>(a, is_static, grid, s);
   if (is_static) {
     AHL_DISPATCH_DTYPE(cfg->dtype, {
-      hipLaunchKernelGGL((k_ir_grad_finalize<D>), dim3(n_tiles), dim3(64), 0, s, (const float*)ws, mb,
+      hipLaunchKernelGGL((k_ir_grad_finalize<D>), dim3(n_tiles), dim3(64), 0, s, (const float*)partial, mb,
                          (int32_t)nkb, a.kb_big, a.kb_small, tl, M, ir, ir_grad, cfg->ir_decay,
                          cfg->ir_input_min_percentage);
     });
@@ -823,7 +862,6 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uin
   return check_launch("ahl_linear_bwd_dx");
 }
 
-static int64_t align256(int64_t v) { return (v + 255) / 256 * 256; }
 
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
                                    int32_t has_keep) {
@@ -845,6 +883,9 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uin
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
+  if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
+      ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && (!keep || (((uintptr_t)keep) & 7u) == 0))
+    return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
   const int planes = (n_tiles + 7) / 8;
   DwArgs a;

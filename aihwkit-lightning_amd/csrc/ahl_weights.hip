@@ -143,13 +143,13 @@ extern "C" {
 
 int ahl_weight_prep(const void* w, int64_t N, int64_t K, int64_t ld, const int32_t* tile_ends_host,
                     int32_t n_tiles, const AhlModifierCfg* cfg, void* wmax, float* tile_max,
-                    float* tile_min, void* w_eff, int64_t ld_eff, void* w_eff_t, void* stream) {
+                    float* tile_min, void* w_eff, int64_t ld_eff, void* stream) {
   if (!w || !cfg || !wmax || !tile_max || !tile_min || N <= 0 || K <= 0 || ld < K) return AHL_ERR_ARG;
   if (w_eff && ld_eff < K) return AHL_ERR_ARG;
   if (w_eff == w) return AHL_ERR_ARG;  // never modifies the parameter storage
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
-  return launch_prep(w, N, K, ld, tl, cfg, true, wmax, tile_max, tile_min, w_eff, ld_eff, w_eff_t,
+  return launch_prep(w, N, K, ld, tl, cfg, true, wmax, tile_max, tile_min, w_eff, ld_eff, nullptr,
                      (hipStream_t)stream);
 }
 

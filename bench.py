@@ -77,9 +77,9 @@ def kernel_rooflines(layer, x, g, reps):
     from aihwkit_lightning.nn.modules.hip_utils import library as L
 
     in_sizes = layer.in_sizes
-    wmax, tile_max, _, w_eff, w_eff_t = OPS.weight_prep(
+    wmax, tile_max, _, w_eff = OPS.weight_prep(
         layer.weight.data, in_sizes, L.AHL_QUANT_NONE, L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02,
-        11, 1, True, True)
+        11, 1, True)
     ir = layer.input_range.detach()
     icfg = [L.AHL_IR_STATIC, 0, 1, 1, 0, 12345, 0]
     fcfg = [254.0, 254.0, 10.0, 0.04, 0.01, 0.95]
@@ -91,14 +91,14 @@ def kernel_rooflines(layer, x, g, reps):
     t = event_time_ms(lambda: OPS.linear_fwd(None, xq, w_eff, layer.bias.data, ir, wmax, tile_max,
                                              in_sizes, icfg, fcfg, True), reps)
     out["linear_fwd"] = t
-    t = event_time_ms(lambda: OPS.linear_bwd_dx(g, keep, flag, w_eff_t, x, ir, in_sizes, icfg, fcfg), reps)
+    t = event_time_ms(lambda: OPS.linear_bwd_dx(g, keep, flag, w_eff, x, ir, in_sizes, icfg, fcfg), reps)
     out["linear_bwd_dx(+ir_grad)"] = t
     t = event_time_ms(lambda: OPS.linear_bwd_dw(g, keep, flag, None, xq, ir, in_sizes, icfg, fcfg), reps)
-    out["linear_bwd_dw(+transposes)"] = t
+    out["linear_bwd_dw"] = t
     out["dac"] = event_time_ms(lambda: OPS.dac(x, ir, in_sizes, icfg, fcfg), reps)
     t = event_time_ms(lambda: OPS.weight_prep(layer.weight.data, in_sizes, L.AHL_QUANT_NONE,
                                               L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02, 11, 1,
-                                              True, True), reps)
+                                              True), reps)
     out["weight_prep"] = t
     return out, flops
 
@@ -139,6 +139,8 @@ def main():
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--kernels-only", action="store_true",
+                        help="only launch the individual kernels (for rocprofv3 runs)")
     ns = parser.parse_args()
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -160,6 +162,10 @@ def main():
         out = layer(x)
         out.backward(g)
 
+    if ns.kernels_only:
+        kernels, _ = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 1))
+        print(json.dumps({"ms_per_launch": kernels}))
+        return
     for _ in range(ns.warmup):
         step()
     torch.cuda.synchronize()
@@ -173,7 +179,7 @@ def main():
     value = step_flops / (ms_per_step * 1e-3) / 1e12
 
     kernels, gemm_flops = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 5))
-    dom = max(("linear_fwd", "linear_bwd_dx(+ir_grad)", "linear_bwd_dw(+transposes)"),
+    dom = max(("linear_fwd", "linear_bwd_dx(+ir_grad)", "linear_bwd_dw"),
               key=lambda k: kernels[k])
     achieved = gemm_flops / (kernels[dom] * 1e-3) / 1e12
     result = {

@@ -144,19 +144,18 @@ int64_t ahl_col_sum_ws_bytes(int64_t cols);
 
 /* ---- weights ------------------------------------------------------------------------------ */
 
-/* Everything the forward needs from the weights, one read of w[N, K]:
+/* Everything the forward needs from the weights:
  *   wmax[t, n]  = max_{k in tile t} |w[n, k]|                       (dtype [T, N])
  *   tile_max[t] = max_n wmax[t, n], tile_min[t] = min_n wmax[t, n]  (float [T])
  *   w_eff       = noise(quantize(w))  (dtype [N, K], ld_eff)   -- only if w_eff != NULL
- *   w_eff_t     = transpose of w_eff  (dtype [K, N], ld N)     -- only if w_eff_t != NULL
- * With quant_type/noise_type NONE, w_eff/w_eff_t receive plain copies of w.
+ * With quant_type/noise_type NONE, w_eff receives a plain copy of w.
  * Never writes to w (the Triton path's in-place store, triton_utils/triton_linear.py:152-156,
  * is deliberately not reproduced).
  * Replaces torch_utils/torch_linear.py:217-251 (amax, clip_and_quantize without learnable
  * clipping, modify_weight) and torch_utils/quant_utils.py:204-233.                       */
 int ahl_weight_prep(const void* w, int64_t N, int64_t K, int64_t ld, const int32_t* tile_ends_host,
                     int32_t n_tiles, const AhlModifierCfg* cfg, void* wmax, float* tile_max,
-                    float* tile_min, void* w_eff, int64_t ld_eff, void* w_eff_t, void* stream);
+                    float* tile_min, void* w_eff, int64_t ld_eff, void* stream);
 
 /* Post-training quantisation in place, per tile, scale from the slice's own abs-max:
  * Replaces AnalogLinear.quantize_weights, nn/modules/linear.py:285-303.
@@ -202,19 +201,19 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
                    const AhlLinearCfg* cfg, void* stream);
 
 /* Input gradient and input-range gradient (torch_utils/torch_linear.py:29-108 backward):
- *   d[:, tile t] = (g * keep_t) @ w_eff[:, tile t]      w_eff_t is the [K, N] transpose
+ *   d[:, tile t] = (g * keep_t) @ w_eff[:, tile t]      w_eff [N, K] as used by the forward
  *   AHL_IR_STATIC: ir_grad[t] per reference InputRangeForward.backward (incl. decay switch),
  *                  dx zeroed where |x| > ir[t]; x[M, K] is the forward input.
  *   otherwise dx = d, ir_grad untouched.
  *   clamp_flag: NULL, or the flag written by ahl_linear_fwd (keep is ignored when it reads 0).
- *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, n_tiles) bytes.
+ *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, N, n_tiles, dtype) bytes.
  * Slot of TritonLinear.backward, triton_utils/triton_linear.py:695-764.                  */
 int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
-                      const void* w_eff_t, const void* x, int64_t ldx, const void* ir, void* dx,
-                      int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
+                      const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
+                      void* dx, int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
-int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int32_t n_tiles);
+int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype);
 
 /* Weight gradient: dw[:, tile t] = (g * keep_t)^T @ DAC(clamp(x[:, tile t])).
  *   xq: the quantised input saved from the forward (ahl_dac), or NULL to re-quantise x here.

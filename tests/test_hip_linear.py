@@ -78,6 +78,12 @@ SHAPES = [
     case("vec_bf16_many_tiles", dtype="bf16", M=128, K=1152, N=128, max_input_size=64,
          ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
          w_scale=0.1, seed=25),
+    case("fast_bf16_clamped", dtype="bf16", M=264, K=512, N=136, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
+         w_scale=0.1, seed=28),
+    case("fast_bf16_dynamic_clamped", dtype="bf16", M=256, K=512, N=256, max_input_size=256,
+         ir_mode="dynamic", inp_res=254, out_res=254, out_bound=0.3, w_scale=0.1, seed=29),
+    case("fast_bf16_plain", dtype="bf16", M=256, K=768, N=256, max_input_size=256, seed=30),
     case("vec_f32_plain", M=200, K=256, N=136, max_input_size=-1, seed=26),
     case("one_token_bf16", dtype="bf16", M=1, K=512, N=512, max_input_size=256, ir_mode="static",
          inp_res=254, out_res=254, out_bound=10.0, seed=27),
