@@ -71,6 +71,17 @@ def tile_bounds(in_sizes: Sequence[int]) -> List[Tuple[int, int]]:
     return out
 
 
+def _acc(dtype: torch.dtype) -> torch.dtype:
+    """Accumulation dtype of a matrix product: fp32 for bf16/fp32 tensors, fp64 for fp64."""
+    return torch.float64 if dtype == torch.float64 else torch.float32
+
+
+def matmul_rounded(a: Tensor, b: Tensor) -> Tensor:
+    """a @ b accumulated in fp32 (fp64 for fp64 inputs) and rounded once to a's dtype."""
+    acc = _acc(a.dtype)
+    return (a.to(acc) @ b.to(acc)).to(a.dtype)
+
+
 def _tiny(dtype: torch.dtype) -> float:
     return torch.finfo(dtype).tiny
 
@@ -196,7 +207,7 @@ def linear_forward(
             w_eff = noisy_weight_tile(w_eff, wmax_t, cfg.weight_noise, cfg.modifier_std,
                                       None if w_xi is None else w_xi[t])
         # one fp32-accumulated product, rounded once to the tensor dtype
-        y = (xq.float() @ w_eff.float().T).to(x.dtype)
+        y = matmul_rounded(xq, w_eff.T)
         if noise_on:
             wr = wmax_t.view(1, -1) if cfg.out_noise_per_channel else wmax_t.max()
             xi = torch.randn_like(y) if out_xi is None else out_xi[t]
@@ -233,8 +244,8 @@ def linear_backward(grad_out: Tensor, saved: Dict) -> Tuple[Tensor, Tensor, Tens
     for t, (lo, hi) in enumerate(tile_bounds(saved["in_sizes"])):
         rec = saved["tiles"][t]
         gy = grad_out if rec["keep"] is None else grad_out * rec["keep"]
-        dw_parts.append((gy.float().T @ rec["xq"].float()).to(dtype))
-        d = (gy.float() @ rec["w_eff"].float()).to(dtype)
+        dw_parts.append(matmul_rounded(gy.T, rec["xq"]))
+        d = matmul_rounded(gy, rec["w_eff"])
         if cfg.ir_mode == IR_STATIC:
             ir_t, up, low = rec["ir"], rec["up"], rec["lo"]
             grad = torch.zeros_like(ir_t)
