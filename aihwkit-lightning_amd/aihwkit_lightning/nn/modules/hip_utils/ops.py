@@ -282,8 +282,9 @@ def linear_fwd(
     cfg = _linear_cfg(ref.dtype, icfg, fcfg)
     y = torch.empty((m_rows, n_out), dtype=ref.dtype, device=ref.device)
     planes = (n_tiles + 7) // 8
-    keep = torch.empty((planes, m_rows, n_out) if want_keep else (0,), dtype=torch.uint8,
-                       device=ref.device)
+    # clamp mask: per plane one 32-bit word per (row quad, column)
+    keep = torch.empty((planes, (m_rows + 3) // 4, n_out, 4) if want_keep else (0,),
+                       dtype=torch.uint8, device=ref.device)
     flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
     L.check(
         lib.ahl_linear_fwd(

@@ -37,6 +37,14 @@ struct Tiling {
 };
 
 // ---------------------------------------------------------------------------------------------
+// Clamp-mask layout ("keep"): one uint32 word per (row quad, column): byte (m % 4) of word
+// [(m / 4) * N + n] of plane (t / 8) holds the 8 tile bits of output element (m, n); bit t % 8
+// is set where the tile-t output stayed inside the ADC range. A lane of a 32x32 MFMA result owns
+// 4 consecutive rows of one column per register group, i.e. exactly one such word.
+AHL_DEV int64_t keep_plane_words(int64_t M, int64_t N) { return ((M + 3) >> 2) * N; }
+AHL_DEV int64_t keep_word(int64_t m, int64_t n, int64_t N) { return (m >> 2) * N + n; }
+
+// ---------------------------------------------------------------------------------------------
 // bf16 <-> f32
 AHL_DEV float bf16_bits_to_f32(uint32_t bits16) { return __uint_as_float(bits16 << 16); }
 AHL_DEV uint32_t f32_to_bf16_bits(float x) {
@@ -115,6 +123,11 @@ AHL_DEV float quant_step(float bound, float res) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// a ^ b ^ c in one instruction (v_bitop3_b32 with truth table 0x96)
+AHL_DEV uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
+  return __builtin_amdgcn_bitop3_b32(a, b, c, 0x96);
+}
+
 // Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11).
 AHL_DEV u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
 #pragma unroll
@@ -122,9 +135,9 @@ AHL_DEV u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
     const uint64_t p0 = (uint64_t)0xD2511F53u * c.x;
     const uint64_t p1 = (uint64_t)0xCD9E8D57u * c.z;
     u32x4 n;
-    n.x = (uint32_t)(p1 >> 32) ^ c.y ^ k0;
+    n.x = xor3((uint32_t)(p1 >> 32), c.y, k0);
     n.y = (uint32_t)p1;
-    n.z = (uint32_t)(p0 >> 32) ^ c.w ^ k1;
+    n.z = xor3((uint32_t)(p0 >> 32), c.w, k1);
     n.w = (uint32_t)p0;
     c = n;
     k0 += 0x9E3779B9u;
@@ -148,14 +161,14 @@ AHL_DEV void box_muller16(uint32_t w, float& n0, float& n1) {
   n1 = r * __builtin_amdgcn_sinf(rev);
 }
 
-// Eight standard normals for one counter value.
-//   output noise: stream 0; group = ((m >> 4) * 2 + ((m >> 2) & 1)) * N + n; normal j belongs to
-//                 row 16 * (m >> 4) + 4 * ((m >> 2) & 1) + (j & 3) + 8 * (j >> 2)  -- the 8 rows one
-//                 lane of a 32x32 MFMA result holds in two consecutive register groups
-//   weight noise: stream 1, tile field 0; group = n * ceil(K / 8) + (k >> 3); normal j is k % 8
-AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, uint64_t group,
-                     float* out8) {
-  u32x4 c = {(uint32_t)group, (uint32_t)(group >> 32), stream_and_tile, (uint32_t)offset};
+// Eight standard normals for one counter value (c0, c1, stream << 24 | tile, offset).
+//   output noise: stream 0; c0 = n (output column), c1 = (m >> 4) * 2 + ((m >> 2) & 1); normal j
+//                 belongs to row 16 * (m >> 4) + 4 * ((m >> 2) & 1) + (j & 3) + 8 * (j >> 2)  -- the 8
+//                 rows one lane of a 32x32 MFMA result holds in two consecutive register groups
+//   weight noise: stream 1, tile field 0; c0 = k >> 3, c1 = n (weight row); normal j is k % 8
+AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, uint32_t c0,
+                     uint32_t c1, float* out8) {
+  u32x4 c = {c0, c1, stream_and_tile, (uint32_t)offset};
   const u32x4 r = philox4x32_10(c, (uint32_t)seed, (uint32_t)(seed >> 32));
   box_muller16(r.x, out8[0], out8[1]);
   box_muller16(r.y, out8[2], out8[3]);

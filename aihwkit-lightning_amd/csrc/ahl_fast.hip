@@ -94,6 +94,12 @@ struct FastFwdArgs {
   uint64_t seed, offset;
 };
 
+AHL_DEV void mma_bf16_zero(const u32x4& a, const u32x4& b, f32x16& c) {
+  const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                              __builtin_bit_cast(bf16x8, b), z, 0, 0, 0);
+}
+
 AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
   c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
@@ -109,33 +115,35 @@ AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
   return BF16::rd((B + B) * a.out_res);
 }
 
-template <int IRMODE, bool NOISE, bool ADC>
-__global__ __launch_bounds__(256, 2) void k_fwd_fast(FastFwdArgs a) {
+template <int IRMODE, bool NOISE, bool ADC, int NBJ>
+__global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs a) {
+  constexpr int BN = 64 * NBJ;   // block columns
+  constexpr int WN = 32 * NBJ;   // wave columns
+  constexpr int NB = 2 * NBJ;    // B vectors per thread and chunk
   extern __shared__ __attribute__((aligned(16))) char lds[];
   char* ldsA = lds;
   char* ldsB = lds + kChunkLdsF;
-  float* rowc = (float*)(lds + 2 * kChunkLdsF);  // dynamic mode: [2][3][128] per-row constants
+  float* rowc = (float*)(lds + (128 + BN) * kLdsStrideF);  // dynamic mode: [2][3][128] per-row constants
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
   const int row0 = tid >> 3, cv = tid & 7;
   const int h = lane >> 5;
 
-  const int64_t nbn = cdiv_dev(a.N, 128);
+  const int64_t nbn = cdiv_dev(a.N, BN);
   const int64_t nb = gridDim.x;
   int64_t logical = blockIdx.x;
   if ((nb & 7) == 0) logical = (logical & 7) * (nb >> 3) + (logical >> 3);
-  const int64_t m0 = (logical / nbn) * 128, n0 = (logical % nbn) * 128;
+  const int64_t m0 = (logical / nbn) * 128, n0 = (logical % nbn) * BN;
   const bool bound_on = ADC || a.clamp_on;
-  const bool full = (m0 + 128 <= a.M) && (n0 + 128 <= a.N);  // no edge predicates needed
 
-  f32x16 acc[2][2];
-  uint32_t totp[2][2][8];   // running total, bf16 pairs: [g*2 + (c>>1)] = rows c, c+1 of group g
-  uint32_t clampbits[2][2][4];
+  f32x16 acc[2][NBJ];
+  uint32_t totp[2][NBJ][8];   // running total, bf16 pairs: [g*2 + (c>>1)] = rows c, c+1 of group g
+  uint32_t clampbits[2][NBJ][4];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < NBJ; ++j) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 #pragma unroll
@@ -145,65 +153,100 @@ __global__ __launch_bounds__(256, 2) void k_fwd_fast(FastFwdArgs a) {
     }
   uint32_t any_clamp = 0u;
 
-  const uint16_t* A = (const uint16_t*)a.xq;
-  const uint16_t* Bw = (const uint16_t*)a.w;
-  u32x4 rawA[4], rawB[4];
+  // Operand loads through buffer descriptors: the per-thread byte offset inside the block's
+  // row panel is computed once, the k position advances as the scalar offset, and rows beyond
+  // the matrix read as zero (out-of-range check of the descriptor) -- no per-chunk address
+  // arithmetic and no predicates.
+  const int64_t rowsA = a.M - m0, rowsB = a.N - n0;
+  const uint64_t bytesA = (uint64_t)rowsA * (uint64_t)a.ldx * 2u, bytesB = (uint64_t)rowsB * (uint64_t)a.ldw * 2u;
+  const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)((const uint16_t*)a.xq + m0 * a.ldx), 0,
+      (int)(bytesA > 0xffffffffull ? 0xffffffffu : (uint32_t)bytesA), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsB = __builtin_amdgcn_make_buffer_rsrc(
+      (void*)((const uint16_t*)a.w + n0 * a.ldw), 0,
+      (int)(bytesB > 0xffffffffull ? 0xffffffffu : (uint32_t)bytesB), 0x00020000);
+  int voA[4], voB[NB];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) voA[j] = (int)(((int64_t)(row0 + 32 * j) * a.ldx + cv * 8) * 2);
+#pragma unroll
+  for (int j = 0; j < NB; ++j) voB[j] = (int)(((int64_t)(row0 + 32 * j) * a.ldw + cv * 8) * 2);
+  u32x4 rawA[4], rawB[NB];
   auto load = [&](int32_t kc) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t ra = m0 + row0 + 32 * j, rb = n0 + row0 + 32 * j;
-      u32x4 z = {0u, 0u, 0u, 0u};
-      rawA[j] = ra < a.M ? ld16(A + ra * a.ldx + kc + cv * 8) : z;
-      rawB[j] = rb < a.N ? ld16(Bw + rb * a.ldw + kc + cv * 8) : z;
-    }
+    for (int j = 0; j < 4; ++j)
+      rawA[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsA, voA[j], kc * 2, 0));
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
+      rawB[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsB, voB[j], kc * 2, 0));
   };
   load(0);
   const int nchunks = a.K / 64, cpt = a.tile / 64;
   int t = 0, cin = 0;
-  for (int ch = 0; ch < nchunks; ++ch) {
+  // registers -> LDS for the chunk held in rawA/rawB; `tt` is its K-tile, `first` whether it
+  // opens that tile (then the dynamic-mode per-row constants of the tile are written too)
+  auto stage = [&](int tt, bool first) {
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 4; ++j)
       *(u32x4*)(ldsA + (row0 + 32 * j) * kLdsStrideF + cv * 16) = rawA[j];
+#pragma unroll
+    for (int j = 0; j < NB; ++j)
       *(u32x4*)(ldsB + (row0 + 32 * j) * kLdsStrideF + cv * 16) = rawB[j];
-    }
-    if (IRMODE == AHL_IR_DYNAMIC && cin == 0 && tid < 128) {
+    if (IRMODE == AHL_IR_DYNAMIC && first && tid < 128) {
       const int64_t m = m0 + tid;
-      const float irm = m < a.M ? BF16::load(a.ir, (int64_t)t * a.M + m) : 0.0f;
-      float* rc = rowc + (t & 1) * 384;
+      const float irm = m < a.M ? BF16::load(a.ir, (int64_t)tt * a.M + m) : 0.0f;
+      float* rc = rowc + (tt & 1) * 384;
       rc[tid] = BF16::rd(a.noise_scale * irm);
       rc[128 + tid] = BF16::rd(irm * a.out_bound);
     }
     __syncthreads();
+  };
+  bool prestaged = false;
+  for (int ch = 0; ch < nchunks; ++ch) {
+    if (!prestaged) stage(t, cin == 0);
+    prestaged = false;
     if (ch + 1 < nchunks) load((ch + 1) * 64);
 
     {
       const int r = lane & 31;
       const char* pa = ldsA + (wm * 64 + r) * kLdsStrideF + h * 16;
-      const char* pb = ldsB + (wn * 64 + r) * kLdsStrideF + h * 16;
+      const char* pb = ldsB + (wn * WN + r) * kLdsStrideF + h * 16;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
         const u32x4 a0 = *(const u32x4*)(pa + s * 32);
         const u32x4 a1 = *(const u32x4*)(pa + 32 * kLdsStrideF + s * 32);
-        const u32x4 b0 = *(const u32x4*)(pb + s * 32);
-        const u32x4 b1 = *(const u32x4*)(pb + 32 * kLdsStrideF + s * 32);
-        mma_bf16(a0, b0, acc[0][0]);
-        mma_bf16(a0, b1, acc[0][1]);
-        mma_bf16(a1, b0, acc[1][0]);
-        mma_bf16(a1, b1, acc[1][1]);
+        u32x4 bf[NBJ];
+#pragma unroll
+        for (int bj = 0; bj < NBJ; ++bj) bf[bj] = *(const u32x4*)(pb + bj * 32 * kLdsStrideF + s * 32);
+        if (s == 0 && cin == 0) {  // first step of a K-tile starts from zero
+#pragma unroll
+          for (int bj = 0; bj < NBJ; ++bj) {
+            mma_bf16_zero(a0, bf[bj], acc[0][bj]);
+            mma_bf16_zero(a1, bf[bj], acc[1][bj]);
+          }
+        } else {
+#pragma unroll
+          for (int bj = 0; bj < NBJ; ++bj) {
+            mma_bf16(a0, bf[bj], acc[0][bj]);
+            mma_bf16(a1, bf[bj], acc[1][bj]);
+          }
+        }
       }
     }
 
     if (++cin < cpt) continue;
     cin = 0;
+    // The next chunk (first of the next tile) is staged before the epilogue so that the
+    // prefetch registers are dead while the epilogue runs.
+    if (ch + 1 < nchunks) { stage(t + 1, true); prestaged = true; }
     // ---------------- per-K-tile epilogue ----------------
     const float ir_t = IRMODE == AHL_IR_STATIC ? BF16::load(a.ir, t) : 0.0f;
     const float tmax = (NOISE || bound_on) ? a.tile_max[t] : 0.0f;
     const float* rc_t = rowc + (t & 1) * 384;
     const bool flush = a.keep != nullptr && a.clamp_on && ((t & 7) == 7 || t == a.n_tiles - 1);
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj) {
-      const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
+    for (int bj = 0; bj < NBJ; ++bj) {
+      const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
       const bool nvalid = n < a.N;
       float wch = 0.0f;
       if ((NOISE || bound_on) && nvalid) wch = BF16::load(a.wmax, (int64_t)t * a.N + n);
@@ -227,16 +270,15 @@ __global__ __launch_bounds__(256, 2) void k_fwd_fast(FastFwdArgs a) {
         for (int gp = 0; gp < 2; ++gp) {
           float xi[8];
           if (NOISE) {
-            const uint64_t mrow = (uint64_t)(m0 + rbase + 16 * gp);
-            const uint64_t grp = ((mrow >> 4) * 2 + ((mrow >> 2) & 1)) * (uint64_t)a.N + (uint64_t)n;
-            normal8(a.seed, a.offset, (uint32_t)t, grp, xi);
+            const uint32_t mrow = (uint32_t)(m0 + rbase + 16 * gp);
+            normal8(a.seed, a.offset, (uint32_t)t, (uint32_t)n, (mrow >> 4) * 2 + ((mrow >> 2) & 1), xi);
           }
 #pragma unroll
           for (int gg = 0; gg < 2; ++gg) {
             const int g = 2 * gp + gg;
             float y[4];
 #pragma unroll
-            for (int c = 0; c < 4; ++c) { y[c] = acc[bi][bj][4 * g + c]; acc[bi][bj][4 * g + c] = 0.0f; }
+            for (int c = 0; c < 4; ++c) y[c] = acc[bi][bj][4 * g + c];
             rd2(y[0], y[1]); rd2(y[2], y[3]);
             float ns[4], Bv[4], rv[4], rcpv[4];
 #pragma unroll
@@ -310,27 +352,23 @@ __global__ __launch_bounds__(256, 2) void k_fwd_fast(FastFwdArgs a) {
       }
     }
     if (flush) {
-      // one byte plane of the clamp mask for the last (up to) 8 tiles; addresses are a 64-bit
-      // base per lane plus 32-bit row offsets
-      const uint32_t valid = (2u << (t & 7)) - 1u;
-      const int64_t mrow0 = m0 + wm * 64 + 4 * h;
-      const int32_t mlim = (int32_t)((a.M - mrow0) < 64 ? (a.M - mrow0) : 64);
-      const int32_t ldn = (int32_t)a.N;
+      // one plane of the clamp mask for the last (up to) 8 tiles: each register of clampbits is
+      // one word of the mask (4 consecutive rows of one column); 32 lanes store 128 contiguous bytes
+      const uint32_t valid = ((2u << (t & 7)) - 1u) * 0x01010101u;
+      uint32_t* plane = (uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N);
+      const int64_t mq0 = (m0 + wm * 64 + 4 * h) >> 2;
 #pragma unroll
-      for (int bj = 0; bj < 2; ++bj) {
-        const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
-        uint8_t* base = a.keep + ((int64_t)(t >> 3) * a.M + mrow0) * a.N + n;
-        const bool nvalid = n < a.N;
+      for (int bj = 0; bj < NBJ; ++bj) {
+        const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
+        uint32_t* wp = plane + mq0 * a.N + n;
+        const int32_t ldn = (int32_t)a.N;
 #pragma unroll
         for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-              const int32_t ro = bi * 32 + 8 * g + c;
-              if (full || (nvalid && ro < mlim))
-                base[ro * ldn] = (uint8_t)(~(clampbits[bi][bj][g] >> (8 * c)) & valid);
-            }
+            const int32_t q = bi * 8 + 2 * g;  // row-quad offset of rows bi*32 + 8*g
+            if (n < a.N && m0 + wm * 64 + bi * 32 + 8 * g + 4 * h < a.M)
+              wp[q * ldn] = ~clampbits[bi][bj][g] & valid;
             clampbits[bi][bj][g] = 0u;
           }
       }
@@ -340,29 +378,37 @@ __global__ __launch_bounds__(256, 2) void k_fwd_fast(FastFwdArgs a) {
 
   if (a.clamp_flag != nullptr && __any(any_clamp != 0u) && lane == 0) atomicOr(a.clamp_flag, 1u);
 
-  // ---- store y = total (+ bias) ----
+  // ---- store y = total (+ bias): transposed through LDS, 16-byte row-contiguous stores ----
   {
-    const int64_t mrow0 = m0 + wm * 64 + 4 * h;
-    const int32_t mlim = (int32_t)((a.M - mrow0) < 64 ? (a.M - mrow0) : 64);
-    const int32_t ldy = (int32_t)a.ldy;
+    constexpr int kOutStride = BN * 2 + 16;  // BN bf16 + 16 bytes pad
+    __syncthreads();                         // every wave is done with the operand buffers
+    char* obase = lds + (wm * 64 + 4 * h) * kOutStride + (wn * WN + (lane & 31)) * 2;
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj) {
-      const int64_t n = n0 + wn * 64 + bj * 32 + (lane & 31);
-      if (!full && n >= a.N) continue;
-      const float b = a.bias ? BF16::load(a.bias, n) : 0.0f;
-      uint16_t* base = (uint16_t*)a.y + mrow0 * a.ldy + n;
+    for (int bj = 0; bj < NBJ; ++bj) {
+      const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
+      const float b = (a.bias && n < a.N) ? BF16::load(a.bias, n) : 0.0f;
 #pragma unroll
       for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int32_t ro = bi * 32 + 8 * (v >> 2) + (v & 3);
-          if (full || ro < mlim) {
-            const uint32_t tp = totp[bi][bj][v >> 1];
-            float o = (v & 1) ? unpack_hi(tp) : unpack_lo(tp);
-            if (a.bias) o = BF16::rd(o + b);
-            base[ro * ldy] = (uint16_t)f32_to_bf16_bits(o);
-          }
+        for (int pr = 0; pr < 8; ++pr) {
+          uint32_t tp = totp[bi][bj][pr];
+          if (a.bias) tp = pack_bf16x2(unpack_lo(tp) + b, unpack_hi(tp) + b);
+          const int ro = bi * 32 + 8 * (pr >> 1) + 2 * (pr & 1);
+          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)tp;
+          *(uint16_t*)(obase + (ro + 1) * kOutStride + bj * 64) = (uint16_t)(tp >> 16);
         }
+    }
+    __syncthreads();
+    constexpr int VPR = BN / 8;          // 16-byte vectors per row
+    constexpr int RPP = 256 / VPR;       // rows per pass
+    const int vcol = tid % VPR, vrow = tid / VPR;
+    const int64_t n = n0 + vcol * 8;
+#pragma unroll
+    for (int j = 0; j < 128 / RPP; ++j) {
+      const int row = vrow + RPP * j;
+      const int64_t m = m0 + row;
+      if (m < a.M && n < a.N)
+        st16((uint16_t*)a.y + m * a.ldy + n, *(const u32x4*)(lds + row * kOutStride + vcol * 16));
     }
   }
 }
@@ -372,8 +418,6 @@ __global__ void k_zero_u32(uint32_t* p) { *p = 0u; }
 }  // namespace ahl
 
 using namespace ahl;
-
-static constexpr int kFastLds = 2 * kChunkLdsF + 2 * 384 * (int)sizeof(float);
 
 // number of significant bits of a positive float's significand
 static int significant_bits(float v) {
@@ -385,15 +429,16 @@ static int significant_bits(float v) {
   return bits;
 }
 
-template <int IRMODE>
-static void launch_fast(const FastFwdArgs& a, bool noise, bool adc, dim3 grid, hipStream_t s) {
-  const dim3 block(256);
+template <int IRMODE, int NBJ>
+static void launch_fast(const FastFwdArgs& a, bool noise, bool adc, hipStream_t s) {
+  constexpr int lds_bytes = (128 + 64 * NBJ) * kLdsStrideF + 2 * 384 * (int)sizeof(float);
+  const dim3 block(256), grid((unsigned)(cdiv(a.M, 128) * cdiv(a.N, 64 * NBJ)));
   if (noise) {
-    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, true>), grid, block, kFastLds, s, a);
-    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, false>), grid, block, kFastLds, s, a);
+    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, true, NBJ>), grid, block, lds_bytes, s, a);
+    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, false, NBJ>), grid, block, lds_bytes, s, a);
   } else {
-    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, true>), grid, block, kFastLds, s, a);
-    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, false>), grid, block, kFastLds, s, a);
+    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, true, NBJ>), grid, block, lds_bytes, s, a);
+    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, false, NBJ>), grid, block, lds_bytes, s, a);
   }
 }
 
@@ -405,7 +450,7 @@ bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, co
   if (cfg->dtype != AHL_BF16 || xq == nullptr) return false;
   if (tl.extra != 0 || tl.base % 64 != 0) return false;
   if (!aligned16(xq) || !aligned16(w) || ldxq % 8 != 0 || ldw % 8 != 0) return false;
-  return K % 64 == 0;
+  return K % 64 == 0;  // the caller also checks N % 8, ldy % 8 and the alignment of y and keep
 }
 
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
@@ -426,13 +471,16 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   a.res_mul_exact = (adc && a.res_is_states && significant_bits(cfg->out_res) <= 8) ? 1 : 0;
   a.two_inv_res = adc ? 2.0f / cfg->out_res : 0.0f;
   a.seed = cfg->seed; a.offset = cfg->offset;
-  const int64_t nb = cdiv(M, 128) * cdiv(N, 128);
-  if (nb > 0x7fffffff) return AHL_ERR_ARG;
-  const dim3 grid((unsigned)nb);
+  if (cdiv(M, 128) * cdiv(N, 64) > 0x7fffffff) return AHL_ERR_ARG;
   if (clamp_flag) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);
-  if (cfg->ir_mode == AHL_IR_NONE) launch_fast<0>(a, noise, adc, grid, s);
-  else if (cfg->ir_mode == AHL_IR_STATIC) launch_fast<1>(a, noise, adc, grid, s);
-  else launch_fast<2>(a, noise, adc, grid, s);
+  // 128 x 64 blocks (wave tile 64 x 32, four blocks per CU) when the epilogue dominates: more
+  // independent blocks per SIMD keep the VALU busy while others are in their MFMA phase;
+  // 128 x 128 blocks (less LDS traffic per MFMA) for the plain product.
+  const bool narrow = false;  // measured: the 128 x 64 variant is ~10 % slower even with noise + ADC on
+  (void)noise;
+  if (cfg->ir_mode == AHL_IR_NONE) { if (narrow) launch_fast<0, 1>(a, noise, adc, s); else launch_fast<0, 2>(a, noise, adc, s); }
+  else if (cfg->ir_mode == AHL_IR_STATIC) { if (narrow) launch_fast<1, 1>(a, noise, adc, s); else launch_fast<1, 2>(a, noise, adc, s); }
+  else { if (narrow) launch_fast<2, 1>(a, noise, adc, s); else launch_fast<2, 2>(a, noise, adc, s); }
   return check_launch("ahl_linear_fwd(fast)");
 }
 

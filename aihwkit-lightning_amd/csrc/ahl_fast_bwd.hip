@@ -52,15 +52,15 @@ AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// zero the elements of a vector of 8 bf16 whose mask byte has bit `bit` clear
-AHL_DEV u32x4 apply_keep(const u32x4& v, const uint8_t* q, int bit) {
-  const uint32_t w0 = *(const uint32_t*)q, w1 = *(const uint32_t*)(q + 4);
+// Zero the elements of a vector of 8 bf16, g[m, n .. n+8), whose clamp-mask bit is clear.
+// q points at the mask word of (m, n); `sh` = 8 * (m % 4) + tile bit.
+AHL_DEV u32x4 apply_keep(const u32x4& v, const uint32_t* q, int sh) {
+  const u32x4 w0 = *(const u32x4*)q, w1 = *(const u32x4*)(q + 4);
   u32x4 o = v;
-  uint32_t m;
-  m = (((w0 >> bit) & 1u) ? 0xffffu : 0u) | (((w0 >> (8 + bit)) & 1u) ? 0xffff0000u : 0u); o.x &= m;
-  m = (((w0 >> (16 + bit)) & 1u) ? 0xffffu : 0u) | (((w0 >> (24 + bit)) & 1u) ? 0xffff0000u : 0u); o.y &= m;
-  m = (((w1 >> bit) & 1u) ? 0xffffu : 0u) | (((w1 >> (8 + bit)) & 1u) ? 0xffff0000u : 0u); o.z &= m;
-  m = (((w1 >> (16 + bit)) & 1u) ? 0xffffu : 0u) | (((w1 >> (24 + bit)) & 1u) ? 0xffff0000u : 0u); o.w &= m;
+  o.x &= (((w0.x >> sh) & 1u) ? 0xffffu : 0u) | (((w0.y >> sh) & 1u) ? 0xffff0000u : 0u);
+  o.y &= (((w0.z >> sh) & 1u) ? 0xffffu : 0u) | (((w0.w >> sh) & 1u) ? 0xffff0000u : 0u);
+  o.z &= (((w1.x >> sh) & 1u) ? 0xffffu : 0u) | (((w1.y >> sh) & 1u) ? 0xffff0000u : 0u);
+  o.w &= (((w1.z >> sh) & 1u) ? 0xffffu : 0u) | (((w1.w >> sh) & 1u) ? 0xffff0000u : 0u);
   return o;
 }
 
@@ -83,7 +83,8 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   const int64_t R = MODE == MODE_DX ? a.M : a.N;      // output rows
   const int64_t L = MODE == MODE_DX ? a.N : a.M;      // contraction length
   const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
-  const uint8_t* plane = use_keep ? a.keep + (int64_t)(t >> 3) * a.M * a.N : nullptr;
+  const uint32_t* plane =
+      use_keep ? (const uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N) : nullptr;
   const int bit = t & 7;
 
   f32x16 acc[4][2];
@@ -105,7 +106,8 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   // Rows of the output tile that lie beyond the matrix are redirected to the last valid row:
   // they only feed accumulators that are never stored. No predicates in the hot loop.
   const uint16_t* pa[4];
-  const uint8_t* pk[4];
+  const uint32_t* pk[4];
+  int psh[4];
   const uint16_t* pb[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -113,23 +115,25 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       int64_t m = r0 + rk_row + 64 * j;
       m = m < a.M ? m : a.M - 1;
       pa[j] = a.g + m * a.ldg + rk_cv * 8;              // + l0 (contraction n)
-      pk[j] = plane ? plane + m * a.N + rk_cv * 8 : nullptr;
+      pk[j] = plane ? plane + keep_word(m, rk_cv * 8, a.N) : nullptr;
+      psh[j] = 8 * (int)(m & 3) + bit;
     } else {
       int64_t n = r0 + km_cv * 8;
       n = n < a.N ? n : a.N - 8;
       pa[j] = a.g + (int64_t)(km_row + 16 * j) * a.ldg + n;  // + l0 * ldg (contraction m)
-      pk[j] = plane ? plane + (int64_t)(km_row + 16 * j) * a.N + n : nullptr;
+      pk[j] = plane ? plane + keep_word(km_row + 16 * j, n, a.N) : nullptr;
+      psh[j] = 8 * ((km_row + 16 * j) & 3) + bit;
     }
     pb[j] = a.b + (int64_t)(km_row + 16 * j) * a.ldb + c0 + km_cv * 8;  // + l0 * ldb
   }
   const int64_t a_step = MODE == MODE_DX ? 64 : 64 * a.ldg;
-  const int64_t k_step = MODE == MODE_DX ? 64 : 64 * a.N;
+  const int64_t k_step = MODE == MODE_DX ? 64 : 16 * a.N;  // 64 rows = 16 row quads
   const int64_t b_step = 64 * a.ldb;
   auto load = [&](bool masked) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       u32x4 v = ld16(pa[j]);
-      if (masked) { v = apply_keep(v, pk[j], bit); pk[j] += k_step; }
+      if (masked) { v = apply_keep(v, pk[j], psh[j]); pk[j] += k_step; }
       rawA[j] = v;
       rawB[j] = ld16(pb[j]);
       pa[j] += a_step;

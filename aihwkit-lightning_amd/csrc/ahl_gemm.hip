@@ -271,9 +271,8 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
             float xi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
             if (a.noise_on) {
               // rows m0 + rbase + 16 * gp + {0..3, 8..11}: one Philox call per lane and pair of groups
-              const uint64_t mrow = (uint64_t)(m0 + rbase + 16 * gp);
-              const uint64_t grp = ((mrow >> 4) * 2 + ((mrow >> 2) & 1)) * (uint64_t)a.N + (uint64_t)n;
-              normal8(a.seed, a.offset, (uint32_t)t, grp, xi);
+              const uint32_t mrow = (uint32_t)(m0 + rbase + 16 * gp);
+            normal8(a.seed, a.offset, (uint32_t)t, (uint32_t)n, (mrow >> 4) * 2 + ((mrow >> 2) & 1), xi);
             }
 #pragma unroll
             for (int gg = 0; gg < 2; ++gg) {
@@ -313,16 +312,13 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
               }
             }
           }
-          // flush one plane of the clamp mask every 8 tiles
+          // flush one plane of the clamp mask every 8 tiles: one word per register group
           if (a.keep != nullptr && a.clamp_on && ((t & 7) == 7 || t == T - 1)) {
-            uint8_t* plane = a.keep + (int64_t)(t >> 3) * a.M * a.N;
+            uint32_t* plane = (uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N);
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-#pragma unroll
-              for (int c = 0; c < 4; ++c) {
-                const int64_t m = m0 + rbase + 8 * g + c;
-                if (m < a.M && nvalid) plane[m * a.N + n] = (uint8_t)(keepbits[bi][bj][g] >> (8 * c));
-              }
+              const int64_t m = m0 + rbase + 8 * g;
+              if (m < a.M && nvalid) plane[keep_word(m, n, a.N)] = keepbits[bi][bj][g];
               keepbits[bi][bj][g] = 0u;
             }
           }
@@ -382,24 +378,21 @@ AHL_DEV void decode_kblock(const Tiling& tl, int32_t kb_big, int32_t kb_small, i
   c1 = tl.start(t + 1);
 }
 
-// Applies the clamp mask of tile t to a vector of gradient values.
-template <class D, bool VEC>
-AHL_DEV u32x4 mask_vec(const u32x4& raw, const uint8_t* keep_plane, int64_t ld, int64_t row,
-                       int64_t n_rows, int32_t k, int32_t k_end, int bit) {
+// Applies the clamp mask of tile t to a vector of gradient values g[m, n .. n+E) (ALONG_N) or
+// g[m .. m+E, n) (!ALONG_N, the transposed operand of the weight gradient).
+template <class D, bool ALONG_N>
+AHL_DEV u32x4 mask_vec(const u32x4& raw, const uint32_t* plane, int64_t N, int64_t m, int64_t n,
+                       int64_t lim, int bit) {
   constexpr int E = D::EPV;
-  if (row >= n_rows || k >= k_end) return raw;
   float e[E];
   D::unpack(raw, e);
-  const uint8_t* q = keep_plane + row * ld + k;
-  if (VEC) {
-    uint32_t w[2];
-    w[0] = *(const uint32_t*)q;
-    w[1] = E == 8 ? *(const uint32_t*)(q + 4) : 0u;
 #pragma unroll
-    for (int i = 0; i < E; ++i) if (!((w[i >> 2] >> (8 * (i & 3) + bit)) & 1u)) e[i] = 0.0f;
-  } else {
-#pragma unroll
-    for (int i = 0; i < E; ++i) if (k + i < k_end && !((q[i] >> bit) & 1)) e[i] = 0.0f;
+  for (int i = 0; i < E; ++i) {
+    const int64_t mi = ALONG_N ? m : m + i, ni = ALONG_N ? n + i : n;
+    if ((ALONG_N ? ni : mi) < lim) {
+      const uint32_t w = plane[keep_word(mi, ni, N)];
+      if (!((w >> (8 * (int)(mi & 3) + bit)) & 1u)) e[i] = 0.0f;
+    }
   }
   return D::pack(e);
 }
@@ -422,7 +415,8 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
   int t; int32_t c0, c1;
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
   const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
-  const uint8_t* plane = use_keep ? a.keep + (int64_t)(t >> 3) * a.M * a.N : nullptr;
+  const uint32_t* plane =
+      use_keep ? (const uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N) : nullptr;
   const int bit = t & 7;
 
   f32x16 acc[2][2];
@@ -442,9 +436,10 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
     u32x4 qa[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      qa[j] = plane ? mask_vec<D, VEC>(rawA[j], plane, a.N, m0 + vp.row0 + 32 * j, a.M,
-                                       kc + vp.cv * D::EPV, kend, bit)
-                    : rawA[j];
+      qa[j] = (plane && m0 + vp.row0 + 32 * j < a.M)
+                  ? mask_vec<D, true>(rawA[j], plane, a.N, m0 + vp.row0 + 32 * j,
+                                      kc + vp.cv * D::EPV, kend, bit)
+                  : rawA[j];
     __syncthreads();
     store_chunk(ldsA, vp, qa);
     store_chunk(ldsB, vp, rawB);
@@ -537,7 +532,7 @@ __global__ __launch_bounds__(64) void k_ir_grad_finalize(const float* __restrict
 // =============================================================================================
 struct DwArgs {
   const void* gt;       // [N, M]
-  const uint8_t* keept; // [P, N, M] or null
+  const uint8_t* keept; // the clamp mask in its native layout, or null
   const uint32_t* clamp_flag;
   const void* xqt;      // [K, M]
   void* dw; int64_t lddw;
@@ -562,7 +557,8 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dw(DwArgs a) {
   int t; int32_t c0, c1;
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
   const bool use_keep = a.keept != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
-  const uint8_t* plane = use_keep ? a.keept + (int64_t)(t >> 3) * a.N * a.M : nullptr;
+  const uint32_t* plane =
+      use_keep ? (const uint32_t*)a.keept + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N) : nullptr;
   const int bit = t & 7;
 
   f32x16 acc[2][2];
@@ -582,9 +578,10 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dw(DwArgs a) {
     u32x4 qa[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      qa[j] = plane ? mask_vec<D, VEC>(rawA[j], plane, a.M, n0 + vp.row0 + 32 * j, a.N,
-                                       kc + vp.cv * D::EPV, kend, bit)
-                    : rawA[j];
+      qa[j] = (plane && n0 + vp.row0 + 32 * j < a.N)
+                  ? mask_vec<D, false>(rawA[j], plane, a.N, kc + vp.cv * D::EPV,
+                                       n0 + vp.row0 + 32 * j, kend, bit)
+                  : rawA[j];
     __syncthreads();
     store_chunk(ldsA, vp, qa);
     store_chunk(ldsB, vp, rawB);
@@ -754,7 +751,8 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
     if (cfg->ir_mode != AHL_IR_NONE && !ir) return AHL_ERR_ARG;
     if ((noise_on || bound_on) && (!wmax || !tile_max)) return AHL_ERR_ARG;
   }
-  if (fast_fwd_eligible(cfg, xq, ldxq, w_eff, ldw, K, tl))
+  if (fast_fwd_eligible(cfg, xq, ldxq, w_eff, ldw, K, tl) && N % 8 == 0 && ldy % 8 == 0 &&
+      aligned16(y) && (!keep || (((uintptr_t)keep) & 3u) == 0))
     return launch_fast_fwd(xq, ldxq, w_eff, ldw, bias, y, ldy, keep, clamp_flag, ir, wmax, tile_max,
                            M, K, N, tl, cfg, (hipStream_t)stream);
   if (!x) return AHL_ERR_UNSUPPORTED;  // only the fast path can start from xq alone
@@ -823,7 +821,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uin
   void* wt = (char*)ws + dx_partial_bytes(M, K, n_tiles);
   const bool fast = fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(w_eff) &&
                     ldg % 8 == 0 && ldw % 8 == 0 && lddx % 8 == 0 &&
-                    (!keep || (((uintptr_t)keep) & 7u) == 0) &&
+                    (!keep || aligned16(keep)) &&
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
     int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
@@ -866,9 +864,9 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uin
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
                                    int32_t has_keep) {
   const int64_t es = dtype == AHL_BF16 ? 2 : 4;
-  int64_t b = align256(N * M * es) + align256(K * M * es);
-  if (has_keep) b += align256((int64_t)((n_tiles + 7) / 8) * N * M);
-  return b;
+  (void)n_tiles;
+  (void)has_keep;
+  return align256(N * M * es) + align256(K * M * es);
 }
 
 int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
@@ -884,10 +882,9 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uin
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
   if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
-      ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && (!keep || (((uintptr_t)keep) & 7u) == 0))
+      ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && (!keep || aligned16(keep)))
     return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
-  const int planes = (n_tiles + 7) / 8;
   DwArgs a;
   a.M = M; a.N = N; a.K = K; a.tl = tl; a.dw = dw; a.lddw = lddw;
   kblocks(tl, &a.kb_big, &a.kb_small);
@@ -901,12 +898,8 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uin
     char* p = (char*)ws;
     E* gt = (E*)p; p += align256(N * M * (int64_t)sizeof(E));
     E* xqt = (E*)p; p += align256(K * M * (int64_t)sizeof(E));
-    uint8_t* keept = keep ? (uint8_t*)p : nullptr;
+    const uint8_t* keept = keep;
     hipLaunchKernelGGL((k_transpose<E>), tgrid_g, dim3(256), 0, s, (const E*)g, M, N, ldg, gt, M);
-    if (keep) {
-      const dim3 tgrid_k((unsigned)cdiv(N, 64), (unsigned)cdiv(M, 64), (unsigned)planes);
-      hipLaunchKernelGGL((k_transpose<uint8_t>), tgrid_k, dim3(256), 0, s, keep, M, N, N, keept, M);
-    }
     if (xq)
       hipLaunchKernelGGL((k_transpose<E>), tgrid_x, dim3(256), 0, s, (const E*)xq, M, K, ldxq, xqt, M);
     else if (cfg->ir_mode == AHL_IR_NONE)

@@ -55,14 +55,13 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a) {
   __shared__ typename D::elem tileT[64][64 + 4];
   const int k0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
   const int kq = threadIdx.x & 7, nr = threadIdx.x >> 3;
-  const int64_t kgroups = (a.K + 7) >> 3;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int64_t n = n0 + nr + 32 * j;
     const int kb = k0 + 8 * kq;
     float xi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if (a.noise_type != AHL_NOISE_NONE && n < a.N && kb < a.K)
-      normal8(a.seed, a.offset, 1u << 24, (uint64_t)n * (uint64_t)kgroups + (uint64_t)(kb >> 3), xi);
+      normal8(a.seed, a.offset, 1u << 24, (uint32_t)(kb >> 3), (uint32_t)n, xi);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int k = kb + e;

@@ -188,9 +188,10 @@ int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_i
  *   tile_max float [T]    from ahl_weight_prep, or NULL likewise
  *   bias     dtype [N] or NULL
  *   y        dtype [M, N]
- *   keep     uint8 [ceil(T/8), M, N] or NULL: bit (t%8) of plane t/8 is set where the tile-t
- *            output was inside [-bound, bound] (the clamp's gradient mask). Written only when
- *            out_bound > 0 and keep != NULL.
+ *   keep     uint8 [ceil(T/8), ceil(M/4), N, 4] or NULL (4-byte aligned): byte (m % 4) of word
+ *            (m / 4, n) of plane t/8 has bit (t % 8) set where the tile-t output of element
+ *            (m, n) was inside [-bound, bound] (the clamp's gradient mask). Written only when
+ *            out_bound > 0 and keep != NULL; consumed by the two backward entry points.
  *   clamp_flag  uint32 [1] or NULL: receives non-zero if any tile output was clamped (or if the
  *            kernel does not track it); the backward entry points skip `keep` when it is zero.
  * Slot of TritonLinear.forward, triton_utils/triton_linear.py:446-690.                   */

@@ -311,8 +311,9 @@ def philox4x32_10(ctr: Sequence[int], key: Sequence[int]) -> Tuple[int, int, int
     return c0, c1, c2, c3
 
 
-def philox_counter(stream_and_tile: int, group: int, offset: int) -> Tuple[int, int, int, int]:
-    """Counter layout of the device generator: (group lo, group hi, stream<<24 | tile, offset lo).
-    Output noise: stream 0, group = (m // 4) * N + n, the 4 normals are rows 4*(m//4)+0..3.
-    Weight noise: stream 1, tile field 0, group = n * ceil(K/4) + k // 4, normals k%4 = 0..3."""
-    return group & _MASK, (group >> 32) & _MASK, stream_and_tile & _MASK, offset & _MASK
+def philox_counter(stream: int, tile: int, c0: int, c1: int, offset: int) -> Tuple[int, int, int, int]:
+    """Counter layout of the device generator: (c0, c1, stream << 24 | tile, offset lo).
+    Output noise: stream 0, c0 = n, c1 = (m // 16) * 2 + ((m // 4) % 2); the 8 normals of a call
+    are rows 16 * (m // 16) + 4 * ((m // 4) % 2) + (j % 4) + 8 * (j // 4).
+    Weight noise: stream 1, tile 0, c0 = k // 8, c1 = n; the 8 normals are k % 8 = 0..7."""
+    return c0 & _MASK, c1 & _MASK, ((stream << 24) | tile) & _MASK, offset & _MASK
