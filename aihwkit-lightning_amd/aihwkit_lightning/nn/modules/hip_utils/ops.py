@@ -281,10 +281,9 @@ def linear_fwd(
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(ref.dtype, icfg, fcfg)
     y = torch.empty((m_rows, n_out), dtype=ref.dtype, device=ref.device)
-    planes = (n_tiles + 7) // 8
-    # clamp mask: per plane one 32-bit word per (row quad, column)
-    keep = torch.empty((planes, (m_rows + 3) // 4, n_out, 4) if want_keep else (0,),
-                       dtype=torch.uint8, device=ref.device)
+    # clamp mask: one bit per (tile, row, column), 32 columns of one row per word
+    keep = torch.empty((n_tiles, (n_out + 31) // 32, m_rows) if want_keep else (0,),
+                       dtype=torch.int32, device=ref.device)
     flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
     L.check(
         lib.ahl_linear_fwd(

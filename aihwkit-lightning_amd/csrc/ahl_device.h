@@ -37,12 +37,12 @@ struct Tiling {
 };
 
 // ---------------------------------------------------------------------------------------------
-// Clamp-mask layout ("keep"): one uint32 word per (row quad, column): byte (m % 4) of word
-// [(m / 4) * N + n] of plane (t / 8) holds the 8 tile bits of output element (m, n); bit t % 8
-// is set where the tile-t output stayed inside the ADC range. A lane of a 32x32 MFMA result owns
-// 4 consecutive rows of one column per register group, i.e. exactly one such word.
-AHL_DEV int64_t keep_plane_words(int64_t M, int64_t N) { return ((M + 3) >> 2) * N; }
-AHL_DEV int64_t keep_word(int64_t m, int64_t n, int64_t N) { return (m >> 2) * N + n; }
+// Clamp-mask layout: one bit per (tile, row, column). Word [(t * ceil(N/32) + n / 32) * M + m]
+// has bit (n % 32) set where the tile-t output of element (m, n) left the ADC range (and so
+// passes no gradient). One 64-lane ballot over a 32x32 MFMA result register yields two such
+// words (rows r and r + 4); the 64 rows of a wave's tile are 256 contiguous bytes.
+AHL_DEV int64_t clamp_plane_words(int64_t M, int64_t N) { return ((N + 31) >> 5) * M; }
+AHL_DEV int64_t clamp_word(int64_t m, int64_t n, int64_t M) { return (n >> 5) * M + m; }
 
 // ---------------------------------------------------------------------------------------------
 // bf16 <-> f32
@@ -178,6 +178,28 @@ AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, u
 
 // ---------------------------------------------------------------------------------------------
 // wave64 reductions (all lanes end up with the result)
+// Records the clamp bits of one register of a 32x32 MFMA result (lane l holds column l % 32 of
+// row `row` for l < 32 and of row `row + 4` for l >= 32, rows counted within the wave's tile)
+// in `words`, where lane L keeps the mask word of row L. Must be called by the whole wave.
+AHL_DEV void clamp_record(bool clamped, int row, uint32_t& words) {
+  const uint64_t b = __builtin_amdgcn_ballot_w64(clamped);
+  const int lane = (int)(threadIdx.x & 63u);
+  words = lane == row ? (uint32_t)b : words;
+  words = lane == row + 4 ? (uint32_t)(b >> 32) : words;
+}
+
+// Zeroes the elements of a vector of 8 bf16 whose bit in the low byte of `bits` is set.
+AHL_DEV u32x4 clamp_apply8(const u32x4& v, uint32_t bits) {
+  // per pair of elements: 0x0000ffff for the even bit, 0xffff0000 for the odd one
+  auto pair = [&](uint32_t x, int i) -> uint32_t {
+    const uint32_t lo = ((bits >> (2 * i)) & 1u) * 0xffffu;
+    const uint32_t hi = (uint32_t)(((int32_t)(bits << (30 - 2 * i))) >> 31) << 16;
+    return x & ~(lo | hi);
+  };
+  u32x4 o = {pair(v.x, 0), pair(v.y, 1), pair(v.z, 2), pair(v.w, 3)};
+  return o;
+}
+
 AHL_DEV float wave_max(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));

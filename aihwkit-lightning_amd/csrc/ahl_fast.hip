@@ -80,7 +80,7 @@ struct FastFwdArgs {
   const void* w; int64_t ldw;    // effective weights, bf16 [N, K]
   const void* bias;
   void* y; int64_t ldy;
-  uint8_t* keep;                 // [planes, M, N] or null
+  uint32_t* keep;                // clamp mask [T, ceil(N/32), M] or null
   uint32_t* clamp_flag;          // set to non-zero if any tile output was clamped; may be null
   const void* ir;                // [T] static, [T, M] dynamic
   const void* wmax;              // [T, N]
@@ -139,7 +139,9 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 
   f32x16 acc[2][NBJ];
   uint32_t totp[2][NBJ][8];   // running total, bf16 pairs: [g*2 + (c>>1)] = rows c, c+1 of group g
-  uint32_t clampbits[2][NBJ][4];
+  uint32_t cwords[NBJ];       // lane L: clamp-mask word of row wm * 64 + L for the current tile
+#pragma unroll
+  for (int j = 0; j < NBJ; ++j) cwords[j] = 0u;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -148,8 +150,6 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 #pragma unroll
       for (int v = 0; v < 8; ++v) totp[i][j][v] = 0u;
-#pragma unroll
-      for (int v = 0; v < 4; ++v) clampbits[i][j][v] = 0u;
     }
   uint32_t any_clamp = 0u;
 
@@ -243,7 +243,6 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
     const float ir_t = IRMODE == AHL_IR_STATIC ? BF16::load(a.ir, t) : 0.0f;
     const float tmax = (NOISE || bound_on) ? a.tile_max[t] : 0.0f;
     const float* rc_t = rowc + (t & 1) * 384;
-    const bool flush = a.keep != nullptr && a.clamp_on && ((t & 7) == 7 || t == a.n_tiles - 1);
 #pragma unroll
     for (int bj = 0; bj < NBJ; ++bj) {
       const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
@@ -331,7 +330,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                   const bool cl = !(fabsf(y[c]) <= Bv[c]);
-                  clampbits[bi][bj][g] |= (cl ? 1u : 0u) << (8 * c + (t & 7));
+                  if (a.keep != nullptr) clamp_record(cl && nvalid, 32 * bi + 8 * g + c, cwords[bj]);
                   y[c] = fminf(fmaxf(y[c], -Bv[c]), Bv[c]);
                 }
                 any_clamp |= over ? 1u : 0u;
@@ -351,26 +350,16 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
         }
       }
     }
-    if (flush) {
-      // one plane of the clamp mask for the last (up to) 8 tiles: each register of clampbits is
-      // one word of the mask (4 consecutive rows of one column); 32 lanes store 128 contiguous bytes
-      const uint32_t valid = ((2u << (t & 7)) - 1u) * 0x01010101u;
-      uint32_t* plane = (uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N);
-      const int64_t mq0 = (m0 + wm * 64 + 4 * h) >> 2;
+    if (a.keep != nullptr && a.clamp_on) {
+      // the clamp-mask words of this tile: per 32-column block, the 64 rows of the wave are
+      // 256 contiguous bytes
+      uint32_t* plane = a.keep + (int64_t)t * clamp_plane_words(a.M, a.N);
+      const int64_t m = m0 + wm * 64 + lane;
 #pragma unroll
       for (int bj = 0; bj < NBJ; ++bj) {
-        const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
-        uint32_t* wp = plane + mq0 * a.N + n;
-        const int32_t ldn = (int32_t)a.N;
-#pragma unroll
-        for (int bi = 0; bi < 2; ++bi)
-#pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const int32_t q = bi * 8 + 2 * g;  // row-quad offset of rows bi*32 + 8*g
-            if (n < a.N && m0 + wm * 64 + bi * 32 + 8 * g + 4 * h < a.M)
-              wp[q * ldn] = ~clampbits[bi][bj][g] & valid;
-            clampbits[bi][bj][g] = 0u;
-          }
+        const int64_t nb0 = n0 + wn * WN + bj * 32;
+        if (m < a.M && nb0 < a.N) plane[clamp_word(m, nb0, a.M)] = cwords[bj];
+        cwords[bj] = 0u;
       }
     }
     t += 1;
@@ -454,7 +443,7 @@ bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, co
 }
 
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
-                    void* y, int64_t ldy, uint8_t* keep, uint32_t* clamp_flag, const void* ir,
+                    void* y, int64_t ldy, uint32_t* keep, uint32_t* clamp_flag, const void* ir,
                     const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
                     const Tiling& tl, const AhlLinearCfg* cfg, hipStream_t s) {
   FastFwdArgs a;

@@ -35,7 +35,7 @@ static constexpr int MODE_DW = 1;
 
 struct BwdArgs {
   const uint16_t* g; int64_t ldg;      // [M, N]
-  const uint8_t* keep;                 // [planes, M, N] or null
+  const uint32_t* keep;                // clamp mask [T, ceil(N/32), M] or null
   const uint32_t* clamp_flag;          // null or the forward's flag
   const uint16_t* b; int64_t ldb;      // DX: W_eff [N, K]; DW: xq [M, K]
   const uint16_t* x; int64_t ldx;      // DX static range: the forward input [M, K]
@@ -50,18 +50,6 @@ struct BwdArgs {
 AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
   c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
-// Zero the elements of a vector of 8 bf16, g[m, n .. n+8), whose clamp-mask bit is clear.
-// q points at the mask word of (m, n); `sh` = 8 * (m % 4) + tile bit.
-AHL_DEV u32x4 apply_keep(const u32x4& v, const uint32_t* q, int sh) {
-  const u32x4 w0 = *(const u32x4*)q, w1 = *(const u32x4*)(q + 4);
-  u32x4 o = v;
-  o.x &= (((w0.x >> sh) & 1u) ? 0xffffu : 0u) | (((w0.y >> sh) & 1u) ? 0xffff0000u : 0u);
-  o.y &= (((w0.z >> sh) & 1u) ? 0xffffu : 0u) | (((w0.w >> sh) & 1u) ? 0xffff0000u : 0u);
-  o.z &= (((w1.x >> sh) & 1u) ? 0xffffu : 0u) | (((w1.y >> sh) & 1u) ? 0xffff0000u : 0u);
-  o.w &= (((w1.z >> sh) & 1u) ? 0xffffu : 0u) | (((w1.w >> sh) & 1u) ? 0xffff0000u : 0u);
-  return o;
 }
 
 template <int MODE>
@@ -83,9 +71,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   const int64_t R = MODE == MODE_DX ? a.M : a.N;      // output rows
   const int64_t L = MODE == MODE_DX ? a.N : a.M;      // contraction length
   const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
-  const uint32_t* plane =
-      use_keep ? (const uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N) : nullptr;
-  const int bit = t & 7;
+  const uint32_t* plane = use_keep ? a.keep + (int64_t)t * clamp_plane_words(a.M, a.N) : nullptr;
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -101,13 +87,14 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   const int rk_row = tid >> 3, rk_cv = tid & 7;
   const int km_row = tid >> 5, km_cv = tid & 31;
   u32x4 rawA[4], rawB[4];
-  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  uint32_t rawK[4] = {0u, 0u, 0u, 0u};  // mask words of the vectors in rawA
 
   // Rows of the output tile that lie beyond the matrix are redirected to the last valid row:
   // they only feed accumulators that are never stored. No predicates in the hot loop.
+  // Clamp mask: the 8 gradient values of one 16-byte vector are one byte of a mask word.
   const uint16_t* pa[4];
   const uint32_t* pk[4];
-  int psh[4];
+  int psh = 0;
   const uint16_t* pb[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -115,34 +102,36 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       int64_t m = r0 + rk_row + 64 * j;
       m = m < a.M ? m : a.M - 1;
       pa[j] = a.g + m * a.ldg + rk_cv * 8;              // + l0 (contraction n)
-      pk[j] = plane ? plane + keep_word(m, rk_cv * 8, a.N) : nullptr;
-      psh[j] = 8 * (int)(m & 3) + bit;
+      pk[j] = plane ? plane + clamp_word(m, rk_cv * 8, a.M) : nullptr;  // + (l0 / 32) * M
+      psh = 8 * (rk_cv & 3);
     } else {
       int64_t n = r0 + km_cv * 8;
       n = n < a.N ? n : a.N - 8;
       pa[j] = a.g + (int64_t)(km_row + 16 * j) * a.ldg + n;  // + l0 * ldg (contraction m)
-      pk[j] = plane ? plane + keep_word(km_row + 16 * j, n, a.N) : nullptr;
-      psh[j] = 8 * ((km_row + 16 * j) & 3) + bit;
+      pk[j] = plane ? plane + clamp_word(km_row + 16 * j, n, a.M) : nullptr;  // + l0
+      psh = 8 * (int)((n >> 3) & 3);
     }
     pb[j] = a.b + (int64_t)(km_row + 16 * j) * a.ldb + c0 + km_cv * 8;  // + l0 * ldb
   }
   const int64_t a_step = MODE == MODE_DX ? 64 : 64 * a.ldg;
-  const int64_t k_step = MODE == MODE_DX ? 64 : 16 * a.N;  // 64 rows = 16 row quads
+  const int64_t k_step = MODE == MODE_DX ? 2 * a.M : 64;   // 64 columns = 2 words; or 64 rows
   const int64_t b_step = 64 * a.ldb;
   auto load = [&](bool masked) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      u32x4 v = ld16(pa[j]);
-      if (masked) { v = apply_keep(v, pk[j], psh[j]); pk[j] += k_step; }
-      rawA[j] = v;
+      rawA[j] = ld16(pa[j]);
+      if (masked) { rawK[j] = *pk[j]; pk[j] += k_step; }
       rawB[j] = ld16(pb[j]);
       pa[j] += a_step;
       pb[j] += b_step;
     }
   };
-  auto stage = [&](char* sa, char* sb) {
+  // The mask is applied here, after the MFMAs of the current chunk, so that nothing waits for
+  // the loads that were issued before them.
+  auto stage = [&](char* sa, char* sb, bool masked) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      if (masked) rawA[j] = clamp_apply8(rawA[j], rawK[j] >> psh);
       if (MODE == MODE_DX) *(u32x4*)(sa + (rk_row + 64 * j) * kRowkStride + rk_cv * 16) = rawA[j];
       else *(u32x4*)(sa + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawA[j];
       *(u32x4*)(sb + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawB[j];
@@ -166,7 +155,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   auto main_loop = [&](auto masked_tag) {
     constexpr bool kMasked = decltype(masked_tag)::value;
     load(kMasked);
-    stage(lds, lds + kOperandLds);
+    stage(lds, lds + kOperandLds, kMasked);
     __syncthreads();
     for (int ch = 0; ch < nchunks; ++ch) {
       const char* sa = lds + (ch & 1) * 2 * kOperandLds;
@@ -191,7 +180,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       }
       if (ch + 1 < nchunks) {
         char* na = lds + ((ch + 1) & 1) * 2 * kOperandLds;
-        stage(na, na + kOperandLds);
+        stage(na, na + kOperandLds, kMasked);
       }
       __syncthreads();
     }
@@ -199,33 +188,61 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   if (plane) main_loop(std::true_type{});
   else main_loop(std::false_type{});
 
-  // ---- epilogue ----
+  // ---- epilogue: the 256 x 256 result goes through LDS (the operand buffers are free after
+  // the loop's last barrier) so that global memory is touched in row-contiguous 16-byte vectors;
+  // the forward input needed by the input-range gradient is fetched the same way ----
   float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
   const bool do_ir = MODE == MODE_DX && a.ir_static != 0;
   const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
-  const int64_t row_w = r0 + wm * 128 + 4 * h;
+  constexpr int kOutStride = 256 * 2 + 16;
+  const int vcol = tid & 31, vrow = tid >> 5;  // 16-byte vector column, row within a pass of 16
+  const uint16_t* xp = do_ir ? a.x + (r0 + vrow) * a.ldx + c0 + vcol * 8 : nullptr;
+  uint16_t* op = a.out + (r0 + vrow) * a.ldo + c0 + vcol * 8;
+  {
+    char* obase = lds + (wm * 128 + 4 * h) * kOutStride + (wn * 64 + (lane & 31)) * 2;
 #pragma unroll
-  for (int bj = 0; bj < 2; ++bj) {
-    const int64_t k = c0 + wn * 64 + bj * 32 + (lane & 31);
-    uint16_t* obase = a.out + row_w * a.ldo + k;
-    const uint16_t* xbase = do_ir ? a.x + row_w * a.ldx + k : nullptr;
+    for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
-    for (int bi = 0; bi < 4; ++bi)
+      for (int bi = 0; bi < 4; ++bi)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
-        if (row_w + ro >= R) continue;
-        float d = BF16::rd(acc[bi][bj][v]);
-        if (do_ir) {
-          const float xv = bf16_bits_to_f32(xbase[(int64_t)ro * a.ldx]);
-          const bool up = xv >= ir_t, lo = xv <= -ir_t;
-          if (up) s_up += fminf(d, 0.0f);
-          if (lo) s_lo += fmaxf(d, 0.0f);
-          if (up || lo) cnt += 1.0f;
-          if (fabsf(xv) > ir_t) d = 0.0f;
+        for (int v = 0; v < 16; ++v) {
+          const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
+          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)f32_to_bf16_bits(acc[bi][bj][v]);
         }
-        obase[(int64_t)ro * a.ldo] = (uint16_t)f32_to_bf16_bits(d);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    u32x4 xr[8];
+    if (do_ir) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int row = vrow + 16 * (8 * half + j);
+        // rows beyond the matrix re-read row r0 + vrow, which always exists
+        xr[j] = ld16(xp + (r0 + row < R ? (int64_t)(16 * (8 * half + j)) * a.ldx : 0));
       }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int row = vrow + 16 * (8 * half + j);
+      u32x4 d4 = *(const u32x4*)(lds + row * kOutStride + vcol * 16);
+      if (r0 + row >= R) continue;
+      if (do_ir) {
+        float d[8], xv[8];
+        BF16::unpack(d4, d);
+        BF16::unpack(xr[j], xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const bool up = xv[i] >= ir_t, lo = xv[i] <= -ir_t;
+          if (up) s_up += fminf(d[i], 0.0f);
+          if (lo) s_lo += fmaxf(d[i], 0.0f);
+          if (up || lo) cnt += 1.0f;
+          if (fabsf(xv[i]) > ir_t) d[i] = 0.0f;
+        }
+        d4 = BF16::pack(d);
+      }
+      st16(op + (int64_t)(16 * (8 * half + j)) * a.ldo, d4);
+    }
   }
   if (do_ir) {
     s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
@@ -250,7 +267,7 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
   return K % 256 == 0 && N % 64 == 0 && M % 64 == 0;
 }
 
-int launch_fast_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, bool ir_static, hipStream_t s) {
@@ -266,7 +283,7 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32
   return check_launch("ahl_linear_bwd_dx(fast)");
 }
 
-int launch_fast_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, int64_t M, int64_t K,
                    int64_t N, const Tiling& tl, hipStream_t s) {
   BwdArgs a;

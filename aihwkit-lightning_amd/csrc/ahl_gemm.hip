@@ -129,7 +129,7 @@ struct FwdArgs {
   const void* w; int64_t ldw;
   const void* bias;
   void* y; int64_t ldy;
-  uint8_t* keep;
+  uint32_t* keep;
   const void* ir;
   const void* wmax;
   const float* tile_max;
@@ -160,15 +160,13 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
   const int T = a.tl.n_tiles;
 
   f32x16 total[2][2], acc[2][2];
-  uint32_t keepbits[2][2][4];
+  uint32_t cwords[2] = {0u, 0u};  // lane L: clamp-mask word of row wm * 64 + L, per column block
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) { total[i][j][v] = 0.0f; acc[i][j][v] = 0.0f; }
-#pragma unroll
-      for (int v = 0; v < 4; ++v) keepbits[i][j][v] = 0u;
     }
 
   // --- state of the chunk being loaded ---
@@ -304,7 +302,7 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
                   }
                   if (a.clamp_on) {
                     const bool kp = (y >= -B) && (y <= B);
-                    keepbits[bi][bj][g] |= (kp ? 1u : 0u) << (8 * c + (t & 7));
+                    if (a.keep != nullptr) clamp_record(!kp && nvalid, 32 * bi + 8 * g + c, cwords[bj]);
                     y = fminf(fmaxf(y, -B), B);
                   }
                 }
@@ -312,16 +310,14 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
               }
             }
           }
-          // flush one plane of the clamp mask every 8 tiles: one word per register group
-          if (a.keep != nullptr && a.clamp_on && ((t & 7) == 7 || t == T - 1)) {
-            uint32_t* plane = (uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N);
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const int64_t m = m0 + rbase + 8 * g;
-              if (m < a.M && nvalid) plane[keep_word(m, n, a.N)] = keepbits[bi][bj][g];
-              keepbits[bi][bj][g] = 0u;
-            }
-          }
+        }
+        // the clamp-mask words of this tile: 64 consecutive rows of one 32-column block
+        if (a.keep != nullptr && a.clamp_on) {
+          const int64_t m = m0 + wm * 64 + lane;
+          const int64_t nb0 = n0 + wn * 64 + bj * 32;
+          if (m < a.M && nb0 < a.N)
+            a.keep[(int64_t)t * clamp_plane_words(a.M, a.N) + clamp_word(m, nb0, a.M)] = cwords[bj];
+          cwords[bj] = 0u;
         }
       }
     }
@@ -355,7 +351,7 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
 // =============================================================================================
 struct DxArgs {
   const void* g; int64_t ldg;
-  const uint8_t* keep;
+  const uint32_t* keep;
   const uint32_t* clamp_flag;
   const void* wt;  // w_eff_t [K, N]
   const void* x; int64_t ldx;
@@ -381,8 +377,8 @@ AHL_DEV void decode_kblock(const Tiling& tl, int32_t kb_big, int32_t kb_small, i
 // Applies the clamp mask of tile t to a vector of gradient values g[m, n .. n+E) (ALONG_N) or
 // g[m .. m+E, n) (!ALONG_N, the transposed operand of the weight gradient).
 template <class D, bool ALONG_N>
-AHL_DEV u32x4 mask_vec(const u32x4& raw, const uint32_t* plane, int64_t N, int64_t m, int64_t n,
-                       int64_t lim, int bit) {
+AHL_DEV u32x4 mask_vec(const u32x4& raw, const uint32_t* plane, int64_t M, int64_t m, int64_t n,
+                       int64_t lim) {
   constexpr int E = D::EPV;
   float e[E];
   D::unpack(raw, e);
@@ -390,8 +386,8 @@ AHL_DEV u32x4 mask_vec(const u32x4& raw, const uint32_t* plane, int64_t N, int64
   for (int i = 0; i < E; ++i) {
     const int64_t mi = ALONG_N ? m : m + i, ni = ALONG_N ? n + i : n;
     if ((ALONG_N ? ni : mi) < lim) {
-      const uint32_t w = plane[keep_word(mi, ni, N)];
-      if (!((w >> (8 * (int)(mi & 3) + bit)) & 1u)) e[i] = 0.0f;
+      const uint32_t w = plane[clamp_word(mi, ni, M)];
+      if ((w >> (int)(ni & 31)) & 1u) e[i] = 0.0f;
     }
   }
   return D::pack(e);
@@ -416,8 +412,7 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
   const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
   const uint32_t* plane =
-      use_keep ? (const uint32_t*)a.keep + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N) : nullptr;
-  const int bit = t & 7;
+      use_keep ? a.keep + (int64_t)t * clamp_plane_words(a.M, a.N) : nullptr;
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -437,8 +432,8 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       qa[j] = (plane && m0 + vp.row0 + 32 * j < a.M)
-                  ? mask_vec<D, true>(rawA[j], plane, a.N, m0 + vp.row0 + 32 * j,
-                                      kc + vp.cv * D::EPV, kend, bit)
+                  ? mask_vec<D, true>(rawA[j], plane, a.M, m0 + vp.row0 + 32 * j,
+                                      kc + vp.cv * D::EPV, kend)
                   : rawA[j];
     __syncthreads();
     store_chunk(ldsA, vp, qa);
@@ -532,7 +527,7 @@ __global__ __launch_bounds__(64) void k_ir_grad_finalize(const float* __restrict
 // =============================================================================================
 struct DwArgs {
   const void* gt;       // [N, M]
-  const uint8_t* keept; // the clamp mask in its native layout, or null
+  const uint32_t* keept; // the clamp mask in its native layout, or null
   const uint32_t* clamp_flag;
   const void* xqt;      // [K, M]
   void* dw; int64_t lddw;
@@ -558,8 +553,7 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dw(DwArgs a) {
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
   const bool use_keep = a.keept != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
   const uint32_t* plane =
-      use_keep ? (const uint32_t*)a.keept + (int64_t)(t >> 3) * keep_plane_words(a.M, a.N) : nullptr;
-  const int bit = t & 7;
+      use_keep ? a.keept + (int64_t)t * clamp_plane_words(a.M, a.N) : nullptr;
 
   f32x16 acc[2][2];
 #pragma unroll
@@ -579,8 +573,8 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dw(DwArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       qa[j] = (plane && n0 + vp.row0 + 32 * j < a.N)
-                  ? mask_vec<D, false>(rawA[j], plane, a.N, kc + vp.cv * D::EPV,
-                                       n0 + vp.row0 + 32 * j, kend, bit)
+                  ? mask_vec<D, false>(rawA[j], plane, a.M, kc + vp.cv * D::EPV,
+                                       n0 + vp.row0 + 32 * j, kend)
                   : rawA[j];
     __syncthreads();
     store_chunk(ldsA, vp, qa);
@@ -684,16 +678,16 @@ namespace ahl {
 bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, const void* w,
                        int64_t ldw, int64_t K, const Tiling& tl);
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
-                    void* y, int64_t ldy, uint8_t* keep, uint32_t* clamp_flag, const void* ir,
+                    void* y, int64_t ldy, uint32_t* keep, uint32_t* clamp_flag, const void* ir,
                     const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
                     const Tiling& tl, const AhlLinearCfg* cfg, hipStream_t s);
 __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N);
-int launch_fast_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, bool ir_static, hipStream_t s);
-int launch_fast_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, int64_t M, int64_t K,
                    int64_t N, const Tiling& tl, hipStream_t s);
 }  // namespace ahl
@@ -736,7 +730,7 @@ static void launch_dx(const DxArgs& a, bool is_static, dim3 grid, hipStream_t s)
 extern "C" {
 
 int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* w_eff,
-                   int64_t ldw, const void* bias, void* y, int64_t ldy, uint8_t* keep,
+                   int64_t ldw, const void* bias, void* y, int64_t ldy, uint32_t* keep,
                    uint32_t* clamp_flag, const void* ir, const void* wmax, const float* tile_max,
                    int64_t M, int64_t K, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
                    const AhlLinearCfg* cfg, void* stream) {
@@ -804,7 +798,7 @@ int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
   return dx_partial_bytes(M, K, n_tiles) + align256(K * N * es);  // partials + transposed weights
 }
 
-int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                       const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                       void* dx, int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
@@ -820,8 +814,8 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uin
   float* partial = (float*)ws;
   void* wt = (char*)ws + dx_partial_bytes(M, K, n_tiles);
   const bool fast = fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(w_eff) &&
-                    ldg % 8 == 0 && ldw % 8 == 0 && lddx % 8 == 0 &&
-                    (!keep || aligned16(keep)) &&
+                    ldg % 8 == 0 && ldw % 8 == 0 && lddx % 8 == 0 && aligned16(dx) &&
+                    (!keep || (((uintptr_t)keep) & 3u) == 0) &&
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
     int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
@@ -869,7 +863,7 @@ int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
   return align256(N * M * es) + align256(K * M * es);
 }
 
-int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                       const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* ir,
                       void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
@@ -882,7 +876,7 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uin
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
   if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
-      ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && (!keep || aligned16(keep)))
+      ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && aligned16(dw) && (!keep || (((uintptr_t)keep) & 3u) == 0))
     return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
   DwArgs a;
@@ -898,7 +892,7 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uin
     char* p = (char*)ws;
     E* gt = (E*)p; p += align256(N * M * (int64_t)sizeof(E));
     E* xqt = (E*)p; p += align256(K * M * (int64_t)sizeof(E));
-    const uint8_t* keept = keep;
+    const uint32_t* keept = keep;
     hipLaunchKernelGGL((k_transpose<E>), tgrid_g, dim3(256), 0, s, (const E*)g, M, N, ldg, gt, M);
     if (xq)
       hipLaunchKernelGGL((k_transpose<E>), tgrid_x, dim3(256), 0, s, (const E*)xq, M, K, ldxq, xqt, M);

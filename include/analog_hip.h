@@ -188,46 +188,46 @@ int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_i
  *   tile_max float [T]    from ahl_weight_prep, or NULL likewise
  *   bias     dtype [N] or NULL
  *   y        dtype [M, N]
- *   keep     uint8 [ceil(T/8), ceil(M/4), N, 4] or NULL (4-byte aligned): byte (m % 4) of word
- *            (m / 4, n) of plane t/8 has bit (t % 8) set where the tile-t output of element
- *            (m, n) was inside [-bound, bound] (the clamp's gradient mask). Written only when
- *            out_bound > 0 and keep != NULL; consumed by the two backward entry points.
+ *   clamp_mask  uint32 [T, ceil(N/32), M] or NULL: bit (n % 32) of word [t][n / 32][m] is set
+ *            where the tile-t output of element (m, n) left [-bound, bound] and was clamped
+ *            (it passes no gradient). Written only when out_bound > 0 and clamp_mask != NULL;
+ *            consumed by the two backward entry points.
  *   clamp_flag  uint32 [1] or NULL: receives non-zero if any tile output was clamped (or if the
- *            kernel does not track it); the backward entry points skip `keep` when it is zero.
+ *            kernel does not track it); the backward entry points skip the mask when it is zero.
  * Slot of TritonLinear.forward, triton_utils/triton_linear.py:446-690.                   */
 int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* w_eff,
-                   int64_t ldw, const void* bias, void* y, int64_t ldy, uint8_t* keep,
+                   int64_t ldw, const void* bias, void* y, int64_t ldy, uint32_t* clamp_mask,
                    uint32_t* clamp_flag, const void* ir, const void* wmax, const float* tile_max,
                    int64_t M, int64_t K, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
                    const AhlLinearCfg* cfg, void* stream);
 
 /* Input gradient and input-range gradient (torch_utils/torch_linear.py:29-108 backward):
- *   d[:, tile t] = (g * keep_t) @ w_eff[:, tile t]      w_eff [N, K] as used by the forward
+ *   d[:, tile t] = (g * !clamped_t) @ w_eff[:, tile t]      w_eff [N, K] as used by the forward
  *   AHL_IR_STATIC: ir_grad[t] per reference InputRangeForward.backward (incl. decay switch),
  *                  dx zeroed where |x| > ir[t]; x[M, K] is the forward input.
  *   otherwise dx = d, ir_grad untouched.
- *   clamp_flag: NULL, or the flag written by ahl_linear_fwd (keep is ignored when it reads 0).
+ *   clamp_flag: NULL, or the flag written by ahl_linear_fwd (the mask is ignored when it reads 0).
  *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, N, n_tiles, dtype) bytes.
  * Slot of TritonLinear.backward, triton_utils/triton_linear.py:695-764.                  */
-int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* clamp_mask, const uint32_t* clamp_flag,
                       const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                       void* dx, int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
 int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype);
 
-/* Weight gradient: dw[:, tile t] = (g * keep_t)^T @ DAC(clamp(x[:, tile t])).
+/* Weight gradient: dw[:, tile t] = (g * !clamped_t)^T @ DAC(clamp(x[:, tile t])).
  *   xq: the quantised input saved from the forward (ahl_dac), or NULL to re-quantise x here.
- *   ws needs ahl_linear_bwd_dw_ws_bytes(M, K, N, n_tiles, dtype, keep != NULL) bytes
- *   (transposed staging copies of g, keep and the quantised input).
+ *   ws needs ahl_linear_bwd_dw_ws_bytes(M, K, N, n_tiles, dtype, clamp_mask != NULL) bytes
+ *   (transposed staging copies of g and the quantised input).
  * Same reference slot as ahl_linear_bwd_dx.                                               */
-int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint8_t* keep, const uint32_t* clamp_flag,
+int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* clamp_mask, const uint32_t* clamp_flag,
                       const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* ir,
                       void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
-                                   int32_t has_keep);
+                                   int32_t has_mask);
 
 #ifdef __cplusplus
 }
