@@ -197,11 +197,15 @@ class HipLinear(Function):
                 grad_inp = dx.view(ctx.inp_shape)
             if ctx.ir_needs_grad and ctx.needs_input_grad[3]:
                 grad_ir = ir_grad
+        want_bias = ctx.has_bias and ctx.needs_input_grad[2]
         if ctx.need_dw:
-            grad_w = OPS.linear_bwd_dw(
+            # the weight-gradient kernel streams all of g and sums its columns on the way
+            grad_w, dbias = OPS.linear_bwd_dw(
                 g2, keep, flag, x2 if xq is None else None, xq, ir_dev, ctx.in_sizes, ctx.icfg,
-                ctx.fcfg,
+                ctx.fcfg, want_bias,
             )
-        if ctx.has_bias and ctx.needs_input_grad[2]:
+            if want_bias:
+                grad_b = dbias
+        elif want_bias:
             grad_b = OPS.col_sum(g2)
         return grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None

@@ -124,8 +124,8 @@ SIGNATURES = {
     "ahl_linear_bwd_dw": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
-         c_void_p, c_int64, c_int64, c_int64, c_int64, _I32P, c_int32, POINTER(AhlLinearCfg),
-         c_void_p, c_void_p],
+         c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32,
+         POINTER(AhlLinearCfg), c_void_p, c_void_p],
     ),
     "ahl_linear_bwd_dw_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32]),
 }

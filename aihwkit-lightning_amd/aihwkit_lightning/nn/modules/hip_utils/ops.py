@@ -89,7 +89,7 @@ LIB.define(
 )
 LIB.define(
     "linear_bwd_dw(Tensor g, Tensor? keep, Tensor? clamp_flag, Tensor? x, Tensor? xq, Tensor? ir, "
-    "int[] in_sizes, int[] icfg, float[] fcfg) -> Tensor"
+    "int[] in_sizes, int[] icfg, float[] fcfg, bool want_bias) -> (Tensor, Tensor)"
 )
 
 
@@ -331,9 +331,10 @@ def linear_bwd_dx(
 def linear_bwd_dw(
     g: Tensor, keep: Optional[Tensor], clamp_flag: Optional[Tensor], x: Optional[Tensor],
     xq: Optional[Tensor], ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
-    fcfg: List[float],
-) -> Tensor:
-    """Weight gradient ``[N, K]`` from the raw input ``x`` or the saved quantised input ``xq``."""
+    fcfg: List[float], want_bias: bool,
+) -> Tuple[Tensor, Tensor]:
+    """Weight gradient ``[N, K]`` from the raw input ``x`` or the saved quantised input ``xq``,
+    and (if wanted, else empty) the bias gradient ``[N]``, the column sums of ``g``."""
     lib = L.load()
     g = _rows2d(g, "g")
     ref = xq if xq is not None else x
@@ -346,18 +347,20 @@ def linear_bwd_dw(
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(g.dtype, icfg, fcfg)
     dw = torch.empty((n_out, k_in), dtype=g.dtype, device=g.device)
+    dbias = torch.empty((n_out,) if want_bias else (0,), dtype=g.dtype, device=g.device)
     ws_bytes = lib.ahl_linear_bwd_dw_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype,
                                               0 if keep is None else 1)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=g.device)
     L.check(
         lib.ahl_linear_bwd_dw(
             _ptr(g), _ld(g), _ptr(keep), _ptr(clamp_flag), _ptr(x), _ld(x) if x is not None else 0,
-            _ptr(xq), _ld(xq) if xq is not None else 0, _ptr(ir), _ptr(dw), k_in, m_rows, k_in,
-            n_out, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(ws), _stream(),
+            _ptr(xq), _ld(xq) if xq is not None else 0, _ptr(ir), _ptr(dw), k_in,
+            _ptr(dbias) if want_bias else None, m_rows, k_in, n_out, L.tile_ends_array(in_sizes),
+            n_tiles, byref(cfg), _ptr(ws), _stream(),
         ),
         "ahl_linear_bwd_dw",
     )
-    return dw
+    return dw, dbias
 
 
 for _name, _fn in [

@@ -42,6 +42,7 @@ struct BwdArgs {
   const uint16_t* ir;                  // DX static range: [T]
   uint16_t* out; int64_t ldo;          // DX: dx [M, K]; DW: dw [N, K]
   float* partial;                      // DX static range: [blocks][4]
+  float* bias_partial;                 // DW: [K / 256][N] partial column sums of g, or null
   int64_t M, N, K;
   int32_t tile;                        // K-tile width (multiple of 256)
   int32_t ir_static;
@@ -128,9 +129,20 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   };
   // The mask is applied here, after the MFMAs of the current chunk, so that nothing waits for
   // the loads that were issued before them.
-  auto stage = [&](char* sa, char* sb, bool masked) {
+  // DW: the bias gradient is the column sum of the unmasked g over all rows. Every block of a
+  // row of blocks streams the same g; block kb of the nkb sums the chunks ch = kb (mod nkb), so
+  // that the extra work is spread evenly, and a small kernel adds the nkb partial sums.
+  float bsum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const int kb_idx = (int)(logical % nkb);
+  auto stage = [&](char* sa, char* sb, bool masked, bool bias) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
+      if (bias) {
+        float e[8];
+        BF16::unpack(rawA[j], e);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) bsum[i] += e[i];
+      }
       if (masked) rawA[j] = clamp_apply8(rawA[j], rawK[j] >> psh);
       if (MODE == MODE_DX) *(u32x4*)(sa + (rk_row + 64 * j) * kRowkStride + rk_cv * 16) = rawA[j];
       else *(u32x4*)(sa + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawA[j];
@@ -152,10 +164,11 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   };
 
   const int nchunks = (int)(L / 64);
-  auto main_loop = [&](auto masked_tag) {
+  auto main_loop = [&](auto masked_tag, auto bias_tag) {
     constexpr bool kMasked = decltype(masked_tag)::value;
+    constexpr bool kBias = decltype(bias_tag)::value;
     load(kMasked);
-    stage(lds, lds + kOperandLds, kMasked);
+    stage(lds, lds + kOperandLds, kMasked, kBias && kb_idx == 0);
     __syncthreads();
     for (int ch = 0; ch < nchunks; ++ch) {
       const char* sa = lds + (ch & 1) * 2 * kOperandLds;
@@ -180,13 +193,31 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       }
       if (ch + 1 < nchunks) {
         char* na = lds + ((ch + 1) & 1) * 2 * kOperandLds;
-        stage(na, na + kOperandLds, kMasked);
+        stage(na, na + kOperandLds, kMasked, kBias && (ch + 1) % (int)nkb == kb_idx);
       }
       __syncthreads();
     }
   };
-  if (plane) main_loop(std::true_type{});
-  else main_loop(std::false_type{});
+  const bool do_bias = MODE == MODE_DW && a.bias_partial != nullptr;
+  if (do_bias) {
+    if (plane) main_loop(std::true_type{}, std::true_type{});
+    else main_loop(std::false_type{}, std::true_type{});
+    // 16 threads (contraction rows km_row + 16 j) hold partial sums of the same 8 columns
+    float* bred = (float*)lds;  // [16][256]; the operand buffers are free after the last barrier
+#pragma unroll
+    for (int i = 0; i < 8; ++i) bred[km_row * 256 + km_cv * 8 + i] = bsum[i];
+    __syncthreads();
+    if (tid < 256 && r0 + tid < a.N) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += bred[r * 256 + tid];
+      a.bias_partial[(int64_t)kb_idx * a.N + r0 + tid] = sum;
+    }
+    __syncthreads();
+  } else {
+    if (plane) main_loop(std::true_type{}, std::false_type{});
+    else main_loop(std::false_type{}, std::false_type{});
+  }
 
   // ---- epilogue: the 256 x 256 result goes through LDS (the operand buffers are free after
   // the loop's last barrier) so that global memory is touched in row-contiguous 16-byte vectors;
@@ -257,6 +288,15 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   }
 }
 
+__global__ __launch_bounds__(256) void k_bias_final(const float* partial, int nkb, int64_t N,
+                                                    uint16_t* dbias) {
+  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (n >= N) return;
+  float s = 0.0f;
+  for (int i = 0; i < nkb; ++i) s += partial[(int64_t)i * N + n];
+  dbias[n] = (uint16_t)f32_to_bf16_bits(s);
+}
+
 // Whether the fast backward kernels can be used: bf16, equal K-tiles of a multiple of 256,
 // 16-byte aligned rows everywhere.
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N) {
@@ -274,7 +314,7 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   BwdArgs a;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
-  a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial;
+  a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
   a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = ir_static ? 1 : 0;
   const int64_t nb = cdiv(M, 256) * (K / 256);
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
@@ -284,17 +324,22 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
 }
 
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
-                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, int64_t M, int64_t K,
-                   int64_t N, const Tiling& tl, hipStream_t s) {
+                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
+                   float* bias_partial, int64_t M, int64_t K, int64_t N, const Tiling& tl,
+                   hipStream_t s) {
   BwdArgs a;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
   a.b = (const uint16_t*)xq; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;
   a.out = (uint16_t*)dw; a.ldo = lddw; a.partial = nullptr;
+  a.bias_partial = dbias ? bias_partial : nullptr;
   a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = 0;
   const int64_t nb = cdiv(N, 256) * (K / 256);
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
   hipLaunchKernelGGL((k_bwd_fast<MODE_DW>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  if (dbias)
+    hipLaunchKernelGGL(k_bias_final, dim3((unsigned)cdiv(N, 256)), dim3(256), 0, s,
+                       (const float*)bias_partial, (int)(K / 256), N, (uint16_t*)dbias);
   return check_launch("ahl_linear_bwd_dw(fast)");
 }
 

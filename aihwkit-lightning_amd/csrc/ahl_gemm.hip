@@ -688,8 +688,9 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, bool ir_static, hipStream_t s);
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
-                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, int64_t M, int64_t K,
-                   int64_t N, const Tiling& tl, hipStream_t s);
+                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
+                   float* bias_partial, int64_t M, int64_t K, int64_t N, const Tiling& tl,
+                   hipStream_t s);
 }  // namespace ahl
 
 template <class D>
@@ -860,12 +861,15 @@ int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
   const int64_t es = dtype == AHL_BF16 ? 2 : 4;
   (void)n_tiles;
   (void)has_keep;
-  return align256(N * M * es) + align256(K * M * es);
+  // the fast path only uses [K / 256][N] floats of partial bias sums at the start of ws
+  const int64_t generic = align256(N * M * es) + align256(K * M * es) + align256(ahl_col_sum_ws_bytes(N));
+  const int64_t fast = align256(cdiv(K, 256) * N * (int64_t)sizeof(float));
+  return generic > fast ? generic : fast;
 }
 
 int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                       const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* ir,
-                      void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
+                      void* dw, int64_t lddw, void* dbias, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream) {
   if (!cfg_ok(cfg) || !g || (!x && !xq) || !dw || !ws || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
@@ -877,7 +881,7 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
   hipStream_t s = (hipStream_t)stream;
   if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
       ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && aligned16(dw) && (!keep || (((uintptr_t)keep) & 3u) == 0))
-    return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, M, K, N, tl, s);
+    return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, dbias, (float*)ws, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
   DwArgs a;
   a.M = M; a.N = N; a.K = K; a.tl = tl; a.dw = dw; a.lddw = lddw;
@@ -907,6 +911,10 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
     const dim3 grid((unsigned)(nbn * nkb)), block(256);
     if (vec) hipLaunchKernelGGL((k_linear_bwd_dw<D, true>), grid, block, kGemmLds, s, a);
     else hipLaunchKernelGGL((k_linear_bwd_dw<D, false>), grid, block, kGemmLds, s, a);
+    if (dbias) {
+      const int rc = ahl_col_sum(g, cfg->dtype, M, N, ldg, dbias, p, stream);
+      if (rc != AHL_OK) return rc;
+    }
   });
   return check_launch("ahl_linear_bwd_dw");
 }

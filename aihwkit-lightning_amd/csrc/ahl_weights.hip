@@ -1,6 +1,5 @@
 // Weight-side kernels: per-tile per-channel abs-max, on-the-fly quantisation and Gaussian weight
-// noise into a scratch copy (plus its transpose for the input-gradient product), and the
-// in-place post-training quantisation.
+// noise into a scratch copy, and the in-place post-training quantisation.
 #include "ahl_host.h"
 #include "ahl_reduce_kernels.h"
 
@@ -43,65 +42,76 @@ struct ModArgs {
   const float* tile_min;  // [T]
   void* w_eff;            // dtype [N, K] (may alias w for the in-place quantiser) or null
   int64_t ld_eff;
-  void* w_eff_t;          // dtype [K, N] or null
   int32_t quant_type, noise_type;
   float n_states, maxq, std_dev;
   uint64_t seed, offset;
 };
 
-// 64 (channels) x 64 (inputs) tile per block; thread = 8 consecutive inputs x 2 channels.
-template <class D>
-__global__ __launch_bounds__(256) void k_weight_modify(ModArgs a) {
-  __shared__ typename D::elem tileT[64][64 + 4];
-  const int k0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
-  const int kq = threadIdx.x & 7, nr = threadIdx.x >> 3;
+// One thread per group of 8 consecutive inputs of one channel (one Philox call gives the 8
+// normals of the group); consecutive threads walk along the row, so that with VEC every wave
+// reads and writes contiguous 16-byte vectors.
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t blocks_per_row) {
+  const int64_t n = blockIdx.x / blocks_per_row;
+  const int32_t kb = (int32_t)((blockIdx.x % blocks_per_row) * 256 + threadIdx.x) * 8;
+  if (kb >= a.K) return;
+  const int32_t klast = kb + 7 < a.K ? kb + 7 : (int32_t)a.K - 1;
+  const bool modify = a.quant_type != AHL_QUANT_NONE || a.noise_type != AHL_NOISE_NONE;
+
+  float v[8];
+  const typename D::elem* src = (const typename D::elem*)a.w + n * a.ld + kb;
+  if (VEC) {
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int64_t n = n0 + nr + 32 * j;
-    const int kb = k0 + 8 * kq;
+    for (int q = 0; q < 8 / D::EPV; ++q) D::unpack(ld16(src + q * D::EPV), v + q * D::EPV);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = kb + e < a.K ? D::load(a.w, n * a.ld + kb + e) : 0.0f;
+  }
+
+  if (modify) {
     float xi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (a.noise_type != AHL_NOISE_NONE && n < a.N && kb < a.K)
+    if (a.noise_type != AHL_NOISE_NONE)
       normal8(a.seed, a.offset, 1u << 24, (uint32_t)(kb >> 3), (uint32_t)n, xi);
+    // constants of a tile for this channel
+    struct TileConst { WQuant q; float nstd; };
+    auto tile_const = [&](int t) {
+      TileConst c;
+      const float wm = D::load(a.wmax, (int64_t)t * a.N + n);
+      const float tmax = a.tile_max[t];
+      c.q.step = 1.0f; c.q.rc = 1.0f; c.q.rcp = 1.0f;
+      if (a.quant_type == AHL_QUANT_DISCRETIZE_PER_CHANNEL) {
+        const bool all_gt1 = D::rd(__fdiv_rn(a.tile_min[t], a.n_states)) > 1.0f;
+        c.q = make_wquant<D>(wm, a.n_states, all_gt1);
+      } else if (a.quant_type == AHL_QUANT_DISCRETIZE) {
+        const bool all_gt1 = D::rd(__fdiv_rn(tmax, a.n_states)) > 1.0f;
+        c.q = make_wquant<D>(tmax, a.n_states, all_gt1);
+      }
+      c.nstd = D::rd(a.std_dev * (a.noise_type == AHL_NOISE_ADD_NORMAL_PER_CHANNEL ? wm : tmax));
+      return c;
+    };
+    const int t0 = a.tl.tile_of(kb), t1 = a.tl.tile_of(klast);
+    TileConst c = tile_const(t0);
+    const int32_t t1_start = t1 != t0 ? a.tl.start(t1) : 0x7fffffff;  // a group spans at most 2 tiles
+    const TileConst c1 = t1 != t0 ? tile_const(t1) : c;
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int k = kb + e;
-      float v = 0.0f;
-      if (n < a.N && k < a.K) {
-        v = D::load(a.w, n * a.ld + k);
-        if (a.quant_type != AHL_QUANT_NONE || a.noise_type != AHL_NOISE_NONE) {
-          const int t = a.tl.tile_of(k);
-          const float wm = D::load(a.wmax, (int64_t)t * a.N + n);
-          const float tmax = a.tile_max[t];
-          if (a.quant_type == AHL_QUANT_DISCRETIZE_PER_CHANNEL) {
-            const bool all_gt1 = D::rd(__fdiv_rn(a.tile_min[t], a.n_states)) > 1.0f;
-            v = wquant_apply<D>(v, make_wquant<D>(wm, a.n_states, all_gt1), a.maxq);
-          } else if (a.quant_type == AHL_QUANT_DISCRETIZE) {
-            const bool all_gt1 = D::rd(__fdiv_rn(tmax, a.n_states)) > 1.0f;
-            v = wquant_apply<D>(v, make_wquant<D>(tmax, a.n_states, all_gt1), a.maxq);
-          }
-          if (a.noise_type != AHL_NOISE_NONE) {
-            const float ref = a.noise_type == AHL_NOISE_ADD_NORMAL_PER_CHANNEL ? wm : tmax;
-            const float nstd = D::rd(a.std_dev * ref);
-            v = D::rd(v + D::rd(nstd * D::rd(xi[e])));
-          }
-        }
-        if (a.w_eff) D::store(a.w_eff, n * a.ld_eff + k, v);
-      }
-      tileT[8 * kq + e][nr + 32 * j] = D::to_elem(v);
+      const TileConst& ce = kb + e >= t1_start ? c1 : c;
+      float x = v[e];
+      if (a.quant_type != AHL_QUANT_NONE) x = wquant_apply<D>(x, ce.q, a.maxq);
+      if (a.noise_type != AHL_NOISE_NONE) x = D::rd(x + D::rd(ce.nstd * D::rd(xi[e])));
+      v[e] = x;
     }
   }
-  if (!a.w_eff_t) return;
-  __syncthreads();
-  const int nq = threadIdx.x & 15, kr = threadIdx.x >> 4;
+
+  if (!a.w_eff) return;
+  typename D::elem* dst = (typename D::elem*)a.w_eff + n * a.ld_eff + kb;
+  if (VEC) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t k = k0 + kr + 16 * j;
-    if (k >= a.K) continue;
+    for (int q = 0; q < 8 / D::EPV; ++q) st16(dst + q * D::EPV, D::pack(v + q * D::EPV));
+  } else {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int64_t n = n0 + 4 * nq + e;
-      if (n < a.N) ((typename D::elem*)a.w_eff_t)[k * a.N + n] = tileT[kr + 16 * j][4 * nq + e];
-    }
+    for (int e = 0; e < 8; ++e)
+      if (kb + e < a.K) D::store(a.w_eff, n * a.ld_eff + kb + e, v[e]);
   }
 }
 
@@ -111,7 +121,7 @@ using namespace ahl;
 
 static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Tiling& tl,
                        const AhlModifierCfg* cfg, bool with_noise, void* wmax, float* tile_max,
-                       float* tile_min, void* w_eff, int64_t ld_eff, void* w_eff_t, hipStream_t s) {
+                       float* tile_min, void* w_eff, int64_t ld_eff, hipStream_t s) {
   const int32_t dtype = cfg->dtype;
   const int32_t noise = with_noise ? cfg->noise_type : AHL_NOISE_NONE;
   if (cfg->quant_type < 0 || cfg->quant_type > 2 || noise < 0 || noise > 2) return AHL_ERR_ARG;
@@ -122,17 +132,23 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
     if (vec) hipLaunchKernelGGL((k_sliced_absmax<D, true>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
     else hipLaunchKernelGGL((k_sliced_absmax<D, false>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
     hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
-    if (w_eff || w_eff_t) {
+    if (w_eff) {
       ModArgs a;
       a.w = w; a.N = N; a.K = K; a.ld = ld; a.tl = tl; a.wmax = wmax; a.tile_max = tile_max;
-      a.tile_min = tile_min; a.w_eff = w_eff; a.ld_eff = ld_eff; a.w_eff_t = w_eff_t;
+      a.tile_min = tile_min; a.w_eff = w_eff; a.ld_eff = ld_eff;
       a.quant_type = cfg->quant_type; a.noise_type = noise;
       const float res = cfg->res;
       a.n_states = cfg->quant_type != AHL_QUANT_NONE ? fmaxf(res, 1.0f / res) : 1.0f;
       // clamp(Tensor, Scalar, Scalar) converts its bounds to the tensor dtype first
       a.maxq = D::kIsBf16 ? host_round_bf16(a.n_states / 2.0f) : a.n_states / 2.0f;
       a.std_dev = cfg->std_dev; a.seed = cfg->seed; a.offset = cfg->offset;
-      hipLaunchKernelGGL((k_weight_modify<D>), dim3((unsigned)cdiv(K, 64), (unsigned)cdiv(N, 64)), dim3(256), 0, s, a);
+      const int64_t bpr = cdiv(cdiv(K, 8), 256);
+      if (bpr * N > 0x7fffffff) return AHL_ERR_ARG;
+      const bool vec_mod = vec && K % 8 == 0 && aligned16(w_eff) && ld_eff % D::EPV == 0;
+      if (vec_mod)
+        hipLaunchKernelGGL((k_weight_modify<D, true>), dim3((unsigned)(bpr * N)), dim3(256), 0, s, a, (uint32_t)bpr);
+      else
+        hipLaunchKernelGGL((k_weight_modify<D, false>), dim3((unsigned)(bpr * N)), dim3(256), 0, s, a, (uint32_t)bpr);
     }
   });
   return check_launch("ahl_weight_prep");
@@ -148,7 +164,7 @@ int ahl_weight_prep(const void* w, int64_t N, int64_t K, int64_t ld, const int32
   if (w_eff == w) return AHL_ERR_ARG;  // never modifies the parameter storage
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
-  return launch_prep(w, N, K, ld, tl, cfg, true, wmax, tile_max, tile_min, w_eff, ld_eff, nullptr,
+  return launch_prep(w, N, K, ld, tl, cfg, true, wmax, tile_max, tile_min, w_eff, ld_eff,
                      (hipStream_t)stream);
 }
 
@@ -159,7 +175,7 @@ int ahl_quantize_weights(void* w, int64_t N, int64_t K, int64_t ld, const int32_
   if (cfg->quant_type == AHL_QUANT_NONE) return AHL_OK;
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
-  return launch_prep(w, N, K, ld, tl, cfg, false, ws_wmax, ws_tile, ws_tile + n_tiles, w, ld, nullptr,
+  return launch_prep(w, N, K, ld, tl, cfg, false, ws_wmax, ws_tile, ws_tile + n_tiles, w, ld,
                      (hipStream_t)stream);
 }
 

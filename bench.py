@@ -93,8 +93,8 @@ def kernel_rooflines(layer, x, g, reps):
     out["linear_fwd"] = t
     t = event_time_ms(lambda: OPS.linear_bwd_dx(g, keep, flag, w_eff, x, ir, in_sizes, icfg, fcfg), reps)
     out["linear_bwd_dx(+ir_grad)"] = t
-    t = event_time_ms(lambda: OPS.linear_bwd_dw(g, keep, flag, None, xq, ir, in_sizes, icfg, fcfg), reps)
-    out["linear_bwd_dw"] = t
+    t = event_time_ms(lambda: OPS.linear_bwd_dw(g, keep, flag, None, xq, ir, in_sizes, icfg, fcfg, True), reps)
+    out["linear_bwd_dw(+bias_grad)"] = t
     out["dac"] = event_time_ms(lambda: OPS.dac(x, ir, in_sizes, icfg, fcfg), reps)
     t = event_time_ms(lambda: OPS.weight_prep(layer.weight.data, in_sizes, L.AHL_QUANT_NONE,
                                               L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02, 11, 1,
@@ -179,7 +179,7 @@ def main():
     value = step_flops / (ms_per_step * 1e-3) / 1e12
 
     kernels, gemm_flops = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 5))
-    dom = max(("linear_fwd", "linear_bwd_dx(+ir_grad)", "linear_bwd_dw"),
+    dom = max(("linear_fwd", "linear_bwd_dx(+ir_grad)", "linear_bwd_dw(+bias_grad)"),
               key=lambda k: kernels[k])
     achieved = gemm_flops / (kernels[dom] * 1e-3) / 1e12
     result = {

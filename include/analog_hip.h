@@ -218,12 +218,15 @@ int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
 
 /* Weight gradient: dw[:, tile t] = (g * !clamped_t)^T @ DAC(clamp(x[:, tile t])).
  *   xq: the quantised input saved from the forward (ahl_dac), or NULL to re-quantise x here.
+ *   dbias: dtype [N] or NULL; receives the bias gradient sum_m g[m, :] (the autograd of the
+ *   bias addition in AnalogLinear.forward, nn/modules/linear.py:120-135), which the kernel
+ *   gets for free while it streams g.
  *   ws needs ahl_linear_bwd_dw_ws_bytes(M, K, N, n_tiles, dtype, clamp_mask != NULL) bytes
  *   (transposed staging copies of g and the quantised input).
  * Same reference slot as ahl_linear_bwd_dx.                                               */
 int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* clamp_mask, const uint32_t* clamp_flag,
                       const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* ir,
-                      void* dw, int64_t lddw, int64_t M, int64_t K, int64_t N,
+                      void* dw, int64_t lddw, void* dbias, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
