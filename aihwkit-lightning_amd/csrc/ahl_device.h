@@ -153,19 +153,16 @@ AHL_DEV u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
 // v_log_f32 is log2, v_sin_f32 / v_cos_f32 take their argument in revolutions.
 AHL_DEV void box_muller16(uint32_t w, float& n0, float& n1) {
   const float a = (float)(w & 0xffffu) + 0.5f;
-  const float b = (float)(w >> 16) + 0.5f;
-  const float r2 = (16.0f - __builtin_amdgcn_logf(a)) * 1.3862943611198906f;  // -2 ln(a / 65536)
+  // radius^2 = -2 ln(a / 65536) = (16 - log2 a) * 2 ln 2
+  const float r2 = __builtin_fmaf(__builtin_amdgcn_logf(a), -1.3862943611198906f, 22.180709777918250f);
   const float r = __builtin_amdgcn_sqrtf(r2);
-  const float rev = b * 1.52587890625e-05f;  // / 65536
+  // angle in revolutions: the high half as the mantissa of a float in [1, 2); v_sin/v_cos are
+  // periodic in whole revolutions, so the leading 1 needs no subtraction
+  const float rev = __uint_as_float(0x3f800000u | ((w >> 9) & 0x007fff80u));
   n0 = r * __builtin_amdgcn_cosf(rev);
   n1 = r * __builtin_amdgcn_sinf(rev);
 }
 
-// Eight standard normals for one counter value (c0, c1, stream << 24 | tile, offset).
-//   output noise: stream 0; c0 = n (output column), c1 = (m >> 4) * 2 + ((m >> 2) & 1); normal j
-//                 belongs to row 16 * (m >> 4) + 4 * ((m >> 2) & 1) + (j & 3) + 8 * (j >> 2)  -- the 8
-//                 rows one lane of a 32x32 MFMA result holds in two consecutive register groups
-//   weight noise: stream 1, tile field 0; c0 = k >> 3, c1 = n (weight row); normal j is k % 8
 AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, uint32_t c0,
                      uint32_t c1, float* out8) {
   u32x4 c = {c0, c1, stream_and_tile, (uint32_t)offset};

@@ -211,24 +211,30 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
       const int r = lane & 31;
       const char* pa = ldsA + (wm * 64 + r) * kLdsStrideF + h * 16;
       const char* pb = ldsB + (wn * WN + r) * kLdsStrideF + h * 16;
+      // fragments of step s + 1 are read while the MFMAs of step s run
+      u32x4 fa[2][2], fb[2][NBJ];
+      auto read_frags = [&](int s, int buf) {
+        fa[buf][0] = *(const u32x4*)(pa + s * 32);
+        fa[buf][1] = *(const u32x4*)(pa + 32 * kLdsStrideF + s * 32);
+#pragma unroll
+        for (int bj = 0; bj < NBJ; ++bj) fb[buf][bj] = *(const u32x4*)(pb + bj * 32 * kLdsStrideF + s * 32);
+      };
+      read_frags(0, 0);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const u32x4 a0 = *(const u32x4*)(pa + s * 32);
-        const u32x4 a1 = *(const u32x4*)(pa + 32 * kLdsStrideF + s * 32);
-        u32x4 bf[NBJ];
-#pragma unroll
-        for (int bj = 0; bj < NBJ; ++bj) bf[bj] = *(const u32x4*)(pb + bj * 32 * kLdsStrideF + s * 32);
+        if (s < 3) read_frags(s + 1, (s + 1) & 1);
+        const u32x4 a0 = fa[s & 1][0], a1 = fa[s & 1][1];
         if (s == 0 && cin == 0) {  // first step of a K-tile starts from zero
 #pragma unroll
           for (int bj = 0; bj < NBJ; ++bj) {
-            mma_bf16_zero(a0, bf[bj], acc[0][bj]);
-            mma_bf16_zero(a1, bf[bj], acc[1][bj]);
+            mma_bf16_zero(a0, fb[s & 1][bj], acc[0][bj]);
+            mma_bf16_zero(a1, fb[s & 1][bj], acc[1][bj]);
           }
         } else {
 #pragma unroll
           for (int bj = 0; bj < NBJ; ++bj) {
-            mma_bf16(a0, bf[bj], acc[0][bj]);
-            mma_bf16(a1, bf[bj], acc[1][bj]);
+            mma_bf16(a0, fb[s & 1][bj], acc[0][bj]);
+            mma_bf16(a1, fb[s & 1][bj], acc[1][bj]);
           }
         }
       }
@@ -302,12 +308,10 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
               }
             }
             if (NOISE) {
-              float nz[4];
+              // y + scale * xi with one rounding: xi is an fp32 normal, so there is no bf16
+              // product of the reference to reproduce, and the sum is rounded once
 #pragma unroll
-              for (int c = 0; c < 4; ++c) nz[c] = ns[c] * xi[4 * gg + c];
-              rd2(nz[0], nz[1]); rd2(nz[2], nz[3]);
-#pragma unroll
-              for (int c = 0; c < 4; ++c) y[c] += nz[c];
+              for (int c = 0; c < 4; ++c) y[c] = __builtin_fmaf(ns[c], xi[4 * gg + c], y[c]);
               rd2(y[0], y[1]); rd2(y[2], y[3]);
             }
             if (ADC) {

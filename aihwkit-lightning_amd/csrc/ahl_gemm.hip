@@ -293,7 +293,7 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
                     }
                   }
                 }
-                if (a.noise_on) y = D::rd(y + D::rd(nscale * xi[4 * gg + c]));
+                if (a.noise_on) y = D::rd(__builtin_fmaf(nscale, xi[4 * gg + c], y));
                 if (a.bound_on) {
                   if (a.adc_on) {
                     float q = D::rd(D::div(y, rc, rcp));

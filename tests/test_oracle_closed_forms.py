@@ -233,7 +233,7 @@ def test_box_muller16_statistics():
     a = np.arange(65536, dtype=np.float64) + 0.5
     r = np.sqrt((16.0 - np.log2(a)) * 2.0 * math.log(2.0))
     assert abs(np.mean(r ** 2) / 2.0 - 1.0) < 1e-3  # E[r^2] = 2 for a unit normal pair
-    b = (np.arange(65536, dtype=np.float64) + 0.5) / 65536.0
+    b = 1.0 + np.arange(65536, dtype=np.float64) / 65536.0  # revolutions, mantissa of a float in [1, 2)
     c, s_ = np.cos(2 * np.pi * b), np.sin(2 * np.pi * b)
     # radius and angle are independent: moments factorise over the grid
     assert abs(c.mean()) < 1e-12 and abs(s_.mean()) < 1e-12
