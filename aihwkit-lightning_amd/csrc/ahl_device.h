@@ -37,6 +37,25 @@ struct Tiling {
 };
 
 // ---------------------------------------------------------------------------------------------
+// Block index -> (row block, column block) of the output. Workgroups go to the 8 XCDs round
+// robin (block b runs on XCD b % 8) and each XCD has its own L2, so (1) every XCD gets one
+// contiguous range of the linear tile order, and (2) that order walks bands of G row blocks
+// column by column: the blocks resident on an XCD at any time then form a compact patch of
+// about G rows by (resident / G) columns and share their operand panels in L2, instead of a
+// 1- or 2-row strip that streams the whole other operand.
+AHL_DEV void block_to_tile(int64_t bid, int64_t nb, int64_t nbm, int64_t nbn, int G, int64_t& bm,
+                           int64_t& bn) {
+  int64_t lin = bid;
+  if ((nb & 7) == 0) lin = (bid & 7) * (nb >> 3) + (bid >> 3);
+  const int64_t per_band = (int64_t)G * nbn;
+  const int64_t band = lin / per_band, in_band = lin % per_band;
+  const int64_t first = band * G;
+  const int64_t gsz = nbm - first < G ? nbm - first : G;
+  bm = first + in_band % gsz;
+  bn = in_band / gsz;
+}
+
+// ---------------------------------------------------------------------------------------------
 // Clamp-mask layout: one bit per (tile, row, column). Word [(t * ceil(N/32) + n / 32) * M + m]
 // has bit (n % 32) set where the tile-t output of element (m, n) left the ADC range (and so
 // passes no gradient). One 64-lane ballot over a 32x32 MFMA result register yields two such

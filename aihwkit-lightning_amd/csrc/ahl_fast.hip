@@ -132,9 +132,9 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 
   const int64_t nbn = cdiv_dev(a.N, BN);
   const int64_t nb = gridDim.x;
-  int64_t logical = blockIdx.x;
-  if ((nb & 7) == 0) logical = (logical & 7) * (nb >> 3) + (logical >> 3);
-  const int64_t m0 = (logical / nbn) * 128, n0 = (logical % nbn) * BN;
+  int64_t bm, bn;
+  block_to_tile(blockIdx.x, nb, cdiv_dev(a.M, 128), nbn, 8, bm, bn);
+  const int64_t m0 = bm * 128, n0 = bn * BN;
   const bool bound_on = ADC || a.clamp_on;
 
   f32x16 acc[2][NBJ];

@@ -64,10 +64,10 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   // ---- block -> output tile. columns of the output are k (both modes), 256 per block ----
   const int64_t nkb = a.K / 256;
   const int64_t nb = gridDim.x;
-  int64_t logical = blockIdx.x;
-  if ((nb & 7) == 0) logical = (logical & 7) * (nb >> 3) + (logical >> 3);
-  const int64_t r0 = (logical / nkb) * 256;          // DX: m0; DW: n0
-  const int64_t c0 = (logical % nkb) * 256;          // k0
+  int64_t brow, bcol;
+  block_to_tile(blockIdx.x, nb, nb / nkb, nkb, 4, brow, bcol);
+  const int64_t r0 = brow * 256;                     // DX: m0; DW: n0
+  const int64_t c0 = bcol * 256;                     // k0
   const int t = (int)(c0 / a.tile);
   const int64_t R = MODE == MODE_DX ? a.M : a.N;      // output rows
   const int64_t L = MODE == MODE_DX ? a.N : a.M;      // contraction length
@@ -133,7 +133,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   // row of blocks streams the same g; block kb of the nkb sums the chunks ch = kb (mod nkb), so
   // that the extra work is spread evenly, and a small kernel adds the nkb partial sums.
   float bsum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const int kb_idx = (int)(logical % nkb);
+  const int kb_idx = (int)bcol;
   auto stage = [&](char* sa, char* sb, bool masked, bool bias) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -282,7 +282,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     if (tid == 0) {
       float u = 0.f, l = 0.f, c = 0.f;
       for (int w = 0; w < 8; ++w) { u += red[w][0]; l += red[w][1]; c += red[w][2]; }
-      float* p = a.partial + logical * 4;
+      float* p = a.partial + (brow * nkb + bcol) * 4;
       p[0] = u; p[1] = l; p[2] = c; p[3] = 0.0f;
     }
   }

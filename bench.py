@@ -100,6 +100,11 @@ def kernel_rooflines(layer, x, g, reps):
                                               L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02, 11, 1,
                                               True), reps)
     out["weight_prep"] = t
+    # a plain device copy of known size (256 MiB read + 256 MiB written): the yardstick that
+    # HBM byte counters of a profiler run of this command are scaled by
+    src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=x.device)
+    dst = torch.empty_like(src)
+    out["copy_256MiB"] = event_time_ms(lambda: dst.copy_(src), reps)
     return out, flops
 
 
