@@ -26,6 +26,14 @@ import torch  # noqa: E402
 
 M_TOKENS, K_IN, N_OUT, TILE = 8192, 4096, 4096, 512
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+# Bytes per launch that the L2s pull from / push to the fabric (HBM or Infinity Cache), from
+# rocprofv3 FETCH_SIZE and WRITE_SIZE runs of `bench.py --kernels-only`, each scaled by what the
+# same counter reads for the 256 MiB copy below (profiles/*_hbm_traffic.txt holds the table).
+MEASURED_TRAFFIC_BYTES = {
+    "linear_fwd": int((697.1 + 96.2) * 2 ** 20),
+    "linear_bwd_dx(+ir_grad)": int((480.3 + 64.0) * 2 ** 20),
+    "linear_bwd_dw(+bias_grad)": int((416.1 + 32.2) * 2 ** 20),
+}
 
 
 def build_layer():
@@ -108,8 +116,9 @@ def kernel_rooflines(layer, x, g, reps):
     return out, flops
 
 
-def cpu_baseline(sample_tokens=1024):
-    """The torch-mode oracle (CPU restatement of the reference) on a token subsample."""
+def cpu_baseline(sample_tokens=M_TOKENS):
+    """The torch-mode oracle (CPU restatement of the reference) on the host cores: the whole
+    workload by default (about 7 s per forward + backward pass on 16 cores)."""
     from oracle import torch_mode as om
 
     threads = min(os.cpu_count() or 1, 16)
@@ -200,7 +209,8 @@ def main():
         },
         "roofline": {
             "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
-            "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4), "traffic": None,
+            "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
             "ms_per_launch": {k: round(v, 4) for k, v in kernels.items()},
         },
     }
