@@ -28,7 +28,8 @@ typedef __attribute__((address_space(3))) s16x4* lds_s16x4_ptr;
 static constexpr int kRowkStride = 144;               // k-contiguous operand: 128 B + 16 B pad
 static constexpr int kKmajStride = 576;               // k-major operand: 512 B + 64 B pad
 static constexpr int kOperandLds = 256 * kRowkStride; // == 64 * kKmajStride == 36864
-static constexpr int kBwdLds = 4 * kOperandLds;       // 2 operands x 2 stages
+static constexpr int kMaskLut = 4 * kOperandLds;      // LDS offset of the clamp-mask table
+static constexpr int kBwdLds = kMaskLut + 256 * 16;   // 2 operands x 2 stages + the table
 
 static constexpr int MODE_DX = 0;
 static constexpr int MODE_DW = 1;
@@ -143,7 +144,11 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) bsum[i] += e[i];
       }
-      if (masked) rawA[j] = clamp_apply8(rawA[j], rawK[j] >> psh);
+      if (masked) {
+        // the mask byte of the vector selects one of 256 precomputed 16-byte AND masks
+        const u32x4 km = *(const u32x4*)(lds + kMaskLut + (((rawK[j] >> psh) & 0xffu) << 4));
+        rawA[j] &= km;
+      }
       if (MODE == MODE_DX) *(u32x4*)(sa + (rk_row + 64 * j) * kRowkStride + rk_cv * 16) = rawA[j];
       else *(u32x4*)(sa + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawA[j];
       *(u32x4*)(sb + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawB[j];
@@ -163,6 +168,14 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     return o;
   };
 
+  if (plane) {  // uniform over the block
+    if (tid < 256) {
+      // entry e: halfword i is all ones unless bit i of e is set
+      const u32x4 ones = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+      *(u32x4*)(lds + kMaskLut + tid * 16) = clamp_apply8(ones, (uint32_t)tid);
+    }
+    __syncthreads();
+  }
   const int nchunks = (int)(L / 64);
   auto main_loop = [&](auto masked_tag, auto bias_tag) {
     constexpr bool kMasked = decltype(masked_tag)::value;
