@@ -14,53 +14,77 @@ int record_hip_error(hipError_t e, const char* where) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Per-tile sum and sum of squares over a block of kStdRows rows, in double.
-static constexpr int kStdRows = 16;
+// Per-tile sum and sum of squares, in double. Every wave owns `rpw` consecutive rows and writes
+// its own partial sums: no block-level synchronisation, and the grid has thousands of waves
+// even for a few thousand rows. The summation order is fixed by (rows, rpw), so results are
+// reproducible run to run.
+static constexpr int kStdRows = 16;  // rows per block of the whole-matrix clip kernels below
+
+// rows per wave: aim at >= 4096 waves, at most 16 rows each
+static int rows_per_wave(int64_t rows) {
+  const int64_t r = rows / 4096;
+  return (int)(r < 1 ? 1 : (r > 16 ? 16 : r));
+}
 
 template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_sliced_sums(const void* __restrict__ x, int64_t rows,
-                                                     int64_t ld, Tiling tl,
+                                                     int64_t ld, Tiling tl, int rpw,
                                                      double* __restrict__ partial) {
-  __shared__ double sh[4][2];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t r0 = (int64_t)blockIdx.x * kStdRows;
-  for (int32_t t = 0; t < tl.n_tiles; ++t) {
-    double s = 0.0, s2 = 0.0;
-    for (int i = wave; i < kStdRows; i += 4) {
-      const int64_t r = r0 + i;
-      if (r >= rows) break;
-      const typename D::elem* row = (const typename D::elem*)x + r * ld;
-      wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
-        s += (double)v;
-        s2 += (double)v * (double)v;
-      });
-    }
-    s = wave_sum(s);
-    s2 = wave_sum(s2);
-    __syncthreads();
-    if (lane == 0) { sh[wave][0] = s; sh[wave][1] = s2; }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      double* p = partial + ((int64_t)blockIdx.x * tl.n_tiles + t) * 2;
-      p[0] = (sh[0][0] + sh[1][0]) + (sh[2][0] + sh[3][0]);
-      p[1] = (sh[0][1] + sh[1][1]) + (sh[2][1] + sh[3][1]);
-    }
-  }
-}
-
-// out[t] = sqrt((S2 - S^2/n) / (n - 1)); one wave per tile, fixed summation order.
-__global__ __launch_bounds__(64) void k_std_finalize(const double* __restrict__ partial,
-                                                     int64_t n_blocks, int64_t rows, Tiling tl,
-                                                     float* __restrict__ out) {
-  const int t = blockIdx.x, lane = threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  // one wave per (group of rpw rows, tile): consecutive waves read consecutive tiles of a row
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t grp = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
+  const int64_t r0 = grp * rpw;
+  if (r0 >= rows) return;
   double s = 0.0, s2 = 0.0;
-  for (int64_t b = lane; b < n_blocks; b += 64) {
-    s += partial[(b * tl.n_tiles + t) * 2];
-    s2 += partial[(b * tl.n_tiles + t) * 2 + 1];
+  for (int i = 0; i < rpw; ++i) {
+    const int64_t r = r0 + i;
+    if (r >= rows) break;
+    const typename D::elem* row = (const typename D::elem*)x + r * ld;
+    wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
+      s += (double)v;
+      s2 += (double)v * (double)v;
+    });
   }
   s = wave_sum(s);
   s2 = wave_sum(s2);
   if (lane == 0) {
+    double* p = partial + wave * 2;  // == (grp * n_tiles + t) * 2
+    p[0] = s;
+    p[1] = s2;
+  }
+}
+
+// out[t] = sqrt((S2 - S^2/n) / (n - 1)); one wave per tile, fixed summation order.
+__global__ __launch_bounds__(256) void k_std_finalize(const double* __restrict__ partial,
+                                                      int64_t n_blocks, int64_t rows, Tiling tl,
+                                                      float* __restrict__ out) {
+  __shared__ double sh[4][2];
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  double s = 0.0, s2 = 0.0;
+  const int64_t stride = (int64_t)tl.n_tiles * 2;
+  const double* p = partial + (int64_t)t * 2;
+  int64_t b = tid;
+  for (; b + 768 < n_blocks; b += 1024) {  // four independent loads in flight per thread
+    const double a0 = p[b * stride], a1 = p[(b + 256) * stride];
+    const double a2 = p[(b + 512) * stride], a3 = p[(b + 768) * stride];
+    const double q0 = p[b * stride + 1], q1 = p[(b + 256) * stride + 1];
+    const double q2 = p[(b + 512) * stride + 1], q3 = p[(b + 768) * stride + 1];
+    s += (a0 + a1) + (a2 + a3);
+    s2 += (q0 + q1) + (q2 + q3);
+  }
+  for (; b < n_blocks; b += 256) {
+    s += p[b * stride];
+    s2 += p[b * stride + 1];
+  }
+  s = wave_sum(s);
+  s2 = wave_sum(s2);
+  if (lane == 0) { sh[wave][0] = s; sh[wave][1] = s2; }
+  __syncthreads();
+  if (tid == 0) {
+    s = (sh[0][0] + sh[1][0]) + (sh[2][0] + sh[3][0]);
+    s2 = (sh[0][1] + sh[1][1]) + (sh[2][1] + sh[3][1]);
     const double n = (double)rows * (double)tl.size(t);
     double var = (s2 - s * s / n) / (n - 1.0);  // n == 1 gives 0/0 = nan like torch
     if (var < 0.0) var = 0.0;
@@ -94,28 +118,25 @@ __global__ void k_ir_init_update(void* ir, void* idx, const float* __restrict__ 
 // negative int, so a signed integer atomicMax implements the float max exactly.
 template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_running_absmax(const void* __restrict__ x, int64_t rows,
-                                                        int64_t ld, Tiling tl, float* cache) {
-  __shared__ float sh[4];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int64_t r0 = (int64_t)blockIdx.x * kStdRows;
-  for (int32_t t = 0; t < tl.n_tiles; ++t) {
-    float m = 0.0f;
-    for (int i = wave; i < kStdRows; i += 4) {
-      const int64_t r = r0 + i;
-      if (r >= rows) break;
-      const typename D::elem* row = (const typename D::elem*)x + r * ld;
-      wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane,
-                               [&](float v) { m = fmaxf(m, fabsf(v)); });
-    }
-    m = wave_max(m);
-    __syncthreads();
-    if (lane == 0) sh[wave] = m;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      const float b = fmaxf(fmaxf(sh[0], sh[1]), fmaxf(sh[2], sh[3]));
-      atomicMax((int*)cache + t, __float_as_int(b));
-    }
+                                                        int64_t ld, Tiling tl, int rpw, float* cache) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t grp = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
+  const int64_t r0 = grp * rpw;
+  if (r0 >= rows) return;
+  float m = 0.0f;
+  for (int i = 0; i < rpw; ++i) {
+    const int64_t r = r0 + i;
+    if (r >= rows) break;
+    const typename D::elem* row = (const typename D::elem*)x + r * ld;
+    wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane,
+                             [&](float v) { m = fmaxf(m, fabsf(v)); });
   }
+  m = wave_max(m);
+  // most waves find the cached maximum already above theirs and skip the atomic
+  if (lane == 0 && __float_as_int(m) > __hip_atomic_load((int*)cache + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+    atomicMax((int*)cache + t, __float_as_int(m));
 }
 
 // ------------------------------------------------------------------------------------------
@@ -289,7 +310,8 @@ int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, 
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid((unsigned)cdiv(rows, 4));
+  if (cdiv(rows * n_tiles, 4) > 0x7fffffff) return AHL_ERR_ARG;
+  const dim3 grid((unsigned)cdiv(rows * n_tiles, 4));
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(x) && (ld % D::EPV == 0);
     if (vec) hipLaunchKernelGGL((k_sliced_absmax<D, true>), grid, dim3(256), 0, s, x, rows, ld, tl, out);
@@ -301,7 +323,8 @@ int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, 
 }
 
 int64_t ahl_sliced_std_ws_bytes(int64_t rows, int32_t n_tiles) {
-  return cdiv(rows, kStdRows) * (int64_t)n_tiles * 2 * (int64_t)sizeof(double);
+  if (rows <= 0 || n_tiles <= 0) return 0;
+  return cdiv(rows, rows_per_wave(rows)) * (int64_t)n_tiles * 2 * (int64_t)sizeof(double);
 }
 
 int ahl_sliced_std(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
@@ -311,13 +334,15 @@ int ahl_sliced_std(const void* x, int32_t dtype, int64_t rows, int64_t cols, int
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
-  const int64_t nb = cdiv(rows, kStdRows);
+  const int rpw = rows_per_wave(rows);
+  const int64_t nw = cdiv(rows, rpw), nb = cdiv(nw * n_tiles, 4);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(x) && (ld % D::EPV == 0);
-    if (vec) hipLaunchKernelGGL((k_sliced_sums<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, (double*)ws_partials);
-    else hipLaunchKernelGGL((k_sliced_sums<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, (double*)ws_partials);
+    if (vec) hipLaunchKernelGGL((k_sliced_sums<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
+    else hipLaunchKernelGGL((k_sliced_sums<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
   });
-  hipLaunchKernelGGL(k_std_finalize, dim3(n_tiles), dim3(64), 0, s, (const double*)ws_partials, nb, rows, tl, out);
+  hipLaunchKernelGGL(k_std_finalize, dim3(n_tiles), dim3(256), 0, s, (const double*)ws_partials, nw, rows, tl, out);
   return check_launch("ahl_sliced_std");
 }
 
@@ -337,11 +362,13 @@ int ahl_running_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols,
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
-  const int64_t nb = cdiv(rows, kStdRows);
+  const int rpw = rows_per_wave(rows);
+  const int64_t nb = cdiv(cdiv(rows, rpw) * n_tiles, 4);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(x) && (ld % D::EPV == 0);
-    if (vec) hipLaunchKernelGGL((k_running_absmax<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, cache);
-    else hipLaunchKernelGGL((k_running_absmax<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, cache);
+    if (vec) hipLaunchKernelGGL((k_running_absmax<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, cache);
+    else hipLaunchKernelGGL((k_running_absmax<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, cache);
   });
   return check_launch("ahl_running_absmax");
 }

@@ -5,22 +5,23 @@
 namespace ahl {
 
 // ------------------------------------------------------------------------------------------
-// out[t, r] = max_{c in tile t} |x[r, c]|. One wave per row, 4 rows per block.
+// out[t, r] = max_{c in tile t} |x[r, c]|. One wave per (row, tile), consecutive waves on
+// consecutive tiles of a row; grid = ceil(rows * n_tiles / 4) blocks of 4 waves.
 template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_sliced_absmax(const void* __restrict__ x, int64_t rows,
                                                        int64_t ld, Tiling tl,
                                                        void* __restrict__ out) {
   const int lane = threadIdx.x & 63;
-  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t r = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
   if (r >= rows) return;
   const typename D::elem* row = (const typename D::elem*)x + r * ld;
-  for (int32_t t = 0; t < tl.n_tiles; ++t) {
-    float m = 0.0f;
-    wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane,
-                             [&](float v) { m = fmaxf(m, fabsf(v)); });
-    m = wave_max(m);
-    if (lane == 0) D::store(out, (int64_t)t * rows + r, m);
-  }
+  float m = 0.0f;
+  wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane,
+                           [&](float v) { m = fmaxf(m, fabsf(v)); });
+  m = wave_max(m);
+  if (lane == 0) D::store(out, (int64_t)t * rows + r, m);
 }
 
 // tile_max[t] = max_r v[t, r], tile_min[t] = min_r v[t, r]; one block per tile.

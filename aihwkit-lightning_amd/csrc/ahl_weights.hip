@@ -128,7 +128,8 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
   if (cfg->quant_type != AHL_QUANT_NONE && !(cfg->res > 0.0f)) return AHL_ERR_ARG;
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(w) && (ld % D::EPV == 0);
-    const dim3 grid((unsigned)cdiv(N, 4));
+    if (cdiv(N * tl.n_tiles, 4) > 0x7fffffff) return AHL_ERR_ARG;
+    const dim3 grid((unsigned)cdiv(N * tl.n_tiles, 4));
     if (vec) hipLaunchKernelGGL((k_sliced_absmax<D, true>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
     else hipLaunchKernelGGL((k_sliced_absmax<D, false>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
     hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);

@@ -116,6 +116,58 @@ def kernel_rooflines(layer, x, g, reps):
     return out, flops
 
 
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
+
+
+def hbm_kernel_rooflines(reps):
+    """The memory-bound kernels of the path at the shapes of the clip / quantise / calibrate
+    configuration: one 8192 x 3072 fp32 weight matrix (6 tiles of 512 inputs), activation batches
+    of 2048 x 3072 fp32. GB/s = algorithmic bytes (each element read once, written where the
+    operation writes) / launch time; fraction of the 8 TB/s HBM peak."""
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+    from aihwkit_lightning.nn.modules.hip_utils import library as L
+
+    gen = torch.Generator().manual_seed(4)
+    n, k, m = 8192, 3072, 2048
+    in_sizes = [512] * 6
+    # 4 weight matrices (403 MB) and 16 activation batches (403 MB), visited in turn, so that
+    # consecutive launches do not find their input in the 256 MB Infinity Cache
+    w0 = (0.02 * torch.randn(n, k, generator=gen)).cuda()
+    ws = [w0] + [w0.clone() for _ in range(3)]
+    x0 = torch.randn(m, k, generator=gen).cuda()
+    xs = [x0] + [x0.clone() for _ in range(15)]
+    xbs = [x0.to(torch.bfloat16).repeat(4, 1) for _ in range(8)]  # 8192 x 3072 bf16 (50 MB each)
+    cache = torch.zeros(6, dtype=torch.float32, device="cuda")
+    irb = torch.full((6,), 3.0, device="cuda", dtype=torch.bfloat16)
+    wb, xbytes = n * k * 4, m * k * 4
+    icfg = [L.AHL_IR_STATIC, 0, 1, 0, 0, 0, 0]
+    fcfg = [254.0, 254.0, 10.0, 0.0, 0.0, 0.95]
+    turn = [0]
+
+    def nxt(lst):
+        turn[0] += 1
+        return lst[turn[0] % len(lst)]
+
+    cases = {
+        "sliced_absmax(W)": (lambda: OPS.sliced_absmax(nxt(ws), in_sizes, True), wb),
+        "sliced_std(x)": (lambda: OPS.sliced_std(nxt(xs), in_sizes), xbytes),
+        "running_absmax(x)": (lambda: OPS.running_absmax(nxt(xs), in_sizes, cache), xbytes),
+        # std pass + clamp pass; the clamp pass re-reads W and writes only changed vectors
+        "clip_weights(W, per channel)": (lambda: OPS.clip_weights(nxt(ws), 3.0, L.AHL_CLIP_PER_CHANNEL), 2 * wb),
+        # abs-max pass + quantise pass (read + write)
+        "quantize_weights(W)": (lambda: OPS.quantize_weights(
+            nxt(ws), in_sizes, L.AHL_QUANT_DISCRETIZE_PER_CHANNEL, 254.0), 3 * wb),
+        "dac(x bf16 8192x3072)": (lambda: OPS.dac(nxt(xbs), irb, in_sizes, icfg, fcfg),
+                                  2 * xbs[0].numel() * 2),
+    }
+    out = {}
+    for name, (fn, nbytes) in cases.items():
+        t = event_time_ms(fn, reps)
+        gbs = nbytes / (t * 1e-3) / 1e9
+        out[name] = {"us": round(t * 1e3, 1), "GB/s": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 3)}
+    return out
+
+
 def cpu_baseline(sample_tokens=M_TOKENS):
     """The torch-mode oracle (CPU restatement of the reference) on the host cores: the whole
     workload by default (about 7 s per forward + backward pass on 16 cores)."""
@@ -214,6 +266,7 @@ def main():
             "ms_per_launch": {k: round(v, 4) for k, v in kernels.items()},
         },
     }
+    result["hbm_kernels"] = hbm_kernel_rooflines(max(ns.steps, 5))
     if not ns.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result))
