@@ -84,45 +84,48 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
   // ---- staging maps ----
-  // k-contiguous operand (DX: g rows m): vector j -> row tid/8 + 64 j, 16-byte column tid%8
-  // k-major operand: vector j -> contraction row tid/32 + 16 j, 16-byte column tid%32
+  // operand A (g): a thread owns 4 consecutive rows, so that the clamp-mask words of its four
+  // vectors are 16 contiguous bytes (one load per chunk):
+  //   DX (k-contiguous, rows m):      vector j -> row 4 (tid/8) + j,  16-byte column tid%8
+  //   DW (k-major, contraction rows): vector j -> row 4 (tid/32) + j, 16-byte column tid%32
+  // operand B (k-major): vector j -> contraction row tid/32 + 16 j, 16-byte column tid%32
   const int rk_row = tid >> 3, rk_cv = tid & 7;
   const int km_row = tid >> 5, km_cv = tid & 31;
   u32x4 rawA[4], rawB[4];
-  uint32_t rawK[4] = {0u, 0u, 0u, 0u};  // mask words of the vectors in rawA
+  u32x4 rawK = {0u, 0u, 0u, 0u};  // mask words of the vectors in rawA
 
   // Rows of the output tile that lie beyond the matrix are redirected to the last valid row:
   // they only feed accumulators that are never stored. No predicates in the hot loop.
   // Clamp mask: the 8 gradient values of one 16-byte vector are one byte of a mask word.
   const uint16_t* pa[4];
-  const uint32_t* pk[4];
+  const uint32_t* pk = nullptr;
   int psh = 0;
   const uint16_t* pb[4];
+  if (MODE == MODE_DX) {
+    int64_t mq = r0 + 4 * rk_row;          // M is a multiple of 64: a row quad is all in or all out
+    mq = mq < a.M ? mq : a.M - 4;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    if (MODE == MODE_DX) {
-      int64_t m = r0 + rk_row + 64 * j;
-      m = m < a.M ? m : a.M - 1;
-      pa[j] = a.g + m * a.ldg + rk_cv * 8;              // + l0 (contraction n)
-      pk[j] = plane ? plane + clamp_word(m, rk_cv * 8, a.M) : nullptr;  // + (l0 / 32) * M
-      psh = 8 * (rk_cv & 3);
-    } else {
-      int64_t n = r0 + km_cv * 8;
-      n = n < a.N ? n : a.N - 8;
-      pa[j] = a.g + (int64_t)(km_row + 16 * j) * a.ldg + n;  // + l0 * ldg (contraction m)
-      pk[j] = plane ? plane + clamp_word(km_row + 16 * j, n, a.M) : nullptr;  // + l0
-      psh = 8 * (int)((n >> 3) & 3);
-    }
-    pb[j] = a.b + (int64_t)(km_row + 16 * j) * a.ldb + c0 + km_cv * 8;  // + l0 * ldb
+    for (int j = 0; j < 4; ++j) pa[j] = a.g + (mq + j) * a.ldg + rk_cv * 8;  // + l0 (contraction n)
+    if (plane) pk = plane + clamp_word(mq, rk_cv * 8, a.M);                  // + (l0 / 32) * M
+    psh = 8 * (rk_cv & 3);
+  } else {
+    int64_t n = r0 + km_cv * 8;
+    n = n < a.N ? n : a.N - 8;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pa[j] = a.g + (int64_t)(4 * km_row + j) * a.ldg + n;  // + l0 * ldg
+    if (plane) pk = plane + clamp_word(4 * km_row, n, a.M);                           // + l0
+    psh = 8 * (int)((n >> 3) & 3);
   }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) pb[j] = a.b + (int64_t)(km_row + 16 * j) * a.ldb + c0 + km_cv * 8;  // + l0 * ldb
   const int64_t a_step = MODE == MODE_DX ? 64 : 64 * a.ldg;
   const int64_t k_step = MODE == MODE_DX ? 2 * a.M : 64;   // 64 columns = 2 words; or 64 rows
   const int64_t b_step = 64 * a.ldb;
   auto load = [&](bool masked) {
+    if (masked) { rawK = ld16(pk); pk += k_step; }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       rawA[j] = ld16(pa[j]);
-      if (masked) { rawK[j] = *pk[j]; pk[j] += k_step; }
       rawB[j] = ld16(pb[j]);
       pa[j] += a_step;
       pb[j] += b_step;
@@ -149,8 +152,8 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
         const u32x4 km = *(const u32x4*)(lds + kMaskLut + (((rawK[j] >> psh) & 0xffu) << 4));
         rawA[j] &= km;
       }
-      if (MODE == MODE_DX) *(u32x4*)(sa + (rk_row + 64 * j) * kRowkStride + rk_cv * 16) = rawA[j];
-      else *(u32x4*)(sa + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawA[j];
+      if (MODE == MODE_DX) *(u32x4*)(sa + (4 * rk_row + j) * kRowkStride + rk_cv * 16) = rawA[j];
+      else *(u32x4*)(sa + (4 * km_row + j) * kKmajStride + km_cv * 16) = rawA[j];
       *(u32x4*)(sb + (km_row + 16 * j) * kKmajStride + km_cv * 16) = rawB[j];
     }
   };

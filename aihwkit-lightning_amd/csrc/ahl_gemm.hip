@@ -816,7 +816,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
   void* wt = (char*)ws + dx_partial_bytes(M, K, n_tiles);
   const bool fast = fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(w_eff) &&
                     ldg % 8 == 0 && ldw % 8 == 0 && lddx % 8 == 0 && aligned16(dx) &&
-                    (!keep || (((uintptr_t)keep) & 3u) == 0) &&
+                    (!keep || aligned16(keep)) &&
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
     int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
@@ -880,7 +880,7 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
   if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
-      ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && aligned16(dw) && (!keep || (((uintptr_t)keep) & 3u) == 0))
+      ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && aligned16(dw) && (!keep || aligned16(keep)))
     return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, dbias, (float*)ws, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
   DwArgs a;
