@@ -42,9 +42,6 @@ def check_supported(rpu_config: TorchInferenceRPUConfig) -> None:
     """Reject configuration branches that the HIP backend does not implement."""
     if rpu_config.clip.type == WeightClipType.LEARNABLE_PER_CHANNEL:
         raise ConfigError("WeightClipType.LEARNABLE_PER_CHANNEL is not implemented by the HIP backend")
-    ir_params = rpu_config.pre_post.input_range
-    if ir_params.enable and ir_params.fast_mode:
-        raise ConfigError("input_range.fast_mode is not implemented by the HIP backend")
 
 
 class HipLinear(Function):
@@ -64,6 +61,8 @@ class HipLinear(Function):
         rpu_config: TorchInferenceRPUConfig,
         training: bool,
         init_active: bool,
+        x_min: Optional[Tensor] = None,
+        x_max: Optional[Tensor] = None,
     ) -> Tensor:
         if not inp.is_cuda:
             raise HipBackendError(
@@ -86,7 +85,15 @@ class HipLinear(Function):
         if apply_out_quantization:
             assert fwd.out_bound > 0, "Out quant. without a bound."
             assert ir_params.enable, "Out quant. without IR."
-        if ir_params.enable and not ir_params.dynamic:
+        # fast_mode takes precedence over dynamic, as in the reference (torch_linear.py:138-153)
+        fast = bool(ir_params.enable and ir_params.fast_mode)
+        if fast:
+            assert x_min is not None, "x_min must be provided"
+            assert x_max is not None, "x_max must be provided"
+            assert input_range is not None, "Input range must be provided"
+            assert input_range_update_idx is not None, "Input range update index must be provided"
+            ir_mode = L.AHL_IR_STATIC
+        elif ir_params.enable and not ir_params.dynamic:
             assert input_range is not None, "Input range must be provided"
             assert input_range_update_idx is not None, "Input range update index must be provided"
             ir_mode = L.AHL_IR_STATIC
@@ -129,6 +136,8 @@ class HipLinear(Function):
             int(rpu_config.clip.type in (WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL,
                                          WeightClipType.LEARNABLE_PER_CHANNEL)),
             int(training), skip_rounding, seed, 0,
+            # fast_mode clamps with torch.clamp: its autograd rule instead of the learned-range one
+            L.AHL_IR_GRAD_CLAMP if fast else L.AHL_IR_GRAD_LEARNED,
         ]
         fcfg = [
             float(fwd.inp_res), float(fwd.out_res), float(fwd.out_bound),
@@ -146,7 +155,12 @@ class HipLinear(Function):
         )
         ir_dev = xq = None
         if ir_mode == L.AHL_IR_STATIC:
-            if training and init_active:
+            if training and init_active and fast:
+                OPS.ir_fast_update(
+                    x2, in_sizes, input_range.data, input_range_update_idx, x_min, x_max,
+                    float(ir_params.init_from_data), float(ir_params.act_range_momentum),
+                )
+            elif training and init_active:
                 std = OPS.sliced_std(x2, in_sizes)
                 OPS.ir_init_update(
                     input_range.data, input_range_update_idx, std, float(ir_params.init_from_data),
@@ -208,4 +222,4 @@ class HipLinear(Function):
                 grad_b = dbias
         elif want_bias:
             grad_b = OPS.col_sum(g2)
-        return grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None
+        return grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None, None, None

@@ -5,19 +5,22 @@ Loading is lazy and failure is loud: there is no software fallback for any entry
 """
 import ctypes
 import os
-from ctypes import c_void_p, c_int32, c_int64, c_float, c_uint64, c_char_p, POINTER, Structure
+from ctypes import (
+    c_void_p, c_int32, c_int64, c_float, c_double, c_uint64, c_char_p, POINTER, Structure,
+)
 
 from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
 AHL_NOISE_NONE, AHL_NOISE_ADD_NORMAL, AHL_NOISE_ADD_NORMAL_PER_CHANNEL = 0, 1, 2
 AHL_QUANT_NONE, AHL_QUANT_DISCRETIZE, AHL_QUANT_DISCRETIZE_PER_CHANNEL = 0, 1, 2
 AHL_CLIP_LAYER, AHL_CLIP_PER_CHANNEL = 0, 1
+AHL_IR_GRAD_LEARNED, AHL_IR_GRAD_CLAMP = 0, 1
 
 STATUS_TEXT = {
     1: "invalid argument",
@@ -44,6 +47,7 @@ class AhlLinearCfg(Structure):
         ("skip_rounding", c_int32),
         ("ir_decay", c_float),
         ("ir_input_min_percentage", c_float),
+        ("ir_grad_rule", c_int32),
         ("seed", c_uint64),
         ("offset", c_uint64),
     ]
@@ -85,6 +89,12 @@ SIGNATURES = {
     "ahl_running_absmax": (
         c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, _I32P, c_int32, c_void_p, c_void_p]
     ),
+    "ahl_ir_fast_update": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int64, c_int64, _I32P, c_int32, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_float, c_double, c_void_p, c_void_p],
+    ),
+    "ahl_ir_fast_update_ws_bytes": (c_int64, [c_int64, c_int32]),
     "ahl_clip_weights": (
         c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_float, c_int32, c_void_p, c_void_p]
     ),

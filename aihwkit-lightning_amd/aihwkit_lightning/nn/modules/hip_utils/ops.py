@@ -52,7 +52,8 @@ def _linear_cfg(dtype: torch.dtype, icfg: List[int], fcfg: List[float]) -> L.Ahl
     cfg = L.AhlLinearCfg()
     cfg.dtype = dtype_id(dtype)
     (cfg.ir_mode, cfg.out_noise_per_channel, cfg.bound_per_channel, cfg.training,
-     cfg.skip_rounding, seed, offset) = icfg
+     cfg.skip_rounding, seed, offset) = icfg[:7]
+    cfg.ir_grad_rule = icfg[7] if len(icfg) > 7 else L.AHL_IR_GRAD_LEARNED
     (cfg.inp_res, cfg.out_res, cfg.out_bound, cfg.out_noise, cfg.ir_decay,
      cfg.ir_input_min_percentage) = fcfg
     cfg.seed, cfg.offset = seed, offset
@@ -68,6 +69,10 @@ LIB.define(
     "float alpha) -> ()"
 )
 LIB.define("running_absmax(Tensor x, int[] in_sizes, Tensor(a!) cache) -> ()")
+LIB.define(
+    "ir_fast_update(Tensor x, int[] in_sizes, Tensor(a!) ir, Tensor(b!) idx, Tensor(c!) x_min, "
+    "Tensor(d!) x_max, float init_from_data, float momentum) -> ()"
+)
 LIB.define("clip_weights(Tensor(a!) w, float sigma, int kind) -> ()")
 LIB.define("col_sum(Tensor x) -> Tensor")
 LIB.define(
@@ -157,6 +162,27 @@ def running_absmax(x: Tensor, in_sizes: List[int], cache: Tensor) -> None:
             len(in_sizes), _ptr(cache), _stream(),
         ),
         "ahl_running_absmax",
+    )
+
+
+def ir_fast_update(x: Tensor, in_sizes: List[int], ir: Tensor, idx: Tensor, x_min: Tensor,
+                   x_max: Tensor, init_from_data: float, momentum: float) -> None:
+    """In-place fast_mode update of the running min / max, the step counter and the range."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    for buf in (ir, idx, x_min, x_max):
+        if not (buf.is_contiguous() and buf.dtype == x.dtype and buf.numel() == len(in_sizes)):
+            raise HipBackendError("input_range, its counter, x_min and x_max must be contiguous "
+                                  "[n_tiles] tensors of the input dtype")
+    ws = torch.empty((lib.ahl_ir_fast_update_ws_bytes(x.size(0), len(in_sizes)),), dtype=torch.uint8,
+                     device=x.device)
+    L.check(
+        lib.ahl_ir_fast_update(
+            _ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), L.tile_ends_array(in_sizes),
+            len(in_sizes), _ptr(ir), _ptr(idx), _ptr(x_min), _ptr(x_max), init_from_data, momentum,
+            _ptr(ws), _stream(),
+        ),
+        "ahl_ir_fast_update",
     )
 
 
@@ -365,7 +391,8 @@ def linear_bwd_dw(
 
 for _name, _fn in [
     ("sliced_absmax", sliced_absmax), ("sliced_std", sliced_std), ("ir_init_update", ir_init_update),
-    ("running_absmax", running_absmax), ("clip_weights", clip_weights), ("col_sum", col_sum),
+    ("running_absmax", running_absmax), ("ir_fast_update", ir_fast_update),
+    ("clip_weights", clip_weights), ("col_sum", col_sum),
     ("weight_prep", weight_prep), ("quantize_weights", quantize_weights),
     ("dac", dac), ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
 ]:

@@ -3,15 +3,17 @@
 // Why the DAC is a separate pass here: quantising an A element costs ~7 VALU instructions
 // (clamp, scale, two bf16 roundings, round-to-even, rescale) and a block that owns BN output
 // columns repeats that work for every one of the N/BN column blocks. At BN = 128 this is ~1.75x
-// the MFMA time of the block, on top of a per-tile epilogue that is already VALU-bound. One
+// the MFMA time of the block, on top of a VALU-heavy per-tile epilogue. One
 // memory-bound pass (k_dac_rows: read x once, write xq once, dynamic abs-max fused in) removes
 // that redundancy; the GEMM then streams xq through LDS untouched. The fused-prologue kernel
 // (ahl_gemm.hip) stays for fp32 and for shapes this path does not take.
 //
 // k_fwd_fast: block 256 threads = 2x2 waves, block tile 128 x 128, wave tile 64 x 64, chunks of 64
 // k; accumulator of the running K-tile in fp32 (64 registers), running total packed as bf16
-// pairs (32 registers) -- the total is a bf16 quantity by the semantics of the path -- so two to
-// three blocks fit on a CU and the VALU epilogue of one overlaps the MFMA phase of another.
+// pairs (32 registers) -- the total is a bf16 quantity by the semantics of the path -- so two
+// blocks fit on a CU and the VALU epilogue of one can overlap the MFMA phase of the other. With
+// this wave tile the kernel reads 64 KB of MFMA fragments from LDS and writes 32 KB into it per
+// 512 MFMA cycles of a SIMD: LDS bandwidth, not the MFMA pipe, bounds the plain product.
 #include "ahl_host.h"
 #include <math.h>
 
@@ -443,7 +445,7 @@ bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, co
   if (cfg->dtype != AHL_BF16 || xq == nullptr) return false;
   if (tl.extra != 0 || tl.base % 64 != 0) return false;
   if (!aligned16(xq) || !aligned16(w) || ldxq % 8 != 0 || ldw % 8 != 0) return false;
-  return K % 64 == 0;  // the caller also checks N % 8, ldy % 8 and the alignment of y and keep
+  return K % 64 == 0;  // the caller also checks N % 8, ldy % 8 and the alignment of y and the clamp mask
 }
 
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
@@ -466,14 +468,11 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   a.seed = cfg->seed; a.offset = cfg->offset;
   if (cdiv(M, 128) * cdiv(N, 64) > 0x7fffffff) return AHL_ERR_ARG;
   if (clamp_flag) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);
-  // 128 x 64 blocks (wave tile 64 x 32, four blocks per CU) when the epilogue dominates: more
-  // independent blocks per SIMD keep the VALU busy while others are in their MFMA phase;
-  // 128 x 128 blocks (less LDS traffic per MFMA) for the plain product.
-  const bool narrow = false;  // measured: the 128 x 64 variant is ~10 % slower even with noise + ADC on
-  (void)noise;
-  if (cfg->ir_mode == AHL_IR_NONE) { if (narrow) launch_fast<0, 1>(a, noise, adc, s); else launch_fast<0, 2>(a, noise, adc, s); }
-  else if (cfg->ir_mode == AHL_IR_STATIC) { if (narrow) launch_fast<1, 1>(a, noise, adc, s); else launch_fast<1, 2>(a, noise, adc, s); }
-  else { if (narrow) launch_fast<2, 1>(a, noise, adc, s); else launch_fast<2, 2>(a, noise, adc, s); }
+  // 128 x 128 blocks (NBJ = 2). Measured alternatives: 128 x 64 blocks (NBJ = 1, three to four
+  // blocks per CU) are ~10 % slower, 256 x 128 blocks (one block of 8 waves per CU) ~15 % slower.
+  if (cfg->ir_mode == AHL_IR_NONE) launch_fast<0, 2>(a, noise, adc, s);
+  else if (cfg->ir_mode == AHL_IR_STATIC) launch_fast<1, 2>(a, noise, adc, s);
+  else launch_fast<2, 2>(a, noise, adc, s);
   return check_launch("ahl_linear_fwd(fast)");
 }
 

@@ -1,6 +1,6 @@
 // bf16 fast path of the backward products.
 //
-//   dX[m, k] = sum_n gy[m, n] * W_eff[n, k]        (MODE_DX)   gy = g, masked by keep bit t(k)
+//   dX[m, k] = sum_n gy[m, n] * W_eff[n, k]        (MODE_DX)   gy = g, zeroed where tile t(k) was clamped
 //   dW[n, k] = sum_m gy[m, n] * xq[m, k]           (MODE_DW)
 //
 // Neither product has both operands contiguous along the contraction index in memory: W_eff
@@ -46,7 +46,7 @@ struct BwdArgs {
   float* bias_partial;                 // DW: [K / 256][N] partial column sums of g, or null
   int64_t M, N, K;
   int32_t tile;                        // K-tile width (multiple of 256)
-  int32_t ir_static;
+  int32_t ir_static;                   // 0: no range gradient; 1 + AHL_IR_GRAD_* otherwise
 };
 
 AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
@@ -280,10 +280,15 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
         BF16::unpack(xr[j], xv);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const bool up = xv[i] >= ir_t, lo = xv[i] <= -ir_t;
-          if (up) s_up += fminf(d[i], 0.0f);
-          if (lo) s_lo += fmaxf(d[i], 0.0f);
-          if (up || lo) cnt += 1.0f;
+          if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
+            const bool up = xv[i] >= ir_t, lo = xv[i] <= -ir_t;
+            if (up) s_up += fminf(d[i], 0.0f);
+            if (lo) s_lo += fmaxf(d[i], 0.0f);
+            if (up || lo) cnt += 1.0f;
+          } else {
+            if (xv[i] > ir_t) s_up += d[i];
+            if (xv[i] < -ir_t) s_lo += d[i];
+          }
           if (fabsf(xv[i]) > ir_t) d[i] = 0.0f;
         }
         d4 = BF16::pack(d);
@@ -326,12 +331,12 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
-                   const Tiling& tl, bool ir_static, hipStream_t s) {
+                   const Tiling& tl, int ir_static, hipStream_t s) {
   BwdArgs a;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
-  a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = ir_static ? 1 : 0;
+  a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = ir_static;
   const int64_t nb = cdiv(M, 256) * (K / 256);
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);

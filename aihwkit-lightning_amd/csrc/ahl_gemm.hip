@@ -361,6 +361,7 @@ struct DxArgs {
   int64_t M, N, K;
   Tiling tl;
   int32_t kb_big, kb_small;  // 128-wide column blocks per tile of size base+1 / base
+  int32_t ir_rule;           // AHL_IR_GRAD_*
 };
 
 // Decodes a column-block index into (tile, first column, end column).
@@ -466,10 +467,15 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
         float d = D::rd(acc[bi][bj][v]);
         if (IRMODE == AHL_IR_STATIC) {
           const float xv = D::load(a.x, m * a.ldx + k);
-          const bool up = xv >= ir_t, lo = xv <= -ir_t;
-          if (up) s_up += fminf(d, 0.0f);
-          if (lo) s_lo += fmaxf(d, 0.0f);
-          if (up || lo) cnt += 1.0f;
+          if (a.ir_rule == AHL_IR_GRAD_LEARNED) {
+            const bool up = xv >= ir_t, lo = xv <= -ir_t;
+            if (up) s_up += fminf(d, 0.0f);
+            if (lo) s_lo += fmaxf(d, 0.0f);
+            if (up || lo) cnt += 1.0f;
+          } else {
+            if (xv > ir_t) s_up += d;
+            if (xv < -ir_t) s_lo += d;
+          }
           if (fabsf(xv) > ir_t) d = 0.0f;
         }
         D::store(a.dx, m * a.lddx + k, d);
@@ -495,7 +501,8 @@ __global__ __launch_bounds__(64) void k_ir_grad_finalize(const float* __restrict
                                                          int64_t m_blocks, int32_t nkb,
                                                          int32_t kb_big, int32_t kb_small,
                                                          Tiling tl, int64_t M, const void* ir,
-                                                         void* ir_grad, float decay, float min_pct) {
+                                                         void* ir_grad, float decay, float min_pct,
+                                                         int32_t rule) {
   const int t = blockIdx.x, lane = threadIdx.x;
   const int32_t first = t < tl.extra ? t * kb_big : tl.extra * kb_big + (t - tl.extra) * kb_small;
   const int32_t count = t < tl.extra ? kb_big : kb_small;
@@ -511,6 +518,10 @@ __global__ __launch_bounds__(64) void k_ir_grad_finalize(const float* __restrict
     const float irv = D::load(ir, t);
     float gr = D::rd(0.0f + D::rd((float)s_up));
     gr = D::rd(gr - D::rd((float)s_lo));
+    if (rule == AHL_IR_GRAD_CLAMP) {  // the two bound gradients, each reduced in dtype, then added
+      D::store(ir_grad, t, gr);
+      return;
+    }
     gr = D::rd(gr * irv);
     if (decay > 0.0f) {
       const float numel = (float)((double)M * (double)tl.size(t));
@@ -523,7 +534,7 @@ __global__ __launch_bounds__(64) void k_ir_grad_finalize(const float* __restrict
 }
 
 // =============================================================================================
-// Weight gradient: dw[n, k] = sum_m gT[n, m] * xqT[k, m], gT masked by keepT bit t
+// Weight gradient: dw[n, k] = sum_m gT[n, m] * xqT[k, m], gT zeroed where tile t was clamped
 // =============================================================================================
 struct DwArgs {
   const void* gt;       // [N, M]
@@ -671,6 +682,7 @@ static bool cfg_ok(const AhlLinearCfg* c) {
   if (!c) return false;
   if (c->dtype != AHL_F32 && c->dtype != AHL_BF16) return false;
   if (c->ir_mode < 0 || c->ir_mode > 2) return false;
+  if (c->ir_grad_rule != AHL_IR_GRAD_LEARNED && c->ir_grad_rule != AHL_IR_GRAD_CLAMP) return false;
   return true;
 }
 
@@ -686,7 +698,7 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
-                   const Tiling& tl, bool ir_static, hipStream_t s);
+                   const Tiling& tl, int ir_static, hipStream_t s);
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    float* bias_partial, int64_t M, int64_t K, int64_t N, const Tiling& tl,
@@ -820,19 +832,21 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
     int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
-                            N, tl, is_static, s);
+                            N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, s);
     if (rc != AHL_OK) return rc;
     if (is_static) {
       const int32_t per_tile = tl.base / 256;
       hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
                          (const float*)partial, cdiv(M, 256), (int32_t)(K / 256), per_tile, per_tile,
-                         tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
+                         tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
+                         cfg->ir_grad_rule);
     }
     return check_launch("ahl_linear_bwd_dx(fast)");
   }
   DxArgs a;
   a.g = g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.wt = wt; a.x = x; a.ldx = ldx;
   a.ir = ir; a.dx = dx; a.lddx = lddx; a.partial = partial; a.M = M; a.N = N; a.K = K; a.tl = tl;
+  a.ir_rule = cfg->ir_grad_rule;
   kblocks(tl, &a.kb_big, &a.kb_small);
   const int64_t nkb = (int64_t)tl.extra * a.kb_big + (int64_t)(n_tiles - tl.extra) * a.kb_small;
   const int64_t mb = cdiv(M, kBM);
@@ -849,7 +863,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     AHL_DISPATCH_DTYPE(cfg->dtype, {
       hipLaunchKernelGGL((k_ir_grad_finalize<D>), dim3(n_tiles), dim3(64), 0, s, (const float*)partial, mb,
                          (int32_t)nkb, a.kb_big, a.kb_small, tl, M, ir, ir_grad, cfg->ir_decay,
-                         cfg->ir_input_min_percentage);
+                         cfg->ir_input_min_percentage, cfg->ir_grad_rule);
     });
   }
   return check_launch("ahl_linear_bwd_dx");

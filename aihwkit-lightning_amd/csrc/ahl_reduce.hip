@@ -140,6 +140,76 @@ __global__ __launch_bounds__(256) void k_running_absmax(const void* __restrict__
 }
 
 // ------------------------------------------------------------------------------------------
+// fast_mode input range (reference torch_utils/torch_linear.py:361-419).
+// Stage 1: signed min and max of every (row group, tile), one wave each.
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_sliced_minmax(const void* __restrict__ x, int64_t rows,
+                                                       int64_t ld, Tiling tl, int rpw,
+                                                       float* __restrict__ partial) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t grp = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
+  const int64_t r0 = grp * rpw;
+  if (r0 >= rows) return;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int i = 0; i < rpw; ++i) {
+    const int64_t r = r0 + i;
+    if (r >= rows) break;
+    const typename D::elem* row = (const typename D::elem*)x + r * ld;
+    wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
+      mn = fminf(mn, v);
+      mx = fmaxf(mx, v);
+    });
+  }
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  if (lane == 0) { partial[wave * 2] = mn; partial[wave * 2 + 1] = mx; }
+}
+
+// Stage 2, one block per tile: finish the min / max, then the update of x_min, x_max, the step
+// counter and the range, every operation rounded to the dtype of the buffers as torch does.
+template <class D>
+__global__ __launch_bounds__(256) void k_ir_fast_update(const float* __restrict__ partial,
+                                                        int64_t n_groups, int32_t n_tiles, void* ir,
+                                                        void* idx, void* x_min, void* x_max,
+                                                        float init_from_data, float momentum,
+                                                        float one_minus_momentum) {
+  __shared__ float sh[4][2];
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float mn = __builtin_inff(), mx = -__builtin_inff();
+  for (int64_t g = tid; g < n_groups; g += 256) {
+    mn = fminf(mn, partial[(g * n_tiles + t) * 2]);
+    mx = fmaxf(mx, partial[(g * n_tiles + t) * 2 + 1]);
+  }
+  mn = wave_min(mn);
+  mx = wave_max(mx);
+  if (lane == 0) { sh[wave][0] = mn; sh[wave][1] = mx; }
+  __syncthreads();
+  if (tid != 0) return;
+  const float act_min = fminf(fminf(sh[0][0], sh[1][0]), fminf(sh[2][0], sh[3][0]));
+  const float act_max = fmaxf(fmaxf(sh[0][1], sh[1][1]), fmaxf(sh[2][1], sh[3][1]));
+  const float step = D::load(idx, t);
+  if (!(step < init_from_data)) return;
+  float lo = D::load(x_min, t), hi = D::load(x_max, t);
+  const float thr = D::rd(1.1e-5f);  // the comparison constant takes the dtype of the buffer
+  if (lo > -thr && hi < thr) {       // still at the initial +-1e-5: start from the first batch
+    lo = D::rd(lo + act_min);
+    hi = D::rd(hi + act_max);
+  } else if (momentum == -1.0f) {    // plain running extrema
+    lo = fminf(lo, act_min);
+    hi = fmaxf(hi, act_max);
+  } else {
+    lo = D::rd(D::rd(lo * momentum) + D::rd(act_min * one_minus_momentum));
+    hi = D::rd(D::rd(hi * momentum) + D::rd(act_max * one_minus_momentum));
+  }
+  D::store(x_min, t, lo);
+  D::store(x_max, t, hi);
+  D::store(idx, t, D::rd(step + 1.0f));
+  D::store(ir, t, fmaxf(fabsf(lo), fabsf(hi)));
+}
+
+// ------------------------------------------------------------------------------------------
 // Weight clipping. Per channel: one wave per row computes the unbiased std of the row in
 // double, then re-reads the row (L2 resident) and stores only the 16-byte vectors in which
 // at least one element changed.
@@ -299,7 +369,7 @@ using namespace ahl;
 // ============================================================================================
 extern "C" {
 
-int ahl_abi_version(void) { return 4; }
+int ahl_abi_version(void) { return 5; }
 const char* ahl_last_hip_error(void) { return ahl::g_err; }
 
 int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
@@ -371,6 +441,33 @@ int ahl_running_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols,
     else hipLaunchKernelGGL((k_running_absmax<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, cache);
   });
   return check_launch("ahl_running_absmax");
+}
+
+int64_t ahl_ir_fast_update_ws_bytes(int64_t rows, int32_t n_tiles) {
+  if (rows <= 0 || n_tiles <= 0) return 0;
+  return cdiv(rows, rows_per_wave(rows)) * (int64_t)n_tiles * 2 * (int64_t)sizeof(float);
+}
+
+int ahl_ir_fast_update(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                       const int32_t* tile_ends_host, int32_t n_tiles, void* ir, void* idx,
+                       void* x_min, void* x_max, float init_from_data, double momentum, void* ws,
+                       void* stream) {
+  if (!x || !ir || !idx || !x_min || !x_max || !ws || rows <= 0 || cols <= 0 || ld < cols)
+    return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  const int rpw = rows_per_wave(rows);
+  const int64_t ng = cdiv(rows, rpw), nb = cdiv(ng * n_tiles, 4);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(x) && (ld % D::EPV == 0);
+    if (vec) hipLaunchKernelGGL((k_sliced_minmax<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (float*)ws);
+    else hipLaunchKernelGGL((k_sliced_minmax<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (float*)ws);
+    hipLaunchKernelGGL((k_ir_fast_update<D>), dim3(n_tiles), dim3(256), 0, s, (const float*)ws, ng, n_tiles,
+                       ir, idx, x_min, x_max, init_from_data, (float)momentum, (float)(1.0 - momentum));
+  });
+  return check_launch("ahl_ir_fast_update");
 }
 
 int64_t ahl_clip_weights_ws_bytes(int64_t rows) {

@@ -47,6 +47,15 @@ extern "C" {
 #define AHL_NOISE_ADD_NORMAL 1              /* std = std_dev * max|W_tile|          */
 #define AHL_NOISE_ADD_NORMAL_PER_CHANNEL 2  /* std = std_dev * max|W_tile[n, :]|    */
 
+/* Backward of the clamp to a static input range (AhlLinearCfg.ir_grad_rule):
+ * AHL_IR_GRAD_LEARNED: StraightThroughClamp + InputRangeForward (torch_utils/torch_linear.py:29-108)
+ *   ir_grad[t] = (sum_{x >= ir} min(d, 0) - sum_{x <= -ir} max(d, 0)) * ir[t] + decay switch
+ * AHL_IR_GRAD_CLAMP: autograd of torch.clamp(x, -ir, ir) with tensor bounds, the fast_mode path
+ *   (torch_utils/torch_linear.py:361-422): ir_grad[t] = sum_{x > ir} d - sum_{x < -ir} d
+ * Both zero dx where |x| > ir[t].                                                         */
+#define AHL_IR_GRAD_LEARNED 0
+#define AHL_IR_GRAD_CLAMP 1
+
 #define AHL_QUANT_NONE 0
 #define AHL_QUANT_DISCRETIZE 1              /* scale from max|W_tile|               */
 #define AHL_QUANT_DISCRETIZE_PER_CHANNEL 2  /* scale from max|W_tile[n, :]|         */
@@ -69,6 +78,7 @@ typedef struct AhlLinearCfg {
   int32_t skip_rounding;         /* the reference's test switch _AIHWKIT_NO_ROUNDING            */
   float ir_decay;                /* pre_post.input_range.decay                                  */
   float ir_input_min_percentage; /* pre_post.input_range.input_min_percentage                   */
+  int32_t ir_grad_rule;          /* AHL_IR_GRAD_*: which backward the static range clamp has     */
   uint64_t seed;                 /* Philox key for this call                                    */
   uint64_t offset;               /* Philox counter offset for this call                         */
 } AhlLinearCfg;
@@ -126,6 +136,19 @@ int ahl_ir_init_update(void* ir, void* idx, const float* std, int32_t dtype, int
  *   (initialise to -inf). Replaces inference/calibration/calibration.py:110-124.         */
 int ahl_running_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
                        const int32_t* tile_ends_host, int32_t n_tiles, float* cache, void* stream);
+
+/* fast_mode input range (TorchLinear.apply_input_range_fast, torch_utils/torch_linear.py:361-419),
+ * the update only: for every tile with idx[t] < init_from_data, the signed min / max of
+ * x[:, tile t] moves x_min[t] / x_max[t] (first batch: added to the initial +-1e-5; momentum -1:
+ * running extrema; else exponential average), idx[t] += 1, ir[t] = max(|x_min[t]|, |x_max[t]|).
+ * ir, idx, x_min, x_max: dtype [T], updated in place on the device, no host sync. The clamp
+ * itself is the AHL_IR_STATIC forward; its backward is AHL_IR_GRAD_CLAMP.
+ * ws needs ahl_ir_fast_update_ws_bytes(rows, n_tiles) bytes.                               */
+int ahl_ir_fast_update(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                       const int32_t* tile_ends_host, int32_t n_tiles, void* ir, void* idx,
+                       void* x_min, void* x_max, float init_from_data, double momentum, void* ws,
+                       void* stream);
+int64_t ahl_ir_fast_update_ws_bytes(int64_t rows, int32_t n_tiles);
 
 /* Weight clipping after an optimizer step, in place on w[rows, cols]:
  *   bound = sigma * std_unbiased(w[r, :]) (AHL_CLIP_PER_CHANNEL) or sigma * std_unbiased(w);

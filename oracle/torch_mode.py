@@ -28,7 +28,7 @@ DISCRETIZE = "discretize"
 DISCRETIZE_PER_CHANNEL = "discretize_per_channel"
 ADD_NORMAL = "add_normal"
 ADD_NORMAL_PER_CHANNEL = "add_normal_per_channel"
-IR_NONE, IR_STATIC, IR_DYNAMIC = "none", "static", "dynamic"
+IR_NONE, IR_STATIC, IR_DYNAMIC, IR_FAST = "none", "static", "dynamic", "fast"
 
 
 @dataclass
@@ -154,6 +154,28 @@ def ir_init_update(x_t: Tensor, ir: Tensor, idx: Tensor, t: int, init_from_data:
         ir[t] = ir[t].abs()
 
 
+def ir_fast_update(x_t: Tensor, ir: Tensor, idx: Tensor, x_min: Tensor, x_max: Tensor, t: int,
+                   init_from_data: float, momentum: float) -> None:
+    """One fast_mode range update of tile t from the data x_t, in place
+    (torch_utils/torch_linear.py:387-419): the running min / max start from the first batch, then
+    follow with momentum (or as plain running extrema for momentum -1); the range is the larger
+    magnitude of the two. All arithmetic is in the dtype of the buffers."""
+    if not idx[t] < init_from_data:
+        return
+    act_min, act_max = x_t.min(), x_t.max()
+    if x_min[t] > -1.1e-5 and x_max[t] < 1.1e-5:
+        x_min[t] = x_min[t] + act_min
+        x_max[t] = x_max[t] + act_max
+    elif momentum == -1:
+        x_min[t] = min(x_min[t], act_min)
+        x_max[t] = max(x_max[t], act_max)
+    else:
+        x_min[t] = x_min[t] * momentum + act_min * (1 - momentum)
+        x_max[t] = x_max[t] * momentum + act_max * (1 - momentum)
+    idx[t] += 1
+    ir[t] = max(x_min[t].abs(), x_max[t].abs())
+
+
 def linear_forward(
     x: Tensor,
     weights: Tensor,
@@ -189,6 +211,11 @@ def linear_forward(
             ir_t = input_range[t]
             rec["up"] = x_t >= ir_t
             rec["lo"] = x_t <= -ir_t
+            xc = torch.clamp(x_t, min=-ir_t, max=ir_t)
+        elif cfg.ir_mode == IR_FAST:
+            # plain torch.clamp with tensor bounds (torch_linear.py:421); its autograd rule is
+            # restated in linear_backward
+            ir_t = input_range[t]
             xc = torch.clamp(x_t, min=-ir_t, max=ir_t)
         elif cfg.ir_mode == IR_DYNAMIC:
             ir_t = x_t.abs().max(dim=-1, keepdim=True)[0]
@@ -240,7 +267,7 @@ def linear_backward(grad_out: Tensor, saved: Dict) -> Tuple[Tensor, Tensor, Tens
     n_tiles = len(saved["in_sizes"])
     dx = torch.zeros_like(x)
     dw_parts = []
-    ir_grad = torch.zeros(n_tiles, dtype=dtype) if cfg.ir_mode == IR_STATIC else None
+    ir_grad = torch.zeros(n_tiles, dtype=dtype) if cfg.ir_mode in (IR_STATIC, IR_FAST) else None
     for t, (lo, hi) in enumerate(tile_bounds(saved["in_sizes"])):
         rec = saved["tiles"][t]
         gy = grad_out if rec["keep"] is None else grad_out * rec["keep"]
@@ -259,6 +286,16 @@ def linear_backward(grad_out: Tensor, saved: Dict) -> Tuple[Tensor, Tensor, Tens
             x_t = x[:, lo:hi]
             d = d.clone()
             d[(up | low) & (x_t.abs() != ir_t)] = 0.0
+        elif cfg.ir_mode == IR_FAST:
+            # autograd of clamp(x, min=-ir, max=ir) with tensor bounds: the gradient goes to x
+            # inside [-ir, ir] (bounds included), to `max` where x > ir and to `min` where
+            # x < -ir; each is reduced to a scalar in the tensor dtype, and min = -ir
+            ir_t, x_t = rec["ir"], x[:, lo:hi]
+            zero = torch.zeros_like(d)
+            g_max = torch.where(x_t > ir_t, d, zero).sum()
+            g_min = torch.where(x_t < -ir_t, d, zero).sum()
+            ir_grad[t] = g_max + (-g_min)
+            d = torch.where((x_t >= -ir_t) & (x_t <= ir_t), d, zero)
         dx[:, lo:hi] = d
     dw = torch.cat(dw_parts, dim=1)
     dbias = grad_out.sum(dim=0)

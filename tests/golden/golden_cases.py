@@ -13,7 +13,7 @@ DEFAULTS = dict(
     clip="none", clip_sigma=-1.0, weight_quant="none", weight_noise="none", modifier_res=0.0,
     modifier_std=0.0, ir_mode="none", ir_init=3.0, init_from_data=0, init_std_alpha=3.0,
     ir_decay=0.001, ir_min_pct=0.95, ir_values=None, training=True, kind="fwd_bwd",
-    seed=0, noise_seed=1234, x_scale=1.0, w_scale=0.02, steps=0,
+    seed=0, noise_seed=1234, x_scale=1.0, w_scale=0.02, steps=0, act_range_momentum=0.95,
 )
 
 
@@ -86,6 +86,20 @@ CASES = [
          ir_mode="static", init_from_data=3, inp_res=254, seed=12),
     case("bf16_ir_init", dtype="bf16", kind="ir_init", steps=4, M=16, K=24, N=8, max_input_size=12,
          ir_mode="static", init_from_data=3, inp_res=254, seed=12),
+    # fast_mode input range: plain clamp to a range that follows the running min / max of the
+    # data; gradients are those of torch.clamp with tensor bounds
+    case("f32_fast_clip", M=12, K=26, N=16, max_input_size=9, ir_mode="fast",
+         ir_values=[0.8, 2.5, 1.5], inp_res=254, out_res=254, out_bound=1.5, clip="channel",
+         clip_sigma=2.5, w_scale=0.3, seed=15),
+    case("bf16_fast_clip", dtype="bf16", M=12, K=26, N=16, max_input_size=9, ir_mode="fast",
+         ir_values=[0.8, 2.5, 1.5], inp_res=254, out_res=254, out_bound=1.5, clip="channel",
+         clip_sigma=2.5, w_scale=0.3, seed=15),
+    case("f32_fast_init", kind="ir_fast_init", steps=5, M=16, K=24, N=8, max_input_size=12,
+         ir_mode="fast", init_from_data=4, inp_res=254, seed=16),
+    case("bf16_fast_init", dtype="bf16", kind="ir_fast_init", steps=5, M=16, K=24, N=8,
+         max_input_size=12, ir_mode="fast", init_from_data=4, inp_res=254, seed=16),
+    case("f32_fast_init_minmax", kind="ir_fast_init", steps=4, M=16, K=24, N=8, max_input_size=12,
+         ir_mode="fast", init_from_data=3, act_range_momentum=-1, inp_res=254, seed=17),
     # optimizer-step clipping
     case("f32_clip_layer", kind="clip", M=4, K=40, N=24, clip="layer", clip_sigma=2.0, w_scale=1.0,
          seed=13),

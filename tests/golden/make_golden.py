@@ -64,6 +64,8 @@ def ref_config(case) -> TorchInferenceRPUConfig:
     ir = cfg.pre_post.input_range
     ir.enable = case["ir_mode"] != "none"
     ir.dynamic = case["ir_mode"] == "dynamic"
+    ir.fast_mode = case["ir_mode"] == "fast"
+    ir.act_range_momentum = case["act_range_momentum"]
     ir.init_value = case["ir_init"]
     ir.init_from_data = case["init_from_data"]
     ir.init_std_alpha = case["init_std_alpha"]
@@ -107,6 +109,17 @@ def run_case(case, store):
             store[f"{name}/out{step}"] = f32(out)
             store[f"{name}/ir{step}"] = f32(layer.input_range.data.clone())
             store[f"{name}/idx{step}"] = f32(layer.input_range_update_idx.clone())
+    elif kind == "ir_fast_init":
+        for step in range(case["steps"]):
+            torch.manual_seed(case["noise_seed"] + step)
+            xs = torch.randn_like(x) * (1.0 + step) + 0.25 * step
+            out = layer(xs)
+            store[f"{name}/x{step}"] = f32(xs)
+            store[f"{name}/out{step}"] = f32(out)
+            store[f"{name}/ir{step}"] = f32(layer.input_range.data.clone())
+            store[f"{name}/idx{step}"] = f32(layer.input_range_update_idx.clone())
+            store[f"{name}/xmin{step}"] = f32(layer.x_min.clone())
+            store[f"{name}/xmax{step}"] = f32(layer.x_max.clone())
     elif kind == "clip":
         optim = AnalogOptimizer(torch.optim.SGD, layer.analog_layers, layer.parameters(), lr=0.0)
         layer(x).sum().backward()

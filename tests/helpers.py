@@ -36,8 +36,8 @@ def oracle_cfg(c) -> om.OracleCfg:
 
 
 def case_input_range(c, n_tiles):
-    """Initial per-tile input range of a case (None unless the range is static)."""
-    if c["ir_mode"] != "static":
+    """Initial per-tile input range of a case (None unless the range is a stored parameter)."""
+    if c["ir_mode"] not in ("static", "fast"):
         return None
     dtype = DTYPES[c["dtype"]]
     if c["ir_values"] is not None:

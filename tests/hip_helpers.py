@@ -47,6 +47,8 @@ def rpu_config(c) -> TorchInferenceRPUConfig:
     ir = cfg.pre_post.input_range
     ir.enable = c["ir_mode"] != "none"
     ir.dynamic = c["ir_mode"] == "dynamic"
+    ir.fast_mode = c["ir_mode"] == "fast"
+    ir.act_range_momentum = c["act_range_momentum"]
     ir.init_value = c["ir_init"]
     ir.init_from_data = c["init_from_data"]
     ir.init_std_alpha = c["init_std_alpha"]

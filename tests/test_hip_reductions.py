@@ -75,6 +75,28 @@ def test_input_range_initialisation_matches_reference(name):
     assert layer._ir_init_active is False or layer._ir_init_calls >= c["init_from_data"]
 
 
+@pytest.mark.parametrize("name", ["f32_fast_init", "bf16_fast_init", "f32_fast_init_minmax"])
+def test_fast_mode_range_sequence_matches_reference(name):
+    """fast_mode training forwards: running min / max, the step counter, the range and the outputs
+    after every step against the reference's recorded sequence. The state is bit-exact: it is a
+    few dtype-rounded operations on exact minima and maxima."""
+    from hip_helpers import make_layer
+
+    c = CASES_BY_NAME[name]
+    dtype = DTYPES[c["dtype"]]
+    layer = make_layer(c)
+    for step in range(c["steps"]):
+        xs = golden_tensor(f"{name}/x{step}", dtype).cuda()
+        out = layer(xs)
+        for key, buf in (("ir", layer.input_range.data), ("idx", layer.input_range_update_idx),
+                         ("xmin", layer.x_min), ("xmax", layer.x_max)):
+            assert torch.equal(buf.float().cpu(), golden_tensor(f"{name}/{key}{step}")), (key, step)
+        ref = golden_tensor(f"{name}/out{step}")
+        err = (out.float().cpu() - ref).abs().max() / ref.abs().mean()
+        assert err < (1e-4 if c["dtype"] == "f32" else 6e-2), (step, float(err))
+    assert layer._ir_init_active is False or layer._ir_init_calls >= c["init_from_data"]
+
+
 @pytest.mark.parametrize("name", ["f32_clip_layer", "f32_clip_channel", "bf16_clip_channel"])
 def test_clip_weights_via_optimizer_matches_reference(name):
     from hip_helpers import make_layer

@@ -32,7 +32,7 @@ def test_forward_backward_matches_reference(case):
             continue
         assert res[key] is not None, f"oracle produced no {key}"
         _exact_or_close(res[key], golden_tensor(gkey), dtype, gkey)
-    if case["ir_mode"] == "static":
+    if case["ir_mode"] in ("static", "fast"):
         assert f"{name}/dir" in golden(), "reference wrote an input-range gradient"
 
 
@@ -54,6 +54,29 @@ def test_input_range_initialisation_sequence(name):
         _exact_or_close(idx, golden_tensor(f"{name}/idx{step}"), dtype, f"idx after step {step}")
         _exact_or_close(out, golden_tensor(f"{name}/out{step}"), dtype, f"out step {step}")
     assert float(idx.max()) == case["init_from_data"], "initialisation must stop at init_from_data"
+
+
+@pytest.mark.parametrize("name", ["f32_fast_init", "bf16_fast_init", "f32_fast_init_minmax"])
+def test_fast_mode_range_sequence(name):
+    case = [c for c in CASES if c["name"] == name][0]
+    dtype = DTYPES[case["dtype"]]
+    _, w, b, _ = make_inputs(case)
+    cfg = oracle_cfg(case)
+    in_sizes = om.split_sizes(case["K"], case["max_input_size"])
+    n_tiles = len(in_sizes)
+    ir = case_input_range(case, n_tiles)
+    idx = torch.zeros(n_tiles, dtype=dtype)
+    x_min = torch.full((n_tiles,), -1e-5, dtype=dtype)  # nn/modules/base.py:149-154
+    x_max = torch.full((n_tiles,), 1e-5, dtype=dtype)
+    for step in range(case["steps"]):
+        xs = golden_tensor(f"{name}/x{step}", dtype)
+        for t, (lo, hi) in enumerate(om.tile_bounds(in_sizes)):
+            om.ir_fast_update(xs[:, lo:hi], ir, idx, x_min, x_max, t, case["init_from_data"],
+                              case["act_range_momentum"])
+        out, _ = om.linear_forward(xs, w, b, cfg, ir, True)
+        for key, val in (("ir", ir), ("idx", idx), ("xmin", x_min), ("xmax", x_max), ("out", out)):
+            _exact_or_close(val, golden_tensor(f"{name}/{key}{step}"), dtype, f"{key} after step {step}")
+    assert float(idx.max()) == case["init_from_data"], "the updates must stop at init_from_data"
 
 
 @pytest.mark.parametrize("name", ["f32_clip_layer", "f32_clip_channel", "bf16_clip_channel"])
