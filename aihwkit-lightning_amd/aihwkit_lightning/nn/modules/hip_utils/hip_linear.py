@@ -39,9 +39,12 @@ def draw_seed() -> int:
 
 
 def check_supported(rpu_config: TorchInferenceRPUConfig) -> None:
-    """Reject configuration branches that the HIP backend does not implement."""
+    """Reject configuration combinations the reference rejects too."""
     if rpu_config.clip.type == WeightClipType.LEARNABLE_PER_CHANNEL:
-        raise ConfigError("WeightClipType.LEARNABLE_PER_CHANNEL is not implemented by the HIP backend")
+        # torch_utils/torch_linear.py:234-238
+        assert rpu_config.modifier.quantization_type in (
+            WeightQuantizationType.NONE, WeightQuantizationType.DISCRETIZE_PER_CHANNEL,
+        ), "You can't learn weight ranges per column but quantize per tensor"
 
 
 class HipLinear(Function):
@@ -63,6 +66,7 @@ class HipLinear(Function):
         init_active: bool,
         x_min: Optional[Tensor] = None,
         x_max: Optional[Tensor] = None,
+        learnable_weight_clip: Optional[Tensor] = None,
     ) -> Tensor:
         if not inp.is_cuda:
             raise HipBackendError(
@@ -112,15 +116,31 @@ class HipLinear(Function):
             )
         w_noise = training and modifier.noise_type != WeightNoiseInjectionType.NONE
         w_quant = modifier.quantization_type != WeightQuantizationType.NONE
-        need_wmax = bound_on or noise_on or w_noise or w_quant
+        learned_clip = rpu_config.clip.type == WeightClipType.LEARNABLE_PER_CHANNEL
+        if learned_clip:
+            assert learnable_weight_clip is not None, "learnable_weight_clip should not be None"
+        need_wmax = bound_on or noise_on or w_noise or w_quant or learned_clip
+        # the clip's gradient comes out of the weight gradient
+        clip_needs_grad = learned_clip and ctx.needs_input_grad[11]
         ir_needs_grad = ir_mode == L.AHL_IR_STATIC and input_range.requires_grad
         need_dx = ctx.needs_input_grad[0] or (ctx.needs_input_grad[3] and ir_needs_grad)
-        need_dw = ctx.needs_input_grad[1]
+        need_dw = ctx.needs_input_grad[1] or clip_needs_grad
 
         seed = draw_seed() if (noise_on or w_noise) else 0
-        wmax = tile_max = None
+        wmax = tile_max = tile_min = None
         w_eff = weights_c
-        if m_rows > 0 and need_wmax:
+        clip_quant = L.AHL_QUANT_DISCRETIZE_PER_CHANNEL if w_quant else L.AHL_QUANT_CLIP_LEARNED
+        if m_rows > 0 and learned_clip:
+            # the clipped (+ quantised, + noisy) weights; the clip is the tile's "wmax" from here on
+            wmax = learnable_weight_clip.detach()
+            if not wmax.is_contiguous():
+                wmax = wmax.contiguous()
+            tile_max, tile_min, w_eff = OPS.weight_prep_clip(
+                weights_c, wmax, in_sizes, clip_quant,
+                NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE,
+                float(modifier.res) if w_quant else 1.0, float(modifier.std_dev), seed, 1,
+            )
+        elif m_rows > 0 and need_wmax:
             res = float(modifier.res) if w_quant else 1.0
             wmax, tile_max, _, eff = OPS.weight_prep(
                 weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
@@ -185,23 +205,27 @@ class HipLinear(Function):
         ctx.in_sizes, ctx.icfg, ctx.fcfg = in_sizes, icfg, fcfg
         ctx.inp_shape, ctx.ir_mode, ctx.has_bias = inp.shape, ir_mode, bias is not None
         ctx.need_dx, ctx.need_dw, ctx.ir_needs_grad = need_dx, need_dw, ir_needs_grad
+        ctx.learned_clip = learned_clip and need_dw
+        ctx.clip_quant, ctx.clip_res = clip_quant, float(modifier.res) if w_quant else 1.0
         need_x = (need_dx and ir_mode == L.AHL_IR_STATIC) or (need_dw and xq is None)
         ctx.save_for_backward(
             x2 if need_x else None, xq if need_dw else None,
             (w_eff if w_eff is not weights else weights.detach()) if need_dx else None,
             keep if want_keep else None, flag if want_keep else None,
             ir_dev.clone() if ir_mode == L.AHL_IR_STATIC else ir_dev,
+            weights_c.detach() if ctx.learned_clip else None,
+            wmax.clone() if ctx.learned_clip else None, tile_min if ctx.learned_clip else None,
         )
         return y.view(out_shape)
 
     @staticmethod
     def backward(ctx, grad_out: Tensor):
-        x2, xq, w_eff, keep, flag, ir_dev = ctx.saved_tensors
+        x2, xq, w_eff, keep, flag, ir_dev, w_plain, clip, clip_tile_min = ctx.saved_tensors
         n_out = grad_out.size(-1)
         g2 = grad_out.reshape(-1, n_out)
         if g2.stride(-1) != 1 or (g2.size(0) > 1 and g2.stride(0) != n_out):
             g2 = g2.contiguous()
-        grad_inp = grad_w = grad_b = grad_ir = None
+        grad_inp = grad_w = grad_b = grad_ir = grad_clip = None
         if ctx.need_dx:
             dx, ir_grad = OPS.linear_bwd_dx(
                 g2, keep, flag, w_eff, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
@@ -220,6 +244,14 @@ class HipLinear(Function):
             )
             if want_bias:
                 grad_b = dbias
+            if ctx.learned_clip:
+                # gradient w.r.t. the clipped weights -> weights (in place) and clip (LSQ rule)
+                grad_clip = OPS.learned_clip_bwd(
+                    grad_w, w_plain, clip, clip_tile_min, ctx.in_sizes, ctx.clip_quant, ctx.clip_res
+                )
         elif want_bias:
             grad_b = OPS.col_sum(g2)
-        return grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None, None, None
+        if not ctx.needs_input_grad[1]:
+            grad_w = None
+        return (grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None, None, None,
+                grad_clip)

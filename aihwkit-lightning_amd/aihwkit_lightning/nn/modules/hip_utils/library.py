@@ -19,6 +19,7 @@ AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
 AHL_NOISE_NONE, AHL_NOISE_ADD_NORMAL, AHL_NOISE_ADD_NORMAL_PER_CHANNEL = 0, 1, 2
 AHL_QUANT_NONE, AHL_QUANT_DISCRETIZE, AHL_QUANT_DISCRETIZE_PER_CHANNEL = 0, 1, 2
+AHL_QUANT_CLIP_LEARNED = 3
 AHL_CLIP_LAYER, AHL_CLIP_PER_CHANNEL = 0, 1
 AHL_IR_GRAD_LEARNED, AHL_IR_GRAD_CLAMP = 0, 1
 
@@ -62,6 +63,7 @@ class AhlModifierCfg(Structure):
         ("noise_type", c_int32),
         ("res", c_float),
         ("std_dev", c_float),
+        ("wmax_given", c_int32),
         ("seed", c_uint64),
         ("offset", c_uint64),
     ]
@@ -88,6 +90,11 @@ SIGNATURES = {
     ),
     "ahl_running_absmax": (
         c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, _I32P, c_int32, c_void_p, c_void_p]
+    ),
+    "ahl_learned_clip_bwd": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int64, _I32P,
+         c_int32, POINTER(AhlModifierCfg), c_void_p],
     ),
     "ahl_ir_fast_update": (
         c_int32,

@@ -81,6 +81,14 @@ LIB.define(
 )
 LIB.define("quantize_weights(Tensor(a!) w, int[] in_sizes, int quant_type, float res) -> ()")
 LIB.define(
+    "weight_prep_clip(Tensor w, Tensor clip, int[] in_sizes, int quant_type, int noise_type, "
+    "float res, float std_dev, int seed, int offset) -> (Tensor, Tensor, Tensor)"
+)
+LIB.define(
+    "learned_clip_bwd(Tensor(a!) dw, Tensor w, Tensor clip, Tensor tile_min, int[] in_sizes, "
+    "int quant_type, float res) -> Tensor"
+)
+LIB.define(
     "dac(Tensor x, Tensor? ir, int[] in_sizes, int[] icfg, float[] fcfg) -> (Tensor, Tensor)"
 )
 LIB.define(
@@ -250,6 +258,54 @@ def weight_prep(
     return wmax, tile_max, tile_min, w_eff
 
 
+def weight_prep_clip(
+    w: Tensor, clip: Tensor, in_sizes: List[int], quant_type: int, noise_type: int, res: float,
+    std_dev: float, seed: int, offset: int,
+) -> Tuple[Tensor, Tensor, Tensor]:
+    """Weights under a learnable per-channel clip ``clip [T, N]`` (which also takes the place of
+    the per-tile abs-max): tile max/min of the clip and the clipped (+ quantised, + noisy) copy."""
+    lib = L.load()
+    if w.dim() != 2 or w.stride(1) != 1:
+        raise HipBackendError("weight must be a row-major 2-D tensor")
+    n_out, n_in = w.shape
+    n_tiles = len(in_sizes)
+    if clip.shape != (n_tiles, n_out) or not clip.is_contiguous() or clip.dtype != w.dtype:
+        raise HipBackendError("learnable_weight_clip must be a contiguous [n_tiles, out] tensor")
+    tile_max = torch.empty((n_tiles,), dtype=torch.float32, device=w.device)
+    tile_min = torch.empty((n_tiles,), dtype=torch.float32, device=w.device)
+    w_eff = torch.empty((n_out, n_in), dtype=w.dtype, device=w.device)
+    cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset)
+    cfg.wmax_given = 1
+    L.check(
+        lib.ahl_weight_prep(
+            _ptr(w), n_out, n_in, _ld(w), L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(clip),
+            _ptr(tile_max), _ptr(tile_min), _ptr(w_eff), n_in, _stream(),
+        ),
+        "ahl_weight_prep",
+    )
+    return tile_max, tile_min, w_eff
+
+
+def learned_clip_bwd(dw: Tensor, w: Tensor, clip: Tensor, tile_min: Tensor, in_sizes: List[int],
+                     quant_type: int, res: float) -> Tensor:
+    """LSQ backward of the learnable clip: ``dw`` (gradient w.r.t. the clipped weights) becomes
+    the gradient w.r.t. the weights in place; returns the gradient of the clip ``[T, N]``."""
+    lib = L.load()
+    if dw.stride(1) != 1 or w.stride(1) != 1:
+        raise HipBackendError("weight and its gradient must be row-major")
+    n_out, n_in = w.shape
+    dclip = torch.empty_like(clip)
+    cfg = _modifier_cfg(w.dtype, quant_type, L.AHL_NOISE_NONE, res, 0.0, 0, 0)
+    L.check(
+        lib.ahl_learned_clip_bwd(
+            _ptr(dw), _ld(dw), _ptr(w), _ld(w), _ptr(clip), _ptr(tile_min), _ptr(dclip), n_out, n_in,
+            L.tile_ends_array(in_sizes), len(in_sizes), byref(cfg), _stream(),
+        ),
+        "ahl_learned_clip_bwd",
+    )
+    return dclip
+
+
 def quantize_weights(w: Tensor, in_sizes: List[int], quant_type: int, res: float) -> None:
     """In-place per-tile weight quantisation with scales from each slice's own abs-max."""
     lib = L.load()
@@ -394,6 +450,7 @@ for _name, _fn in [
     ("running_absmax", running_absmax), ("ir_fast_update", ir_fast_update),
     ("clip_weights", clip_weights), ("col_sum", col_sum),
     ("weight_prep", weight_prep), ("quantize_weights", quantize_weights),
+    ("weight_prep_clip", weight_prep_clip), ("learned_clip_bwd", learned_clip_bwd),
     ("dac", dac), ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
 ]:
     LIB.impl(_name, _fn, "CUDA")

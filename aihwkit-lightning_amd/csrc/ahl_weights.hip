@@ -26,11 +26,23 @@ AHL_DEV WQuant make_wquant(float wm, float n_states, bool all_gt1) {
 }
 
 template <class D>
-AHL_DEV float wquant_apply(float w, const WQuant& q, float maxq) {
+AHL_DEV float wquant_apply(float w, const WQuant& q, float maxq, bool round = true) {
   float v = D::rd(D::div(w, q.rc, q.rcp));
   v = fminf(fmaxf(v, -maxq), maxq);
-  v = rintf(v);
+  if (round) v = rintf(v);
   return D::rd(v * q.step);
+}
+
+// Step of the learnable clip without a quantiser (UniformQuantize with res = clip, bound 0.5):
+// alpha = 1, so the step is the clip itself, or its inverse if every clip of the tile is > 1.
+template <class D>
+AHL_DEV WQuant make_wclip(float clip, bool all_gt1) {
+  WQuant q;
+  q.step = all_gt1 ? D::rd(__fdiv_rn(1.0f, clip)) : clip;
+  if (q.step == 0.0f) q.step = 1.0f;
+  q.rc = fmaxf(q.step, kTinyF32);
+  q.rcp = __fdiv_rn(1.0f, q.rc);
+  return q;
 }
 
 struct ModArgs {
@@ -85,6 +97,8 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t block
       } else if (a.quant_type == AHL_QUANT_DISCRETIZE) {
         const bool all_gt1 = D::rd(__fdiv_rn(tmax, a.n_states)) > 1.0f;
         c.q = make_wquant<D>(tmax, a.n_states, all_gt1);
+      } else if (a.quant_type == AHL_QUANT_CLIP_LEARNED) {
+        c.q = make_wclip<D>(wm, a.tile_min[t] > 1.0f);
       }
       c.nstd = D::rd(a.std_dev * (a.noise_type == AHL_NOISE_ADD_NORMAL_PER_CHANNEL ? wm : tmax));
       return c;
@@ -97,7 +111,8 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t block
     for (int e = 0; e < 8; ++e) {
       const TileConst& ce = kb + e >= t1_start ? c1 : c;
       float x = v[e];
-      if (a.quant_type != AHL_QUANT_NONE) x = wquant_apply<D>(x, ce.q, a.maxq);
+      if (a.quant_type != AHL_QUANT_NONE)
+        x = wquant_apply<D>(x, ce.q, a.maxq, a.quant_type != AHL_QUANT_CLIP_LEARNED);
       if (a.noise_type != AHL_NOISE_NONE) x = D::rd(x + D::rd(ce.nstd * D::rd(xi[e])));
       v[e] = x;
     }
@@ -115,6 +130,56 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t block
   }
 }
 
+// LSQ backward of the learnable clip: one wave per (channel, tile).
+struct ClipBwdArgs {
+  void* dw; int64_t lddw;
+  const void* w; int64_t ldw;
+  const void* clip;        // dtype [T, N]
+  const float* tile_min;   // [T]
+  void* dclip;             // dtype [T, N]
+  int64_t N;
+  Tiling tl;
+  int32_t quant_type;
+  float n_states, maxq, maxq_exact;
+};
+
+template <class D>
+__global__ __launch_bounds__(256) void k_learned_clip_bwd(ClipBwdArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t n = wave / a.tl.n_tiles;
+  const int32_t t = (int32_t)(wave % a.tl.n_tiles);
+  if (n >= a.N) return;
+  const bool quant = a.quant_type == AHL_QUANT_DISCRETIZE_PER_CHANNEL;
+  const float clip = D::load(a.clip, (int64_t)t * a.N + n);
+  WQuant q;
+  if (quant) q = make_wquant<D>(clip, a.n_states, D::rd(__fdiv_rn(a.tile_min[t], a.n_states)) > 1.0f);
+  else q = make_wclip<D>(clip, a.tile_min[t] > 1.0f);
+  // grad_scale in double like the Python expression, then the fp32 scalar of the tensor op
+  const double numel = (double)a.N * (double)a.tl.size(t);
+  const float gs = (float)(quant ? 2.0 * sqrt((double)a.maxq_exact / numel) : 1.0 / sqrt(numel));
+  float acc = 0.0f;
+  for (int32_t k = a.tl.start(t) + lane; k < a.tl.start(t + 1); k += 64) {
+    const float w = D::load(a.w, n * a.ldw + k);
+    const float g = D::load(a.dw, n * a.lddw + k);
+    const float qw = D::rd(D::div(w, q.rc, q.rcp));
+    const bool small = qw < -a.maxq, big = qw > a.maxq;
+    // (indicator terms) * grad * grad_scale, evaluated in fp32 as torch promotes them
+    float term;
+    if (small) term = -a.maxq_exact;
+    else if (big) term = a.maxq_exact;
+    else term = quant ? D::rd(-qw + rintf(qw)) : 0.0f;
+    acc += (term * g) * gs;
+    if (small || big) D::store(a.dw, n * a.lddw + k, 0.0f);
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) {
+    float r = D::rd(acc);                                // cast to the parameter dtype
+    if (quant) r = D::rd(__fdiv_rn(r, a.n_states));       // through clip / n_states
+    D::store(a.dclip, (int64_t)t * a.N + n, r);
+  }
+}
+
 }  // namespace ahl
 
 using namespace ahl;
@@ -124,14 +189,21 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
                        float* tile_min, void* w_eff, int64_t ld_eff, hipStream_t s) {
   const int32_t dtype = cfg->dtype;
   const int32_t noise = with_noise ? cfg->noise_type : AHL_NOISE_NONE;
-  if (cfg->quant_type < 0 || cfg->quant_type > 2 || noise < 0 || noise > 2) return AHL_ERR_ARG;
-  if (cfg->quant_type != AHL_QUANT_NONE && !(cfg->res > 0.0f)) return AHL_ERR_ARG;
+  if (cfg->quant_type < 0 || cfg->quant_type > 3 || noise < 0 || noise > 2) return AHL_ERR_ARG;
+  const bool clip_only = cfg->quant_type == AHL_QUANT_CLIP_LEARNED;
+  if (clip_only && !cfg->wmax_given) return AHL_ERR_ARG;
+  if (cfg->quant_type != AHL_QUANT_NONE && !clip_only && !(cfg->res > 0.0f)) return AHL_ERR_ARG;
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(w) && (ld % D::EPV == 0);
     if (cdiv(N * tl.n_tiles, 4) > 0x7fffffff) return AHL_ERR_ARG;
     const dim3 grid((unsigned)cdiv(N * tl.n_tiles, 4));
-    if (vec) hipLaunchKernelGGL((k_sliced_absmax<D, true>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
-    else hipLaunchKernelGGL((k_sliced_absmax<D, false>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
+    if (cfg->wmax_given) {
+      // wmax holds the learnable clip: nothing to reduce
+    } else if (vec) {
+      hipLaunchKernelGGL((k_sliced_absmax<D, true>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
+    } else {
+      hipLaunchKernelGGL((k_sliced_absmax<D, false>), grid, dim3(256), 0, s, w, N, ld, tl, wmax);
+    }
     hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
     if (w_eff) {
       ModArgs a;
@@ -139,9 +211,10 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       a.tile_min = tile_min; a.w_eff = w_eff; a.ld_eff = ld_eff;
       a.quant_type = cfg->quant_type; a.noise_type = noise;
       const float res = cfg->res;
-      a.n_states = cfg->quant_type != AHL_QUANT_NONE ? fmaxf(res, 1.0f / res) : 1.0f;
+      a.n_states = (cfg->quant_type != AHL_QUANT_NONE && !clip_only) ? fmaxf(res, 1.0f / res) : 1.0f;
       // clamp(Tensor, Scalar, Scalar) converts its bounds to the tensor dtype first
       a.maxq = D::kIsBf16 ? host_round_bf16(a.n_states / 2.0f) : a.n_states / 2.0f;
+      if (clip_only) a.maxq = 1.0f;
       a.std_dev = cfg->std_dev; a.seed = cfg->seed; a.offset = cfg->offset;
       const int64_t bpr = cdiv(cdiv(K, 8), 256);
       if (bpr * N > 0x7fffffff) return AHL_ERR_ARG;
@@ -167,6 +240,31 @@ int ahl_weight_prep(const void* w, int64_t N, int64_t K, int64_t ld, const int32
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   return launch_prep(w, N, K, ld, tl, cfg, true, wmax, tile_max, tile_min, w_eff, ld_eff,
                      (hipStream_t)stream);
+}
+
+int ahl_learned_clip_bwd(void* dw, int64_t lddw, const void* w, int64_t ldw, const void* clip,
+                         const float* tile_min, void* dclip, int64_t N, int64_t K,
+                         const int32_t* tile_ends_host, int32_t n_tiles, const AhlModifierCfg* cfg,
+                         void* stream) {
+  if (!dw || !w || !clip || !tile_min || !dclip || !cfg || N <= 0 || K <= 0 || lddw < K || ldw < K)
+    return AHL_ERR_ARG;
+  const bool quant = cfg->quant_type == AHL_QUANT_DISCRETIZE_PER_CHANNEL;
+  if (!quant && cfg->quant_type != AHL_QUANT_CLIP_LEARNED) return AHL_ERR_ARG;
+  if (quant && !(cfg->res > 0.0f)) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  ClipBwdArgs a;
+  a.dw = dw; a.lddw = lddw; a.w = w; a.ldw = ldw; a.clip = clip; a.tile_min = tile_min;
+  a.dclip = dclip; a.N = N; a.tl = tl; a.quant_type = cfg->quant_type;
+  a.n_states = quant ? fmaxf(cfg->res, 1.0f / cfg->res) : 1.0f;
+  a.maxq_exact = quant ? a.n_states / 2.0f : 1.0f;
+  a.maxq = (cfg->dtype == AHL_BF16) ? host_round_bf16(a.maxq_exact) : a.maxq_exact;
+  const int64_t nb = cdiv(N * n_tiles, 4);
+  if (nb > 0x7fffffff) return AHL_ERR_ARG;
+  AHL_DISPATCH_DTYPE(cfg->dtype, {
+    hipLaunchKernelGGL((k_learned_clip_bwd<D>), dim3((unsigned)nb), dim3(256), 0, (hipStream_t)stream, a);
+  });
+  return check_launch("ahl_learned_clip_bwd");
 }
 
 int ahl_quantize_weights(void* w, int64_t N, int64_t K, int64_t ld, const int32_t* tile_ends_host,

@@ -59,6 +59,8 @@ extern "C" {
 #define AHL_QUANT_NONE 0
 #define AHL_QUANT_DISCRETIZE 1              /* scale from max|W_tile|               */
 #define AHL_QUANT_DISCRETIZE_PER_CHANNEL 2  /* scale from max|W_tile[n, :]|         */
+#define AHL_QUANT_CLIP_LEARNED 3            /* no quantiser, clamp(w / c, -1, 1) * c with the
+                                               learnable clip c (needs wmax_given)   */
 
 #define AHL_CLIP_LAYER 0        /* one std over the whole matrix   */
 #define AHL_CLIP_PER_CHANNEL 1  /* one std per output channel (row) */
@@ -91,6 +93,9 @@ typedef struct AhlModifierCfg {
   int32_t noise_type; /* AHL_NOISE_* (ignored by ahl_quantize_weights)                          */
   float res;          /* modifier.res (number of states, or its inverse)                        */
   float std_dev;      /* modifier.std_dev                                                       */
+  int32_t wmax_given; /* != 0: wmax[T, N] is an input (clip.type LEARNABLE_PER_CHANNEL: the
+                         learnable_weight_clip takes the place of the per-tile abs-max,
+                         torch_utils/torch_linear.py:222-244) instead of being computed            */
   uint64_t seed;
   uint64_t offset;
 } AhlModifierCfg;
@@ -238,6 +243,20 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* clamp_mask, co
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
 int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype);
+
+/* Backward of the learnable weight clip (UniformQuantize.backward with learn_res,
+ * torch_utils/quant_utils.py:123-153, as called from clip_and_quantize :184-233).
+ *   dw    dtype [N, K], in/out: on entry the gradient w.r.t. the clipped (and quantised) weights,
+ *         on exit the gradient w.r.t. the weights (zero where a weight was clipped)
+ *   w     dtype [N, K]  the weights of the forward;  clip dtype [T, N]  learnable_weight_clip
+ *   tile_min float [T]  as returned by ahl_weight_prep for that clip
+ *   dclip dtype [T, N]  gradient of the clip (LSQ rule, scaled by 1/sqrt(numel) without and
+ *         2 sqrt(max_state / numel) with a quantiser, numel = N * tile width)
+ *   cfg->quant_type: AHL_QUANT_CLIP_LEARNED or AHL_QUANT_DISCRETIZE_PER_CHANNEL.            */
+int ahl_learned_clip_bwd(void* dw, int64_t lddw, const void* w, int64_t ldw, const void* clip,
+                         const float* tile_min, void* dclip, int64_t N, int64_t K,
+                         const int32_t* tile_ends_host, int32_t n_tiles, const AhlModifierCfg* cfg,
+                         void* stream);
 
 /* Weight gradient: dw[:, tile t] = (g * !clamped_t)^T @ DAC(clamp(x[:, tile t])).
  *   xq: the quantised input saved from the forward (ahl_dac), or NULL to re-quantise x here.

@@ -42,6 +42,7 @@ class OracleCfg:
     out_noise: float = 0.0
     out_noise_per_channel: bool = False
     bound_per_channel: bool = False  # clip type is one of the per-channel kinds
+    clip_learnable: bool = False     # clip type LEARNABLE_PER_CHANNEL
     ir_mode: str = IR_NONE
     ir_decay: float = 0.001
     ir_input_min_percentage: float = 0.95
@@ -128,6 +129,57 @@ def quantize_weight_tile(w_t: Tensor, wmax_t: Tensor, kind: str, res: float) -> 
     return quantize(w_t, step, False, n_states / 2)
 
 
+def learned_clip_tile(w_t: Tensor, lwc_t: Tensor, kind: str, res: float) -> Tuple[Tensor, Dict]:
+    """Weights of one tile under LEARNABLE_PER_CHANNEL clipping (clip_and_quantize,
+    torch_utils/quant_utils.py:184-233, through UniformQuantize.forward :63-107). ``lwc_t`` is the
+    learnable clip of the tile, [N, 1].
+    No quantiser: clamp(w / c, -1, 1) * c (res = c, bound 0.5, max state 1, no rounding);
+    DISCRETIZE_PER_CHANNEL: round(clamp(w / (2 c / n), +-n/2)) * (2 c / n).
+    Returns the weights and what :func:`learned_clip_backward` needs."""
+    assert kind in (NONE, DISCRETIZE_PER_CHANNEL), "per-channel clip cannot feed a per-tensor quantiser"
+    tiny = _tiny(w_t.dtype)
+    if kind == NONE:
+        alpha, max_q, skip, passed = 1.0, 1.0, True, lwc_t
+        chain = 1.0
+    else:
+        n_states = max(res, 1 / res)
+        alpha, max_q, skip, passed = 2.0, n_states / 2, False, lwc_t / n_states
+        chain = n_states
+    step = alpha / passed if bool((passed > 1.0).all()) else alpha * passed
+    step = step.clone()
+    step[step == 0.0] = 1.0
+    cstep = step.clamp_min(tiny)
+    out = torch.clamp(w_t / cstep, min=-max_q, max=max_q)
+    if not skip:
+        out = out.round()
+    out = out * step
+    numel = w_t.numel()
+    grad_scale = 1 / sqrt(numel) if skip else 2 * sqrt(max_q / numel)
+    return out, dict(w=w_t, cstep=cstep, max_q=max_q, skip=skip, grad_scale=grad_scale, chain=chain)
+
+
+def learned_clip_backward(grad_w_eff: Tensor, ctx: Dict) -> Tuple[Tensor, Tensor]:
+    """LSQ backward of :func:`learned_clip_tile` (UniformQuantize.backward,
+    torch_utils/quant_utils.py:123-153, written with the same tensor expressions so that the
+    dtype promotions are torch's own): gradient to the weights where they were not clipped, and
+    to the clip value [N] (through ``lwc / n_states`` when a quantiser follows)."""
+    w, cstep, max_q = ctx["w"], ctx["cstep"], ctx["max_q"]
+    q_w = w / cstep
+    small = (q_w < -max_q).float()
+    big = (q_w > max_q).float()
+    middle = 1.0 - small - big
+    if ctx["skip"]:
+        grad_res = (small * (-max_q) + big * max_q) * grad_w_eff * ctx["grad_scale"]
+    else:
+        grad_res = ((small * (-max_q) + big * max_q + middle * (-q_w + q_w.round()))
+                    * grad_w_eff * ctx["grad_scale"])
+    grad_res = torch.sum(grad_res, dim=-1, keepdim=True).to(w.dtype)  # autograd casts to the input dtype
+    grad_w = (middle * grad_w_eff).to(w.dtype)
+    if ctx["chain"] != 1.0:
+        grad_res = grad_res / ctx["chain"]
+    return grad_w, grad_res.view(-1)
+
+
 def noisy_weight_tile(w_t: Tensor, wmax_t: Tensor, kind: str, std_dev: float,
                       xi: Optional[Tensor] = None) -> Tensor:
     """w + std_dev * wmax * N(0,1) per tile (ADD_NORMAL) or per tile and channel
@@ -185,6 +237,7 @@ def linear_forward(
     training: bool,
     out_xi: Optional[Sequence[Tensor]] = None,
     w_xi: Optional[Sequence[Tensor]] = None,
+    learnable_weight_clip: Optional[Tensor] = None,
 ) -> Tuple[Tensor, Dict]:
     """Forward of one layer call on x[M, K] (torch_utils/torch_linear.py:116-314), tile by tile:
     input range -> DAC -> weight quantiser/noise -> product -> output noise -> ADC -> clamp ->
@@ -200,7 +253,7 @@ def linear_forward(
     bound_on = adc_on or cfg.out_bound > 0
     noise_on = training and cfg.out_noise > 0
     w_noise_on = training and cfg.weight_noise != NONE
-    need_wmax = bound_on or noise_on or w_noise_on or cfg.weight_quant != NONE
+    need_wmax = bound_on or noise_on or w_noise_on or cfg.weight_quant != NONE or cfg.clip_learnable
     out = 0.0
     saved: Dict = {"cfg": cfg, "in_sizes": in_sizes, "x": x, "tiles": []}
     for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
@@ -229,7 +282,14 @@ def linear_forward(
             xq = xc
         w_t = weights[:, lo:hi]
         wmax_t = w_t.abs().amax(dim=-1, keepdim=True) if need_wmax else None
-        w_eff = quantize_weight_tile(w_t, wmax_t, cfg.weight_quant, cfg.modifier_res)
+        if cfg.clip_learnable:
+            # the clipped weights, and from here on the learned clip is the tile's "wmax"
+            # (torch_linear.py:222-244)
+            lwc_t = learnable_weight_clip[t].unsqueeze(-1)
+            w_eff, rec["lsq"] = learned_clip_tile(w_t, lwc_t, cfg.weight_quant, cfg.modifier_res)
+            wmax_t = lwc_t.view_as(wmax_t)
+        else:
+            w_eff = quantize_weight_tile(w_t, wmax_t, cfg.weight_quant, cfg.modifier_res)
         if w_noise_on:
             w_eff = noisy_weight_tile(w_eff, wmax_t, cfg.weight_noise, cfg.modifier_std,
                                       None if w_xi is None else w_xi[t])
@@ -260,7 +320,8 @@ def linear_backward(grad_out: Tensor, saved: Dict) -> Tuple[Tensor, Tensor, Tens
     """Explicit backward of :func:`linear_forward` = what autograd computes for the reference
     graph: clamp mask (torch.clamp), straight-through ADC/DAC (quant_utils.py:152-156), product,
     input-range gradient (torch_linear.py:92-106) and straight-through input clamp
-    (torch_linear.py:44-54). Returns (dx, dw, dbias, ir_grad or None)."""
+    (torch_linear.py:44-54). Returns (dx, dw, dbias, ir_grad or None); with a learnable weight
+    clip its gradient [T, N] is stored as ``saved["dlwc"]``."""
     cfg: OracleCfg = saved["cfg"]
     x = saved["x"]
     dtype = x.dtype
@@ -271,7 +332,11 @@ def linear_backward(grad_out: Tensor, saved: Dict) -> Tuple[Tensor, Tensor, Tens
     for t, (lo, hi) in enumerate(tile_bounds(saved["in_sizes"])):
         rec = saved["tiles"][t]
         gy = grad_out if rec["keep"] is None else grad_out * rec["keep"]
-        dw_parts.append(matmul_rounded(gy.T, rec["xq"]))
+        dw_t = matmul_rounded(gy.T, rec["xq"])
+        if "lsq" in rec:
+            dw_t, dlwc_t = learned_clip_backward(dw_t, rec["lsq"])
+            saved.setdefault("dlwc", []).append(dlwc_t)
+        dw_parts.append(dw_t)
         d = matmul_rounded(gy, rec["w_eff"])
         if cfg.ir_mode == IR_STATIC:
             ir_t, up, low = rec["ir"], rec["up"], rec["lo"]
@@ -299,6 +364,8 @@ def linear_backward(grad_out: Tensor, saved: Dict) -> Tuple[Tensor, Tensor, Tens
         dx[:, lo:hi] = d
     dw = torch.cat(dw_parts, dim=1)
     dbias = grad_out.sum(dim=0)
+    if "dlwc" in saved:  # gradient of learnable_weight_clip [T, N], left in ``saved``
+        saved["dlwc"] = torch.stack(saved["dlwc"])
     return dx, dw, dbias, ir_grad
 
 

@@ -13,7 +13,7 @@ DEFAULTS = dict(
     clip="none", clip_sigma=-1.0, weight_quant="none", weight_noise="none", modifier_res=0.0,
     modifier_std=0.0, ir_mode="none", ir_init=3.0, init_from_data=0, init_std_alpha=3.0,
     ir_decay=0.001, ir_min_pct=0.95, ir_values=None, training=True, kind="fwd_bwd",
-    seed=0, noise_seed=1234, x_scale=1.0, w_scale=0.02, steps=0, act_range_momentum=0.95,
+    seed=0, noise_seed=1234, x_scale=1.0, w_scale=0.02, steps=0, act_range_momentum=0.95, lwc_scale=1.0,
 )
 
 
@@ -100,6 +100,24 @@ CASES = [
          max_input_size=12, ir_mode="fast", init_from_data=4, inp_res=254, seed=16),
     case("f32_fast_init_minmax", kind="ir_fast_init", steps=4, M=16, K=24, N=8, max_input_size=12,
          ir_mode="fast", init_from_data=3, act_range_momentum=-1, inp_res=254, seed=17),
+    # learnable per-channel weight clip (LSQ): clip only, clip + on-the-fly quantisation, and clip
+    # + weight noise (whose scale is then the learned clip); the clip values start at lwc_scale
+    # times the per-tile per-channel abs-max so that some weights are actually clipped
+    case("f32_lsq_clip", M=10, K=24, N=12, max_input_size=12, ir_mode="static", clip="learnable",
+         lwc_scale=0.6, w_scale=0.3, seed=18, **_ADC8),
+    case("bf16_lsq_clip", dtype="bf16", M=10, K=24, N=12, max_input_size=12, ir_mode="static",
+         clip="learnable", lwc_scale=0.6, w_scale=0.3, seed=18, **_ADC8),
+    case("f32_lsq_quant", M=10, K=24, N=12, max_input_size=12, ir_mode="static", clip="learnable",
+         lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30, w_scale=0.3, seed=19,
+         **_ADC8),
+    case("bf16_lsq_quant", dtype="bf16", M=10, K=24, N=12, max_input_size=12, ir_mode="static",
+         clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30,
+         w_scale=0.3, seed=19, **_ADC8),
+    case("f32_lsq_clip_wnoise", M=10, K=24, N=12, max_input_size=12, ir_mode="static",
+         clip="learnable", lwc_scale=0.6, weight_noise="add_normal_per_channel", modifier_std=0.05,
+         w_scale=0.3, seed=20, **_ADC8),
+    case("f32_lsq_clip_big", M=6, K=16, N=8, max_input_size=8, clip="learnable", lwc_scale=0.6,
+         w_scale=4.0, seed=21),
     # optimizer-step clipping
     case("f32_clip_layer", kind="clip", M=4, K=40, N=24, clip="layer", clip_sigma=2.0, w_scale=1.0,
          seed=13),
@@ -117,6 +135,16 @@ CASES = [
 ]
 
 CASES_BY_NAME = {c["name"]: c for c in CASES}
+
+
+def make_learnable_clip(c, w):
+    """Initial learnable_weight_clip [T, N] of a case: lwc_scale x per-tile per-channel abs-max."""
+    k, mx = c["K"], c["max_input_size"]
+    n_tiles = 1 if mx <= 0 else -(-k // mx)
+    base, extra = divmod(k, n_tiles)
+    sizes = [base + 1 if i < extra else base for i in range(n_tiles)]
+    parts = torch.split(w.abs().float(), sizes, dim=1)
+    return (torch.stack([p.amax(dim=1) for p in parts]) * c["lwc_scale"]).to(w.dtype)
 
 
 def make_inputs(c):

@@ -19,7 +19,7 @@ import torch
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, HERE)
-from golden_cases import CASES, DTYPES, make_inputs  # noqa: E402  pylint: disable=wrong-import-position
+from golden_cases import CASES, DTYPES, make_inputs, make_learnable_clip  # noqa: E402  pylint: disable=wrong-import-position
 
 from aihwkit_lightning.nn import AnalogLinear  # noqa: E402  (the reference)
 from aihwkit_lightning.optim import AnalogOptimizer  # noqa: E402
@@ -34,6 +34,7 @@ CLIP = {
     "none": WeightClipType.NONE,
     "layer": WeightClipType.LAYER_GAUSSIAN,
     "channel": WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL,
+    "learnable": WeightClipType.LEARNABLE_PER_CHANNEL,
 }
 QUANT = {
     "none": WeightQuantizationType.NONE,
@@ -86,6 +87,8 @@ def run_case(case, store):
     layer.set_weights_and_biases(w, b)
     if case["ir_values"] is not None and layer.input_range is not None:
         layer.input_range.data = torch.tensor(case["ir_values"], dtype=dtype)
+    if case["clip"] == "learnable":
+        layer.learnable_weight_clip.data = make_learnable_clip(case, w)
     layer.train(case["training"])
     kind = case["kind"]
     if kind == "fwd_bwd":
@@ -100,6 +103,8 @@ def run_case(case, store):
             store[f"{name}/db"] = f32(layer.bias.grad)
         if layer.input_range is not None and layer.input_range.grad is not None:
             store[f"{name}/dir"] = f32(layer.input_range.grad)
+        if case["clip"] == "learnable":
+            store[f"{name}/dlwc"] = f32(layer.learnable_weight_clip.grad)
     elif kind == "ir_init":
         for step in range(case["steps"]):
             torch.manual_seed(case["noise_seed"] + step)

@@ -4,7 +4,7 @@ import os
 import numpy as np
 import torch
 
-from golden_cases import CASES_BY_NAME, DTYPES, make_inputs
+from golden_cases import CASES_BY_NAME, DTYPES, make_inputs, make_learnable_clip
 from oracle import torch_mode as om
 
 GOLDEN_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "linear_cases.npz")
@@ -28,7 +28,8 @@ def oracle_cfg(c) -> om.OracleCfg:
     return om.OracleCfg(
         max_input_size=c["max_input_size"], inp_res=c["inp_res"], out_res=c["out_res"],
         out_bound=c["out_bound"], out_noise=c["out_noise"],
-        out_noise_per_channel=c["out_noise_per_channel"], bound_per_channel=c["clip"] == "channel",
+        out_noise_per_channel=c["out_noise_per_channel"],
+        bound_per_channel=c["clip"] in ("channel", "learnable"), clip_learnable=c["clip"] == "learnable",
         ir_mode=c["ir_mode"], ir_decay=c["ir_decay"], ir_input_min_percentage=c["ir_min_pct"],
         weight_quant=c["weight_quant"], weight_noise=c["weight_noise"],
         modifier_res=c["modifier_res"], modifier_std=c["modifier_std"],
@@ -52,9 +53,11 @@ def oracle_fwd_bwd(c):
     in_sizes = om.split_sizes(c["K"], c["max_input_size"])
     ir = case_input_range(c, len(in_sizes))
     torch.manual_seed(c["noise_seed"])
-    out, saved = om.linear_forward(x, w, b, cfg, ir, c["training"])
+    lwc = make_learnable_clip(c, w) if c["clip"] == "learnable" else None
+    out, saved = om.linear_forward(x, w, b, cfg, ir, c["training"], learnable_weight_clip=lwc)
     dx, dw, db, dir_ = om.linear_backward(g, saved)
-    return dict(out=out, dx=dx, dw=dw, db=db if b is not None else None, dir=dir_)
+    return dict(out=out, dx=dx, dw=dw, db=db if b is not None else None, dir=dir_,
+                dlwc=saved.get("dlwc"))
 
 
 def rel_scale_mismatch(got, ref, rtol):

@@ -1,7 +1,7 @@
 """Helpers of the GPU parity tests: build the product layer for a case, run it, fetch results."""
 import torch
 
-from golden_cases import DTYPES, make_inputs
+from golden_cases import DTYPES, make_inputs, make_learnable_clip
 from helpers import case_input_range
 
 from aihwkit_lightning.nn import AnalogLinear
@@ -16,6 +16,7 @@ CLIP = {
     "none": WeightClipType.NONE,
     "layer": WeightClipType.LAYER_GAUSSIAN,
     "channel": WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL,
+    "learnable": WeightClipType.LEARNABLE_PER_CHANNEL,
 }
 QUANT = {
     "none": WeightQuantizationType.NONE,
@@ -64,6 +65,8 @@ def make_layer(c, device="cuda", inputs=None):
     layer = AnalogLinear(c["K"], c["N"], bias=b is not None, dtype=dtype, rpu_config=rpu_config(c))
     layer.set_weights_and_biases(w, b)
     layer = layer.to(device)
+    if c["clip"] == "learnable":
+        layer.learnable_weight_clip.data = make_learnable_clip(c, w).to(device)
     ir = case_input_range(c, len(layer.in_sizes))
     if ir is not None:
         layer.input_range.data = ir.to(device)
@@ -85,4 +88,6 @@ def hip_fwd_bwd(c, inputs=None):
         res["db"] = layer.bias.grad.cpu()
     if layer.input_range is not None and layer.input_range.grad is not None:
         res["dir"] = layer.input_range.grad.cpu()
+    if layer.learnable_weight_clip is not None and layer.learnable_weight_clip.grad is not None:
+        res["dlwc"] = layer.learnable_weight_clip.grad.cpu()
     return res

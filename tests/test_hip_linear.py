@@ -41,10 +41,10 @@ def check_against(res, ref, c, tag):
     lsb = adc_lsb(c)
     assert_close_lsb(res["out"], ref["out"].float().to(res["out"].dtype), rtol, lsb, what=f"{tag} out")
     # gradients: an output LSB flip never enters them (straight-through), only clamp-mask flips
-    for key in ("dx", "dw", "db", "dir"):
+    for key in ("dx", "dw", "db", "dir", "dlwc"):
         if ref.get(key) is None:
             continue
-        assert res[key] is not None, f"{tag}: no {key} from the HIP path"
+        assert res.get(key) is not None, f"{tag}: no {key} from the HIP path"
         assert_close_lsb(res[key].float(), ref[key].float(), rtol, None, what=f"{tag} {key}")
 
 
@@ -56,7 +56,7 @@ def test_golden_cases_match_oracle_and_reference(c):
     ref = oracle_fwd_bwd(c)
     check_against(res, ref, c, c["name"] + " vs oracle")
     gold = {k: golden_tensor(f"{c['name']}/{k}") if f"{c['name']}/{k}" in golden() else None
-            for k in ("out", "dx", "dw", "db", "dir")}
+            for k in ("out", "dx", "dw", "db", "dir", "dlwc")}
     check_against(res, gold, c, c["name"] + " vs reference")
 
 

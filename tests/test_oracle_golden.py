@@ -26,7 +26,7 @@ def test_forward_backward_matches_reference(case):
     res = oracle_fwd_bwd(case)
     dtype = DTYPES[case["dtype"]]
     name = case["name"]
-    for key in ("out", "dx", "dw", "db", "dir"):
+    for key in ("out", "dx", "dw", "db", "dir", "dlwc"):
         gkey = f"{name}/{key}"
         if gkey not in golden():
             continue
@@ -34,6 +34,8 @@ def test_forward_backward_matches_reference(case):
         _exact_or_close(res[key], golden_tensor(gkey), dtype, gkey)
     if case["ir_mode"] in ("static", "fast"):
         assert f"{name}/dir" in golden(), "reference wrote an input-range gradient"
+    if case["clip"] == "learnable":
+        assert f"{name}/dlwc" in golden(), "reference wrote a gradient of the learnable clip"
 
 
 @pytest.mark.parametrize("name", ["f32_ir_init", "bf16_ir_init"])
