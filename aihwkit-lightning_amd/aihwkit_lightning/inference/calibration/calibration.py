@@ -14,6 +14,7 @@ from torch.utils.hooks import RemovableHandle
 
 from ...exceptions import ConfigError
 from ...nn import AnalogLinear
+from ...nn.modules.conv import _AnalogConvNd
 from ...nn.modules.hip_utils.ops import OPS
 from ...simulator.configs import TorchInferenceRPUConfig, WeightNoiseInjectionType
 
@@ -32,6 +33,9 @@ def _max_pre_forward(mod: AnalogLinear, args: Tuple, kwargs: Dict, cache: Dict[s
                      key: str) -> None:
     """Forward pre-hook: fold this batch into the layer's running per-tile abs-max."""
     x_input: Tensor = args[0] if len(args) > 0 else kwargs["inp"]
+    if isinstance(mod, _AnalogConvNd):
+        # the tiles of a convolution see patches, not the image (reference calibration.py:82-93)
+        x_input = mod.patch_rows(x_input)
     x_input = x_input.reshape(-1, x_input.size(-1))
     if key not in cache:
         cache[key] = torch.full((len(mod.in_sizes),), float("-inf"), dtype=torch.float32,

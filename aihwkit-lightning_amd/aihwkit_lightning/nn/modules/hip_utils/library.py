@@ -13,7 +13,7 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
@@ -69,11 +69,30 @@ class AhlModifierCfg(Structure):
     ]
 
 
+class AhlConvGeom(Structure):
+    """Mirror of ``struct AhlConvGeom``."""
+
+    _fields_ = [
+        ("batch", c_int32),
+        ("channels", c_int32),
+        ("in_size", c_int32 * 3),
+        ("kernel", c_int32 * 3),
+        ("stride", c_int32 * 3),
+        ("padding", c_int32 * 3),
+        ("dilation", c_int32 * 3),
+    ]
+
+
 _I32P = POINTER(c_int32)
 
 # name -> (restype, argtypes); every exported symbol of include/analog_hip.h
 SIGNATURES = {
     "ahl_abi_version": (c_int32, []),
+    "ahl_conv_out_size": (c_int32, [POINTER(AhlConvGeom), _I32P]),
+    "ahl_im2col": (c_int32, [c_void_p, POINTER(AhlConvGeom), c_int32, c_void_p, c_int64, c_void_p]),
+    "ahl_col2im": (c_int32, [c_void_p, c_int64, POINTER(AhlConvGeom), c_int32, c_void_p, c_void_p]),
+    "ahl_transpose_batched": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int64, c_int64,
+                                        c_void_p, c_int64, c_void_p]),
     "ahl_last_hip_error": (c_char_p, []),
     "ahl_sliced_absmax": (
         c_int32,

@@ -104,6 +104,78 @@ LIB.define(
     "linear_bwd_dw(Tensor g, Tensor? keep, Tensor? clamp_flag, Tensor? x, Tensor? xq, Tensor? ir, "
     "int[] in_sizes, int[] icfg, float[] fcfg, bool want_bias) -> (Tensor, Tensor)"
 )
+LIB.define("im2col(Tensor x, int[] geom) -> Tensor")
+LIB.define("col2im(Tensor dcols, int[] geom) -> Tensor")
+LIB.define("transpose_batched(Tensor src) -> Tensor")
+
+
+def conv_geom(geom: List[int]) -> L.AhlConvGeom:
+    """``[batch, channels, in(3), kernel(3), stride(3), padding(3), dilation(3)]`` as the ABI's
+    geometry struct."""
+    if len(geom) != 17:
+        raise HipBackendError(f"a convolution geometry has 17 integers, got {len(geom)}")
+    out = L.AhlConvGeom()
+    out.batch, out.channels = int(geom[0]), int(geom[1])
+    for i in range(3):
+        out.in_size[i] = int(geom[2 + i])
+        out.kernel[i] = int(geom[5 + i])
+        out.stride[i] = int(geom[8 + i])
+        out.padding[i] = int(geom[11 + i])
+        out.dilation[i] = int(geom[14 + i])
+    return out
+
+
+def conv_out_size(geom: List[int]) -> List[int]:
+    """Output extents (3) of a convolution geometry; host arithmetic in the library."""
+    out = (L.c_int32 * 3)()
+    L.check(L.load().ahl_conv_out_size(byref(conv_geom(geom)), out), "ahl_conv_out_size")
+    return [int(v) for v in out]
+
+
+def im2col(x: Tensor, geom: List[int]) -> Tensor:
+    """Patches ``[B, L, C * kD * kH * kW]`` of ``x [B, C, D, H, W]``."""
+    lib = L.load()
+    x = x.contiguous()
+    cgeom = conv_geom(geom)
+    if x.numel() != geom[0] * geom[1] * geom[2] * geom[3] * geom[4]:
+        raise HipBackendError(f"input of shape {tuple(x.shape)} does not match geometry {geom}")
+    out_size = conv_out_size(geom)
+    n_pos = out_size[0] * out_size[1] * out_size[2]
+    k_in = geom[1] * geom[5] * geom[6] * geom[7]
+    cols = torch.empty((geom[0], n_pos, k_in), dtype=x.dtype, device=x.device)
+    L.check(lib.ahl_im2col(_ptr(x), byref(cgeom), dtype_id(x.dtype), _ptr(cols), k_in, _stream()),
+            "ahl_im2col")
+    return cols
+
+
+def col2im(dcols: Tensor, geom: List[int]) -> Tensor:
+    """Adjoint of :func:`im2col`: ``[B, L, K]`` patch gradients to ``[B, C, D, H, W]``."""
+    lib = L.load()
+    dcols = dcols.contiguous()
+    cgeom = conv_geom(geom)
+    out_size = conv_out_size(geom)
+    k_in = geom[1] * geom[5] * geom[6] * geom[7]
+    if dcols.numel() != geom[0] * out_size[0] * out_size[1] * out_size[2] * k_in:
+        raise HipBackendError(f"patches of shape {tuple(dcols.shape)} do not match geometry {geom}")
+    dx = torch.empty((geom[0], geom[1], geom[2], geom[3], geom[4]), dtype=dcols.dtype,
+                     device=dcols.device)
+    L.check(lib.ahl_col2im(_ptr(dcols), k_in, byref(cgeom), dtype_id(dcols.dtype), _ptr(dx),
+                           _stream()), "ahl_col2im")
+    return dx
+
+
+def transpose_batched(src: Tensor) -> Tensor:
+    """``dst[b, c, r] = src[b, r, c]`` as a new contiguous tensor."""
+    lib = L.load()
+    if src.dim() != 3:
+        raise HipBackendError(f"transpose_batched takes a 3-D tensor, got {tuple(src.shape)}")
+    src = src.contiguous()
+    batch, rows, cols = src.shape
+    dst = torch.empty((batch, cols, rows), dtype=src.dtype, device=src.device)
+    if src.numel() > 0:
+        L.check(lib.ahl_transpose_batched(_ptr(src), cols, dtype_id(src.dtype), batch, rows, cols,
+                                          _ptr(dst), rows, _stream()), "ahl_transpose_batched")
+    return dst
 
 
 def sliced_absmax(x: Tensor, in_sizes: List[int], tile_stats: bool) -> Tuple[Tensor, Tensor, Tensor]:
@@ -451,6 +523,7 @@ for _name, _fn in [
     ("clip_weights", clip_weights), ("col_sum", col_sum),
     ("weight_prep", weight_prep), ("quantize_weights", quantize_weights),
     ("weight_prep_clip", weight_prep_clip), ("learned_clip_bwd", learned_clip_bwd),
+    ("im2col", im2col), ("col2im", col2im), ("transpose_batched", transpose_batched),
     ("dac", dac), ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
 ]:
     LIB.impl(_name, _fn, "CUDA")

@@ -1,0 +1,272 @@
+// Data movement that turns a convolution into the tiled analog matrix product: patch extraction
+// (im2col), its adjoint (col2im) and the batched transpose between the [tokens, channels] layout
+// of the matrix product and the [channels, positions] layout of a convolution output.
+//
+// All three are pure HBM kernels. Patches are written as rows of a [B * L, C * kD * kH * kW]
+// matrix (L output positions per image), channel-major then kernel offsets with the last spatial
+// dimension fastest: the order of `weight.view(out_channels, -1)` of a torch convolution weight,
+// so the K-tiles of the analog layer cut the same columns as in the reference
+// (nn/modules/conv.py:310-325 for 1-d/2-d through torch's unfold, :40-103 for 3-d).
+// 1-d and 2-d convolutions use the same code with leading sizes of one.
+#include "ahl_host.h"
+
+namespace ahl {
+
+struct ConvGeom {
+  int32_t B, C;
+  int32_t in[3], out[3], ker[3], str[3], pad[3], dil[3];
+  int32_t kvol;  // kernel offsets per channel
+  int64_t L;     // output positions per image
+  int64_t K;     // patch length C * kvol
+};
+
+// Output extent of one dimension (torch's convolution arithmetic); <= 0 means "does not fit".
+static int64_t conv_extent(int64_t in, int64_t ker, int64_t str, int64_t pad, int64_t dil) {
+  const int64_t span = in + 2 * pad - dil * (ker - 1) - 1;
+  if (span < 0) return 0;
+  return span / str + 1;
+}
+
+static bool make_geom(const AhlConvGeom* a, ConvGeom* g) {
+  if (a == nullptr || a->batch <= 0 || a->channels <= 0) return false;
+  g->B = a->batch;
+  g->C = a->channels;
+  int64_t kvol = 1, L = 1, vol = 1;
+  for (int d = 0; d < 3; ++d) {
+    if (a->in_size[d] <= 0 || a->kernel[d] <= 0 || a->stride[d] <= 0 || a->padding[d] < 0 ||
+        a->dilation[d] <= 0)
+      return false;
+    g->in[d] = a->in_size[d];
+    g->ker[d] = a->kernel[d];
+    g->str[d] = a->stride[d];
+    g->pad[d] = a->padding[d];
+    g->dil[d] = a->dilation[d];
+    const int64_t o = conv_extent(a->in_size[d], a->kernel[d], a->stride[d], a->padding[d],
+                                  a->dilation[d]);
+    if (o <= 0 || o > 0x7fffffff) return false;
+    g->out[d] = (int32_t)o;
+    kvol *= a->kernel[d];
+    L *= o;
+    vol *= a->in_size[d];
+    if (kvol > 0x7fffffff || vol > 0x7fffffff || L > 0x7fffffff) return false;
+  }
+  if (kvol * a->channels > 0x7fffffff) return false;
+  g->kvol = (int32_t)kvol;
+  g->L = L;
+  g->K = kvol * a->channels;
+  return true;
+}
+
+// One thread gathers VEC consecutive patch entries (consecutive kernel offsets, carrying into
+// the next kernel row / plane / channel) and writes them with one store. Threads of a wave walk
+// along the patch, so the writes are contiguous; the reads of neighbouring offsets touch
+// neighbouring input elements and mostly hit L2, since every input element is reused by up to
+// kvol patches.
+template <class E, int VEC>
+__global__ __launch_bounds__(256) void k_im2col(const E* __restrict__ x, E* __restrict__ cols,
+                                                int64_t ldc, ConvGeom g, int64_t groups_per_row,
+                                                int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const int64_t m = idx / groups_per_row;
+  const int32_t k0 = (int32_t)(idx - m * groups_per_row) * VEC;
+  const int64_t b = m / g.L;
+  int32_t l = (int32_t)(m - b * g.L);
+  const int32_t ow = l % g.out[2];
+  l /= g.out[2];
+  const int32_t oh = l % g.out[1];
+  const int32_t od = l / g.out[1];
+  int32_t c = k0 / g.kvol;
+  int32_t r = k0 - c * g.kvol;
+  int32_t kw = r % g.ker[2];
+  r /= g.ker[2];
+  int32_t kh = r % g.ker[1];
+  int32_t kd = r / g.ker[1];
+  const int32_t id0 = od * g.str[0] - g.pad[0];
+  const int32_t ih0 = oh * g.str[1] - g.pad[1];
+  const int32_t iw0 = ow * g.str[2] - g.pad[2];
+  const int64_t plane = (int64_t)g.in[1] * g.in[2];
+  E v[VEC];
+#pragma unroll
+  for (int j = 0; j < VEC; ++j) {
+    E val = (E)0;
+    if (k0 + j < g.K) {
+      const int32_t id = id0 + kd * g.dil[0], ih = ih0 + kh * g.dil[1], iw = iw0 + kw * g.dil[2];
+      if (id >= 0 && id < g.in[0] && ih >= 0 && ih < g.in[1] && iw >= 0 && iw < g.in[2])
+        val = x[((b * g.C + c) * g.in[0] + id) * plane + (int64_t)ih * g.in[2] + iw];
+    }
+    v[j] = val;
+    if (++kw == g.ker[2]) {
+      kw = 0;
+      if (++kh == g.ker[1]) {
+        kh = 0;
+        if (++kd == g.ker[0]) {
+          kd = 0;
+          ++c;
+        }
+      }
+    }
+  }
+  E* dst = cols + m * ldc + k0;
+  if constexpr (VEC * sizeof(E) == 16) {
+    u32x4 pk;
+    __builtin_memcpy(&pk, v, 16);
+    *(u32x4*)dst = pk;
+  } else {
+#pragma unroll
+    for (int j = 0; j < VEC; ++j)
+      if (k0 + j < g.K) dst[j] = v[j];
+  }
+}
+
+// Adjoint of k_im2col as a gather: one thread per input element sums, in fp32 and in a fixed
+// order (ascending kernel offset), the patch entries that were copied from it, and rounds once.
+// No atomics, so the result is reproducible.
+template <class D>
+__global__ __launch_bounds__(256) void k_col2im(const void* __restrict__ dcols, int64_t ldc,
+                                                ConvGeom g, void* __restrict__ dx, int64_t total) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  int64_t r = idx;
+  const int32_t w = (int32_t)(r % g.in[2]);
+  r /= g.in[2];
+  const int32_t h = (int32_t)(r % g.in[1]);
+  r /= g.in[1];
+  const int32_t d = (int32_t)(r % g.in[0]);
+  r /= g.in[0];
+  const int32_t c = (int32_t)(r % g.C);
+  const int64_t b = r / g.C;
+  float acc = 0.f;
+  for (int32_t kd = 0; kd < g.ker[0]; ++kd) {
+    const int32_t td = d + g.pad[0] - kd * g.dil[0];
+    if (td < 0 || td % g.str[0] != 0) continue;
+    const int32_t od = td / g.str[0];
+    if (od >= g.out[0]) continue;
+    for (int32_t kh = 0; kh < g.ker[1]; ++kh) {
+      const int32_t th = h + g.pad[1] - kh * g.dil[1];
+      if (th < 0 || th % g.str[1] != 0) continue;
+      const int32_t oh = th / g.str[1];
+      if (oh >= g.out[1]) continue;
+      for (int32_t kw = 0; kw < g.ker[2]; ++kw) {
+        const int32_t tw = w + g.pad[2] - kw * g.dil[2];
+        if (tw < 0 || tw % g.str[2] != 0) continue;
+        const int32_t ow = tw / g.str[2];
+        if (ow >= g.out[2]) continue;
+        const int64_t l = ((int64_t)od * g.out[1] + oh) * g.out[2] + ow;
+        const int64_t k = (int64_t)c * g.kvol + ((int64_t)kd * g.ker[1] + kh) * g.ker[2] + kw;
+        acc += D::load(dcols, (b * g.L + l) * ldc + k);
+      }
+    }
+  }
+  D::store(dx, idx, acc);
+}
+
+// dst[b][c][r] = src[b][r][c]; 32 x 32 tiles through LDS (padded against bank conflicts) so that
+// both the reads and the writes are contiguous.
+template <class E>
+__global__ __launch_bounds__(256) void k_transpose_batched(const E* __restrict__ src,
+                                                           int64_t ld_src, int64_t rows,
+                                                           int64_t cols, E* __restrict__ dst,
+                                                           int64_t ld_dst, int64_t tiles_c,
+                                                           int64_t tiles_per_mat) {
+  __shared__ E tile[32][33];
+  const int64_t bid = blockIdx.x;
+  const int64_t b = bid / tiles_per_mat;
+  const int64_t t = bid - b * tiles_per_mat;
+  const int64_t r0 = (t / tiles_c) * 32, c0 = (t % tiles_c) * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const E* s = src + b * rows * ld_src;
+  E* d = dst + b * cols * ld_dst;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t rr = r0 + ty + 8 * i, cc = c0 + tx;
+    if (rr < rows && cc < cols) tile[ty + 8 * i][tx] = s[rr * ld_src + cc];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int64_t cc = c0 + ty + 8 * i, rr = r0 + tx;
+    if (rr < rows && cc < cols) d[cc * ld_dst + rr] = tile[tx][ty + 8 * i];
+  }
+}
+
+template <class E, int VEC>
+static int launch_im2col(const void* x, void* cols, int64_t ldc, const ConvGeom& g,
+                         hipStream_t st) {
+  const int64_t M = (int64_t)g.B * g.L;
+  const int64_t gpr = cdiv(g.K, VEC);
+  const int64_t total = M * gpr;
+  const int64_t blocks = cdiv(total, 256);
+  if (blocks > 0x7fffffff) return AHL_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL((k_im2col<E, VEC>), dim3((unsigned)blocks), dim3(256), 0, st, (const E*)x,
+                     (E*)cols, ldc, g, gpr, total);
+  return check_launch("k_im2col");
+}
+
+}  // namespace ahl
+
+using namespace ahl;
+
+extern "C" int ahl_conv_out_size(const AhlConvGeom* geom, int32_t* out_size) {
+  ConvGeom g;
+  if (out_size == nullptr || !make_geom(geom, &g)) return AHL_ERR_ARG;
+  for (int d = 0; d < 3; ++d) out_size[d] = g.out[d];
+  return AHL_OK;
+}
+
+extern "C" int ahl_im2col(const void* x, const AhlConvGeom* geom, int32_t dtype, void* cols,
+                          int64_t ldc, void* stream) {
+  ConvGeom g;
+  if (x == nullptr || cols == nullptr || !make_geom(geom, &g) || ldc < g.K) return AHL_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == AHL_F32) {
+    if (g.K % 4 == 0 && ldc % 4 == 0 && aligned16(cols))
+      return launch_im2col<uint32_t, 4>(x, cols, ldc, g, st);
+    return launch_im2col<uint32_t, 1>(x, cols, ldc, g, st);
+  }
+  if (dtype == AHL_BF16) {
+    if (g.K % 8 == 0 && ldc % 8 == 0 && aligned16(cols))
+      return launch_im2col<uint16_t, 8>(x, cols, ldc, g, st);
+    return launch_im2col<uint16_t, 1>(x, cols, ldc, g, st);
+  }
+  return AHL_ERR_ARG;
+}
+
+extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geom, int32_t dtype,
+                          void* dx, void* stream) {
+  ConvGeom g;
+  if (dcols == nullptr || dx == nullptr || !make_geom(geom, &g) || ldc < g.K) return AHL_ERR_ARG;
+  const int64_t total = (int64_t)g.B * g.C * g.in[0] * g.in[1] * g.in[2];
+  const int64_t blocks = cdiv(total, 256);
+  if (blocks > 0x7fffffff) return AHL_ERR_UNSUPPORTED;
+  AHL_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((k_col2im<D>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       dcols, ldc, g, dx, total);
+  });
+  return check_launch("k_col2im");
+}
+
+extern "C" int ahl_transpose_batched(const void* src, int64_t ld_src, int32_t dtype, int64_t batch,
+                                     int64_t rows, int64_t cols, void* dst, int64_t ld_dst,
+                                     void* stream) {
+  if (src == nullptr || dst == nullptr || batch <= 0 || rows <= 0 || cols <= 0 || ld_src < cols ||
+      ld_dst < rows)
+    return AHL_ERR_ARG;
+  const int64_t tiles_c = cdiv(cols, 32), tiles_r = cdiv(rows, 32);
+  const int64_t per_mat = tiles_c * tiles_r;
+  if (per_mat > 0x7fffffff || batch > 0x7fffffff / per_mat) return AHL_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)(per_mat * batch));
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == AHL_F32) {
+    hipLaunchKernelGGL((k_transpose_batched<uint32_t>), grid, dim3(256), 0, st,
+                       (const uint32_t*)src, ld_src, rows, cols, (uint32_t*)dst, ld_dst, tiles_c,
+                       per_mat);
+  } else if (dtype == AHL_BF16) {
+    hipLaunchKernelGGL((k_transpose_batched<uint16_t>), grid, dim3(256), 0, st,
+                       (const uint16_t*)src, ld_src, rows, cols, (uint16_t*)dst, ld_dst, tiles_c,
+                       per_mat);
+  } else {
+    return AHL_ERR_ARG;
+  }
+  return check_launch("k_transpose_batched");
+}

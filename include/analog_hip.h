@@ -274,6 +274,42 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* clamp_mask, co
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
                                    int32_t has_mask);
 
+/* ---- convolution as the same matrix product (nn/modules/conv.py:121-367) -------------------
+ * A convolution layer of the reference unfolds its input into patches, runs the AnalogLinear
+ * operator on them with weight.view(out_channels, -1), and transposes the result back. The three
+ * entry points below are the data movement of that wrapper; the operator itself is
+ * ahl_linear_fwd / ahl_linear_bwd_*. 1-d and 2-d layers use leading sizes of one.              */
+typedef struct AhlConvGeom {
+  int32_t batch, channels;
+  int32_t in_size[3];  /* D, H, W of the input                                                  */
+  int32_t kernel[3], stride[3], padding[3], dilation[3];
+} AhlConvGeom;
+
+/* Host only: out_size[d] = (in + 2 pad - dil (ker - 1) - 1) / stride + 1, the output extent
+ * computed in _AnalogConvNd.forward (nn/modules/conv.py:357-362, :826-846). AHL_ERR_ARG if the
+ * kernel does not fit.                                                                         */
+int ahl_conv_out_size(const AhlConvGeom* geom, int32_t* out_size);
+
+/* cols[(b * L + l), c * kvol + (kd * kH + kh) * kW + kw] = x[b, c, od*sD - pD + kd*dD, ...] or 0
+ * outside the input; x dtype [B, C, D, H, W] contiguous, cols dtype [B * L, K] with row stride
+ * ldc, L = product of the output extents, K = C * kD * kH * kW. Replaces
+ * unfold(inp, ...).transpose(-1, -2).contiguous() (nn/modules/conv.py:310-322) and
+ * unfold3d(...).transpose(-1, -2).contiguous() (:40-103, :777-792).                            */
+int ahl_im2col(const void* x, const AhlConvGeom* geom, int32_t dtype, void* cols, int64_t ldc,
+               void* stream);
+
+/* Adjoint of ahl_im2col (the autograd of the unfold above): dx[b, c, d, h, w] = sum of the
+ * dcols entries that ahl_im2col copied from that element, accumulated in fp32 in ascending
+ * kernel-offset order and rounded once.                                                        */
+int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geom, int32_t dtype, void* dx,
+               void* stream);
+
+/* dst[b][c][r] = src[b][r][c] for `batch` row-major matrices of rows x cols (row strides ld_src
+ * and ld_dst, matrices back to back). Replaces out.transpose(-1, -2).contiguous()
+ * (nn/modules/conv.py:356) and its autograd.                                                   */
+int ahl_transpose_batched(const void* src, int64_t ld_src, int32_t dtype, int64_t batch,
+                          int64_t rows, int64_t cols, void* dst, int64_t ld_dst, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,16 +48,18 @@ def test_struct_layout_matches_ctypes():
     from aihwkit_lightning.nn.modules.hip_utils import library as L
 
     src = ('#include <stdio.h>\n#include <stddef.h>\n#include "analog_hip.h"\n'
-           'int main(void){printf("%zu %zu %zu %zu %zu\\n", sizeof(AhlLinearCfg), '
+           'int main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu\\n", sizeof(AhlLinearCfg), '
            'offsetof(AhlLinearCfg, seed), offsetof(AhlLinearCfg, ir_decay), sizeof(AhlModifierCfg), '
-           'offsetof(AhlModifierCfg, seed)); return 0;}\n')
+           'offsetof(AhlModifierCfg, seed), sizeof(AhlConvGeom), offsetof(AhlConvGeom, kernel), '
+           'offsetof(AhlConvGeom, dilation)); return 0;}\n')
     exe = "/tmp/ahl_layout_probe"
     proc = subprocess.run(["gcc", "-I", os.path.dirname(HEADER), "-x", "c", "-", "-o", exe],
                           input=src, text=True, capture_output=True)
     assert proc.returncode == 0, proc.stderr
     got = [int(v) for v in subprocess.run([exe], capture_output=True, text=True).stdout.split()]
     want = [ctypes.sizeof(L.AhlLinearCfg), L.AhlLinearCfg.seed.offset, L.AhlLinearCfg.ir_decay.offset,
-            ctypes.sizeof(L.AhlModifierCfg), L.AhlModifierCfg.seed.offset]
+            ctypes.sizeof(L.AhlModifierCfg), L.AhlModifierCfg.seed.offset,
+            ctypes.sizeof(L.AhlConvGeom), L.AhlConvGeom.kernel.offset, L.AhlConvGeom.dilation.offset]
     assert got == want
 
 

@@ -1,0 +1,201 @@
+"""GPU parity of the analog convolutions (AnalogConv1d/2d/3d -> custom ops -> C ABI) against the
+CPU oracle and the reference's golden vectors, and of the three data-movement entry points
+(ahl_im2col, ahl_col2im, ahl_transpose_batched), which are pure copies / fixed-order sums and
+therefore compared bit for bit.
+
+Layer acceptance rule as for the linear operator: 1e-5 (fp32) / 1e-2 (bf16) relative to the
+tensor scale, elements outside that at most one ADC LSB off and at most 0.1 % of the tensor.
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from conv_cases import CONV_CASES, conv_case, make_conv_inputs
+from golden_cases import DTYPES
+from helpers import assert_close_lsb, case_input_range, oracle_cfg
+from oracle import conv_mode as oc
+from oracle import torch_mode as om
+
+pytestmark = pytest.mark.gpu
+
+CONV_GOLDEN = dict(np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                                        "conv_cases.npz")))
+RTOL = {"f32": 1e-5, "bf16": 1e-2}
+
+GEOMS = [
+    # batch, C, size(3), kernel(3), stride(3), padding(3), dilation(3)
+    (2, 3, (1, 9, 8), (1, 3, 3), (1, 2, 1), (0, 1, 0), (1, 1, 2)),   # K = 27: scalar stores
+    (3, 8, (1, 1, 37), (1, 1, 5), (1, 1, 2), (0, 0, 2), (1, 1, 1)),  # 1-d, K = 40: vector stores
+    (2, 4, (5, 6, 7), (2, 3, 2), (1, 2, 1), (1, 0, 1), (1, 1, 1)),   # 3-d, K = 48
+    (1, 16, (1, 33, 29), (1, 3, 3), (1, 1, 1), (0, 1, 1), (1, 1, 1)),  # K = 144, odd sizes
+    (2, 2, (3, 4, 5), (3, 4, 5), (1, 1, 1), (0, 0, 0), (1, 1, 1)),   # kernel == input
+]
+
+
+def _geom_list(geom):
+    batch, chan, size, kernel, stride, padding, dilation = geom
+    return [batch, chan, *size, *kernel, *stride, *padding, *dilation]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("geom", GEOMS, ids=[f"geom{i}" for i in range(len(GEOMS))])
+def test_patch_kernels_bit_exact(geom, dtype):
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS, conv_out_size
+
+    batch, chan, size, kernel, stride, padding, dilation = geom
+    gen = torch.Generator().manual_seed(7)
+    x = torch.randn(batch, chan, *size, generator=gen).to(dtype)
+    want_cols, out = oc.conv_patches(x, kernel, stride, padding, dilation)
+    assert conv_out_size(_geom_list(geom)) == out
+    cols = OPS.im2col(x.cuda(), _geom_list(geom))
+    assert torch.equal(cols.cpu(), want_cols)
+    g = torch.randn(want_cols.shape, generator=gen).to(dtype)
+    want_dx = oc.conv_fold(g, x.shape, kernel, stride, padding, dilation)
+    dx = OPS.col2im(g.cuda(), _geom_list(geom))
+    assert torch.equal(dx.cpu(), want_dx)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 33, 65), (2, 64, 32), (5, 7, 130), (1, 300, 17)])
+def test_transpose_batched_bit_exact(shape, dtype):
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+
+    src = torch.randn(*shape, generator=torch.Generator().manual_seed(8)).to(dtype)
+    got = OPS.transpose_batched(src.cuda())
+    assert got.is_contiguous() and torch.equal(got.cpu(), src.transpose(1, 2).contiguous())
+
+
+def make_conv_layer(c, w, b):
+    from hip_helpers import rpu_config
+    from aihwkit_lightning.nn import AnalogConv1d, AnalogConv2d, AnalogConv3d
+
+    cls = {1: AnalogConv1d, 2: AnalogConv2d, 3: AnalogConv3d}[c["ndim"]]
+    one = c["ndim"] == 1
+    pick = (lambda v: v[0]) if one else (lambda v: v)
+    layer = cls(c["C"], c["N"], pick(c["kernel"]), stride=pick(c["stride"]),
+                padding=pick(c["padding"]), dilation=pick(c["dilation"]), bias=b is not None,
+                dtype=DTYPES[c["dtype"]], rpu_config=rpu_config(c))
+    layer.set_weights_and_biases(w.unsqueeze(-2) if one else w, b)
+    layer = layer.cuda()
+    ir = case_input_range(c, len(layer.in_sizes))
+    if ir is not None:
+        layer.input_range.data = ir.cuda()
+    layer.train(c["training"])
+    return layer
+
+
+def hip_conv_fwd_bwd(c, inputs):
+    x, w, b, g = inputs
+    layer = make_conv_layer(c, w, b)
+    xin = x.cuda().requires_grad_(True)
+    torch.manual_seed(c["noise_seed"])
+    out = layer(xin)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+    wgrad = layer.weight.grad.cpu()
+    res = dict(out=out.detach().cpu(), dx=xin.grad.cpu(),
+               dw=wgrad.squeeze(-2) if c["ndim"] == 1 else wgrad, db=None, dir=None)
+    if b is not None:
+        res["db"] = layer.bias.grad.cpu()
+    if layer.input_range is not None and layer.input_range.grad is not None:
+        res["dir"] = layer.input_range.grad.cpu()
+    return res
+
+
+def oracle_conv_fwd_bwd(c, inputs):
+    x, w, b, g = inputs
+    batched = c["batch"] > 0
+    xb, gb = (x, g) if batched else (x.unsqueeze(0), g.unsqueeze(0))
+    ir = case_input_range(c, len(om.split_sizes(w[0].numel(), c["max_input_size"])))
+    torch.manual_seed(c["noise_seed"])
+    out, saved = oc.conv_forward(xb, w, b, c["stride"], c["padding"], c["dilation"], oracle_cfg(c),
+                                 ir, c["training"])
+    dx, dw, db, dir_ = oc.conv_backward(gb, saved)
+    if not batched:
+        out, dx = out.squeeze(0), dx.squeeze(0)
+    return dict(out=out, dx=dx, dw=dw, db=db if b is not None else None, dir=dir_)
+
+
+def check(res, ref, c, tag):
+    from test_hip_linear import adc_lsb
+
+    rtol = RTOL[c["dtype"]]
+    assert_close_lsb(res["out"].float(), ref["out"].float(), rtol, adc_lsb(c), what=f"{tag} out")
+    for key in ("dx", "dw", "db", "dir"):
+        if ref.get(key) is None:
+            continue
+        assert res.get(key) is not None, f"{tag}: no {key} from the HIP path"
+        assert_close_lsb(res[key].float(), ref[key].float(), rtol, None, what=f"{tag} {key}")
+
+
+NOISELESS = [c for c in CONV_CASES if c["out_noise"] == 0 and c["weight_noise"] == "none"]
+
+
+@pytest.mark.parametrize("c", NOISELESS, ids=[c["name"] for c in NOISELESS])
+def test_golden_convolutions_match_oracle_and_reference(c):
+    inputs = make_conv_inputs(c)
+    res = hip_conv_fwd_bwd(c, inputs)
+    check(res, oracle_conv_fwd_bwd(c, inputs), c, c["name"] + " vs oracle")
+    gold = {k: torch.from_numpy(CONV_GOLDEN[f"{c['name']}/{k}"])
+            if f"{c['name']}/{k}" in CONV_GOLDEN else None for k in ("out", "dx", "dw", "db", "dir")}
+    check(res, gold, c, c["name"] + " vs reference")
+
+
+_ADC = dict(inp_res=254, out_res=254, out_bound=10.0, clip="channel", clip_sigma=2.5, ir_decay=0.01)
+SHAPES = [
+    # ResNet-like 3x3 layer: K = 576 in three tiles of 192, 1568 patches
+    conv_case("conv2d_bf16_resnet", 2, 2, 64, (28, 28), (3, 3), (1, 1), (1, 1), N=128, dtype="bf16",
+              max_input_size=256, ir_mode="static", ir_init=3.0, seed=50, **_ADC),
+    conv_case("conv2d_f32_strided", 2, 3, 16, (19, 17), (5, 3), (2, 2), (2, 1), N=40,
+              max_input_size=128, ir_mode="static", ir_init=3.0, seed=51, **_ADC),
+    conv_case("conv1d_bf16_long", 1, 4, 32, (200,), (7,), (3,), (3,), N=64, dtype="bf16",
+              max_input_size=128, ir_mode="dynamic", seed=52, **_ADC),
+    conv_case("conv3d_bf16_video", 3, 2, 8, (6, 14, 14), (3, 3, 3), (1, 2, 2), (1, 1, 1), N=32,
+              dtype="bf16", max_input_size=128, ir_mode="static", ir_init=3.0, seed=53, **_ADC),
+]
+
+
+@pytest.mark.parametrize("c", SHAPES, ids=[c["name"] for c in SHAPES])
+def test_seeded_convolutions_match_oracle(c):
+    inputs = make_conv_inputs(c)
+    check(hip_conv_fwd_bwd(c, inputs), oracle_conv_fwd_bwd(c, inputs), c, c["name"])
+
+
+def test_conv1d_state_dict_round_trip_with_torch():
+    """An AnalogConv1d saves and loads nn.Conv1d-shaped weights (reference conv.py:497-512)."""
+    from hip_helpers import rpu_config
+    from aihwkit_lightning.nn import AnalogConv1d
+
+    c = CONV_CASES[1]
+    digital = torch.nn.Conv1d(4, 6, 3, stride=2, padding=1).cuda()
+    analog = AnalogConv1d.from_digital(digital, rpu_config(c))
+    assert analog.weight.shape == (6, 4, 1, 3) and analog.state_dict()["weight"].shape == (6, 4, 3)
+    x = torch.randn(3, 4, 11, device="cuda")
+    assert torch.allclose(analog(x), digital(x), rtol=1e-5, atol=1e-5)
+    other = AnalogConv1d(4, 6, 3, stride=2, padding=1, rpu_config=rpu_config(c)).cuda()
+    other.load_state_dict(analog.state_dict())
+    assert torch.equal(other.weight, analog.weight)
+    back = AnalogConv1d.to_digital(other)
+    assert torch.equal(back.weight, digital.weight)
+
+
+def test_calibration_max_sees_patches():
+    """reference tests/test_calibration.py:139-158 for AnalogConv2d: after MAX calibration the
+    range of tile t is the abs-max of the unfolded input over that tile's patch entries."""
+    from aihwkit_lightning.inference import calibrate_input_ranges, InputRangeCalibrationType
+    from aihwkit_lightning.nn import AnalogConv2d
+    from aihwkit_lightning.simulator.configs import TorchInferenceRPUConfig
+
+    cfg = TorchInferenceRPUConfig()
+    cfg.mapping.max_input_size = 10
+    layer = AnalogConv2d(3, 4, 3, stride=2, padding=1, rpu_config=cfg).cuda().eval()
+    gen = torch.Generator().manual_seed(9)
+    batches = [torch.randn(2, 3, 9, 8, generator=gen) for _ in range(4)]
+    calibrate_input_ranges(layer, InputRangeCalibrationType.MAX,
+                           iter([((b.cuda(),), {}) for b in batches]), verbose=False)
+    rows = [oc.conv_patches(b.unsqueeze(2), [1, 3, 3], [1, 2, 2], [0, 1, 1], [1, 1, 1])[0]
+            .reshape(-1, 27) for b in batches]
+    assert torch.equal(layer.input_range.data.cpu(), om.calibrate_max(rows, layer.in_sizes))
+    assert layer(batches[0].cuda()).shape == (2, 4, 5, 4)

@@ -123,3 +123,106 @@ def test_analog_optimizer_clips_after_every_step():
     assert torch.allclose(layer.weight.detach(), before - 0.1)
     opt.step()
     assert len(calls) == 2
+
+
+# ------------------------------------------------------------------ convolutions and conversion
+def test_conv_layers_tile_the_patch_dimension():
+    """nn/modules/conv.py:167-189: in_features = C * prod(kernel), split like a linear layer;
+    a 1-d layer stores a height-one 2-d kernel but saves the nn.Conv1d shape."""
+    from aihwkit_lightning.nn import AnalogConv1d, AnalogConv2d, AnalogConv3d
+
+    cfg = _cfg(max_input_size=10)
+    c1 = AnalogConv1d(3, 4, 3, padding=1, rpu_config=cfg)
+    assert c1.weight.shape == (4, 3, 1, 3) and c1.in_features == 9 and c1.in_sizes == [9]
+    assert c1.state_dict()["weight"].shape == (4, 3, 3)
+    assert c1.kernel_size == (1, 3) and c1.padding == (0, 1)
+    c2 = AnalogConv2d(3, 5, (3, 2), stride=2, rpu_config=cfg)
+    assert c2.in_features == 18 and c2.in_sizes == [9, 9] and c2.input_range.shape == (2,)
+    assert c2.upper_end_of_slices.tolist() == [9, 18]
+    c3 = AnalogConv3d(2, 5, (2, 3, 3), rpu_config=cfg)
+    assert c3.in_features == 36 and c3.in_sizes == [9, 9, 9, 9] and c3.out_features == 5
+    assert c2.geometry((2, 3, 9, 8)) == [2, 3, 1, 9, 8, 1, 3, 2, 1, 2, 2, 0, 0, 0, 1, 1, 1]
+    with pytest.raises(ValueError):
+        c2.geometry((2, 4, 9, 8))
+
+
+def test_conv_layers_reject_what_the_reference_rejects():
+    from aihwkit_lightning.nn import AnalogConv1d, AnalogConv2d, AnalogConv3d
+
+    cfg = _cfg()
+    with pytest.raises(ValueError):
+        AnalogConv2d(4, 4, 3, groups=2, rpu_config=cfg)
+    with pytest.raises(ValueError):
+        AnalogConv2d(4, 4, 3, padding_mode="reflect", rpu_config=cfg)
+    with pytest.raises(ValueError):
+        AnalogConv1d(4, 4, 3, dilation=2, rpu_config=cfg)
+    with pytest.raises(AssertionError):
+        AnalogConv3d(4, 4, 3, dilation=2, rpu_config=cfg)
+    with pytest.raises(AssertionError):
+        AnalogConv2d(4, 4, 3)
+
+
+def test_conv_output_size_in_the_library():
+    """ahl_conv_out_size is host arithmetic: it runs without a GPU."""
+    from aihwkit_lightning.exceptions import HipBackendError
+    from aihwkit_lightning.nn.modules.hip_utils.ops import conv_out_size
+
+    geom = [2, 3, 5, 9, 8, 2, 3, 3, 1, 2, 1, 1, 1, 0, 1, 1, 2]
+    want = [(5 + 2 - 1 - 1) // 1 + 1, (9 + 2 - 2 - 1) // 2 + 1, (8 - 4 - 1) // 1 + 1]
+    assert conv_out_size(geom) == want
+    with pytest.raises(HipBackendError):  # kernel larger than the padded input
+        conv_out_size([1, 1, 1, 2, 2, 1, 3, 3, 1, 1, 1, 0, 0, 0, 1, 1, 1])
+
+
+class _Net(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.conv1 = torch.nn.Conv1d(3, 3, 3, padding=1)
+        self.conv2 = torch.nn.Conv2d(3, 10, 3)
+        self.seq = torch.nn.Sequential(torch.nn.Linear(4, 5), torch.nn.ReLU(), torch.nn.Linear(5, 2))
+        self.rnn = torch.nn.GRU(4, 4)
+
+
+def test_convert_to_analog_and_back():
+    """tests/test_conversion.py of the reference: default map, empty map, in place, exclusion,
+    per-layer config hook, round trip of the weights."""
+    from aihwkit_lightning.exceptions import ArgumentError
+    from aihwkit_lightning.nn import AnalogConv1d, AnalogConv2d
+    from aihwkit_lightning.nn.conversion import convert_to_analog, convert_to_digital
+
+    model = _Net()
+    analog = convert_to_analog(model, _cfg())
+    assert isinstance(analog, AnalogWrapper)
+    assert isinstance(analog.conv1, AnalogConv1d) and isinstance(analog.conv2, AnalogConv2d)
+    assert isinstance(analog.seq, AnalogSequential) and isinstance(analog.seq[0], AnalogLinear)
+    assert isinstance(analog.rnn, torch.nn.GRU), "recurrent layers stay digital in this build"
+    assert isinstance(model.conv1, torch.nn.Conv1d), "without inplace the model is copied"
+    assert len(list(analog.analog_layers())) == 4
+    assert analog.conv1.rpu_config is not analog.conv2.rpu_config
+
+    untouched = convert_to_analog(model, _cfg(), conversion_map={})
+    assert isinstance(untouched.conv1, torch.nn.Conv1d) and isinstance(untouched, AnalogWrapper)
+    partial = convert_to_analog(model, _cfg(), exclude_modules=["seq.0", "conv2"])
+    assert isinstance(partial.conv2, torch.nn.Conv2d) and isinstance(partial.seq[0], torch.nn.Linear)
+    assert isinstance(partial.seq[2], AnalogLinear)
+
+    def per_layer(name, _module, config):
+        config.mapping.max_input_size = 2 if name == "seq.2" else 3
+        return config
+
+    tuned = convert_to_analog(model, _cfg(), specific_rpu_config_fun=per_layer)
+    assert tuned.seq[2].in_sizes == [2, 2, 1] and tuned.seq[0].in_sizes == [2, 2]
+
+    in_place = _Net()
+    convert_to_analog(in_place, _cfg(), inplace=True)
+    assert isinstance(in_place.conv1, AnalogConv1d) and isinstance(in_place.seq[2], AnalogLinear)
+
+    digital = convert_to_digital(analog)
+    assert type(digital) is _Net and isinstance(digital.conv1, torch.nn.Conv1d)
+    assert isinstance(digital.seq, torch.nn.Sequential) and isinstance(digital.seq[0], torch.nn.Linear)
+    for name, param in model.state_dict().items():
+        assert torch.equal(param, digital.state_dict()[name]), name
+    with pytest.raises(ArgumentError):
+        convert_to_analog(model, _cfg(), conversion_map=[])
+    with pytest.raises(ArgumentError):
+        convert_to_digital(analog, conversion_set=[])
