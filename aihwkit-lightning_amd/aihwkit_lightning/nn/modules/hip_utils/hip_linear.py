@@ -11,7 +11,7 @@ from torch import Tensor
 from torch.autograd import Function
 
 from . import library as L
-from .ops import OPS
+from .ops import OPS, tile_stride
 from ....exceptions import ConfigError, HipBackendError
 from ....simulator.configs import (
     TorchInferenceRPUConfig,
@@ -150,6 +150,18 @@ class HipLinear(Function):
             if w_noise or w_quant:
                 w_eff = eff
 
+        # bf16 splits whose tiles do not start on the MFMA kernels' 256-column block boundaries:
+        # the quantised input and the effective weights are kept in a padded tile layout instead
+        # (stride > 0), unless the padding would blow the work up more than the slower general
+        # kernels do, or the shape does not fit the fast backward at all
+        stride = 0
+        dense_fwd_ok = len(set(in_sizes)) == 1 and in_sizes[0] % 64 == 0
+        if (inp.dtype == torch.bfloat16 and m_rows > 0 and m_rows % 64 == 0 and n_out % 64 == 0
+                and weights_c.data_ptr() % 16 == 0):
+            stride = tile_stride(k_in, len(in_sizes), inp.dtype)
+            if stride * len(in_sizes) > 4 * k_in or (dense_fwd_ok and not (need_dx or need_dw)):
+                stride = 0
+
         skip_rounding = 1 if os.environ.get("_AIHWKIT_NO_ROUNDING", False) else 0
         icfg = [
             ir_mode, int(fwd.out_noise_per_channel),
@@ -158,6 +170,7 @@ class HipLinear(Function):
             int(training), skip_rounding, seed, 0,
             # fast_mode clamps with torch.clamp: its autograd rule instead of the learned-range one
             L.AHL_IR_GRAD_CLAMP if fast else L.AHL_IR_GRAD_LEARNED,
+            stride,
         ]
         fcfg = [
             float(fwd.inp_res), float(fwd.out_res), float(fwd.out_bound),
@@ -170,9 +183,9 @@ class HipLinear(Function):
         # bf16 with equal tiles of a multiple of 64 inputs: clamp + DAC (+ dynamic abs-max) run as
         # one memory-bound pass and the matrix kernel streams the quantised input; otherwise the
         # clamp + DAC are fused into the matrix kernel's A-tile staging.
-        split_dac = (
-            inp.dtype == torch.bfloat16 and len(set(in_sizes)) == 1 and in_sizes[0] % 64 == 0
-        )
+        split_dac = stride > 0 or (inp.dtype == torch.bfloat16 and dense_fwd_ok)
+        if stride > 0:
+            w_eff = OPS.pad_tiles(w_eff, in_sizes, stride)
         ir_dev = xq = None
         if ir_mode == L.AHL_IR_STATIC:
             if training and init_active and fast:

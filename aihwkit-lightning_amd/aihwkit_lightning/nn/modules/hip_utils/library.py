@@ -13,7 +13,7 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
@@ -49,6 +49,7 @@ class AhlLinearCfg(Structure):
         ("ir_decay", c_float),
         ("ir_input_min_percentage", c_float),
         ("ir_grad_rule", c_int32),
+        ("tile_stride", c_int32),
         ("seed", c_uint64),
         ("offset", c_uint64),
     ]
@@ -156,14 +157,20 @@ SIGNATURES = {
          c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32,
          POINTER(AhlLinearCfg), c_void_p, c_void_p],
     ),
-    "ahl_linear_bwd_dx_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32]),
+    "ahl_linear_bwd_dx_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int64]),
     "ahl_linear_bwd_dw": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
          c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32,
          POINTER(AhlLinearCfg), c_void_p, c_void_p],
     ),
-    "ahl_linear_bwd_dw_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32]),
+    "ahl_linear_bwd_dw_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32,
+                                             c_int64]),
+    "ahl_tile_stride": (c_int64, [c_int64, c_int32, c_int32]),
+    "ahl_pad_tiles": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int64, _I32P, c_int32, c_int64,
+                                c_void_p, c_int64, c_void_p]),
+    "ahl_unpad_tiles": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int64, _I32P, c_int32,
+                                  c_int64, c_void_p, c_int64, c_void_p]),
 }
 
 _LIB = None

@@ -54,6 +54,7 @@ def _linear_cfg(dtype: torch.dtype, icfg: List[int], fcfg: List[float]) -> L.Ahl
     (cfg.ir_mode, cfg.out_noise_per_channel, cfg.bound_per_channel, cfg.training,
      cfg.skip_rounding, seed, offset) = icfg[:7]
     cfg.ir_grad_rule = icfg[7] if len(icfg) > 7 else L.AHL_IR_GRAD_LEARNED
+    cfg.tile_stride = icfg[8] if len(icfg) > 8 else 0
     (cfg.inp_res, cfg.out_res, cfg.out_bound, cfg.out_noise, cfg.ir_decay,
      cfg.ir_input_min_percentage) = fcfg
     cfg.seed, cfg.offset = seed, offset
@@ -104,9 +105,42 @@ LIB.define(
     "linear_bwd_dw(Tensor g, Tensor? keep, Tensor? clamp_flag, Tensor? x, Tensor? xq, Tensor? ir, "
     "int[] in_sizes, int[] icfg, float[] fcfg, bool want_bias) -> (Tensor, Tensor)"
 )
+LIB.define("pad_tiles(Tensor x, int[] in_sizes, int stride) -> Tensor")
+LIB.define("unpad_tiles(Tensor x, int[] in_sizes, int stride) -> Tensor")
 LIB.define("im2col(Tensor x, int[] geom) -> Tensor")
 LIB.define("col2im(Tensor dcols, int[] geom) -> Tensor")
 LIB.define("transpose_batched(Tensor src) -> Tensor")
+
+
+def tile_stride(k_in: int, n_tiles: int, dtype: torch.dtype) -> int:
+    """Column stride of the padded tile layout the fast kernels want for this split, or 0 when
+    the dense layout already suits them (host arithmetic in the library)."""
+    return int(L.load().ahl_tile_stride(k_in, n_tiles, dtype_id(dtype)))
+
+
+def pad_tiles(x: Tensor, in_sizes: List[int], stride: int) -> Tensor:
+    """Dense ``[rows, K]`` to the padded tile layout ``[rows, T * stride]``."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    rows, k_in = x.shape
+    n_tiles = len(in_sizes)
+    out = torch.empty((rows, n_tiles * stride), dtype=x.dtype, device=x.device)
+    L.check(lib.ahl_pad_tiles(_ptr(x), _ld(x), dtype_id(x.dtype), rows, k_in,
+                              L.tile_ends_array(in_sizes), n_tiles, stride, _ptr(out),
+                              n_tiles * stride, _stream()), "ahl_pad_tiles")
+    return out
+
+
+def unpad_tiles(x: Tensor, in_sizes: List[int], stride: int) -> Tensor:
+    """Padded tile layout ``[rows, T * stride]`` back to dense ``[rows, K]``."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    rows, k_in, n_tiles = x.size(0), sum(in_sizes), len(in_sizes)
+    out = torch.empty((rows, k_in), dtype=x.dtype, device=x.device)
+    L.check(lib.ahl_unpad_tiles(_ptr(x), _ld(x), dtype_id(x.dtype), rows, k_in,
+                                L.tile_ends_array(in_sizes), n_tiles, stride, _ptr(out), k_in,
+                                _stream()), "ahl_unpad_tiles")
+    return out
 
 
 def conv_geom(geom: List[int]) -> L.AhlConvGeom:
@@ -404,12 +438,14 @@ def dac(x: Tensor, ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
     m_rows, k_in = x.shape
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(x.dtype, icfg, fcfg)
-    xq = torch.empty((m_rows, k_in), dtype=x.dtype, device=x.device)
+    # padded tile layout: n_tiles * stride columns per row
+    q_cols = n_tiles * cfg.tile_stride if cfg.tile_stride > 0 else k_in
+    xq = torch.empty((m_rows, q_cols), dtype=x.dtype, device=x.device)
     dynamic = cfg.ir_mode == L.AHL_IR_DYNAMIC
     ir_dyn = torch.empty((n_tiles, m_rows) if dynamic else (0,), dtype=x.dtype, device=x.device)
     L.check(
         lib.ahl_dac(
-            _ptr(x), _ld(x), _ptr(xq), k_in, _ptr(ir), _ptr(ir_dyn) if dynamic else None, m_rows,
+            _ptr(x), _ld(x), _ptr(xq), q_cols, _ptr(ir), _ptr(ir_dyn) if dynamic else None, m_rows,
             k_in, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _stream(),
         ),
         "ahl_dac",
@@ -430,7 +466,7 @@ def linear_fwd(
         x = _rows2d(x, "x")
     if xq is not None:
         xq = _rows2d(xq, "xq")
-    m_rows, k_in = ref.shape
+    m_rows, k_in = ref.size(0), sum(in_sizes)
     n_out = w_eff.size(0)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(ref.dtype, icfg, fcfg)
@@ -460,13 +496,14 @@ def linear_bwd_dx(
     lib = L.load()
     g = _rows2d(g, "g")
     m_rows, n_out = g.shape
-    k_in = w_eff.size(1)
+    k_in = sum(in_sizes)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(g.dtype, icfg, fcfg)
     static = cfg.ir_mode == L.AHL_IR_STATIC
     dx = torch.empty((m_rows, k_in), dtype=g.dtype, device=g.device)
     ir_grad = torch.empty((n_tiles,) if static else (0,), dtype=g.dtype, device=g.device)
-    ws = torch.empty((lib.ahl_linear_bwd_dx_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype),),
+    ws = torch.empty((lib.ahl_linear_bwd_dx_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype,
+                                                     cfg.tile_stride),),
                      dtype=torch.uint8, device=g.device)
     if x is not None:
         x = _rows2d(x, "x")
@@ -497,13 +534,13 @@ def linear_bwd_dw(
     if xq is not None:
         xq = _rows2d(xq, "xq")
     m_rows, n_out = g.shape
-    k_in = ref.size(1)
+    k_in = sum(in_sizes)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(g.dtype, icfg, fcfg)
     dw = torch.empty((n_out, k_in), dtype=g.dtype, device=g.device)
     dbias = torch.empty((n_out,) if want_bias else (0,), dtype=g.dtype, device=g.device)
     ws_bytes = lib.ahl_linear_bwd_dw_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype,
-                                              0 if keep is None else 1)
+                                              0 if keep is None else 1, cfg.tile_stride)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=g.device)
     L.check(
         lib.ahl_linear_bwd_dw(
@@ -523,6 +560,7 @@ for _name, _fn in [
     ("clip_weights", clip_weights), ("col_sum", col_sum),
     ("weight_prep", weight_prep), ("quantize_weights", quantize_weights),
     ("weight_prep_clip", weight_prep_clip), ("learned_clip_bwd", learned_clip_bwd),
+    ("pad_tiles", pad_tiles), ("unpad_tiles", unpad_tiles),
     ("im2col", im2col), ("col2im", col2im), ("transpose_batched", transpose_batched),
     ("dac", dac), ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
 ]:

@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void k_dac_rows(const void* __restrict__ x, in
                                                   const void* __restrict__ ir_in,
                                                   void* __restrict__ ir_out, int64_t M, Tiling tl,
                                                   float inp_res, int32_t dac_on,
-                                                  int32_t skip_rounding) {
+                                                  int32_t skip_rounding, int32_t qstride) {
   const int lane = threadIdx.x & 63;
   const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (m >= M) return;
@@ -62,17 +62,31 @@ __global__ __launch_bounds__(256) void k_dac_rows(const void* __restrict__ x, in
       if (dac_on) return dac_apply<D, IRMODE == AHL_IR_STATIC, true>(v, dac, skip_rounding != 0);
       return dac_apply<D, IRMODE == AHL_IR_STATIC, false>(v, dac, false);
     };
+    // padded tile layout (qstride > 0): tile t of xq starts at column t * qstride and is
+    // zero-filled up to the next tile
+    typename D::elem* qt = qstride > 0 ? qrow + ((int64_t)t * qstride - c0) : qrow;
     if (VEC) {  // tile bounds are multiples of E on this path
       for (int32_t v = c0 / E + lane; v < c1 / E; v += 64) {
         float e[E];
         D::unpack(ld16(row + (int64_t)v * E), e);
 #pragma unroll
         for (int i = 0; i < E; ++i) e[i] = f(e[i]);
-        st16(qrow + (int64_t)v * E, D::pack(e));
+        st16(qt + (int64_t)v * E, D::pack(e));
       }
     } else {
-      for (int32_t c = c0 + lane; c < c1; c += 64) D::store(qrow, c, f(D::load(row, c)));
+      // element-wise, four independent loads per lane and pass
+      int32_t c = c0 + lane;
+      for (; c + 192 < c1; c += 256) {
+        float e[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) e[i] = D::load(row, c + 64 * i);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) D::store(qt, c + 64 * i, f(e[i]));
+      }
+      for (; c < c1; c += 64) D::store(qt, c, f(D::load(row, c)));
     }
+    if (qstride > 0)
+      for (int32_t c = c1 + lane; c < c0 + qstride; c += 64) D::store(qt, c, 0.0f);
   }
 }
 
@@ -88,7 +102,8 @@ struct FastFwdArgs {
   const void* wmax;              // [T, N]
   const float* tile_max;         // [T]
   int64_t M, N;
-  int32_t K, tile;               // all tiles have `tile` columns (multiple of 64)
+  int32_t tile;                  // columns of a tile that hold data, rounded up to 64
+  int32_t tile_stride;           // columns from one tile start to the next (>= tile)
   int32_t n_tiles;
   float out_bound, out_res, two_inv_res;
   float noise_scale;
@@ -182,7 +197,11 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
       rawB[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsB, voB[j], kc * 2, 0));
   };
   load(0);
-  const int nchunks = a.K / 64, cpt = a.tile / 64;
+  const int cpt = a.tile / 64, nchunks = a.n_tiles * cpt;
+  // k offset of the chunk after the one being loaded: next 64 columns, or the next tile's start
+  int32_t knext = 64;
+  int lcin = 1;  // position inside its tile of the chunk at knext
+  if (lcin == cpt) { lcin = 0; knext = a.tile_stride; }
   int t = 0, cin = 0;
   // registers -> LDS for the chunk held in rawA/rawB; `tt` is its K-tile, `first` whether it
   // opens that tile (then the dynamic-mode per-row constants of the tile are written too)
@@ -207,7 +226,11 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
   for (int ch = 0; ch < nchunks; ++ch) {
     if (!prestaged) stage(t, cin == 0);
     prestaged = false;
-    if (ch + 1 < nchunks) load((ch + 1) * 64);
+    if (ch + 1 < nchunks) {
+      load(knext);
+      knext += 64;
+      if (++lcin == cpt) { lcin = 0; knext += a.tile_stride - a.tile; }
+    }
 
     {
       const int r = lane & 31;
@@ -443,8 +466,13 @@ namespace ahl {
 bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, const void* w,
                        int64_t ldw, int64_t K, const Tiling& tl) {
   if (cfg->dtype != AHL_BF16 || xq == nullptr) return false;
-  if (tl.extra != 0 || tl.base % 64 != 0) return false;
   if (!aligned16(xq) || !aligned16(w) || ldxq % 8 != 0 || ldw % 8 != 0) return false;
+  if (cfg->tile_stride > 0) {  // padded tile layout: any split
+    const int64_t padded = (int64_t)tl.n_tiles * cfg->tile_stride;
+    return cfg->tile_stride % 256 == 0 && cfg->tile_stride >= widest_tile(tl) && ldxq >= padded &&
+           ldw >= padded && padded <= 0x3fffffff;
+  }
+  if (tl.extra != 0 || tl.base % 64 != 0) return false;
   return K % 64 == 0;  // the caller also checks N % 8, ldy % 8 and the alignment of y and the clamp mask
 }
 
@@ -455,7 +483,15 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   FastFwdArgs a;
   a.xq = xq; a.ldx = ldxq; a.w = w_eff; a.ldw = ldw; a.bias = bias; a.y = y; a.ldy = ldy;
   a.keep = keep; a.clamp_flag = clamp_flag; a.ir = ir; a.wmax = wmax; a.tile_max = tile_max;
-  a.M = M; a.N = N; a.K = (int32_t)K; a.tile = tl.base; a.n_tiles = tl.n_tiles;
+  a.M = M; a.N = N; a.n_tiles = tl.n_tiles;
+  if (cfg->tile_stride > 0) {  // padded tile layout: only the chunks that hold data are visited
+    a.tile = (int32_t)cdiv(widest_tile(tl), 64) * 64;
+    a.tile_stride = cfg->tile_stride;
+  } else {
+    a.tile = tl.base;
+    a.tile_stride = tl.base;
+  }
+  (void)K;
   a.out_bound = cfg->out_bound; a.out_res = cfg->out_res;
   const bool noise = cfg->training && cfg->out_noise > 0.0f;
   const bool adc = cfg->out_res > 0.0f;
@@ -480,7 +516,7 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
 
 #define AHL_DAC(V, I)                                                                          \
   hipLaunchKernelGGL((k_dac_rows<D, V, I>), grid, block, 0, s, x, ldx, xq, ldxq, ir_in, ir_out, M, \
-                     tl, cfg->inp_res, dac_on, cfg->skip_rounding)
+                     tl, cfg->inp_res, dac_on, cfg->skip_rounding, qstride)
 
 extern "C" {
 
@@ -493,6 +529,9 @@ int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_i
   if (cfg->ir_mode == AHL_IR_NONE && cfg->inp_res > 0.0f) return AHL_ERR_ARG;
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
+  const int32_t qstride = cfg->tile_stride;
+  if (qstride < 0 || qstride % 256 != 0) return AHL_ERR_ARG;
+  if (qstride > 0 && (qstride < widest_tile(tl) || ldxq < (int64_t)n_tiles * qstride)) return AHL_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)cdiv(M, 4)), block(256);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;

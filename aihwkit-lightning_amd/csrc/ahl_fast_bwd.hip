@@ -47,6 +47,10 @@ struct BwdArgs {
   int64_t M, N, K;
   int32_t tile;                        // K-tile width (multiple of 256)
   int32_t ir_static;                   // 0: no range gradient; 1 + AHL_IR_GRAD_* otherwise
+  int32_t slices;                      // DW: the contraction (rows m) is cut into this many
+                                       // slices, one block each; > 1 when N x K alone gives
+                                       // too few blocks to fill the chip
+  float* split;                        // slices > 1: fp32 partial results [slices][N][K]
 };
 
 AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
@@ -64,9 +68,10 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
 
   // ---- block -> output tile. columns of the output are k (both modes), 256 per block ----
   const int64_t nkb = a.K / 256;
-  const int64_t nb = gridDim.x;
+  const int64_t nb = gridDim.x / a.slices;            // output tiles
+  const int slice = (int)(blockIdx.x / nb);
   int64_t brow, bcol;
-  block_to_tile(blockIdx.x, nb, nb / nkb, nkb, 4, brow, bcol);
+  block_to_tile(blockIdx.x % nb, nb, nb / nkb, nkb, 4, brow, bcol);
   const int64_t r0 = brow * 256;                     // DX: m0; DW: n0
   const int64_t c0 = bcol * 256;                     // k0
   const int t = (int)(c0 / a.tile);
@@ -121,6 +126,19 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   const int64_t a_step = MODE == MODE_DX ? 64 : 64 * a.ldg;
   const int64_t k_step = MODE == MODE_DX ? 2 * a.M : 64;   // 64 columns = 2 words; or 64 rows
   const int64_t b_step = 64 * a.ldb;
+  // this block's share of the contraction: chunks [ch0, ch0 + nchunks)
+  const int chunks_all = (int)(L / 64);
+  const int per_slice = (chunks_all + a.slices - 1) / a.slices;
+  const int ch0 = slice * per_slice;
+  const int nchunks = chunks_all - ch0 < per_slice ? chunks_all - ch0 : per_slice;
+  if (ch0 > 0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      pa[j] += (int64_t)ch0 * a_step;
+      pb[j] += (int64_t)ch0 * b_step;
+    }
+    if (pk) pk += (int64_t)ch0 * k_step;
+  }
   auto load = [&](bool masked) {
     if (masked) { rawK = ld16(pk); pk += k_step; }
 #pragma unroll
@@ -179,12 +197,11 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     }
     __syncthreads();
   }
-  const int nchunks = (int)(L / 64);
   auto main_loop = [&](auto masked_tag, auto bias_tag) {
     constexpr bool kMasked = decltype(masked_tag)::value;
     constexpr bool kBias = decltype(bias_tag)::value;
     load(kMasked);
-    stage(lds, lds + kOperandLds, kMasked, kBias && kb_idx == 0);
+    stage(lds, lds + kOperandLds, kMasked, kBias && ch0 % (int)nkb == kb_idx);
     __syncthreads();
     for (int ch = 0; ch < nchunks; ++ch) {
       const char* sa = lds + (ch & 1) * 2 * kOperandLds;
@@ -209,7 +226,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       }
       if (ch + 1 < nchunks) {
         char* na = lds + ((ch + 1) & 1) * 2 * kOperandLds;
-        stage(na, na + kOperandLds, kMasked, kBias && (ch + 1) % (int)nkb == kb_idx);
+        stage(na, na + kOperandLds, kMasked, kBias && (ch0 + ch + 1) % (int)nkb == kb_idx);
       }
       __syncthreads();
     }
@@ -227,12 +244,29 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       float sum = 0.0f;
 #pragma unroll
       for (int r = 0; r < 16; ++r) sum += bred[r * 256 + tid];
-      a.bias_partial[(int64_t)kb_idx * a.N + r0 + tid] = sum;
+      a.bias_partial[((int64_t)slice * nkb + kb_idx) * a.N + r0 + tid] = sum;
     }
     __syncthreads();
   } else {
     if (plane) main_loop(std::true_type{}, std::false_type{});
     else main_loop(std::false_type{}, std::false_type{});
+  }
+
+  if (MODE == MODE_DW && a.slices > 1) {
+    // partial result of this slice, fp32, straight from the accumulators: for fixed (bi, bj, v)
+    // the 32 lanes of a half wave write 128 contiguous bytes of one row
+    float* sp = a.split + ((int64_t)slice * a.N) * a.K;
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t row = r0 + wm * 128 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (row >= R) continue;
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+          sp[row * a.K + c0 + wn * 64 + bj * 32 + (lane & 31)] = acc[bi][bj][v];
+      }
+    return;
   }
 
   // ---- epilogue: the 256 x 256 result goes through LDS (the operand buffers are free after
@@ -309,6 +343,19 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   }
 }
 
+// out[r, c] = bf16(sum over slices of split[s][r][c]), slices added in order
+__global__ __launch_bounds__(256) void k_split_reduce(const float* __restrict__ split, int slices,
+                                                      int64_t R, int64_t K, uint16_t* __restrict__ out,
+                                                      int64_t ldo) {
+  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (idx >= R * K) return;
+  const int64_t r = idx / K, c = idx - r * K;  // K is a multiple of 256: the 4 share a row
+  f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < slices; ++s) sum += *(const f32x4*)(split + (int64_t)s * R * K + idx);
+  u32x2 pk = {pack_bf16x2(sum.x, sum.y), pack_bf16x2(sum.z, sum.w)};
+  *(u32x2*)(out + r * ldo + c) = pk;
+}
+
 __global__ __launch_bounds__(256) void k_bias_final(const float* partial, int nkb, int64_t N,
                                                     uint16_t* dbias) {
   const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -337,6 +384,7 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
   a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = ir_static;
+  a.slices = 1; a.split = nullptr;
   const int64_t nb = cdiv(M, 256) * (K / 256);
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
@@ -344,23 +392,53 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   return check_launch("ahl_linear_bwd_dx(fast)");
 }
 
+// Slices of the contraction for the weight gradient: N x K / 65536 output tiles are too few to
+// fill 256 CUs when the layer is narrow (a convolution with many patches and few channels), so
+// the rows m are cut until there are about 256 blocks, each with at least 8 chunks of 64 rows.
+int fast_dw_slices(int64_t M, int64_t K, int64_t N) {
+  const int64_t tiles = cdiv(N, 256) * (K / 256);
+  if (tiles >= 128) return 1;
+  int64_t s = cdiv(256, tiles);
+  const int64_t chunks = M / 64, most = chunks / 8;
+  if (s > most) s = most;
+  if (s <= 1) return 1;
+  // every slice gets ceil(chunks / s) chunks; drop the slices that would be left empty
+  return (int)cdiv(chunks, cdiv(chunks, s));
+}
+
+// Workspace of launch_fast_dw: [partial bias sums: slices x K/256 x N floats | slices > 1:
+// partial results slices x N x K floats]
+int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N) {
+  const int64_t slices = fast_dw_slices(M, K, N);
+  const int64_t bias = (slices * (K / 256) * N * 4 + 255) / 256 * 256;
+  return bias + (slices > 1 ? slices * N * K * 4 : 0);
+}
+
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
-                   float* bias_partial, int64_t M, int64_t K, int64_t N, const Tiling& tl,
+                   void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
                    hipStream_t s) {
   BwdArgs a;
+  const int slices = fast_dw_slices(M, K, N);
+  float* bias_partial = (float*)ws;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
   a.b = (const uint16_t*)xq; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;
   a.out = (uint16_t*)dw; a.ldo = lddw; a.partial = nullptr;
   a.bias_partial = dbias ? bias_partial : nullptr;
   a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = 0;
-  const int64_t nb = cdiv(N, 256) * (K / 256);
+  a.slices = slices;
+  a.split = slices > 1
+      ? (float*)((char*)ws + ((int64_t)slices * (K / 256) * N * 4 + 255) / 256 * 256) : nullptr;
+  const int64_t nb = cdiv(N, 256) * (K / 256) * slices;
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
   hipLaunchKernelGGL((k_bwd_fast<MODE_DW>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  if (slices > 1)
+    hipLaunchKernelGGL(k_split_reduce, dim3((unsigned)cdiv(N * K, 1024)), dim3(256), 0, s,
+                       (const float*)a.split, slices, N, K, (uint16_t*)dw, lddw);
   if (dbias)
     hipLaunchKernelGGL(k_bias_final, dim3((unsigned)cdiv(N, 256)), dim3(256), 0, s,
-                       (const float*)bias_partial, (int)(K / 256), N, (uint16_t*)dbias);
+                       (const float*)bias_partial, (int)(K / 256) * slices, N, (uint16_t*)dbias);
   return check_launch("ahl_linear_bwd_dw(fast)");
 }
 

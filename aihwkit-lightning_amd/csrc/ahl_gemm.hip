@@ -683,6 +683,7 @@ static bool cfg_ok(const AhlLinearCfg* c) {
   if (c->dtype != AHL_F32 && c->dtype != AHL_BF16) return false;
   if (c->ir_mode < 0 || c->ir_mode > 2) return false;
   if (c->ir_grad_rule != AHL_IR_GRAD_LEARNED && c->ir_grad_rule != AHL_IR_GRAD_CLAMP) return false;
+  if (c->tile_stride < 0 || c->tile_stride % 256 != 0) return false;
   return true;
 }
 
@@ -701,8 +702,13 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
                    const Tiling& tl, int ir_static, hipStream_t s);
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
-                   float* bias_partial, int64_t M, int64_t K, int64_t N, const Tiling& tl,
+                   void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
                    hipStream_t s);
+int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N);
+int launch_pad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows, const Tiling& tl,
+                     int64_t stride, void* dst, int64_t ld_dst, hipStream_t s);
+int launch_unpad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows, int64_t K,
+                       const Tiling& tl, int64_t stride, void* dst, int64_t ld_dst, hipStream_t s);
 }  // namespace ahl
 
 template <class D>
@@ -762,7 +768,8 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
       aligned16(y) && (!keep || (((uintptr_t)keep) & 3u) == 0))
     return launch_fast_fwd(xq, ldxq, w_eff, ldw, bias, y, ldy, keep, clamp_flag, ir, wmax, tile_max,
                            M, K, N, tl, cfg, (hipStream_t)stream);
-  if (!x) return AHL_ERR_UNSUPPORTED;  // only the fast path can start from xq alone
+  // only the fast path can start from xq alone or read the padded tile layout
+  if (!x || cfg->tile_stride > 0) return AHL_ERR_UNSUPPORTED;
   FwdArgs a;
   a.x = x; a.ldx = ldx; a.w = w_eff; a.ldw = ldw; a.bias = bias; a.y = y; a.ldy = ldy;
   a.keep = keep; a.ir = ir; a.wmax = wmax; a.tile_max = tile_max; a.M = M; a.N = N; a.tl = tl;
@@ -805,9 +812,19 @@ static int64_t dx_partial_bytes(int64_t M, int64_t K, int32_t n_tiles) {
   return align256(cdiv(M, kBM) * nkb * 4 * (int64_t)sizeof(float));
 }
 
-int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype) {
+// Workspace of the padded-layout backward: [partials | x padded | dx padded]
+static int64_t dx_padded_partial_bytes(int64_t M, int64_t padded) {
+  return align256(cdiv(M, 256) * (padded / 256) * 4 * (int64_t)sizeof(float));
+}
+
+int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
+                                   int64_t tile_stride) {
   if (n_tiles <= 0 || K <= 0 || M <= 0 || N <= 0) return 0;
   const int64_t es = dtype == AHL_BF16 ? 2 : 4;
+  if (tile_stride > 0) {
+    const int64_t padded = (int64_t)n_tiles * tile_stride;
+    return dx_padded_partial_bytes(M, padded) + 2 * align256(M * padded * es);
+  }
   return dx_partial_bytes(M, K, n_tiles) + align256(K * N * es);  // partials + transposed weights
 }
 
@@ -825,6 +842,35 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
   float* partial = (float*)ws;
+  if (cfg->tile_stride > 0) {
+    // w_eff is in the padded tile layout: pad x, run the MFMA kernel on aligned tiles of
+    // `stride` columns, copy the data columns of the result into the dense dx
+    const int64_t stride = cfg->tile_stride, padded = (int64_t)n_tiles * stride;
+    if (stride < widest_tile(tl) || ldw < padded || padded > 0x3fffffff) return AHL_ERR_ARG;
+    if (cfg->dtype != AHL_BF16 || M % 64 != 0 || N % 64 != 0 || !aligned16(g) || !aligned16(w_eff) ||
+        ldg % 8 != 0 || ldw % 8 != 0 || (keep && !aligned16(keep)))
+      return AHL_ERR_UNSUPPORTED;
+    char* p = (char*)ws + dx_padded_partial_bytes(M, padded);
+    void* xpad = p;
+    void* dxp = p + align256(M * padded * 2);
+    int rc;
+    if (is_static) {
+      rc = launch_pad_tiles(x, ldx, AHL_BF16, M, tl, stride, xpad, padded, s);
+      if (rc != AHL_OK) return rc;
+    }
+    const Tiling ptl{n_tiles, (int32_t)stride, 0};
+    rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, xpad, padded, ir, dxp, padded, partial,
+                        M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0, s);
+    if (rc != AHL_OK) return rc;
+    if (is_static) {
+      const int32_t per_tile = (int32_t)(stride / 256);
+      hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
+                         (const float*)partial, cdiv(M, 256), (int32_t)(padded / 256), per_tile,
+                         per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
+                         cfg->ir_grad_rule);
+    }
+    return launch_unpad_tiles(dxp, padded, AHL_BF16, M, K, tl, stride, dx, lddx, s);
+  }
   void* wt = (char*)ws + dx_partial_bytes(M, K, n_tiles);
   const bool fast = fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(w_eff) &&
                     ldg % 8 == 0 && ldw % 8 == 0 && lddx % 8 == 0 && aligned16(dx) &&
@@ -871,13 +917,15 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
 
 
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
-                                   int32_t has_keep) {
+                                   int32_t has_keep, int64_t tile_stride) {
   const int64_t es = dtype == AHL_BF16 ? 2 : 4;
-  (void)n_tiles;
   (void)has_keep;
-  // the fast path only uses [K / 256][N] floats of partial bias sums at the start of ws
+  if (tile_stride > 0) {  // [workspace of the MFMA kernel | dw in the padded tile layout]
+    const int64_t padded = (int64_t)n_tiles * tile_stride;
+    return align256(fast_dw_ws_bytes(M, padded, N)) + align256(N * padded * es);
+  }
   const int64_t generic = align256(N * M * es) + align256(K * M * es) + align256(ahl_col_sum_ws_bytes(N));
-  const int64_t fast = align256(cdiv(K, 256) * N * (int64_t)sizeof(float));
+  const int64_t fast = K % 256 == 0 ? align256(fast_dw_ws_bytes(M, K, N)) : 0;
   return generic > fast ? generic : fast;
 }
 
@@ -893,9 +941,24 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
   Tiling tl;
   if (!make_tiling(tile_ends_host, n_tiles, K, &tl)) return AHL_ERR_TILING;
   hipStream_t s = (hipStream_t)stream;
+  if (cfg->tile_stride > 0) {
+    // xq is in the padded tile layout: the MFMA kernel writes dw in the same layout into the
+    // workspace, then the data columns are copied into the dense dw
+    const int64_t stride = cfg->tile_stride, padded = (int64_t)n_tiles * stride;
+    if (!xq || stride < widest_tile(tl) || ldxq < padded || padded > 0x3fffffff) return AHL_ERR_ARG;
+    if (cfg->dtype != AHL_BF16 || M % 64 != 0 || N % 64 != 0 || !aligned16(g) || !aligned16(xq) ||
+        ldg % 8 != 0 || ldxq % 8 != 0 || (keep && !aligned16(keep)))
+      return AHL_ERR_UNSUPPORTED;
+    void* dwp = (char*)ws + align256(fast_dw_ws_bytes(M, padded, N));
+    const Tiling ptl{n_tiles, (int32_t)stride, 0};
+    const int rc = launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dwp, padded, dbias, ws, M,
+                                  padded, N, ptl, s);
+    if (rc != AHL_OK) return rc;
+    return launch_unpad_tiles(dwp, padded, AHL_BF16, N, K, tl, stride, dw, lddw, s);
+  }
   if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
       ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && aligned16(dw) && (!keep || aligned16(keep)))
-    return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, dbias, (float*)ws, M, K, N, tl, s);
+    return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, dbias, ws, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
   DwArgs a;
   a.M = M; a.N = N; a.K = K; a.tl = tl; a.dw = dw; a.lddw = lddw;

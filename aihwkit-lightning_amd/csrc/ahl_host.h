@@ -31,6 +31,9 @@ inline bool make_tiling(const int32_t* ends, int32_t n_tiles, int64_t K, Tiling*
   return true;
 }
 
+// Columns of the widest tile of a split (host side; Tiling's own accessors are device code).
+inline int32_t widest_tile(const Tiling& tl) { return tl.base + (tl.extra > 0 ? 1 : 0); }
+
 // Round-to-nearest-even of a float to bfloat16 precision, on the host.
 inline float host_round_bf16(float x) {
   uint32_t u;

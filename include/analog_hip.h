@@ -81,6 +81,8 @@ typedef struct AhlLinearCfg {
   float ir_decay;                /* pre_post.input_range.decay                                  */
   float ir_input_min_percentage; /* pre_post.input_range.input_min_percentage                   */
   int32_t ir_grad_rule;          /* AHL_IR_GRAD_*: which backward the static range clamp has     */
+  int32_t tile_stride;           /* 0: xq and w_eff are dense [rows, K]. > 0: they are in the
+                                    padded tile layout with this stride (see ahl_tile_stride)    */
   uint64_t seed;                 /* Philox key for this call                                    */
   uint64_t offset;               /* Philox counter offset for this call                         */
 } AhlLinearCfg;
@@ -99,6 +101,31 @@ typedef struct AhlModifierCfg {
   uint64_t seed;
   uint64_t offset;
 } AhlModifierCfg;
+
+/* ---- padded tile layout ------------------------------------------------------------------
+ * The MFMA kernels of the bf16 path want every K-tile to start on a 256-column boundary. The
+ * reference's split rule (nn/modules/linear.py:155-170) gives that only for some shapes
+ * (4096 inputs in tiles of 512 do, 11008 in tiles of 512 or 2304 in tiles of 576 do not). For
+ * the others the two operands the library produces itself -- the quantised input xq (ahl_dac)
+ * and the effective weights w_eff -- can be kept in a padded layout: tile t starts at column
+ * t * tile_stride, holds its size(t) columns and is zero up to the next tile; a row has
+ * n_tiles * tile_stride columns. Zeros add nothing to any product, so results do not change.
+ * Tensors the caller owns (x, y, dx, dw) stay dense.                                          */
+
+/* The stride the fast kernels want for this split: 0 if the dense layout already suits them or
+ * the dtype has no fast kernels, else ceil(K / n_tiles) rounded up to a multiple of 256.       */
+int64_t ahl_tile_stride(int64_t K, int32_t n_tiles, int32_t dtype);
+
+/* dst[r, t * tile_stride + j] = src[r, start(t) + j] for j < size(t), 0 for the rest of the
+ * stride; src dtype [rows, K] (row stride ld_src), dst dtype [rows, n_tiles * tile_stride].    */
+int ahl_pad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows, int64_t K,
+                  const int32_t* tile_ends_host, int32_t n_tiles, int64_t tile_stride, void* dst,
+                  int64_t ld_dst, void* stream);
+
+/* The inverse copy: dst[r, start(t) + j] = src[r, t * tile_stride + j].                        */
+int ahl_unpad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows, int64_t K,
+                    const int32_t* tile_ends_host, int32_t n_tiles, int64_t tile_stride, void* dst,
+                    int64_t ld_dst, void* stream);
 
 /* ---- library ------------------------------------------------------------------------------ */
 
@@ -199,7 +226,9 @@ int ahl_quantize_weights(void* w, int64_t N, int64_t K, int64_t ld, const int32_
  *   AHL_IR_DYNAMIC: ir_out[t, m] = max_k |x[m, tile t]| (dtype [T, M]), xq = DAC(x) with it
  *   AHL_IR_NONE   : xq = x
  * Replaces torch_utils/torch_linear.py:155-192 (apply_input_range forward, dynamic abs-max,
- * UniformQuantize of the input). ahl_linear_fwd accepts the result as `xq`.               */
+ * UniformQuantize of the input). ahl_linear_fwd accepts the result as `xq`.
+ * With cfg->tile_stride > 0 xq is written in the padded tile layout (ldxq >= n_tiles *
+ * tile_stride), padding zeroed.                                                            */
 int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_in, void* ir_out,
             int64_t M, int64_t K, const int32_t* tile_ends_host, int32_t n_tiles,
             const AhlLinearCfg* cfg, void* stream);
@@ -210,7 +239,9 @@ int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_i
  *   bias added last.
  *   x        dtype [M, K] raw input; the clamp + DAC then run fused in the A-tile staging.
  *   xq       dtype [M, K] from ahl_dac, or NULL. bf16 calls whose tiles are equal multiples of
- *            64 take a faster kernel when xq is given (x may then be NULL).
+ *            64 take a faster kernel when xq is given (x may then be NULL); with
+ *            cfg->tile_stride > 0, xq and w_eff are in the padded tile layout and every split
+ *            takes that kernel (bf16 only; AHL_ERR_UNSUPPORTED otherwise).
  *   ir       dtype [T] (AHL_IR_STATIC) or [T, M] (AHL_IR_DYNAMIC) or NULL (AHL_IR_NONE)
  *   wmax     dtype [T, N] from ahl_weight_prep, or NULL when neither noise nor bound is on
  *   tile_max float [T]    from ahl_weight_prep, or NULL likewise
@@ -235,14 +266,17 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
  *                  dx zeroed where |x| > ir[t]; x[M, K] is the forward input.
  *   otherwise dx = d, ir_grad untouched.
  *   clamp_flag: NULL, or the flag written by ahl_linear_fwd (the mask is ignored when it reads 0).
- *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, N, n_tiles, dtype) bytes.
+ *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, N, n_tiles, dtype, cfg->tile_stride) bytes.
+ *   With cfg->tile_stride > 0, w_eff is in the padded tile layout (x and dx stay dense; the
+ *   call pads and un-pads them inside the workspace); needs bf16 and M, N multiples of 64.
  * Slot of TritonLinear.backward, triton_utils/triton_linear.py:695-764.                  */
 int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* clamp_mask, const uint32_t* clamp_flag,
                       const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                       void* dx, int64_t lddx, void* ir_grad, int64_t M, int64_t K, int64_t N,
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
-int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype);
+int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
+                                   int64_t tile_stride);
 
 /* Backward of the learnable weight clip (UniformQuantize.backward with learn_res,
  * torch_utils/quant_utils.py:123-153, as called from clip_and_quantize :184-233).
@@ -263,7 +297,9 @@ int ahl_learned_clip_bwd(void* dw, int64_t lddw, const void* w, int64_t ldw, con
  *   dbias: dtype [N] or NULL; receives the bias gradient sum_m g[m, :] (the autograd of the
  *   bias addition in AnalogLinear.forward, nn/modules/linear.py:120-135), which the kernel
  *   gets for free while it streams g.
- *   ws needs ahl_linear_bwd_dw_ws_bytes(M, K, N, n_tiles, dtype, clamp_mask != NULL) bytes
+ *   With cfg->tile_stride > 0, xq is in the padded tile layout (dw stays dense).
+ *   ws needs ahl_linear_bwd_dw_ws_bytes(M, K, N, n_tiles, dtype, clamp_mask != NULL,
+ *   cfg->tile_stride) bytes
  *   (transposed staging copies of g and the quantised input).
  * Same reference slot as ahl_linear_bwd_dx.                                               */
 int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* clamp_mask, const uint32_t* clamp_flag,
@@ -272,7 +308,7 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* clamp_mask, co
                       const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg,
                       void* ws, void* stream);
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
-                                   int32_t has_mask);
+                                   int32_t has_mask, int64_t tile_stride);
 
 /* ---- convolution as the same matrix product (nn/modules/conv.py:121-367) -------------------
  * A convolution layer of the reference unfolds its input into patches, runs the AnalogLinear

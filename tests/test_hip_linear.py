@@ -87,6 +87,28 @@ SHAPES = [
     case("vec_f32_plain", M=200, K=256, N=136, max_input_size=-1, seed=26),
     case("one_token_bf16", dtype="bf16", M=1, K=512, N=512, max_input_size=256, ir_mode="static",
          inp_res=254, out_res=254, out_bound=10.0, seed=27),
+    # splits whose tiles do not start on 256-column boundaries: padded tile layout of xq / w_eff
+    case("pad_bf16_uneven_clamped", dtype="bf16", M=256, K=1000, N=128, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
+         w_scale=0.1, seed=31),
+    case("pad_bf16_extra_tiles", dtype="bf16", M=192, K=1003, N=64, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=10.0, clip="channel", clip_sigma=2.5,
+         ir_decay=0.01, ir_values=[1.5, 2.0, 2.5, 3.0], seed=32),
+    case("pad_bf16_576_dynamic", dtype="bf16", M=128, K=1152, N=192, max_input_size=576,
+         ir_mode="dynamic", inp_res=254, out_res=254, out_bound=0.3, w_scale=0.1, seed=33),
+    case("pad_bf16_plain", dtype="bf16", M=64, K=300, N=64, max_input_size=128, seed=34),
+    case("pad_bf16_fast_mode", dtype="bf16", M=128, K=520, N=64, max_input_size=256, ir_mode="fast",
+         ir_values=[0.8, 2.5, 1.5], inp_res=254, out_res=254, out_bound=1.5, clip="channel",
+         clip_sigma=2.5, w_scale=0.3, seed=35),
+    # narrow layers with many rows: the weight-gradient kernel cuts the rows into slices
+    case("sliced_dw_bf16_clamped", dtype="bf16", M=1536, K=512, N=128, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
+         w_scale=0.1, seed=37),
+    case("pad_bf16_sliced_dw", dtype="bf16", M=1088, K=1000, N=64, max_input_size=256,
+         ir_mode="dynamic", inp_res=254, out_res=254, out_bound=0.3, w_scale=0.1, seed=38),
+    case("pad_bf16_lsq", dtype="bf16", M=64, K=200, N=64, max_input_size=100, ir_mode="static",
+         clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30,
+         w_scale=0.3, inp_res=254, out_res=254, out_bound=10.0, seed=36),
 ]
 
 
@@ -183,3 +205,32 @@ def test_weight_noise_statistics(kind):
         assert abs(float(z.std()) - 1.0) < 0.01
     # the forward used the same noisy weights
     assert torch.allclose(out.detach().cpu(), x @ w_eff.T, atol=1e-4)
+
+
+@pytest.mark.parametrize("c", [c for c in SHAPES if c["name"].startswith("pad_")],
+                         ids=lambda c: c["name"])
+def test_padded_layout_is_what_runs(c):
+    """The pad_* shapes must actually take the padded tile layout (a non-zero stride from the
+    library), or the cases above would only exercise the general kernels."""
+    from aihwkit_lightning.nn.modules.hip_utils.ops import tile_stride
+
+    n_tiles = len(om.split_sizes(c["K"], c["max_input_size"]))
+    stride = tile_stride(c["K"], n_tiles, torch.bfloat16)
+    assert stride > 0 and stride % 256 == 0 and stride * n_tiles <= 4 * c["K"]
+    assert c["M"] % 64 == 0 and c["N"] % 64 == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("rows,k_in,max_size", [(5, 1003, 256), (64, 300, 128), (3, 7, 2), (130, 2304, 576)])
+def test_pad_unpad_tiles_bit_exact(rows, k_in, max_size, dtype):
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+
+    sizes = om.split_sizes(k_in, max_size)
+    stride = (max(sizes) + 255) // 256 * 256
+    x = torch.randn(rows, k_in, generator=torch.Generator().manual_seed(5)).to(dtype)
+    want = torch.zeros(rows, len(sizes) * stride, dtype=dtype)
+    for t, (lo, hi) in enumerate(om.tile_bounds(sizes)):
+        want[:, t * stride:t * stride + hi - lo] = x[:, lo:hi]
+    padded = OPS.pad_tiles(x.cuda(), sizes, stride)
+    assert torch.equal(padded.cpu(), want)
+    assert torch.equal(OPS.unpad_tiles(padded, sizes, stride).cpu(), x)

@@ -226,3 +226,16 @@ def test_convert_to_analog_and_back():
         convert_to_analog(model, _cfg(), conversion_map=[])
     with pytest.raises(ArgumentError):
         convert_to_digital(analog, conversion_set=[])
+
+
+def test_tile_stride_rule():
+    """Host arithmetic of the library: aligned splits stay dense, others get a stride that is a
+    multiple of 256 and holds the widest tile; fp32 has no padded layout."""
+    from aihwkit_lightning.nn.modules.hip_utils.ops import tile_stride
+
+    assert tile_stride(4096, 8, torch.bfloat16) == 0
+    assert tile_stride(11008, 22, torch.bfloat16) == 512      # tiles of 501 / 500
+    assert tile_stride(2304, 4, torch.bfloat16) == 768        # tiles of 576
+    assert tile_stride(768, 2, torch.bfloat16) == 512         # tiles of 384
+    assert tile_stride(1003, 4, torch.bfloat16) == 256
+    assert tile_stride(11008, 22, torch.float32) == 0
