@@ -119,6 +119,70 @@ __global__ __launch_bounds__(256) void k_im2col(const E* __restrict__ x, E* __re
   }
 }
 
+// Tiled variant for rows that can be written in 16-byte vectors: a block produces 64 patches x
+// one 128-byte span of the patch dimension. Gather phase: each wave takes one patch entry
+// (c, kd, kh, kw) at a time -- uniform over the wave -- and its 64 lanes read it for 64 consecutive
+// patches, i.e. (for stride 1) 64 consecutive input elements: coalesced reads. The tile is turned
+// in LDS (row stride of 33 words: conflict-free writes) and written out as row-contiguous
+// 16-byte vectors.
+template <class E>
+__global__ __launch_bounds__(256) void k_im2col_tiled(const E* __restrict__ x, E* __restrict__ cols,
+                                                      int64_t ldc, ConvGeom g, int64_t M,
+                                                      int32_t k_tiles) {
+  constexpr int KT = 128 / (int)sizeof(E);  // patch entries per tile: 64 bf16 or 32 fp32
+  constexpr int EPV = 16 / (int)sizeof(E);  // entries per 16-byte vector
+  constexpr int VPR = KT / EPV;             // vectors per tile row: 8
+  __shared__ uint32_t tile[64 * 33];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t m0 = (int64_t)(blockIdx.x / k_tiles) * 64;
+  const int32_t k0 = (int32_t)(blockIdx.x % k_tiles) * KT;
+  // this lane's patch
+  const int64_t m = m0 + lane;
+  const bool mvalid = m < M;
+  const int64_t mm = mvalid ? m : M - 1;
+  const int64_t b = mm / g.L;
+  int32_t l = (int32_t)(mm - b * g.L);
+  const int32_t ow = l % g.out[2];
+  l /= g.out[2];
+  const int32_t oh = l % g.out[1];
+  const int32_t od = l / g.out[1];
+  const int32_t id0 = od * g.str[0] - g.pad[0];
+  const int32_t ih0 = oh * g.str[1] - g.pad[1];
+  const int32_t iw0 = ow * g.str[2] - g.pad[2];
+  const int64_t plane = (int64_t)g.in[1] * g.in[2];
+  const E* xb = x + b * g.C * g.in[0] * plane;
+  E* trow = (E*)tile;
+  constexpr int RS = 33 * 4 / (int)sizeof(E);  // tile row stride in entries
+  for (int kk = wave; kk < KT; kk += 4) {
+    const int32_t k = k0 + kk;  // uniform over the wave
+    E val = (E)0;
+    if (k < g.K) {
+      const int32_t c = k / g.kvol;
+      int32_t r = k - c * g.kvol;
+      const int32_t kw = r % g.ker[2];
+      r /= g.ker[2];
+      const int32_t kh = r % g.ker[1];
+      const int32_t kd = r / g.ker[1];
+      const int32_t id = id0 + kd * g.dil[0], ih = ih0 + kh * g.dil[1], iw = iw0 + kw * g.dil[2];
+      if (id >= 0 && id < g.in[0] && ih >= 0 && ih < g.in[1] && iw >= 0 && iw < g.in[2])
+        val = xb[((int64_t)c * g.in[0] + id) * plane + (int64_t)ih * g.in[2] + iw];
+    }
+    trow[lane * RS + kk] = val;
+  }
+  __syncthreads();
+  const int vcol = tid % VPR, vrow = tid / VPR;  // 32 rows per pass
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    const int p = vrow + 32 * pass;
+    const int32_t k = k0 + vcol * EPV;
+    if (m0 + p < M && k < g.K) {  // K is a multiple of EPV on this path
+      const uint32_t* src = tile + p * 33 + vcol * 4;
+      u32x4 v = {src[0], src[1], src[2], src[3]};
+      *(u32x4*)(cols + (m0 + p) * ldc + k) = v;
+    }
+  }
+}
+
 // Adjoint of k_im2col as a gather: one thread per input element sums, in fp32 and in a fixed
 // order (ascending kernel offset), the patch entries that were copied from it, and rounds once.
 // No atomics, so the result is reproducible.
@@ -159,6 +223,92 @@ __global__ __launch_bounds__(256) void k_col2im(const void* __restrict__ dcols, 
     }
   }
   D::store(dx, idx, acc);
+}
+
+// Tiled variant: a block computes 64 consecutive input elements of one image row for 8
+// channels. Every patch row that can contribute lies, for each kernel offset (kd, kh), in one
+// contiguous range of output columns; the block stages those ranges' entries of its 8 channels
+// (8 * kvol contiguous entries per patch row, loaded as 16-byte vectors) in LDS and then sums from
+// LDS, in the same ascending kernel-offset order as k_col2im, so both give the same bits.
+struct FoldPlan {
+  int32_t ow_span;   // staged output columns per (kd, kh)
+  int32_t row_vecs;  // 16-byte vectors per staged patch row (8 * kvol entries)
+  int32_t w_tiles;   // blocks along the input row
+};
+
+template <class D>
+__global__ __launch_bounds__(512) void k_col2im_tiled(const void* __restrict__ dcols, int64_t ldc,
+                                                      ConvGeom g, FoldPlan fp,
+                                                      void* __restrict__ dx) {
+  typedef typename D::elem E;
+  constexpr int EPV = D::EPV;
+  extern __shared__ __attribute__((aligned(16))) char fold_lds[];
+  const int tid = threadIdx.x;
+  // block -> (image b, channel group, d, h, column tile)
+  int64_t r = blockIdx.x;
+  const int32_t wt = (int32_t)(r % fp.w_tiles);
+  r /= fp.w_tiles;
+  const int32_t h = (int32_t)(r % g.in[1]);
+  r /= g.in[1];
+  const int32_t d = (int32_t)(r % g.in[0]);
+  r /= g.in[0];
+  const int32_t cg = (int32_t)(r % (g.C / 8));
+  const int64_t b = r / (g.C / 8);
+  const int32_t w0 = wt * 64;
+  const int32_t w_last = (w0 + 63 < g.in[2] ? w0 + 63 : g.in[2] - 1);
+  // output columns that can touch [w0, w_last]: ow = (w + pad - kw * dil) / str
+  const int32_t reach = (g.ker[2] - 1) * g.dil[2];
+  int32_t ow_min = w0 + g.pad[2] - reach;
+  ow_min = ow_min <= 0 ? 0 : (ow_min + g.str[2] - 1) / g.str[2];
+  int32_t ow_max = (w_last + g.pad[2]) / g.str[2];
+  if (ow_max > g.out[2] - 1) ow_max = g.out[2] - 1;
+  const int32_t span = ow_max - ow_min + 1;  // <= fp.ow_span by construction; may be <= 0
+  const int32_t row_bytes = fp.row_vecs * 16;
+  const int32_t kbase = cg * 8 * g.kvol;       // first patch entry of the channel group
+  // ---- stage: for every (kd, kh) with a valid output row, `span` patch rows ----
+  const int32_t combos = g.ker[0] * g.ker[1];
+  const int32_t vec_total = combos * fp.ow_span * fp.row_vecs;
+  for (int32_t v = tid; v < vec_total; v += 512) {
+    const int32_t vc = v % fp.row_vecs;
+    int32_t q = v / fp.row_vecs;
+    const int32_t oi = q % fp.ow_span;
+    q /= fp.ow_span;
+    const int32_t kh = q % g.ker[1], kd = q / g.ker[1];
+    const int32_t td = d + g.pad[0] - kd * g.dil[0], th = h + g.pad[1] - kh * g.dil[1];
+    u32x4 val = {0u, 0u, 0u, 0u};
+    if (oi < span && td >= 0 && th >= 0 && td % g.str[0] == 0 && th % g.str[1] == 0) {
+      const int32_t od = td / g.str[0], oh = th / g.str[1];
+      if (od < g.out[0] && oh < g.out[1]) {
+        const int64_t l = ((int64_t)od * g.out[1] + oh) * g.out[2] + ow_min + oi;
+        val = ld16((const E*)dcols + (b * g.L + l) * ldc + kbase + vc * EPV);
+      }
+    }
+    *(u32x4*)(fold_lds + ((int64_t)(kd * g.ker[1] + kh) * fp.ow_span + oi) * row_bytes + vc * 16) = val;
+  }
+  __syncthreads();
+  // ---- sum: thread = (channel tid / 64 of the group, column tid % 64) ----
+  const int32_t w = w0 + (tid & 63), cl = tid >> 6;
+  if (w >= g.in[2]) return;
+  float acc = 0.f;
+  for (int32_t kd = 0; kd < g.ker[0]; ++kd) {
+    const int32_t td = d + g.pad[0] - kd * g.dil[0];
+    if (td < 0 || td % g.str[0] != 0 || td / g.str[0] >= g.out[0]) continue;
+    for (int32_t kh = 0; kh < g.ker[1]; ++kh) {
+      const int32_t th = h + g.pad[1] - kh * g.dil[1];
+      if (th < 0 || th % g.str[1] != 0 || th / g.str[1] >= g.out[1]) continue;
+      const char* rows = fold_lds + (int64_t)(kd * g.ker[1] + kh) * fp.ow_span * row_bytes;
+      for (int32_t kw = 0; kw < g.ker[2]; ++kw) {
+        const int32_t tw = w + g.pad[2] - kw * g.dil[2];
+        if (tw < 0 || tw % g.str[2] != 0) continue;
+        const int32_t ow = tw / g.str[2];
+        if (ow >= g.out[2]) continue;
+        const int32_t k = cl * g.kvol + (kd * g.ker[1] + kh) * g.ker[2] + kw;
+        acc += D::load(rows + (int64_t)(ow - ow_min) * row_bytes, k);
+      }
+    }
+  }
+  const int64_t plane = (int64_t)g.in[1] * g.in[2];
+  D::store(dx, (((b * g.C + cg * 8 + cl) * g.in[0] + d) * plane) + (int64_t)h * g.in[2] + w, acc);
 }
 
 // dst[b][c][r] = src[b][r][c]; 32 x 32 tiles through LDS (padded against bank conflicts) so that
@@ -214,6 +364,19 @@ extern "C" int ahl_conv_out_size(const AhlConvGeom* geom, int32_t* out_size) {
   return AHL_OK;
 }
 
+template <class E>
+static int launch_im2col_tiled(const void* x, void* cols, int64_t ldc, const ConvGeom& g,
+                               hipStream_t st) {
+  constexpr int KT = 128 / (int)sizeof(E);
+  const int64_t M = (int64_t)g.B * g.L;
+  const int64_t k_tiles = cdiv(g.K, KT);
+  const int64_t blocks = cdiv(M, 64) * k_tiles;
+  if (blocks > 0x7fffffff) return AHL_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL((k_im2col_tiled<E>), dim3((unsigned)blocks), dim3(256), 0, st, (const E*)x,
+                     (E*)cols, ldc, g, M, (int32_t)k_tiles);
+  return check_launch("k_im2col_tiled");
+}
+
 extern "C" int ahl_im2col(const void* x, const AhlConvGeom* geom, int32_t dtype, void* cols,
                           int64_t ldc, void* stream) {
   ConvGeom g;
@@ -221,12 +384,12 @@ extern "C" int ahl_im2col(const void* x, const AhlConvGeom* geom, int32_t dtype,
   hipStream_t st = (hipStream_t)stream;
   if (dtype == AHL_F32) {
     if (g.K % 4 == 0 && ldc % 4 == 0 && aligned16(cols))
-      return launch_im2col<uint32_t, 4>(x, cols, ldc, g, st);
+      return launch_im2col_tiled<uint32_t>(x, cols, ldc, g, st);
     return launch_im2col<uint32_t, 1>(x, cols, ldc, g, st);
   }
   if (dtype == AHL_BF16) {
     if (g.K % 8 == 0 && ldc % 8 == 0 && aligned16(cols))
-      return launch_im2col<uint16_t, 8>(x, cols, ldc, g, st);
+      return launch_im2col_tiled<uint16_t>(x, cols, ldc, g, st);
     return launch_im2col<uint16_t, 1>(x, cols, ldc, g, st);
   }
   return AHL_ERR_ARG;
@@ -237,6 +400,27 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
   ConvGeom g;
   if (dcols == nullptr || dx == nullptr || !make_geom(geom, &g) || ldc < g.K) return AHL_ERR_ARG;
   const int64_t total = (int64_t)g.B * g.C * g.in[0] * g.in[1] * g.in[2];
+  // tiled kernel: channel groups of 8 whose 8 * kvol patch entries are whole 16-byte vectors
+  {
+    const int epv = dtype == AHL_BF16 ? 8 : 4;
+    const int64_t row_entries = 8 * (int64_t)g.kvol;
+    // widest range of output columns one block of 64 input columns can reach
+    const int64_t ow_span = (63 + (int64_t)(g.ker[2] - 1) * g.dil[2]) / g.str[2] + 2;
+    const int64_t lds_bytes = (int64_t)g.ker[0] * g.ker[1] * ow_span * row_entries * (dtype == AHL_BF16 ? 2 : 4);
+    const int64_t w_tiles = cdiv(g.in[2], 64);
+    const int64_t tblocks = (int64_t)g.B * (g.C / 8) * g.in[0] * g.in[1] * w_tiles;
+    if ((dtype == AHL_BF16 || dtype == AHL_F32) && g.C % 8 == 0 && row_entries % epv == 0 &&
+        ldc % epv == 0 && aligned16(dcols) && lds_bytes <= 96 * 1024 && tblocks <= 0x7fffffff) {
+      FoldPlan fp{(int32_t)ow_span, (int32_t)(row_entries / epv), (int32_t)w_tiles};
+      AHL_DISPATCH_DTYPE(dtype, {
+        hipFuncSetAttribute((const void*)k_col2im_tiled<D>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        hipLaunchKernelGGL((k_col2im_tiled<D>), dim3((unsigned)tblocks), dim3(512), (size_t)lds_bytes,
+                           (hipStream_t)stream, dcols, ldc, g, fp, dx);
+      });
+      return check_launch("k_col2im_tiled");
+    }
+  }
   const int64_t blocks = cdiv(total, 256);
   if (blocks > 0x7fffffff) return AHL_ERR_UNSUPPORTED;
   AHL_DISPATCH_DTYPE(dtype, {

@@ -47,6 +47,9 @@ struct BwdArgs {
   int64_t M, N, K;
   int32_t tile;                        // K-tile width (multiple of 256)
   int32_t ir_static;                   // 0: no range gradient; 1 + AHL_IR_GRAD_* otherwise
+  int32_t dense_tile;                  // DX: 0, or the true tile width when x and dx are dense
+                                       // while W_eff is in the padded tile layout (K, tile then
+                                       // describe the padded columns); a multiple of 8
   int32_t slices;                      // DW: the contraction (rows m) is cut into this many
                                        // slices, one block each; > 1 when N x K alone gives
                                        // too few blocks to fill the chip
@@ -277,8 +280,17 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
   constexpr int kOutStride = 256 * 2 + 16;
   const int vcol = tid & 31, vrow = tid >> 5;  // 16-byte vector column, row within a pass of 16
-  const uint16_t* xp = do_ir ? a.x + (r0 + vrow) * a.ldx + c0 + vcol * 8 : nullptr;
-  uint16_t* op = a.out + (r0 + vrow) * a.ldo + c0 + vcol * 8;
+  // column of this thread's vectors in x / dx: the operand column itself, or, with dense x / dx
+  // next to a padded W_eff, the same offset inside the dense tile (padding columns: no vector)
+  int64_t ocol = c0 + vcol * 8;
+  bool ovalid = true;
+  if (MODE == MODE_DX && a.dense_tile > 0) {
+    const int64_t in_tile = ocol - (int64_t)t * a.tile;
+    ovalid = in_tile < a.dense_tile;
+    ocol = ovalid ? (int64_t)t * a.dense_tile + in_tile : 0;
+  }
+  const uint16_t* xp = do_ir ? a.x + (r0 + vrow) * a.ldx + ocol : nullptr;
+  uint16_t* op = a.out + (r0 + vrow) * a.ldo + ocol;
   {
     char* obase = lds + (wm * 128 + 4 * h) * kOutStride + (wn * 64 + (lane & 31)) * 2;
 #pragma unroll
@@ -295,7 +307,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     u32x4 xr[8];
-    if (do_ir) {
+    if (do_ir && ovalid) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int row = vrow + 16 * (8 * half + j);
@@ -307,7 +319,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     for (int j = 0; j < 8; ++j) {
       const int row = vrow + 16 * (8 * half + j);
       u32x4 d4 = *(const u32x4*)(lds + row * kOutStride + vcol * 16);
-      if (r0 + row >= R) continue;
+      if (r0 + row >= R || !ovalid) continue;
       if (do_ir) {
         float d[8], xv[8];
         BF16::unpack(d4, d);
@@ -378,8 +390,9 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
-                   const Tiling& tl, int ir_static, hipStream_t s) {
+                   const Tiling& tl, int ir_static, int32_t dense_tile, hipStream_t s) {
   BwdArgs a;
+  a.dense_tile = dense_tile;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
@@ -425,7 +438,7 @@ int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   a.b = (const uint16_t*)xq; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;
   a.out = (uint16_t*)dw; a.ldo = lddw; a.partial = nullptr;
   a.bias_partial = dbias ? bias_partial : nullptr;
-  a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = 0;
+  a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = 0; a.dense_tile = 0;
   a.slices = slices;
   a.split = slices > 1
       ? (float*)((char*)ws + ((int64_t)slices * (K / 256) * N * 4 + 255) / 256 * 256) : nullptr;

@@ -699,7 +699,7 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
-                   const Tiling& tl, int ir_static, hipStream_t s);
+                   const Tiling& tl, int ir_static, int32_t dense_tile, hipStream_t s);
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
@@ -850,20 +850,34 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     if (cfg->dtype != AHL_BF16 || M % 64 != 0 || N % 64 != 0 || !aligned16(g) || !aligned16(w_eff) ||
         ldg % 8 != 0 || ldw % 8 != 0 || (keep && !aligned16(keep)))
       return AHL_ERR_UNSUPPORTED;
+    const Tiling ptl{n_tiles, (int32_t)stride, 0};
+    const int32_t per_tile = (int32_t)(stride / 256);
+    int rc;
+    if (tl.extra == 0 && tl.base % 8 == 0 && lddx % 8 == 0 && aligned16(dx) &&
+        (!is_static || (ldx % 8 == 0 && aligned16(x)))) {
+      // equal tiles of a multiple of 8 columns: the kernel's 16-byte vectors of x and dx map
+      // one to one onto the dense matrices, no padded copies needed
+      rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M,
+                          padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0, tl.base, s);
+      if (rc != AHL_OK) return rc;
+      if (is_static)
+        hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
+                           (const float*)partial, cdiv(M, 256), (int32_t)(padded / 256), per_tile,
+                           per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
+                           cfg->ir_grad_rule);
+      return check_launch("ahl_linear_bwd_dx(fast, padded weights)");
+    }
     char* p = (char*)ws + dx_padded_partial_bytes(M, padded);
     void* xpad = p;
     void* dxp = p + align256(M * padded * 2);
-    int rc;
     if (is_static) {
       rc = launch_pad_tiles(x, ldx, AHL_BF16, M, tl, stride, xpad, padded, s);
       if (rc != AHL_OK) return rc;
     }
-    const Tiling ptl{n_tiles, (int32_t)stride, 0};
     rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, xpad, padded, ir, dxp, padded, partial,
-                        M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0, s);
+                        M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, s);
     if (rc != AHL_OK) return rc;
     if (is_static) {
-      const int32_t per_tile = (int32_t)(stride / 256);
       hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
                          (const float*)partial, cdiv(M, 256), (int32_t)(padded / 256), per_tile,
                          per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
@@ -878,7 +892,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
     int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
-                            N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, s);
+                            N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, s);
     if (rc != AHL_OK) return rc;
     if (is_static) {
       const int32_t per_tile = tl.base / 256;

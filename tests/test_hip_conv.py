@@ -31,6 +31,11 @@ GEOMS = [
     (2, 4, (5, 6, 7), (2, 3, 2), (1, 2, 1), (1, 0, 1), (1, 1, 1)),   # 3-d, K = 48
     (1, 16, (1, 33, 29), (1, 3, 3), (1, 1, 1), (0, 1, 1), (1, 1, 1)),  # K = 144, odd sizes
     (2, 2, (3, 4, 5), (3, 4, 5), (1, 1, 1), (0, 0, 0), (1, 1, 1)),   # kernel == input
+    # channel counts that are multiples of 8: the tiled fold kernel
+    (2, 8, (4, 9, 70), (2, 3, 3), (1, 2, 1), (1, 1, 1), (1, 1, 1)),   # 3-d, two column tiles
+    (2, 16, (1, 17, 131), (1, 3, 5), (1, 2, 3), (0, 1, 2), (1, 2, 2)),  # strides and dilations
+    (1, 8, (1, 5, 200), (1, 1, 7), (1, 1, 4), (0, 0, 0), (1, 1, 1)),   # stride > 1 along the row
+    (3, 24, (1, 12, 12), (1, 1, 1), (1, 1, 1), (0, 0, 0), (1, 1, 1)),   # 1 x 1 kernel
 ]
 
 

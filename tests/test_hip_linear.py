@@ -97,6 +97,10 @@ SHAPES = [
     case("pad_bf16_576_dynamic", dtype="bf16", M=128, K=1152, N=192, max_input_size=576,
          ir_mode="dynamic", inp_res=254, out_res=254, out_bound=0.3, w_scale=0.1, seed=33),
     case("pad_bf16_plain", dtype="bf16", M=64, K=300, N=64, max_input_size=128, seed=34),
+    # equal tiles of a multiple of 8: padded operands, dense x / dx straight from the kernel
+    case("pad_bf16_384_static_clamped", dtype="bf16", M=320, K=768, N=128, max_input_size=384,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01,
+         ir_values=[1.5, 2.5], w_scale=0.1, seed=39),
     case("pad_bf16_fast_mode", dtype="bf16", M=128, K=520, N=64, max_input_size=256, ir_mode="fast",
          ir_values=[0.8, 2.5, 1.5], inp_res=254, out_res=254, out_bound=1.5, clip="channel",
          clip_sigma=2.5, w_scale=0.3, seed=35),
