@@ -30,7 +30,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 # rocprofv3 FETCH_SIZE and WRITE_SIZE runs of `bench.py --kernels-only`, each scaled by what the
 # same counter reads for the 256 MiB copy below (profiles/*_hbm_traffic.txt holds the table).
 MEASURED_TRAFFIC_BYTES = {
-    "linear_fwd": int((697.1 + 96.2) * 2 ** 20),
+    "linear_fwd": int((707.2 + 96.2) * 2 ** 20),
     "linear_bwd_dx(+ir_grad)": int((480.3 + 64.0) * 2 ** 20),
     "linear_bwd_dw(+bias_grad)": int((416.1 + 32.2) * 2 ** 20),
 }
@@ -64,6 +64,83 @@ def build_layer():
     x = torch.randn(M_TOKENS, K_IN, generator=gen).to(torch.bfloat16)
     g = torch.randn(M_TOKENS, N_OUT, generator=gen).to(torch.bfloat16)
     return layer, x, g
+
+
+def _analog_cfg(tile, noise=True):
+    from aihwkit_lightning.simulator.configs import (
+        TorchInferenceRPUConfig, WeightClipType, WeightNoiseInjectionType,
+    )
+
+    cfg = TorchInferenceRPUConfig()
+    cfg.mapping.max_input_size = tile
+    cfg.forward.inp_res = 254
+    cfg.forward.out_res = 254
+    cfg.forward.out_bound = 10.0
+    cfg.forward.out_noise = 0.04 if noise else 0.0
+    cfg.clip.type = WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL
+    cfg.clip.sigma = 2.5
+    if noise:
+        cfg.modifier.noise_type = WeightNoiseInjectionType.ADD_NORMAL_PER_CHANNEL
+        cfg.modifier.std_dev = 0.02
+    ir = cfg.pre_post.input_range
+    ir.enable, ir.dynamic, ir.learn_input_range = True, False, True
+    ir.init_value, ir.init_from_data, ir.decay, ir.input_min_percentage = 3.0, 0, 0.01, 0.95
+    return cfg
+
+
+# Workloads next to the headline one (`--workload NAME`, each prints its own line; the default
+# run measures the headline workload only), same analog configuration. They exercise what the
+# headline shape does not: a split whose tiles do not start on 256-column boundaries (padded tile
+# layout of the operands) and a convolution (patch extraction, narrow weight gradient).
+OTHER_WORKLOADS = {
+    "linear_11008": "AnalogLinear 11008->4096 bf16, 8192 tokens, 22 tiles of 501/500, fwd+bwd",
+    "conv2d_256": "AnalogConv2d 256->256 3x3 pad 1 bf16, 128 x 28 x 28 input, 4 tiles of 576, "
+                  "fwd+bwd",
+}
+
+
+def build_other(name):
+    """(layer, x, grad_out, flops per step) of one of OTHER_WORKLOADS, on the device."""
+    from aihwkit_lightning.nn import AnalogConv2d, AnalogLinear
+
+    gen = torch.Generator().manual_seed(3)
+    if name == "linear_11008":
+        layer = AnalogLinear(11008, 4096, bias=True, dtype=torch.bfloat16, rpu_config=_analog_cfg(512))
+        x = torch.randn(8192, 11008, generator=gen).to(torch.bfloat16)
+        g = torch.randn(8192, 4096, generator=gen).to(torch.bfloat16)
+        flops = 3 * 2.0 * 8192 * 11008 * 4096
+    elif name == "conv2d_256":
+        layer = AnalogConv2d(256, 256, 3, padding=1, bias=True, dtype=torch.bfloat16,
+                             rpu_config=_analog_cfg(576))
+        x = torch.randn(128, 256, 28, 28, generator=gen).to(torch.bfloat16)
+        g = torch.randn(128, 256, 28, 28, generator=gen).to(torch.bfloat16)
+        flops = 3 * 2.0 * (128 * 28 * 28) * (256 * 9) * 256
+    else:
+        raise ValueError(name)
+    with torch.no_grad():
+        layer.weight.mul_(0.02 / layer.weight.std())
+    return layer.cuda().train(), x.cuda().requires_grad_(True), g.cuda(), flops
+
+
+def time_other(name, steps, warmup):
+    """ms per fwd+bwd step and TFLOP/s of one of OTHER_WORKLOADS (wall clock around K steps)."""
+    layer, x, g, flops = build_other(name)
+
+    def step():
+        x.grad = None
+        layer.zero_grad(set_to_none=True)
+        layer(x).backward(g)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    return {"workload": OTHER_WORKLOADS[name], "ms_per_step": round(ms, 4),
+            "tflops": round(flops / (ms * 1e-3) / 1e12, 2)}
 
 
 def event_time_ms(fn, reps):
@@ -207,6 +284,8 @@ def main():
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--kernels-only", action="store_true",
                         help="only launch the individual kernels (for rocprofv3 runs)")
+    parser.add_argument("--workload", default="linear", choices=["linear", *OTHER_WORKLOADS],
+                        help="'linear' is the headline workload; the others print their own line")
     ns = parser.parse_args()
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)",
@@ -215,6 +294,17 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
+
+    if ns.workload != "linear":
+        torch.manual_seed(0)
+        res = time_other(ns.workload, ns.steps, ns.warmup)
+        print(json.dumps({
+            "metric": "fwd+bwd TFLOP/s", "value": res["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
+            "steps": ns.steps, "warmup": ns.warmup, "ms_per_step": res["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "data": "synthetic", "config": {"workload": res["workload"]},
+        }))
+        return
 
     layer, x, g = build_layer()
     layer = layer.cuda().train()
