@@ -65,6 +65,12 @@ LIB = torch.library.Library("aihwkit_hip", "DEF")
 
 LIB.define("sliced_absmax(Tensor x, int[] in_sizes, bool tile_stats) -> (Tensor, Tensor, Tensor)")
 LIB.define("sliced_std(Tensor x, int[] in_sizes) -> Tensor")
+LIB.define("row_nonzero(Tensor x) -> Tensor")
+LIB.define("sliced_std_kept(Tensor x, int[] in_sizes) -> Tensor")
+LIB.define("sliced_quantile(Tensor x, int[] in_sizes, float q) -> Tensor")
+LIB.define(
+    "ir_moving_update(Tensor(a!) ir, Tensor(b!) idx, Tensor val, float alpha, bool val_in_dtype) -> ()"
+)
 LIB.define(
     "ir_init_update(Tensor(a!) ir, Tensor(b!) idx, Tensor std, float init_from_data, "
     "float alpha) -> ()"
@@ -248,6 +254,70 @@ def sliced_std(x: Tensor, in_sizes: List[int]) -> Tensor:
         "ahl_sliced_std",
     )
     return out
+
+
+def row_nonzero(x: Tensor) -> Tensor:
+    """uint8 ``[rows]``: 1 for every row of ``x`` that is not all zero."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    kept = torch.empty((x.size(0),), dtype=torch.uint8, device=x.device)
+    count = torch.empty((1,), dtype=torch.int32, device=x.device)
+    L.check(
+        lib.ahl_row_nonzero(_ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), _ptr(kept),
+                            _ptr(count), _stream()),
+        "ahl_row_nonzero",
+    )
+    return kept
+
+
+def sliced_std_kept(x: Tensor, in_sizes: List[int]) -> Tensor:
+    """Unbiased std of every K-tile over the rows that are not all zero, float32 ``[T]``."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    n_tiles = len(in_sizes)
+    out = torch.empty((n_tiles,), dtype=torch.float32, device=x.device)
+    ws = torch.empty((lib.ahl_sliced_std_kept_ws_bytes(x.size(0), n_tiles),), dtype=torch.uint8,
+                     device=x.device)
+    L.check(
+        lib.ahl_sliced_std_kept(
+            _ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), L.tile_ends_array(in_sizes),
+            n_tiles, _ptr(out), _ptr(ws), _stream(),
+        ),
+        "ahl_sliced_std_kept",
+    )
+    return out
+
+
+def sliced_quantile(x: Tensor, in_sizes: List[int], q: float) -> Tensor:
+    """``torch.quantile(x[kept rows, tile].float().flatten(), q)`` of every K-tile, float32
+    ``[T]``; kept rows are those that are not all zero."""
+    lib = L.load()
+    x = _rows2d(x, "x")
+    n_tiles = len(in_sizes)
+    out = torch.empty((n_tiles,), dtype=torch.float32, device=x.device)
+    ws = torch.empty((lib.ahl_sliced_quantile_ws_bytes(x.size(0), n_tiles),), dtype=torch.uint8,
+                     device=x.device)
+    L.check(
+        lib.ahl_sliced_quantile(
+            _ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), L.tile_ends_array(in_sizes),
+            n_tiles, float(q), _ptr(out), _ptr(ws), _stream(),
+        ),
+        "ahl_sliced_quantile",
+    )
+    return out
+
+
+def ir_moving_update(ir: Tensor, idx: Tensor, val: Tensor, alpha: float, val_in_dtype: bool) -> None:
+    """In-place moving-average step of the calibrated ranges; ``idx`` is int32 ``[T]``."""
+    lib = L.load()
+    if not (ir.is_contiguous() and idx.is_contiguous() and idx.dtype == torch.int32
+            and val.dtype == torch.float32 and val.is_contiguous()):
+        raise HipBackendError("ir_moving_update: contiguous ir, int32 idx and float32 val expected")
+    L.check(
+        lib.ahl_ir_moving_update(_ptr(ir), _ptr(idx), _ptr(val), dtype_id(ir.dtype), ir.numel(),
+                                 float(alpha), int(val_in_dtype), _stream()),
+        "ahl_ir_moving_update",
+    )
 
 
 def ir_init_update(ir: Tensor, idx: Tensor, std: Tensor, init_from_data: float, alpha: float) -> None:
@@ -555,7 +625,9 @@ def linear_bwd_dw(
 
 
 for _name, _fn in [
-    ("sliced_absmax", sliced_absmax), ("sliced_std", sliced_std), ("ir_init_update", ir_init_update),
+    ("sliced_absmax", sliced_absmax), ("sliced_std", sliced_std),
+    ("row_nonzero", row_nonzero), ("sliced_std_kept", sliced_std_kept), ("sliced_quantile", sliced_quantile),
+    ("ir_moving_update", ir_moving_update), ("ir_init_update", ir_init_update),
     ("running_absmax", running_absmax), ("ir_fast_update", ir_fast_update),
     ("clip_weights", clip_weights), ("col_sum", col_sum),
     ("weight_prep", weight_prep), ("quantize_weights", quantize_weights),

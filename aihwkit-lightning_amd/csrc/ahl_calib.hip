@@ -1,0 +1,265 @@
+// Statistics of the post-training input-range calibration that need more than a reduction
+// (reference inference/calibration/calibration.py:57-152): the q-quantile of every K-tile of a
+// batch over the rows that are not all zero, and the moving-average update of the ranges.
+//
+// The quantile is exact: torch.quantile's linear interpolation between the two neighbouring
+// order statistics, which are found by a most-significant-digit radix selection on the
+// order-preserving integer image of the fp32 values -- four histogram passes of 8 bits over the
+// data (integer atomics only: deterministic), one pass for the successor of the selected value.
+// No sort, no copy of the data; everything stays on the device, so a calibration run never
+// synchronises with the host.
+#include "ahl_host.h"
+#include "ahl_reduce_kernels.h"
+#include <math.h>
+
+namespace ahl {
+
+// order-preserving map fp32 -> uint32 (negative values reversed below the positive ones)
+AHL_DEV uint32_t f32_key(float v) {
+  const uint32_t u = __float_as_uint(v);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+AHL_DEV float key_f32(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+
+// per-tile selection state
+struct SelState {
+  uint32_t prefix;    // digits of the selected key found so far (right-aligned)
+  uint32_t k_rem;     // rank of the wanted element among the elements that match the prefix
+  uint32_t lo;        // rank of the lower order statistic
+  uint32_t need_hi;   // the interpolation needs the next order statistic too
+  float weight;       // interpolation weight of the upper order statistic
+  uint32_t n_le;      // elements <= the selected value (set by the last pick)
+  uint32_t next_key;  // smallest key above the selected one (0xffffffff: none)
+  uint32_t has_nan;
+  uint32_t n;         // elements of the tile over the kept rows
+  uint32_t pad[3];
+};
+static_assert(sizeof(SelState) == 48, "layout");
+
+// n, rank and weight per tile: rank = q * (n - 1) evaluated in fp32 as torch.quantile does for
+// an fp32 input (aten/src/ATen/native/Sorting.cpp quantile_compute)
+__global__ void k_select_init(SelState* st, uint32_t* hist, const uint32_t* n_kept, Tiling tl,
+                              float q) {
+  const int t = blockIdx.x, i = threadIdx.x;
+  hist[t * 256 + i] = 0u;
+  if (i != 0) return;
+  const uint64_t n64 = (uint64_t)*n_kept * (uint64_t)tl.size(t);
+  SelState s;
+  s.n = (uint32_t)n64;
+  s.prefix = 0u; s.n_le = 0u; s.next_key = 0xffffffffu; s.has_nan = 0u;
+  s.pad[0] = s.pad[1] = s.pad[2] = 0u;
+  if (n64 == 0) { s.k_rem = 0u; s.lo = 0u; s.need_hi = 0u; s.weight = 0.0f; st[t] = s; return; }
+  const float rank = q * (float)(n64 - 1);
+  const float below = floorf(rank);
+  s.lo = (uint32_t)below;
+  s.k_rem = s.lo;
+  s.weight = rank - below;
+  s.need_hi = ceilf(rank) > below ? 1u : 0u;
+  st[t] = s;
+}
+
+// Histogram of digit `pass` (0 = most significant byte) over the kept elements of every tile
+// whose higher digits equal the tile's prefix. One wave per (group of rows, tile); per-wave
+// histogram in LDS, then one integer atomic per non-empty bin.
+template <class D>
+__global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x, int64_t rows,
+                                                     int64_t ld, const uint8_t* __restrict__ kept,
+                                                     Tiling tl, int rpw, int pass,
+                                                     SelState* __restrict__ st,
+                                                     uint32_t* __restrict__ hist) {
+  __shared__ uint32_t lh[4][256];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  for (int i = lane; i < 256; i += 64) lh[w][i] = 0u;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + w;
+  const int64_t grp = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
+  const int64_t r0 = grp * rpw;
+  if (r0 < rows) {  // no early return: nothing below synchronises across waves, but keep it simple
+    const uint32_t prefix = st[t].prefix;
+    const int shift = 24 - 8 * pass;
+    bool nan = false;
+    for (int i = 0; i < rpw; ++i) {
+      const int64_t r = r0 + i;
+      if (r >= rows) break;
+      if (!kept[r]) continue;
+      const typename D::elem* row = (const typename D::elem*)x + r * ld;
+      for (int32_t c = tl.start(t) + lane; c < tl.start(t + 1); c += 64) {
+        const float v = D::load(row, c);
+        nan |= (v != v);
+        const uint32_t key = f32_key(v);
+        // digits above this pass must match the prefix found so far
+        if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&lh[w][(key >> shift) & 255u], 1u);
+      }
+    }
+    if (pass == 0 && __builtin_amdgcn_ballot_w64(nan) != 0ull && lane == 0) atomicOr(&st[t].has_nan, 1u);
+    for (int i = lane; i < 256; i += 64) {
+      const uint32_t c = lh[w][i];
+      if (c) atomicAdd(&hist[t * 256 + i], c);
+    }
+  }
+}
+
+// The bin that holds rank k_rem: extend the prefix, rebase the rank, clear the histogram.
+__global__ void k_select_pick(SelState* st, uint32_t* hist, int pass) {
+  const int t = blockIdx.x;
+  if (threadIdx.x == 0) {
+    SelState s = st[t];
+    if (s.n != 0) {
+      uint32_t cum = 0u;
+      int b = 0;
+      for (; b < 255; ++b) {
+        const uint32_t c = hist[t * 256 + b];
+        if (cum + c > s.k_rem) break;
+        cum += c;
+      }
+      s.prefix = (s.prefix << 8) | (uint32_t)b;
+      s.k_rem -= cum;
+      if (pass == 3) s.n_le = (s.lo - s.k_rem) + hist[t * 256 + b];  // below + equal
+      st[t] = s;
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[t * 256 + i] = 0u;
+}
+
+// next_key[t] = smallest key above the selected one
+template <class D>
+__global__ __launch_bounds__(256) void k_select_next(const void* __restrict__ x, int64_t rows,
+                                                     int64_t ld, const uint8_t* __restrict__ kept,
+                                                     Tiling tl, int rpw, SelState* __restrict__ st) {
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t grp = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
+  const int64_t r0 = grp * rpw;
+  if (r0 >= rows) return;
+  const uint32_t sel = st[t].prefix;
+  uint32_t best = 0xffffffffu;
+  for (int i = 0; i < rpw; ++i) {
+    const int64_t r = r0 + i;
+    if (r >= rows) break;
+    if (!kept[r]) continue;
+    const typename D::elem* row = (const typename D::elem*)x + r * ld;
+    for (int32_t c = tl.start(t) + lane; c < tl.start(t + 1); c += 64) {
+      const uint32_t key = f32_key(D::load(row, c));
+      if (key > sel && key < best) best = key;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)best, off, 64);
+    best = o < best ? o : best;
+  }
+  if (lane == 0 && best != 0xffffffffu) atomicMin(&st[t].next_key, best);
+}
+
+// out[t] = lerp(x_(lo), x_(lo+1), weight) with torch's two-sided lerp formula
+__global__ void k_select_final(const SelState* st, int32_t n_tiles, float* out) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_tiles) return;
+  const SelState s = st[t];
+  if (s.n == 0 || s.has_nan) { out[t] = __builtin_nanf(""); return; }
+  const float lo = key_f32(s.prefix);
+  float hi = lo;
+  if (s.need_hi && s.n_le < s.lo + 2u && s.next_key != 0xffffffffu) hi = key_f32(s.next_key);
+  const float w = s.weight, diff = hi - lo;
+  out[t] = w < 0.5f ? lo + w * diff : hi - diff * (1.0f - w);
+}
+
+// input_range[t] <- (input_range[t] * idx[t] + val[t]) / (idx[t] + 1), idx[t] += 1: the moving
+// average of calibration.py:126-147. The reference evaluates it on a 0-dim fp32 tensor (Python
+// float times an int32 tensor element), then casts to the range's dtype.
+template <class D>
+__global__ void k_ir_moving_update(void* ir, int32_t* idx, const float* __restrict__ val,
+                                   int32_t n_tiles, double alpha, int32_t val_in_dtype) {
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  if (t >= n_tiles) return;
+  const float old = D::load(ir, t);
+  const int32_t i = idx[t];
+  // the statistic as the Python float the reference holds: alpha * std (std in the tensor dtype)
+  // or the fp32 quantile
+  const float stat = val_in_dtype ? D::rd(val[t]) : val[t];
+  const float v = (float)(alpha * (double)stat);
+  const float num = old * (float)i + v;
+  D::store(ir, t, __fdiv_rn(num, (float)(i + 1)));
+  idx[t] = i + 1;
+}
+
+static int select_rpw(int64_t rows) {
+  const int64_t r = rows / 4096;
+  return (int)(r < 1 ? 1 : (r > 16 ? 16 : r));
+}
+
+}  // namespace ahl
+
+using namespace ahl;
+
+extern "C" {
+
+// workspace: [SelState[T] | hist[T][256] | kept-row counter | kept flags, one byte per row]
+int64_t ahl_sliced_quantile_ws_bytes(int64_t rows, int32_t n_tiles) {
+  if (rows <= 0 || n_tiles <= 0) return 0;
+  const int64_t head = ((int64_t)n_tiles * (int64_t)(sizeof(SelState) + 1024) + 255) / 256 * 256;
+  return head + 256 + rows;
+}
+
+int ahl_sliced_quantile(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                        const int32_t* tile_ends_host, int32_t n_tiles, float q, float* out,
+                        void* ws, void* stream) {
+  if (!x || !out || !ws || rows <= 0 || cols <= 0 || ld < cols) return AHL_ERR_ARG;
+  if (!(q >= 0.0f && q <= 1.0f)) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
+  if (rows * (int64_t)widest_tile(tl) > 0xffffffffll) return AHL_ERR_UNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  SelState* st = (SelState*)ws;
+  uint32_t* hist = (uint32_t*)(st + n_tiles);
+  const int64_t head = ((int64_t)n_tiles * (int64_t)(sizeof(SelState) + 1024) + 255) / 256 * 256;
+  uint32_t* n_kept = (uint32_t*)((char*)ws + head);
+  uint8_t* kept = (uint8_t*)n_kept + 256;
+  const int rpw = select_rpw(rows);
+  const int64_t nb = cdiv(cdiv(rows, rpw) * n_tiles, 4);
+  if (nb > 0x7fffffff || cdiv(rows, 4) > 0x7fffffff) return AHL_ERR_ARG;
+  hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, s, n_kept, 0u, 1);
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(x) && (ld % D::EPV == 0);
+    if (vec) hipLaunchKernelGGL((k_row_nonzero<D, true>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
+    else hipLaunchKernelGGL((k_row_nonzero<D, false>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
+    hipLaunchKernelGGL(k_select_init, dim3(n_tiles), dim3(256), 0, s, st, hist, (const uint32_t*)n_kept, tl, q);
+    for (int pass = 0; pass < 4; ++pass) {
+      hipLaunchKernelGGL((k_select_hist<D>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist);
+      hipLaunchKernelGGL(k_select_pick, dim3(n_tiles), dim3(256), 0, s, st, hist, pass);
+    }
+    hipLaunchKernelGGL((k_select_next<D>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, st);
+  });
+  hipLaunchKernelGGL(k_select_final, dim3((unsigned)cdiv(n_tiles, 64)), dim3(64), 0, s, (const SelState*)st, n_tiles, out);
+  return check_launch("ahl_sliced_quantile");
+}
+
+int ahl_row_nonzero(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                    uint8_t* kept, uint32_t* n_kept, void* stream) {
+  if (!x || !kept || !n_kept || rows <= 0 || cols <= 0 || ld < cols) return AHL_ERR_ARG;
+  if (cols > 0x7fffffff || cdiv(rows, 4) > 0x7fffffff) return AHL_ERR_UNSUPPORTED;
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, s, n_kept, 0u, 1);
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(x) && (ld % D::EPV == 0);
+    if (vec) hipLaunchKernelGGL((k_row_nonzero<D, true>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
+    else hipLaunchKernelGGL((k_row_nonzero<D, false>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
+  });
+  return check_launch("ahl_row_nonzero");
+}
+
+int ahl_ir_moving_update(void* ir, int32_t* idx, const float* val, int32_t dtype, int32_t n_tiles,
+                         double alpha, int32_t val_in_dtype, void* stream) {
+  if (!ir || !idx || !val || n_tiles <= 0) return AHL_ERR_ARG;
+  AHL_DISPATCH_DTYPE(dtype, {
+    hipLaunchKernelGGL((k_ir_moving_update<D>), dim3((unsigned)cdiv(n_tiles, 64)), dim3(64), 0,
+                       (hipStream_t)stream, ir, idx, val, n_tiles, alpha, val_in_dtype);
+  });
+  return check_launch("ahl_ir_moving_update");
+}
+
+}  // extern "C"

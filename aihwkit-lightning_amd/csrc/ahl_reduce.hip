@@ -59,7 +59,8 @@ __global__ __launch_bounds__(256) void k_sliced_sums(const void* __restrict__ x,
 // out[t] = sqrt((S2 - S^2/n) / (n - 1)); one wave per tile, fixed summation order.
 __global__ __launch_bounds__(256) void k_std_finalize(const double* __restrict__ partial,
                                                       int64_t n_blocks, int64_t rows, Tiling tl,
-                                                      float* __restrict__ out) {
+                                                      float* __restrict__ out,
+                                                      const uint32_t* __restrict__ rows_kept) {
   __shared__ double sh[4][2];
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   double s = 0.0, s2 = 0.0;
@@ -85,7 +86,8 @@ __global__ __launch_bounds__(256) void k_std_finalize(const double* __restrict__
   if (tid == 0) {
     s = (sh[0][0] + sh[1][0]) + (sh[2][0] + sh[3][0]);
     s2 = (sh[0][1] + sh[1][1]) + (sh[2][1] + sh[3][1]);
-    const double n = (double)rows * (double)tl.size(t);
+    // all-zero rows add nothing to either sum: leaving them out only changes the count
+    const double n = (double)(rows_kept ? (int64_t)*rows_kept : rows) * (double)tl.size(t);
     double var = (s2 - s * s / n) / (n - 1.0);  // n == 1 gives 0/0 = nan like torch
     if (var < 0.0) var = 0.0;
     out[t] = (float)sqrt(var);
@@ -369,7 +371,7 @@ using namespace ahl;
 // ============================================================================================
 extern "C" {
 
-int ahl_abi_version(void) { return 7; }
+int ahl_abi_version(void) { return 8; }
 const char* ahl_last_hip_error(void) { return ahl::g_err; }
 
 int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
@@ -412,8 +414,43 @@ int ahl_sliced_std(const void* x, int32_t dtype, int64_t rows, int64_t cols, int
     if (vec) hipLaunchKernelGGL((k_sliced_sums<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
     else hipLaunchKernelGGL((k_sliced_sums<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
   });
-  hipLaunchKernelGGL(k_std_finalize, dim3(n_tiles), dim3(256), 0, s, (const double*)ws_partials, nw, rows, tl, out);
+  hipLaunchKernelGGL(k_std_finalize, dim3(n_tiles), dim3(256), 0, s, (const double*)ws_partials, nw, rows, tl, out,
+                     (const uint32_t*)nullptr);
   return check_launch("ahl_sliced_std");
+}
+
+// workspace: [partial sums of ahl_sliced_std | kept-row counter | kept flags, one byte per row]
+int64_t ahl_sliced_std_kept_ws_bytes(int64_t rows, int32_t n_tiles) {
+  return (ahl_sliced_std_ws_bytes(rows, n_tiles) + 255) / 256 * 256 + 256 + rows;
+}
+
+int ahl_sliced_std_kept(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                        const int32_t* tile_ends_host, int32_t n_tiles, float* out, void* ws,
+                        void* stream) {
+  if (!x || !out || !ws || rows <= 0 || cols <= 0 || ld < cols) return AHL_ERR_ARG;
+  Tiling tl;
+  if (!make_tiling(tile_ends_host, n_tiles, cols, &tl)) return AHL_ERR_TILING;
+  hipStream_t s = (hipStream_t)stream;
+  const int rpw = rows_per_wave(rows);
+  const int64_t nw = cdiv(rows, rpw), nb = cdiv(nw * n_tiles, 4);
+  if (nb > 0x7fffffff || cdiv(rows, 4) > 0x7fffffff) return AHL_ERR_ARG;
+  double* partial = (double*)ws;
+  uint32_t* n_kept = (uint32_t*)((char*)ws + (ahl_sliced_std_ws_bytes(rows, n_tiles) + 255) / 256 * 256);
+  uint8_t* kept = (uint8_t*)n_kept + 256;
+  hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, s, n_kept, 0u, 1);
+  AHL_DISPATCH_DTYPE(dtype, {
+    const bool vec = aligned16(x) && (ld % D::EPV == 0);
+    if (vec) {
+      hipLaunchKernelGGL((k_row_nonzero<D, true>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
+      hipLaunchKernelGGL((k_sliced_sums<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, partial);
+    } else {
+      hipLaunchKernelGGL((k_row_nonzero<D, false>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
+      hipLaunchKernelGGL((k_sliced_sums<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, partial);
+    }
+  });
+  hipLaunchKernelGGL(k_std_finalize, dim3(n_tiles), dim3(256), 0, s, (const double*)partial, nw, rows, tl, out,
+                     (const uint32_t*)n_kept);
+  return check_launch("ahl_sliced_std_kept");
 }
 
 int ahl_ir_init_update(void* ir, void* idx, const float* std, int32_t dtype, int32_t n_tiles,

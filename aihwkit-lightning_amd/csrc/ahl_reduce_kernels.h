@@ -47,4 +47,30 @@ __global__ __launch_bounds__(256) void k_tile_minmax(const void* __restrict__ v,
   }
 }
 
+// p[0..n) = v (a fill kernel instead of a memset node, so callers may capture it in a graph)
+static __global__ void k_fill_u32(uint32_t* p, uint32_t v, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// kept[r] = 1 unless every element of row r is zero (-0.0 counts as zero, NaN does not);
+// *n_kept += number of kept rows. One wave per row.
+template <class D, bool VEC>
+__global__ __launch_bounds__(256) void k_row_nonzero(const void* __restrict__ x, int64_t rows,
+                                                     int64_t cols, int64_t ld,
+                                                     uint8_t* __restrict__ kept,
+                                                     uint32_t* __restrict__ n_kept) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  const typename D::elem* row = (const typename D::elem*)x + r * ld;
+  bool any = false;
+  wave_row_foreach<D, VEC>(row, 0, (int32_t)cols, lane, [&](float v) { any |= (v != 0.0f); });
+  const bool keep = __builtin_amdgcn_ballot_w64(any) != 0ull;
+  if (lane == 0) {
+    kept[r] = keep ? 1 : 0;
+    if (keep) atomicAdd(n_kept, 1u);
+  }
+}
+
 }  // namespace ahl

@@ -156,6 +156,37 @@ int ahl_sliced_std(const void* x, int32_t dtype, int64_t rows, int64_t cols, int
                    void* stream);
 int64_t ahl_sliced_std_ws_bytes(int64_t rows, int32_t n_tiles);
 
+/* ---- calibration statistics (inference/calibration/calibration.py:57-152) -------------------
+ * The reference drops the rows of a batch that are entirely zero before it takes a statistic
+ * (`x_input[~(x_input == 0.0).all(-1)]`, calibration.py:95); "kept rows" below are the others. */
+
+/* kept[r] = 1 unless x[r, :] == 0 everywhere (uint8 [rows]); *n_kept = number of kept rows.     */
+int ahl_row_nonzero(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                    uint8_t* kept, uint32_t* n_kept, void* stream);
+
+/* out[t] = unbiased std of x[kept rows, tile t] as float (MOVING_STD, calibration.py:140-142).
+ * ws needs ahl_sliced_std_kept_ws_bytes(rows, n_tiles) bytes.                                  */
+int ahl_sliced_std_kept(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                        const int32_t* tile_ends_host, int32_t n_tiles, float* out, void* ws,
+                        void* stream);
+int64_t ahl_sliced_std_kept_ws_bytes(int64_t rows, int32_t n_tiles);
+
+/* out[t] = torch.quantile(x[kept rows, tile t].float().flatten(), q) (linear interpolation;
+ * NaN if the tile holds a NaN or no row is kept), exact, by radix selection on the device
+ * (MOVING_QUANTILE and CACHE_QUANTILE, calibration.py:133-138, :305-313).
+ * ws needs ahl_sliced_quantile_ws_bytes(rows, n_tiles) bytes.                                  */
+int ahl_sliced_quantile(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
+                        const int32_t* tile_ends_host, int32_t n_tiles, float q, float* out,
+                        void* ws, void* stream);
+int64_t ahl_sliced_quantile_ws_bytes(int64_t rows, int32_t n_tiles);
+
+/* Moving average of the calibrated range (calibration.py:144-147), on the device:
+ *   ir[t] = dtype((float(ir[t]) * idx[t] + float(alpha * val[t])) / (idx[t] + 1)); idx[t] += 1
+ * ir dtype [T], idx int32 [T], val float [T]; val_in_dtype != 0 rounds val to dtype first (a std
+ * that torch returns in the tensor dtype).                                                     */
+int ahl_ir_moving_update(void* ir, int32_t* idx, const float* val, int32_t dtype, int32_t n_tiles,
+                         double alpha, int32_t val_in_dtype, void* stream);
+
 /* Input-range initialisation from data, all tiles, no host sync:
  *   if idx[t] < init_from_data: if std[t] > 0 { ir[t] = (ir[t]*idx[t] + alpha*std[t])/(idx[t]+1);
  *   idx[t] += 1 }  ir[t] = |ir[t]|.   ir and idx are dtype [n_tiles], updated in place.

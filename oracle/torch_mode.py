@@ -13,7 +13,8 @@ op rounds to that dtype exactly as torch does for the reference.
 How the oracle itself is pinned (see ``tests/test_oracle_*.py``): golden vectors written by the
 real reference (``tests/golden/make_golden.py``), the closed forms in the reference's own tests
 (clipping, weight modifier, calibration max, quantisation idempotence), reductions to
-``F.linear`` / brute force, and Philox known-answer vectors.
+``F.linear`` / brute force, ``torch.quantile`` for the quantile restatement, and Philox
+known-answer vectors.
 """
 from dataclasses import dataclass
 from math import sqrt
@@ -395,6 +396,81 @@ def calibrate_max(batches: Sequence[Tensor], in_sizes: Sequence[int]) -> Tensor:
         for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
             cache[t] = max(cache[t], x[:, lo:hi].abs().max())
     return cache
+
+
+def kept_rows(x: Tensor) -> Tensor:
+    """Rows of x[n, K] that are not all zero (calibration.py:94-95)."""
+    x = x.reshape(-1, x.size(-1))
+    return x[~(x == 0.0).all(-1)]
+
+
+def quantile_linear(values: Tensor, q: float) -> Tensor:
+    """q-quantile with linear interpolation of a 1-d fp32 tensor, restated from the definition
+    torch.quantile implements (aten/src/ATen/native/Sorting.cpp, quantile_compute): the rank
+    q * (n - 1) is evaluated in fp32, the two neighbouring order statistics are blended with the
+    two-sided lerp formula. NaN for an empty input or one that holds a NaN."""
+    values = values.float().flatten()
+    n = values.numel()
+    if n == 0 or bool(torch.isnan(values).any()):
+        return torch.tensor(float("nan"))
+    ordered = torch.sort(values).values
+    rank = torch.tensor(q, dtype=torch.float32) * torch.tensor(float(n - 1), dtype=torch.float32)
+    below = torch.floor(rank)
+    weight = rank - below
+    lo = ordered[int(below)]
+    hi = ordered[int(torch.ceil(rank))]
+    diff = hi - lo
+    return lo + weight * diff if float(weight) < 0.5 else hi - diff * (1.0 - weight)
+
+
+def moving_update(ir: Tensor, idx: Tensor, t: int, val: float) -> None:
+    """input_range[t] <- (input_range[t] * idx[t] + val) / (idx[t] + 1); idx[t] += 1, evaluated as
+    the reference does: Python float times an int32 tensor element gives an fp32 0-dim tensor,
+    the result is cast to the range's dtype (calibration.py:144-147)."""
+    old_val = ir[t].item()
+    new_val = (old_val * idx[t] + val) / (idx[t] + 1)
+    ir[t] = new_val.type_as(ir)
+    idx[t] += 1
+
+
+def calibrate_moving(batches: Sequence[Tensor], in_sizes: Sequence[int], kind: str, dtype,
+                     alpha: float = 3.0, q: float = 0.99995) -> Tuple[Tensor, Tensor]:
+    """MOVING_STD / MOVING_QUANTILE (calibration.py:126-147): per batch and tile the statistic
+    of the kept rows (alpha * std in the data dtype, or the quantile of the fp32 values, or the
+    abs-max when q == 1), folded into a running mean that starts from 3.0. Returns the final
+    ranges and the trace of ranges seen before each batch."""
+    n_tiles = len(in_sizes)
+    ir = torch.full((n_tiles,), 3.0, dtype=dtype)
+    idx = torch.zeros(n_tiles, dtype=torch.int32)
+    trace = []
+    for x in batches:
+        trace.append(ir.float().clone())
+        rows = kept_rows(x)
+        for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
+            part = rows[:, lo:hi]
+            if kind == "MovingStd":
+                val = alpha * part.std().item()
+            elif q == 1.0:
+                val = part.abs().max().item()
+            else:
+                val = quantile_linear(part, q).item()
+            moving_update(ir, idx, t, val)
+    return ir, torch.stack(trace)
+
+
+def calibrate_cache_quantile(batches: Sequence[Tensor], in_sizes: Sequence[int], q: float,
+                             max_samples: int, dtype) -> Tensor:
+    """CACHE_QUANTILE (calibration.py:100-110, :305-313): the kept rows of every batch join a
+    cache that is re-drawn to at most max_samples rows with torch.randperm (global CPU
+    generator); the range of a tile is the quantile of the cached fp32 values."""
+    cache = torch.zeros(0, sum(in_sizes))
+    for x in batches:
+        cache = torch.cat([cache, kept_rows(x).float()])
+        cache = cache[torch.randperm(cache.size(0))[:max_samples]]
+    out = torch.empty(len(in_sizes), dtype=dtype)
+    for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
+        out[t] = quantile_linear(cache[:, lo:hi], q).item()
+    return out
 
 
 # --------------------------------------------------------------------------------------------
