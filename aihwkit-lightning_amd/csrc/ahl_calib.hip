@@ -69,9 +69,12 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
                                                      Tiling tl, int rpw, int pass,
                                                      SelState* __restrict__ st,
                                                      uint32_t* __restrict__ hist) {
-  __shared__ uint32_t lh[4][256];
+  // eight copies of the wave's histogram, one per lane residue: the leading digits of real data
+  // fall into a handful of bins, and a single copy would serialise the LDS atomics of a wave
+  __shared__ uint32_t lh[4][8][256];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  for (int i = lane; i < 256; i += 64) lh[w][i] = 0u;
+  for (int i = lane; i < 2048; i += 64) (&lh[w][0][0])[i] = 0u;
+  uint32_t* mine = lh[w][lane & 7];
   const int64_t wave = (int64_t)blockIdx.x * 4 + w;
   const int64_t grp = wave / tl.n_tiles;
   const int32_t t = (int32_t)(wave % tl.n_tiles);
@@ -90,12 +93,14 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
         nan |= (v != v);
         const uint32_t key = f32_key(v);
         // digits above this pass must match the prefix found so far
-        if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&lh[w][(key >> shift) & 255u], 1u);
+        if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1u);
       }
     }
     if (pass == 0 && __builtin_amdgcn_ballot_w64(nan) != 0ull && lane == 0) atomicOr(&st[t].has_nan, 1u);
     for (int i = lane; i < 256; i += 64) {
-      const uint32_t c = lh[w][i];
+      uint32_t c = 0u;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) c += lh[w][j][i];
       if (c) atomicAdd(&hist[t * 256 + i], c);
     }
   }

@@ -79,3 +79,75 @@ def test_full_size_analog_matches_oracle(ir_mode):
             continue
         assert_close_lsb(res[key].float(), ref[key].float(), 1e-2, flip[key], max_frac=1e-3,
                          what=f"{c['name']} {key}")
+
+
+def test_llama_mlp_block_matches_oracle():
+    """Configuration 4 of the baseline: a LLaMA-style MLP block (hidden 3072, intermediate 8192,
+    SiLU gating: down(silu(gate(x)) * up(x))), bf16, 4096 tokens, tiles of 512, 8-bit DAC/ADC,
+    forward + backward through three analog layers, noise off for a deterministic comparison.
+
+    The block composes three layers, so a rounding-boundary tie in one layer's ADC reaches the
+    next layer's input: element-wise bounds do not compose. Compared instead: every layer on the
+    oracle's own input for that layer (element-wise, the path's tolerance), and the block's
+    output and input gradient against the oracle's in the mean (1 % of the mean magnitude).
+    """
+    import torch.nn.functional as F
+    from hip_helpers import make_layer
+    from helpers import oracle_cfg
+    from oracle import torch_mode as om
+
+    hidden, inter, tokens = 3072, 8192, 4096
+    common = dict(dtype="bf16", max_input_size=512, ir_mode="static", inp_res=254, out_res=254,
+                  out_bound=10.0, clip="channel", clip_sigma=2.5, ir_decay=0.01, bias=False)
+    cases = {
+        "gate": case("mlp_gate", M=tokens, K=hidden, N=inter, ir_init=3.0, w_scale=0.02, seed=43, **common),
+        "up": case("mlp_up", M=tokens, K=hidden, N=inter, ir_init=3.0, w_scale=0.02, seed=44, **common),
+        "down": case("mlp_down", M=tokens, K=inter, N=hidden, ir_init=1.0, w_scale=0.02, seed=45, **common),
+    }
+    weights = {k: make_inputs(c)[1] for k, c in cases.items()}
+    x = make_inputs(cases["gate"])[0]
+    g = make_inputs(cases["down"])[3]
+    layers = {k: make_layer(c, inputs=(None, weights[k], None, None)) for k, c in cases.items()}
+
+    # ---- HIP block ----
+    xd = x.cuda().requires_grad_(True)
+    gate, up = layers["gate"](xd), layers["up"](xd)
+    act = F.silu(gate) * up
+    out = layers["down"](act)
+    out.backward(g.cuda())
+    torch.cuda.synchronize()
+
+    # ---- oracle block (explicit backward per layer, torch autograd for the gating) ----
+    torch.set_num_threads(16)
+    ir3 = lambda c: torch.full((len(om.split_sizes(c["K"], 512)),), c["ir_init"], dtype=torch.bfloat16)  # noqa: E731
+    o_gate, s_gate = om.linear_forward(x, weights["gate"], None, oracle_cfg(cases["gate"]), ir3(cases["gate"]), True)
+    o_up, s_up = om.linear_forward(x, weights["up"], None, oracle_cfg(cases["up"]), ir3(cases["up"]), True)
+    gate_r, up_r = o_gate.clone().requires_grad_(True), o_up.clone().requires_grad_(True)
+    act_r = F.silu(gate_r) * up_r
+    o_out, s_down = om.linear_forward(act_r.detach(), weights["down"], None, oracle_cfg(cases["down"]),
+                                      ir3(cases["down"]), True)
+    d_act, dw_down, _, _ = om.linear_backward(g, s_down)
+    act_r.backward(d_act)
+    dx_gate, dw_gate, _, _ = om.linear_backward(gate_r.grad, s_gate)
+    dx_up, dw_up, _, _ = om.linear_backward(up_r.grad, s_up)
+    dx_ref = dx_gate + dx_up
+
+    def mean_close(got, ref, what):
+        got, ref = got.float().cpu(), ref.float()
+        err = float((got - ref).abs().mean()) / float(ref.abs().mean())
+        assert err < 1e-2, f"{what}: mean error {err:.3e} of the mean magnitude"
+
+    # one ADC step of one tile (0.02) moves the bf16 running sum to the neighbouring bf16 value:
+    # 2^-5 for the largest outputs here (magnitude 4 to 8)
+    lsb = 2.0 ** -5
+    assert_close_lsb(gate.detach().float().cpu(), o_gate.float(), 1e-2, lsb, max_frac=1e-4, what="gate out")
+    assert_close_lsb(up.detach().float().cpu(), o_up.float(), 1e-2, lsb, max_frac=1e-4, what="up out")
+    mean_close(out.detach(), o_out, "block output")
+    mean_close(xd.grad, dx_ref, "block input gradient")
+    mean_close(layers["down"].weight.grad, dw_down, "down-projection weight gradient")
+    mean_close(layers["gate"].weight.grad, dw_gate, "gate-projection weight gradient")
+    mean_close(layers["up"].weight.grad, dw_up, "up-projection weight gradient")
+    # the down projection on the oracle's own activations: element-wise
+    down_on_ref = layers["down"](act_r.detach().cuda())
+    assert_close_lsb(down_on_ref.detach().float().cpu(), o_out.float(), 1e-2, lsb, max_frac=1e-4,
+                     what="down out on the oracle's activations")
