@@ -314,11 +314,17 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
             for (int c = 0; c < 4; ++c) { ns[c] = nscale; Bv[c] = B; rv[c] = r; rcpv[c] = rcp; }
             if (IRMODE == AHL_IR_DYNAMIC && (NOISE || bound_on)) {
+              // the four rows of this group are consecutive: one 16-byte LDS read per constant
+              const int rl0 = rbase + 8 * g;
+              if (NOISE) {
+                const f32x4 nr = *(const f32x4*)(rc_t + rl0);
 #pragma unroll
-              for (int c = 0; c < 4; ++c) {
-                const int rl = rbase + 8 * g + c;
-                if (NOISE) ns[c] = wr * rc_t[rl];
-                if (bound_on) Bv[c] = rc_t[128 + rl] * wb;
+                for (int c = 0; c < 4; ++c) ns[c] = wr * nr[c];
+              }
+              if (bound_on) {
+                const f32x4 br = *(const f32x4*)(rc_t + 128 + rl0);
+#pragma unroll
+                for (int c = 0; c < 4; ++c) Bv[c] = br[c] * wb;
               }
               if (NOISE) { rd2(ns[0], ns[1]); rd2(ns[2], ns[3]); }
               if (bound_on) {
