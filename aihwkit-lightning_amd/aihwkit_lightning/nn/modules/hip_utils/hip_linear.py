@@ -225,7 +225,9 @@ class HipLinear(Function):
             x2 if need_x else None, xq if need_dw else None,
             (w_eff if w_eff is not weights else weights.detach()) if need_dx else None,
             keep if want_keep else None, flag if want_keep else None,
-            ir_dev.clone() if ir_mode == L.AHL_IR_STATIC else ir_dev,
+            # while the range is still initialised from data, the next forward rewrites it in
+            # place (possibly before this call's backward): keep this call's values then
+            ir_dev.clone() if (ir_mode == L.AHL_IR_STATIC and init_active) else ir_dev,
             weights_c.detach() if ctx.learned_clip else None,
             wmax.clone() if ctx.learned_clip else None, tile_min if ctx.learned_clip else None,
         )
