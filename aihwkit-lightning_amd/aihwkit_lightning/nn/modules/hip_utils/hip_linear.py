@@ -156,7 +156,7 @@ class HipLinear(Function):
         # kernels do, or the shape does not fit the fast backward at all
         stride = 0
         dense_fwd_ok = len(set(in_sizes)) == 1 and in_sizes[0] % 64 == 0
-        if (inp.dtype == torch.bfloat16 and m_rows > 0 and m_rows % 64 == 0 and n_out % 64 == 0
+        if (inp.dtype == torch.bfloat16 and m_rows > 0 and n_out % 8 == 0
                 and weights_c.data_ptr() % 16 == 0):
             stride = tile_stride(k_in, len(in_sizes), inp.dtype)
             if stride * len(in_sizes) > 4 * k_in or (dense_fwd_ok and not (need_dx or need_dw)):

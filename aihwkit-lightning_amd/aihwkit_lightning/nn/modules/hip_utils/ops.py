@@ -542,7 +542,8 @@ def linear_fwd(
     cfg = _linear_cfg(ref.dtype, icfg, fcfg)
     y = torch.empty((m_rows, n_out), dtype=ref.dtype, device=ref.device)
     # clamp mask: one bit per (tile, row, column), 32 columns of one row per word
-    keep = torch.empty((n_tiles, (n_out + 31) // 32, m_rows) if want_keep else (0,),
+    # rows padded to a multiple of 64 (the kernels never write or use the padding rows)
+    keep = torch.empty((n_tiles, (n_out + 31) // 32, (m_rows + 63) // 64 * 64) if want_keep else (0,),
                        dtype=torch.int32, device=ref.device)
     flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
     L.check(

@@ -60,8 +60,11 @@ AHL_DEV void block_to_tile(int64_t bid, int64_t nb, int64_t nbm, int64_t nbn, in
 // has bit (n % 32) set where the tile-t output of element (m, n) left the ADC range (and so
 // passes no gradient). One 64-lane ballot over a 32x32 MFMA result register yields two such
 // words (rows r and r + 4); the 64 rows of a wave's tile are 256 contiguous bytes.
-AHL_DEV int64_t clamp_plane_words(int64_t M, int64_t N) { return ((N + 31) >> 5) * M; }
-AHL_DEV int64_t clamp_word(int64_t m, int64_t n, int64_t M) { return (n >> 5) * M + m; }
+// The row dimension of the mask is padded to a multiple of 64, so that the words of four
+// consecutive rows are always one aligned 16-byte vector inside the plane, whatever M is.
+AHL_DEV int64_t clamp_rows(int64_t M) { return (M + 63) & ~(int64_t)63; }
+AHL_DEV int64_t clamp_plane_words(int64_t M, int64_t N) { return ((N + 31) >> 5) * clamp_rows(M); }
+AHL_DEV int64_t clamp_word(int64_t m, int64_t n, int64_t M) { return (n >> 5) * clamp_rows(M) + m; }
 
 // ---------------------------------------------------------------------------------------------
 // bf16 <-> f32

@@ -110,11 +110,14 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   int psh = 0;
   const uint16_t* pb[4];
   if (MODE == MODE_DX) {
-    int64_t mq = r0 + 4 * rk_row;          // M is a multiple of 64: a row quad is all in or all out
-    mq = mq < a.M ? mq : a.M - 4;
+    int64_t mq = r0 + 4 * rk_row;          // first row of this thread's quad
+    mq = mq < a.M ? mq : (a.M - 1) & ~(int64_t)3;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) pa[j] = a.g + (mq + j) * a.ldg + rk_cv * 8;  // + l0 (contraction n)
-    if (plane) pk = plane + clamp_word(mq, rk_cv * 8, a.M);                  // + (l0 / 32) * M
+    for (int j = 0; j < 4; ++j) {
+      const int64_t mr = mq + j < a.M ? mq + j : a.M - 1;
+      pa[j] = a.g + mr * a.ldg + rk_cv * 8;                                  // + l0 (contraction n)
+    }
+    if (plane) pk = plane + clamp_word(mq, rk_cv * 8, a.M);                  // + (l0 / 32) * rows
     psh = 8 * (rk_cv & 3);
   } else {
     int64_t n = r0 + km_cv * 8;
@@ -127,10 +130,14 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
 #pragma unroll
   for (int j = 0; j < 4; ++j) pb[j] = a.b + (int64_t)(km_row + 16 * j) * a.ldb + c0 + km_cv * 8;  // + l0 * ldb
   const int64_t a_step = MODE == MODE_DX ? 64 : 64 * a.ldg;
-  const int64_t k_step = MODE == MODE_DX ? 2 * a.M : 64;   // 64 columns = 2 words; or 64 rows
+  const int64_t k_step = MODE == MODE_DX ? 2 * clamp_rows(a.M) : 64;   // 64 columns = 2 words; or 64 rows
   const int64_t b_step = 64 * a.ldb;
+  // l_next: contraction offset of the chunk the next load() fetches. Only the last chunk of a
+  // contraction length that is not a multiple of 64 takes the predicated path: contraction
+  // indices beyond L read as zero (and are never touched in memory).
+  int64_t l_next = 0;
   // this block's share of the contraction: chunks [ch0, ch0 + nchunks)
-  const int chunks_all = (int)(L / 64);
+  const int chunks_all = (int)((L + 63) / 64);  // the last chunk may be partial
   const int per_slice = (chunks_all + a.slices - 1) / a.slices;
   const int ch0 = slice * per_slice;
   const int nchunks = chunks_all - ch0 < per_slice ? chunks_all - ch0 : per_slice;
@@ -141,16 +148,42 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       pb[j] += (int64_t)ch0 * b_step;
     }
     if (pk) pk += (int64_t)ch0 * k_step;
+    l_next = (int64_t)ch0 * 64;
   }
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
   auto load = [&](bool masked) {
-    if (masked) { rawK = ld16(pk); pk += k_step; }
+    if (l_next + 64 <= L) {
+      if (masked) rawK = ld16(pk);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        rawA[j] = ld16(pa[j]);
+        rawB[j] = ld16(pb[j]);
+      }
+    } else {
+      // DX: contraction = columns of g (8 per vector, L a multiple of 8) and rows of W_eff;
+      // DW: contraction = rows of g and of xq
+      const bool a_col_ok = l_next + rk_cv * 8 < L;
+      if (masked) {
+        rawK = zero4;
+        if (MODE == MODE_DW || a_col_ok) rawK = ld16(pk);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool a_ok = MODE == MODE_DX ? a_col_ok : (l_next + 4 * km_row + j < L);
+        const bool b_ok = l_next + km_row + 16 * j < L;
+        rawA[j] = zero4;
+        rawB[j] = zero4;
+        if (a_ok) rawA[j] = ld16(pa[j]);
+        if (b_ok) rawB[j] = ld16(pb[j]);
+      }
+    }
+    if (masked) pk += k_step;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      rawA[j] = ld16(pa[j]);
-      rawB[j] = ld16(pb[j]);
       pa[j] += a_step;
       pb[j] += b_step;
     }
+    l_next += 64;
   };
   // The mask is applied here, after the MFMAs of the current chunk, so that nothing waits for
   // the loads that were issued before them.
@@ -289,7 +322,6 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     ovalid = in_tile < a.dense_tile;
     ocol = ovalid ? (int64_t)t * a.dense_tile + in_tile : 0;
   }
-  const uint16_t* xp = do_ir ? a.x + (r0 + vrow) * a.ldx + ocol : nullptr;
   uint16_t* op = a.out + (r0 + vrow) * a.ldo + ocol;
   {
     char* obase = lds + (wm * 128 + 4 * h) * kOutStride + (wn * 64 + (lane & 31)) * 2;
@@ -311,8 +343,9 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const int row = vrow + 16 * (8 * half + j);
-        // rows beyond the matrix re-read row r0 + vrow, which always exists
-        xr[j] = ld16(xp + (r0 + row < R ? (int64_t)(16 * (8 * half + j)) * a.ldx : 0));
+        // rows beyond the matrix re-read the last row (the values are not used)
+        const int64_t xrow = r0 + row < R ? r0 + row : R - 1;
+        xr[j] = ld16(a.x + xrow * a.ldx + ocol);
       }
     }
 #pragma unroll
@@ -377,14 +410,13 @@ __global__ __launch_bounds__(256) void k_bias_final(const float* partial, int nk
   dbias[n] = (uint16_t)f32_to_bf16_bits(s);
 }
 
-// Whether the fast backward kernels can be used: bf16, equal K-tiles of a multiple of 256,
-// 16-byte aligned rows everywhere.
+// Whether the fast backward kernels can be used: bf16, equal K-tiles of a multiple of 256
+// columns, output channels in whole 16-byte vectors. Any number of rows M: a contraction length
+// that is not a multiple of 64 ends in one predicated chunk.
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N) {
   if (dtype != AHL_BF16) return false;
   if (tl.extra != 0 || tl.base % 256 != 0) return false;
-  // the contraction length (N for dX, M for dW) must be a multiple of 64 so that the hot loop
-  // needs no predicates; output rows beyond the matrix are handled by clamping the row index
-  return K % 256 == 0 && N % 64 == 0 && M % 64 == 0;
+  return K % 256 == 0 && N % 8 == 0 && N >= 8 && M >= 1;
 }
 
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
@@ -412,7 +444,7 @@ int fast_dw_slices(int64_t M, int64_t K, int64_t N) {
   const int64_t tiles = cdiv(N, 256) * (K / 256);
   if (tiles >= 128) return 1;
   int64_t s = cdiv(256, tiles);
-  const int64_t chunks = M / 64, most = chunks / 8;
+  const int64_t chunks = cdiv(M, 64), most = chunks / 8;
   if (s > most) s = most;
   if (s <= 1) return 1;
   // every slice gets ceil(chunks / s) chunks; drop the slices that would be left empty

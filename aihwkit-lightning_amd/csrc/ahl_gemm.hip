@@ -847,7 +847,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     // `stride` columns, copy the data columns of the result into the dense dx
     const int64_t stride = cfg->tile_stride, padded = (int64_t)n_tiles * stride;
     if (stride < widest_tile(tl) || ldw < padded || padded > 0x3fffffff) return AHL_ERR_ARG;
-    if (cfg->dtype != AHL_BF16 || M % 64 != 0 || N % 64 != 0 || !aligned16(g) || !aligned16(w_eff) ||
+    if (cfg->dtype != AHL_BF16 || N % 8 != 0 || N < 8 || !aligned16(g) || !aligned16(w_eff) ||
         ldg % 8 != 0 || ldw % 8 != 0 || (keep && !aligned16(keep)))
       return AHL_ERR_UNSUPPORTED;
     const Tiling ptl{n_tiles, (int32_t)stride, 0};
@@ -960,7 +960,7 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
     // workspace, then the data columns are copied into the dense dw
     const int64_t stride = cfg->tile_stride, padded = (int64_t)n_tiles * stride;
     if (!xq || stride < widest_tile(tl) || ldxq < padded || padded > 0x3fffffff) return AHL_ERR_ARG;
-    if (cfg->dtype != AHL_BF16 || M % 64 != 0 || N % 64 != 0 || !aligned16(g) || !aligned16(xq) ||
+    if (cfg->dtype != AHL_BF16 || N % 8 != 0 || N < 8 || !aligned16(g) || !aligned16(xq) ||
         ldg % 8 != 0 || ldxq % 8 != 0 || (keep && !aligned16(keep)))
       return AHL_ERR_UNSUPPORTED;
     void* dwp = (char*)ws + align256(fast_dw_ws_bytes(M, padded, N));

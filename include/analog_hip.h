@@ -278,7 +278,8 @@ int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_i
  *   tile_max float [T]    from ahl_weight_prep, or NULL likewise
  *   bias     dtype [N] or NULL
  *   y        dtype [M, N]
- *   clamp_mask  uint32 [T, ceil(N/32), M] or NULL: bit (n % 32) of word [t][n / 32][m] is set
+ *   clamp_mask  uint32 [T, ceil(N/32), Mr] or NULL, Mr = M rounded up to a multiple of 64 (rows
+ *            beyond M are never written): bit (n % 32) of word [t][n / 32][m] is set
  *            where the tile-t output of element (m, n) left [-bound, bound] and was clamped
  *            (it passes no gradient). Written only when out_bound > 0 and clamp_mask != NULL;
  *            consumed by the two backward entry points.
