@@ -61,7 +61,9 @@ AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-template <int MODE>
+// TAIL: the contraction length is not a multiple of 64 (its last chunk is loaded with
+// predicates); the TAIL = false instantiation has no trace of that in its hot loop.
+template <int MODE, bool TAIL>
 __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   __shared__ float red[8][3];
@@ -152,7 +154,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   }
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   auto load = [&](bool masked) {
-    if (l_next + 64 <= L) {
+    if (!TAIL || l_next + 64 <= L) {
       if (masked) rawK = ld16(pk);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -183,7 +185,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       pa[j] += a_step;
       pb[j] += b_step;
     }
-    l_next += 64;
+    if (TAIL) l_next += 64;
   };
   // The mask is applied here, after the MFMAs of the current chunk, so that nothing waits for
   // the loads that were issued before them.
@@ -432,8 +434,13 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   a.slices = 1; a.split = nullptr;
   const int64_t nb = cdiv(M, 256) * (K / 256);
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
-  hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-  hipLaunchKernelGGL((k_bwd_fast<MODE_DX>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  if (N % 64 == 0) {
+    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    hipLaunchKernelGGL((k_bwd_fast<MODE_DX, false>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  } else {
+    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    hipLaunchKernelGGL((k_bwd_fast<MODE_DX, true>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  }
   return check_launch("ahl_linear_bwd_dx(fast)");
 }
 
@@ -476,8 +483,13 @@ int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint3
       ? (float*)((char*)ws + ((int64_t)slices * (K / 256) * N * 4 + 255) / 256 * 256) : nullptr;
   const int64_t nb = cdiv(N, 256) * (K / 256) * slices;
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
-  hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-  hipLaunchKernelGGL((k_bwd_fast<MODE_DW>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  if (M % 64 == 0) {
+    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    hipLaunchKernelGGL((k_bwd_fast<MODE_DW, false>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  } else {
+    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+    hipLaunchKernelGGL((k_bwd_fast<MODE_DW, true>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  }
   if (slices > 1)
     hipLaunchKernelGGL(k_split_reduce, dim3((unsigned)cdiv(N * K, 1024)), dim3(256), 0, s,
                        (const float*)a.split, slices, N, K, (uint16_t*)dw, lddw);
