@@ -578,6 +578,8 @@ def linear_bwd_dx(
                      dtype=torch.uint8, device=g.device)
     if x is not None:
         x = _rows2d(x, "x")
+        if cfg.tile_stride > 0 and (x.data_ptr() % 16 != 0 or _ld(x) != k_in):
+            x = x.clone(memory_format=torch.contiguous_format)  # same row stride and alignment as dx
     L.check(
         lib.ahl_linear_bwd_dx(
             _ptr(g), _ld(g), _ptr(keep), _ptr(clamp_flag), _ptr(w_eff), _ld(w_eff), _ptr(x),

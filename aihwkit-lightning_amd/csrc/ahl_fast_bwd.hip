@@ -50,6 +50,9 @@ struct BwdArgs {
   int32_t dense_tile;                  // DX: 0, or the true tile width when x and dx are dense
                                        // while W_eff is in the padded tile layout (K, tile then
                                        // describe the padded columns); a multiple of 8
+  int32_t dense_base, dense_extra;     // DX: dense_base > 0: x and dx are dense with the split
+                                       // (base, extra) of any widths; the epilogue then works
+                                       // element by element instead of in 16-byte vectors
   int32_t slices;                      // DW: the contraction (rows m) is cut into this many
                                        // slices, one block each; > 1 when N x K alone gives
                                        // too few blocks to fill the chip
@@ -338,6 +341,60 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
         }
   }
   __syncthreads();
+  if (MODE == MODE_DX && a.dense_base > 0) {
+    // Dense x / dx whose tiles start at arbitrary columns. Per output row the block owns one
+    // contiguous run of dense columns; it is written as 16-byte vectors from the first 16-byte
+    // boundary of dx on (x has the same alignment: the launcher checks ldx == ldo and the base
+    // pointers), the few elements before and after as single 2-byte accesses. Sub-dword
+    // accesses for everything cost more than the padded copies they replace. A half wave
+    // handles one row per pass; wave w owns rows 32 w .. 32 w + 31.
+    const int32_t tw = a.dense_base + (t < a.dense_extra ? 1 : 0);
+    const int64_t dstart = (int64_t)t * a.dense_base + (t < a.dense_extra ? t : a.dense_extra);
+    const int64_t in0 = c0 - (int64_t)t * a.tile;  // block's first column inside the padded tile
+    const int count = (int)(tw - in0 < 256 ? tw - in0 : 256);  // columns with data (may be <= 0)
+    const int hw = lane >> 5, l32 = lane & 31;
+    auto element = [&](float d, float x1) -> float {
+      if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
+        const bool up = x1 >= ir_t, lo = x1 <= -ir_t;
+        if (up) s_up += fminf(d, 0.0f);
+        if (lo) s_lo += fmaxf(d, 0.0f);
+        if (up || lo) cnt += 1.0f;
+      } else {
+        if (x1 > ir_t) s_up += d;
+        if (x1 < -ir_t) s_lo += d;
+      }
+      return fabsf(x1) > ir_t ? 0.0f : d;
+    };
+    for (int rr = 0; rr < 32; rr += 2) {
+      const int row = wave * 32 + rr + hw;
+      if (count <= 0 || r0 + row >= R) continue;
+      const int64_t e0 = (r0 + row) * a.ldo + dstart + in0;   // first element of the run in dx (and x)
+      const int head = (int)((8 - (e0 & 7)) & 7) < count ? (int)((8 - (e0 & 7)) & 7) : count;
+      const int nv = (count - head) >> 3;
+      const int tail0 = head + 8 * nv;                        // first column of the tail
+      const char* lrow = lds + row * kOutStride;
+      if (l32 < nv) {
+        const int j = head + 8 * l32;
+        float d[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d[i] = bf16_bits_to_f32(*(const uint16_t*)(lrow + (j + i) * 2));
+        if (do_ir) {
+          float xv[8];
+          BF16::unpack(ld16(a.x + e0 + j), xv);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) d[i] = element(d[i], xv[i]);
+        }
+        st16(a.out + e0 + j, BF16::pack(d));
+      }
+      // up to 7 elements before the first and after the last vector
+      const int j1 = l32 < head ? l32 : tail0 + (l32 - head);
+      if (l32 < head + (count - tail0)) {
+        float d = bf16_bits_to_f32(*(const uint16_t*)(lrow + j1 * 2));
+        if (do_ir) d = element(d, bf16_bits_to_f32(a.x[e0 + j1]));
+        a.out[e0 + j1] = (uint16_t)f32_to_bf16_bits(d);
+      }
+    }
+  } else
 #pragma unroll
   for (int half = 0; half < 2; ++half) {
     u32x4 xr[8];
@@ -424,9 +481,12 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
-                   const Tiling& tl, int ir_static, int32_t dense_tile, hipStream_t s) {
+                   const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
+                   hipStream_t s) {
   BwdArgs a;
   a.dense_tile = dense_tile;
+  a.dense_base = dense ? dense->base : 0;
+  a.dense_extra = dense ? dense->extra : 0;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
@@ -478,6 +538,7 @@ int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   a.out = (uint16_t*)dw; a.ldo = lddw; a.partial = nullptr;
   a.bias_partial = dbias ? bias_partial : nullptr;
   a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = 0; a.dense_tile = 0;
+  a.dense_base = 0; a.dense_extra = 0;
   a.slices = slices;
   a.split = slices > 1
       ? (float*)((char*)ws + ((int64_t)slices * (K / 256) * N * 4 + 255) / 256 * 256) : nullptr;

@@ -699,7 +699,8 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
-                   const Tiling& tl, int ir_static, int32_t dense_tile, hipStream_t s);
+                   const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
+                   hipStream_t s);
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
@@ -812,7 +813,7 @@ static int64_t dx_partial_bytes(int64_t M, int64_t K, int32_t n_tiles) {
   return align256(cdiv(M, kBM) * nkb * 4 * (int64_t)sizeof(float));
 }
 
-// Workspace of the padded-layout backward: [partials | x padded | dx padded]
+// Workspace of the padded-layout backward: the input-range partial sums
 static int64_t dx_padded_partial_bytes(int64_t M, int64_t padded) {
   return align256(cdiv(M, 256) * (padded / 256) * 4 * (int64_t)sizeof(float));
 }
@@ -821,9 +822,9 @@ int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
                                    int64_t tile_stride) {
   if (n_tiles <= 0 || K <= 0 || M <= 0 || N <= 0) return 0;
   const int64_t es = dtype == AHL_BF16 ? 2 : 4;
-  if (tile_stride > 0) {
+  if (tile_stride > 0) {  // only the input-range partial sums; x and dx are used in place
     const int64_t padded = (int64_t)n_tiles * tile_stride;
-    return dx_padded_partial_bytes(M, padded) + 2 * align256(M * padded * es);
+    return dx_padded_partial_bytes(M, padded);
   }
   return dx_partial_bytes(M, K, n_tiles) + align256(K * N * es);  // partials + transposed weights
 }
@@ -843,8 +844,8 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
   hipStream_t s = (hipStream_t)stream;
   float* partial = (float*)ws;
   if (cfg->tile_stride > 0) {
-    // w_eff is in the padded tile layout: pad x, run the MFMA kernel on aligned tiles of
-    // `stride` columns, copy the data columns of the result into the dense dx
+    // w_eff is in the padded tile layout: the MFMA kernel runs on aligned tiles of `stride`
+    // columns and maps its output columns back onto the dense x / dx in its epilogue
     const int64_t stride = cfg->tile_stride, padded = (int64_t)n_tiles * stride;
     if (stride < widest_tile(tl) || ldw < padded || padded > 0x3fffffff) return AHL_ERR_ARG;
     if (cfg->dtype != AHL_BF16 || N % 8 != 0 || N < 8 || !aligned16(g) || !aligned16(w_eff) ||
@@ -852,38 +853,24 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
       return AHL_ERR_UNSUPPORTED;
     const Tiling ptl{n_tiles, (int32_t)stride, 0};
     const int32_t per_tile = (int32_t)(stride / 256);
-    int rc;
-    if (tl.extra == 0 && tl.base % 8 == 0 && lddx % 8 == 0 && aligned16(dx) &&
-        (!is_static || (ldx % 8 == 0 && aligned16(x)))) {
-      // equal tiles of a multiple of 8 columns: the kernel's 16-byte vectors of x and dx map
-      // one to one onto the dense matrices, no padded copies needed
-      rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M,
-                          padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0, tl.base, s);
-      if (rc != AHL_OK) return rc;
-      if (is_static)
-        hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
-                           (const float*)partial, cdiv(M, 256), (int32_t)(padded / 256), per_tile,
-                           per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
-                           cfg->ir_grad_rule);
-      return check_launch("ahl_linear_bwd_dx(fast, padded weights)");
-    }
-    char* p = (char*)ws + dx_padded_partial_bytes(M, padded);
-    void* xpad = p;
-    void* dxp = p + align256(M * padded * 2);
-    if (is_static) {
-      rc = launch_pad_tiles(x, ldx, AHL_BF16, M, tl, stride, xpad, padded, s);
-      if (rc != AHL_OK) return rc;
-    }
-    rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, xpad, padded, ir, dxp, padded, partial,
-                        M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, s);
+    // x and dx stay dense. Equal tiles of a multiple of 8 columns: the kernel's 16-byte vectors
+    // of x and dx map one to one onto the dense matrices; any other split: its epilogue works
+    // element by element (coalesced 2-byte accesses). No padded copies either way.
+    const bool vectors = tl.extra == 0 && tl.base % 8 == 0 && lddx % 8 == 0 && aligned16(dx) &&
+                         (!is_static || (ldx % 8 == 0 && aligned16(x)));
+    // the element-wise epilogue addresses x and dx with one offset and aligns its vectors on dx
+    if (!vectors && (!aligned16(dx) || (is_static && (!aligned16(x) || ldx != lddx))))
+      return AHL_ERR_UNSUPPORTED;
+    const int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial,
+                                  M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0,
+                                  vectors ? tl.base : 0, vectors ? nullptr : &tl, s);
     if (rc != AHL_OK) return rc;
-    if (is_static) {
+    if (is_static)
       hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
                          (const float*)partial, cdiv(M, 256), (int32_t)(padded / 256), per_tile,
                          per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
                          cfg->ir_grad_rule);
-    }
-    return launch_unpad_tiles(dxp, padded, AHL_BF16, M, K, tl, stride, dx, lddx, s);
+    return check_launch("ahl_linear_bwd_dx(fast, padded weights)");
   }
   void* wt = (char*)ws + dx_partial_bytes(M, K, n_tiles);
   const bool fast = fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(w_eff) &&
@@ -892,7 +879,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
     int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
-                            N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, s);
+                            N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, nullptr, s);
     if (rc != AHL_OK) return rc;
     if (is_static) {
       const int32_t per_tile = tl.base / 256;

@@ -299,8 +299,8 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
  *   otherwise dx = d, ir_grad untouched.
  *   clamp_flag: NULL, or the flag written by ahl_linear_fwd (the mask is ignored when it reads 0).
  *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, N, n_tiles, dtype, cfg->tile_stride) bytes.
- *   With cfg->tile_stride > 0, w_eff is in the padded tile layout (x and dx stay dense; the
- *   call pads and un-pads them inside the workspace); needs bf16 and M, N multiples of 64.
+ *   With cfg->tile_stride > 0, w_eff is in the padded tile layout (x and dx stay dense: the
+ *   kernel maps its columns back in the epilogue); needs bf16 and N a multiple of 8.
  * Slot of TritonLinear.backward, triton_utils/triton_linear.py:695-764.                  */
 int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* clamp_mask, const uint32_t* clamp_flag,
                       const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
