@@ -225,15 +225,19 @@ __global__ __launch_bounds__(256) void k_col2im(const void* __restrict__ dcols, 
   D::store(dx, idx, acc);
 }
 
-// Tiled variant: a block computes 64 consecutive input elements of one image row for 8
-// channels. Every patch row that can contribute lies, for each kernel offset (kd, kh), in one
-// contiguous range of output columns; the block stages those ranges' entries of its 8 channels
-// (8 * kvol contiguous entries per patch row, loaded as 16-byte vectors) in LDS and then sums from
-// LDS, in the same ascending kernel-offset order as k_col2im, so both give the same bits.
+// Tiled variant: a block computes a patch of rpb rows x cpb columns (rpb * cpb = 64; cpb is the
+// smallest power of two that covers the image width, at most 64, so narrow images still fill
+// the lanes) of one image plane for 8 channels. Every patch row that can contribute lies in a
+// small window of output rows and a contiguous range of output columns; the block stages that
+// window's entries of its 8 channels (8 * kvol contiguous entries per patch row, loaded as
+// 16-byte vectors) in LDS once and then sums from LDS, in the same ascending kernel-offset order
+// as k_col2im, so both give the same bits.
 struct FoldPlan {
-  int32_t ow_span;   // staged output columns per (kd, kh)
-  int32_t row_vecs;  // 16-byte vectors per staged patch row (8 * kvol entries)
-  int32_t w_tiles;   // blocks along the input row
+  int32_t cpb, rpb;   // columns and rows of the image patch of a block
+  int32_t ow_span;    // staged output columns
+  int32_t oh_span;    // staged output rows
+  int32_t row_vecs;   // 16-byte vectors per staged patch row (8 * kvol entries)
+  int32_t w_tiles, h_tiles;
 };
 
 template <class D>
@@ -244,51 +248,51 @@ __global__ __launch_bounds__(512) void k_col2im_tiled(const void* __restrict__ d
   constexpr int EPV = D::EPV;
   extern __shared__ __attribute__((aligned(16))) char fold_lds[];
   const int tid = threadIdx.x;
-  // block -> (image b, channel group, d, h, column tile)
+  // block -> (image b, channel group, d, row tile, column tile)
   int64_t r = blockIdx.x;
   const int32_t wt = (int32_t)(r % fp.w_tiles);
   r /= fp.w_tiles;
-  const int32_t h = (int32_t)(r % g.in[1]);
-  r /= g.in[1];
+  const int32_t ht = (int32_t)(r % fp.h_tiles);
+  r /= fp.h_tiles;
   const int32_t d = (int32_t)(r % g.in[0]);
   r /= g.in[0];
   const int32_t cg = (int32_t)(r % (g.C / 8));
   const int64_t b = r / (g.C / 8);
-  const int32_t w0 = wt * 64;
-  const int32_t w_last = (w0 + 63 < g.in[2] ? w0 + 63 : g.in[2] - 1);
-  // output columns that can touch [w0, w_last]: ow = (w + pad - kw * dil) / str
-  const int32_t reach = (g.ker[2] - 1) * g.dil[2];
-  int32_t ow_min = w0 + g.pad[2] - reach;
+  const int32_t w0 = wt * fp.cpb, h0 = ht * fp.rpb;
+  const int32_t w_last = (w0 + fp.cpb - 1 < g.in[2] ? w0 + fp.cpb - 1 : g.in[2] - 1);
+  const int32_t h_last = (h0 + fp.rpb - 1 < g.in[1] ? h0 + fp.rpb - 1 : g.in[1] - 1);
+  // output columns / rows that can touch the patch: o = (i + pad - k * dil) / str
+  int32_t ow_min = w0 + g.pad[2] - (g.ker[2] - 1) * g.dil[2];
   ow_min = ow_min <= 0 ? 0 : (ow_min + g.str[2] - 1) / g.str[2];
   int32_t ow_max = (w_last + g.pad[2]) / g.str[2];
   if (ow_max > g.out[2] - 1) ow_max = g.out[2] - 1;
-  const int32_t span = ow_max - ow_min + 1;  // <= fp.ow_span by construction; may be <= 0
+  int32_t oh_min = h0 + g.pad[1] - (g.ker[1] - 1) * g.dil[1];
+  oh_min = oh_min <= 0 ? 0 : (oh_min + g.str[1] - 1) / g.str[1];
+  int32_t oh_max = (h_last + g.pad[1]) / g.str[1];
+  if (oh_max > g.out[1] - 1) oh_max = g.out[1] - 1;
+  const int32_t wspan = ow_max - ow_min + 1, hspan = oh_max - oh_min + 1;  // <= the plan's spans
   const int32_t row_bytes = fp.row_vecs * 16;
   const int32_t kbase = cg * 8 * g.kvol;       // first patch entry of the channel group
-  // ---- stage: for every (kd, kh) with a valid output row, `span` patch rows ----
-  const int32_t combos = g.ker[0] * g.ker[1];
-  const int32_t vec_total = combos * fp.ow_span * fp.row_vecs;
+  // ---- stage: for every kd with a valid output plane, hspan x wspan patch rows ----
+  const int32_t vec_total = g.ker[0] * fp.oh_span * fp.ow_span * fp.row_vecs;
   for (int32_t v = tid; v < vec_total; v += 512) {
     const int32_t vc = v % fp.row_vecs;
     int32_t q = v / fp.row_vecs;
     const int32_t oi = q % fp.ow_span;
     q /= fp.ow_span;
-    const int32_t kh = q % g.ker[1], kd = q / g.ker[1];
-    const int32_t td = d + g.pad[0] - kd * g.dil[0], th = h + g.pad[1] - kh * g.dil[1];
-    u32x4 val = {0u, 0u, 0u, 0u};
-    if (oi < span && td >= 0 && th >= 0 && td % g.str[0] == 0 && th % g.str[1] == 0) {
-      const int32_t od = td / g.str[0], oh = th / g.str[1];
-      if (od < g.out[0] && oh < g.out[1]) {
-        const int64_t l = ((int64_t)od * g.out[1] + oh) * g.out[2] + ow_min + oi;
-        val = ld16((const E*)dcols + (b * g.L + l) * ldc + kbase + vc * EPV);
-      }
+    const int32_t hi = q % fp.oh_span, kd = q / fp.oh_span;
+    const int32_t td = d + g.pad[0] - kd * g.dil[0];
+    if (oi < wspan && hi < hspan && td >= 0 && td % g.str[0] == 0 && td / g.str[0] < g.out[0]) {
+      const int64_t l = ((int64_t)(td / g.str[0]) * g.out[1] + oh_min + hi) * g.out[2] + ow_min + oi;
+      *(u32x4*)(fold_lds + (((int64_t)kd * fp.oh_span + hi) * fp.ow_span + oi) * row_bytes + vc * 16) =
+          ld16((const E*)dcols + (b * g.L + l) * ldc + kbase + vc * EPV);
     }
-    *(u32x4*)(fold_lds + ((int64_t)(kd * g.ker[1] + kh) * fp.ow_span + oi) * row_bytes + vc * 16) = val;
   }
   __syncthreads();
-  // ---- sum: thread = (channel tid / 64 of the group, column tid % 64) ----
-  const int32_t w = w0 + (tid & 63), cl = tid >> 6;
-  if (w >= g.in[2]) return;
+  // ---- sum: thread = (channel tid / 64 of the group, pixel tid % 64 of the patch) ----
+  const int32_t pix = tid & 63, cl = tid >> 6;
+  const int32_t w = w0 + pix % fp.cpb, h = h0 + pix / fp.cpb;
+  if (w >= g.in[2] || h >= g.in[1]) return;
   float acc = 0.f;
   for (int32_t kd = 0; kd < g.ker[0]; ++kd) {
     const int32_t td = d + g.pad[0] - kd * g.dil[0];
@@ -296,7 +300,8 @@ __global__ __launch_bounds__(512) void k_col2im_tiled(const void* __restrict__ d
     for (int32_t kh = 0; kh < g.ker[1]; ++kh) {
       const int32_t th = h + g.pad[1] - kh * g.dil[1];
       if (th < 0 || th % g.str[1] != 0 || th / g.str[1] >= g.out[1]) continue;
-      const char* rows = fold_lds + (int64_t)(kd * g.ker[1] + kh) * fp.ow_span * row_bytes;
+      const char* rows = fold_lds +
+          (((int64_t)kd * fp.oh_span + (th / g.str[1] - oh_min)) * fp.ow_span) * row_bytes;
       for (int32_t kw = 0; kw < g.ker[2]; ++kw) {
         const int32_t tw = w + g.pad[2] - kw * g.dil[2];
         if (tw < 0 || tw % g.str[2] != 0) continue;
@@ -404,14 +409,19 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
   {
     const int epv = dtype == AHL_BF16 ? 8 : 4;
     const int64_t row_entries = 8 * (int64_t)g.kvol;
-    // widest range of output columns one block of 64 input columns can reach
-    const int64_t ow_span = (63 + (int64_t)(g.ker[2] - 1) * g.dil[2]) / g.str[2] + 2;
-    const int64_t lds_bytes = (int64_t)g.ker[0] * g.ker[1] * ow_span * row_entries * (dtype == AHL_BF16 ? 2 : 4);
-    const int64_t w_tiles = cdiv(g.in[2], 64);
-    const int64_t tblocks = (int64_t)g.B * (g.C / 8) * g.in[0] * g.in[1] * w_tiles;
+    int32_t cpb = 64;
+    while (cpb > 8 && cpb / 2 >= g.in[2]) cpb /= 2;
+    const int32_t rpb = 64 / cpb;
+    // widest window of output columns / rows that one block's image patch can reach
+    const int64_t ow_span = (cpb - 1 + (int64_t)(g.ker[2] - 1) * g.dil[2]) / g.str[2] + 2;
+    const int64_t oh_span = (rpb - 1 + (int64_t)(g.ker[1] - 1) * g.dil[1]) / g.str[1] + 2;
+    const int64_t lds_bytes = (int64_t)g.ker[0] * oh_span * ow_span * row_entries * (dtype == AHL_BF16 ? 2 : 4);
+    const int64_t w_tiles = cdiv(g.in[2], cpb), h_tiles = cdiv(g.in[1], rpb);
+    const int64_t tblocks = (int64_t)g.B * (g.C / 8) * g.in[0] * h_tiles * w_tiles;
     if ((dtype == AHL_BF16 || dtype == AHL_F32) && g.C % 8 == 0 && row_entries % epv == 0 &&
         ldc % epv == 0 && aligned16(dcols) && lds_bytes <= 96 * 1024 && tblocks <= 0x7fffffff) {
-      FoldPlan fp{(int32_t)ow_span, (int32_t)(row_entries / epv), (int32_t)w_tiles};
+      FoldPlan fp{cpb, rpb, (int32_t)ow_span, (int32_t)oh_span, (int32_t)(row_entries / epv),
+                  (int32_t)w_tiles, (int32_t)h_tiles};
       AHL_DISPATCH_DTYPE(dtype, {
         hipFuncSetAttribute((const void*)k_col2im_tiled<D>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);

@@ -36,6 +36,9 @@ GEOMS = [
     (2, 16, (1, 17, 131), (1, 3, 5), (1, 2, 3), (0, 1, 2), (1, 2, 2)),  # strides and dilations
     (1, 8, (1, 5, 200), (1, 1, 7), (1, 1, 4), (0, 0, 0), (1, 1, 1)),   # stride > 1 along the row
     (3, 24, (1, 12, 12), (1, 1, 1), (1, 1, 1), (0, 0, 0), (1, 1, 1)),   # 1 x 1 kernel
+    (2, 8, (1, 9, 7), (1, 3, 3), (1, 2, 1), (0, 1, 1), (1, 1, 1)),     # narrow image: 8 x 8 pixel patches
+    (1, 8, (2, 30, 28), (2, 5, 3), (1, 3, 2), (0, 2, 1), (1, 1, 1)),   # 2 x 32 patches, strides, 3-d
+    (2, 16, (1, 14, 14), (1, 3, 3), (1, 1, 1), (0, 1, 1), (1, 2, 2)),  # 4 x 16 patches, dilation
 ]
 
 
