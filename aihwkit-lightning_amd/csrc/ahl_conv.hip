@@ -153,17 +153,32 @@ __global__ __launch_bounds__(256) void k_im2col_tiled(const E* __restrict__ x, E
   const E* xb = x + b * g.C * g.in[0] * plane;
   E* trow = (E*)tile;
   constexpr int RS = 33 * 4 / (int)sizeof(E);  // tile row stride in entries
-  for (int kk = wave; kk < KT; kk += 4) {
-    const int32_t k = k0 + kk;  // uniform over the wave
-    E val = (E)0;
+  // (channel, kd * dil, kh * dil, kw * dil) of the tile's patch entries, decomposed once per
+  // block instead of once per load (three integer divisions each); channel < 0: beyond K
+  __shared__ int32_t entry[KT][4];
+  if (tid < KT) {
+    const int32_t k = k0 + tid;
+    int32_t c = -1, kd = 0, kh = 0, kw = 0;
     if (k < g.K) {
-      const int32_t c = k / g.kvol;
+      c = k / g.kvol;
       int32_t r = k - c * g.kvol;
-      const int32_t kw = r % g.ker[2];
+      kw = r % g.ker[2];
       r /= g.ker[2];
-      const int32_t kh = r % g.ker[1];
-      const int32_t kd = r / g.ker[1];
-      const int32_t id = id0 + kd * g.dil[0], ih = ih0 + kh * g.dil[1], iw = iw0 + kw * g.dil[2];
+      kh = r % g.ker[1];
+      kd = r / g.ker[1];
+    }
+    entry[tid][0] = c;
+    entry[tid][1] = kd * g.dil[0];
+    entry[tid][2] = kh * g.dil[1];
+    entry[tid][3] = kw * g.dil[2];
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (int kk = wave; kk < KT; kk += 4) {
+    const int32_t c = entry[kk][0];  // uniform over the wave
+    E val = (E)0;
+    if (c >= 0) {
+      const int32_t id = id0 + entry[kk][1], ih = ih0 + entry[kk][2], iw = iw0 + entry[kk][3];
       if (id >= 0 && id < g.in[0] && ih >= 0 && ih < g.in[1] && iw >= 0 && iw < g.in[2])
         val = xb[((int64_t)c * g.in[0] + id) * plane + (int64_t)ih * g.in[2] + iw];
     }
@@ -225,6 +240,22 @@ __global__ __launch_bounds__(256) void k_col2im(const void* __restrict__ dcols, 
   D::store(dx, idx, acc);
 }
 
+// Quotient and remainder of a small non-negative int by a run-time divisor through the fp32
+// reciprocal (exact for a < 2^22 after one correction step): a handful of instructions instead
+// of the ~40 of an integer division, which otherwise dominate the address arithmetic below.
+struct SmallDiv {
+  int32_t d;
+  float inv;
+  AHL_DEV int32_t quot(int32_t a) const {
+    int32_t q = (int32_t)((float)a * inv);
+    const int32_t r = a - q * d;
+    if (r >= d) ++q;
+    if (r < 0) --q;
+    return q;
+  }
+};
+static SmallDiv make_small_div(int32_t d) { return SmallDiv{d, 1.0f / (float)d}; }
+
 // Tiled variant: a block computes a patch of rpb rows x cpb columns (rpb * cpb = 64; cpb is the
 // smallest power of two that covers the image width, at most 64, so narrow images still fill
 // the lanes) of one image plane for 8 channels. Every patch row that can contribute lies in a
@@ -238,6 +269,7 @@ struct FoldPlan {
   int32_t oh_span;    // staged output rows
   int32_t row_vecs;   // 16-byte vectors per staged patch row (8 * kvol entries)
   int32_t w_tiles, h_tiles;
+  SmallDiv by_row_vecs, by_ow_span, by_oh_span, by_cpb, by_str[3];
 };
 
 template <class D>
@@ -276,14 +308,16 @@ __global__ __launch_bounds__(512) void k_col2im_tiled(const void* __restrict__ d
   // ---- stage: for every kd with a valid output plane, hspan x wspan patch rows ----
   const int32_t vec_total = g.ker[0] * fp.oh_span * fp.ow_span * fp.row_vecs;
   for (int32_t v = tid; v < vec_total; v += 512) {
-    const int32_t vc = v % fp.row_vecs;
-    int32_t q = v / fp.row_vecs;
-    const int32_t oi = q % fp.ow_span;
-    q /= fp.ow_span;
-    const int32_t hi = q % fp.oh_span, kd = q / fp.oh_span;
+    int32_t q = fp.by_row_vecs.quot(v);
+    const int32_t vc = v - q * fp.row_vecs;
+    int32_t q2 = fp.by_ow_span.quot(q);
+    const int32_t oi = q - q2 * fp.ow_span;
+    const int32_t kd = fp.by_oh_span.quot(q2);
+    const int32_t hi = q2 - kd * fp.oh_span;
     const int32_t td = d + g.pad[0] - kd * g.dil[0];
-    if (oi < wspan && hi < hspan && td >= 0 && td % g.str[0] == 0 && td / g.str[0] < g.out[0]) {
-      const int64_t l = ((int64_t)(td / g.str[0]) * g.out[1] + oh_min + hi) * g.out[2] + ow_min + oi;
+    const int32_t od = td >= 0 ? fp.by_str[0].quot(td) : -1;
+    if (oi < wspan && hi < hspan && od >= 0 && od * g.str[0] == td && od < g.out[0]) {
+      const int64_t l = ((int64_t)od * g.out[1] + oh_min + hi) * g.out[2] + ow_min + oi;
       *(u32x4*)(fold_lds + (((int64_t)kd * fp.oh_span + hi) * fp.ow_span + oi) * row_bytes + vc * 16) =
           ld16((const E*)dcols + (b * g.L + l) * ldc + kbase + vc * EPV);
     }
@@ -291,22 +325,27 @@ __global__ __launch_bounds__(512) void k_col2im_tiled(const void* __restrict__ d
   __syncthreads();
   // ---- sum: thread = (channel tid / 64 of the group, pixel tid % 64 of the patch) ----
   const int32_t pix = tid & 63, cl = tid >> 6;
-  const int32_t w = w0 + pix % fp.cpb, h = h0 + pix / fp.cpb;
+  const int32_t prow = fp.by_cpb.quot(pix);
+  const int32_t w = w0 + pix - prow * fp.cpb, h = h0 + prow;
   if (w >= g.in[2] || h >= g.in[1]) return;
   float acc = 0.f;
   for (int32_t kd = 0; kd < g.ker[0]; ++kd) {
     const int32_t td = d + g.pad[0] - kd * g.dil[0];
-    if (td < 0 || td % g.str[0] != 0 || td / g.str[0] >= g.out[0]) continue;
+    if (td < 0) continue;
+    const int32_t od = fp.by_str[0].quot(td);
+    if (od * g.str[0] != td || od >= g.out[0]) continue;
     for (int32_t kh = 0; kh < g.ker[1]; ++kh) {
       const int32_t th = h + g.pad[1] - kh * g.dil[1];
-      if (th < 0 || th % g.str[1] != 0 || th / g.str[1] >= g.out[1]) continue;
+      if (th < 0) continue;
+      const int32_t oh = fp.by_str[1].quot(th);
+      if (oh * g.str[1] != th || oh >= g.out[1]) continue;
       const char* rows = fold_lds +
-          (((int64_t)kd * fp.oh_span + (th / g.str[1] - oh_min)) * fp.ow_span) * row_bytes;
+          (((int64_t)kd * fp.oh_span + (oh - oh_min)) * fp.ow_span) * row_bytes;
       for (int32_t kw = 0; kw < g.ker[2]; ++kw) {
         const int32_t tw = w + g.pad[2] - kw * g.dil[2];
-        if (tw < 0 || tw % g.str[2] != 0) continue;
-        const int32_t ow = tw / g.str[2];
-        if (ow >= g.out[2]) continue;
+        if (tw < 0) continue;
+        const int32_t ow = fp.by_str[2].quot(tw);
+        if (ow * g.str[2] != tw || ow >= g.out[2]) continue;
         const int32_t k = cl * g.kvol + (kd * g.ker[1] + kh) * g.ker[2] + kw;
         acc += D::load(rows + (int64_t)(ow - ow_min) * row_bytes, k);
       }
@@ -419,9 +458,14 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
     const int64_t w_tiles = cdiv(g.in[2], cpb), h_tiles = cdiv(g.in[1], rpb);
     const int64_t tblocks = (int64_t)g.B * (g.C / 8) * g.in[0] * h_tiles * w_tiles;
     if ((dtype == AHL_BF16 || dtype == AHL_F32) && g.C % 8 == 0 && row_entries % epv == 0 &&
-        ldc % epv == 0 && aligned16(dcols) && lds_bytes <= 96 * 1024 && tblocks <= 0x7fffffff) {
+        ldc % epv == 0 && aligned16(dcols) && lds_bytes <= 96 * 1024 && tblocks <= 0x7fffffff &&
+        g.in[0] + g.pad[0] < (1 << 22) && g.in[1] + g.pad[1] < (1 << 22) &&
+        g.in[2] + g.pad[2] < (1 << 22)) {
       FoldPlan fp{cpb, rpb, (int32_t)ow_span, (int32_t)oh_span, (int32_t)(row_entries / epv),
-                  (int32_t)w_tiles, (int32_t)h_tiles};
+                  (int32_t)w_tiles, (int32_t)h_tiles,
+                  make_small_div((int32_t)(row_entries / epv)), make_small_div((int32_t)ow_span),
+                  make_small_div((int32_t)oh_span), make_small_div(cpb),
+                  {make_small_div(g.str[0]), make_small_div(g.str[1]), make_small_div(g.str[2])}};
       AHL_DISPATCH_DTYPE(dtype, {
         hipFuncSetAttribute((const void*)k_col2im_tiled<D>,
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
