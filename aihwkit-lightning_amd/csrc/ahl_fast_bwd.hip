@@ -460,13 +460,25 @@ __global__ __launch_bounds__(256) void k_split_reduce(const float* __restrict__ 
   *(u32x2*)(out + r * ldo + c) = pk;
 }
 
-__global__ __launch_bounds__(256) void k_bias_final(const float* partial, int nkb, int64_t N,
+// dbias[n] = bf16(sum of the partial rows): 16 columns per block, 16 threads per column that
+// each add every 16th row, combined in a fixed order (the partial rows can be hundreds when the
+// weight gradient is sliced)
+__global__ __launch_bounds__(256) void k_bias_final(const float* partial, int rows, int64_t N,
                                                     uint16_t* dbias) {
-  const int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (n >= N) return;
+  __shared__ float part[16][17];
+  const int col = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  const int64_t n = (int64_t)blockIdx.x * 16 + col;
   float s = 0.0f;
-  for (int i = 0; i < nkb; ++i) s += partial[(int64_t)i * N + n];
-  dbias[n] = (uint16_t)f32_to_bf16_bits(s);
+  if (n < N)
+    for (int i = grp; i < rows; i += 16) s += partial[(int64_t)i * N + n];
+  part[grp][col] = s;
+  __syncthreads();
+  if (grp == 0 && n < N) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sum += part[i][col];
+    dbias[n] = (uint16_t)f32_to_bf16_bits(sum);
+  }
 }
 
 // Whether the fast backward kernels can be used: bf16, equal K-tiles of a multiple of 256
@@ -555,7 +567,7 @@ int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint3
     hipLaunchKernelGGL(k_split_reduce, dim3((unsigned)cdiv(N * K, 1024)), dim3(256), 0, s,
                        (const float*)a.split, slices, N, K, (uint16_t*)dw, lddw);
   if (dbias)
-    hipLaunchKernelGGL(k_bias_final, dim3((unsigned)cdiv(N, 256)), dim3(256), 0, s,
+    hipLaunchKernelGGL(k_bias_final, dim3((unsigned)cdiv(N, 16)), dim3(256), 0, s,
                        (const float*)bias_partial, (int)(K / 256) * slices, N, (uint16_t*)dbias);
   return check_launch("ahl_linear_bwd_dw(fast)");
 }
