@@ -256,3 +256,24 @@ def test_pad_unpad_tiles_bit_exact(rows, k_in, max_size, dtype):
     padded = OPS.pad_tiles(x.cuda(), sizes, stride)
     assert torch.equal(padded.cpu(), want)
     assert torch.equal(OPS.unpad_tiles(padded, sizes, stride).cpu(), x)
+
+
+def test_misaligned_input_with_padded_layout():
+    """An input whose storage does not start on a 16-byte boundary (a view into a larger buffer)
+    through the padded-layout path: the input-gradient kernel wants x aligned like dx, the op
+    makes the copy."""
+    from hip_helpers import make_layer
+
+    c = [s for s in SHAPES if s["name"] == "pad_bf16_extra_tiles"][0]
+    x, w, b, g = make_inputs(c)
+    layer = make_layer(c, inputs=(x, w, b, g))
+    flat = torch.zeros(x.numel() + 8, dtype=x.dtype, device="cuda")
+    flat[3:3 + x.numel()] = x.cuda().reshape(-1)
+    xin = flat[3:3 + x.numel()].view_as(x).requires_grad_(True)
+    assert xin.data_ptr() % 16 != 0
+    out = layer(xin)
+    out.backward(g.cuda())
+    ref = oracle_fwd_bwd(c)
+    res = dict(out=out.detach().cpu(), dx=xin.grad.cpu(), dw=layer.weight.grad.cpu(),
+               db=layer.bias.grad.cpu(), dir=layer.input_range.grad.cpu())
+    check_against(res, ref, c, "misaligned x")
