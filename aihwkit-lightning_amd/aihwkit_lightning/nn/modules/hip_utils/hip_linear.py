@@ -120,6 +120,8 @@ class HipLinear(Function):
         if learned_clip:
             assert learnable_weight_clip is not None, "learnable_weight_clip should not be None"
         need_wmax = bound_on or noise_on or w_noise or w_quant or learned_clip
+        per_channel_bound = rpu_config.clip.type in (WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL,
+                                                     WeightClipType.LEARNABLE_PER_CHANNEL)
         # the clip's gradient comes out of the weight gradient
         clip_needs_grad = learned_clip and ctx.needs_input_grad[11]
         ir_needs_grad = ir_mode == L.AHL_IR_STATIC and input_range.requires_grad
@@ -146,6 +148,9 @@ class HipLinear(Function):
                 weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
                 NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE, res,
                 float(modifier.std_dev), seed, 1, w_noise or w_quant,
+                # per-tile maxima are only read when the ADC bound or the output noise scale with
+                # the whole tile instead of the channel
+                (not bound_on or per_channel_bound) and (not noise_on or fwd.out_noise_per_channel),
             )
             if w_noise or w_quant:
                 w_eff = eff
@@ -164,9 +169,7 @@ class HipLinear(Function):
 
         skip_rounding = 1 if os.environ.get("_AIHWKIT_NO_ROUNDING", False) else 0
         icfg = [
-            ir_mode, int(fwd.out_noise_per_channel),
-            int(rpu_config.clip.type in (WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL,
-                                         WeightClipType.LEARNABLE_PER_CHANNEL)),
+            ir_mode, int(fwd.out_noise_per_channel), int(per_channel_bound),
             int(training), skip_rounding, seed, 0,
             # fast_mode clamps with torch.clamp: its autograd rule instead of the learned-range one
             L.AHL_IR_GRAD_CLAMP if fast else L.AHL_IR_GRAD_LEARNED,

@@ -13,7 +13,7 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
@@ -65,6 +65,7 @@ class AhlModifierCfg(Structure):
         ("res", c_float),
         ("std_dev", c_float),
         ("wmax_given", c_int32),
+        ("skip_tile_stats", c_int32),
         ("seed", c_uint64),
         ("offset", c_uint64),
     ]

@@ -84,7 +84,8 @@ LIB.define("clip_weights(Tensor(a!) w, float sigma, int kind) -> ()")
 LIB.define("col_sum(Tensor x) -> Tensor")
 LIB.define(
     "weight_prep(Tensor w, int[] in_sizes, int quant_type, int noise_type, float res, "
-    "float std_dev, int seed, int offset, bool want_eff) -> (Tensor, Tensor, Tensor, Tensor)"
+    "float std_dev, int seed, int offset, bool want_eff, bool skip_tile_stats=False) "
+    "-> (Tensor, Tensor, Tensor, Tensor)"
 )
 LIB.define("quantize_weights(Tensor(a!) w, int[] in_sizes, int quant_type, float res) -> ()")
 LIB.define(
@@ -410,9 +411,10 @@ def _modifier_cfg(dtype, quant_type, noise_type, res, std_dev, seed, offset) -> 
 
 def weight_prep(
     w: Tensor, in_sizes: List[int], quant_type: int, noise_type: int, res: float, std_dev: float,
-    seed: int, offset: int, want_eff: bool,
+    seed: int, offset: int, want_eff: bool, skip_tile_stats: bool = False,
 ) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
-    """wmax ``[T, N]``, tile max/min ``[T]`` and, if wanted, the modified copy ``[N, K]``."""
+    """wmax ``[T, N]``, tile max/min ``[T]`` and, if wanted, the modified copy ``[N, K]``.
+    ``skip_tile_stats``: the caller does not use tile max/min (they may come back unwritten)."""
     lib = L.load()
     if w.dim() != 2 or w.stride(1) != 1:
         raise HipBackendError("weight must be a row-major 2-D tensor")
@@ -424,6 +426,7 @@ def weight_prep(
     tile_min = torch.empty((n_tiles,), dtype=torch.float32, device=dev)
     w_eff = torch.empty((n_out, n_in) if want_eff else (0,), dtype=w.dtype, device=dev)
     cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset)
+    cfg.skip_tile_stats = int(skip_tile_stats)
     L.check(
         lib.ahl_weight_prep(
             _ptr(w), n_out, n_in, _ld(w), L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(wmax),

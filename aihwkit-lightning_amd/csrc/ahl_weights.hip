@@ -130,6 +130,58 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t block
   }
 }
 
+// Abs-max and per-channel weight noise in one pass over W, for the common training
+// configuration (no quantiser, noise scaled by the channel's own maximum): one wave per (channel,
+// tile) reads its segment as 16-byte vectors, reduces the maximum, writes wmax[t, n] and then
+// the noisy copy -- from registers for segments of up to 1024 inputs, else from a second
+// (cache-resident) read. Same Philox counters and the same arithmetic as k_weight_modify.
+template <class D>
+__global__ __launch_bounds__(256) void k_weight_prep_rows(ModArgs a, void* __restrict__ wmax_out) {
+  constexpr int E = D::EPV;       // elements per 16-byte vector
+  constexpr int VPG = 8 / E;      // vectors per group of 8 inputs (one Philox call)
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t n = wave / a.tl.n_tiles;
+  const int32_t t = (int32_t)(wave % a.tl.n_tiles);
+  if (n >= a.N) return;
+  const int32_t g0 = a.tl.start(t) >> 3, g1 = a.tl.start(t + 1) >> 3;  // groups of 8 inputs
+  const typename D::elem* row = (const typename D::elem*)a.w + n * a.ld;
+  typename D::elem* dst = (typename D::elem*)a.w_eff + n * a.ld_eff;
+  float keep[2][8];
+  float mx = 0.0f;
+  int it = 0;
+  for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
+    float v[8];
+#pragma unroll
+    for (int q = 0; q < VPG; ++q) D::unpack(ld16(row + (int64_t)g * 8 + q * E), v + q * E);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
+    if (it < 2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) keep[it][e] = v[e];
+    }
+  }
+  mx = wave_max(mx);
+  if (lane == 0) D::store(wmax_out, (int64_t)t * a.N + n, mx);
+  const float nstd = D::rd(a.std_dev * D::rd(mx));
+  it = 0;
+  for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
+    float v[8], xi[8];
+    if (it < 2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = keep[it][e];
+    } else {
+#pragma unroll
+      for (int q = 0; q < VPG; ++q) D::unpack(ld16(row + (int64_t)g * 8 + q * E), v + q * E);
+    }
+    normal8(a.seed, a.offset, 1u << 24, (uint32_t)g, (uint32_t)n, xi);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = D::rd(v[e] + D::rd(nstd * D::rd(xi[e])));
+#pragma unroll
+    for (int q = 0; q < VPG; ++q) st16(dst + (int64_t)g * 8 + q * E, D::pack(v + q * E));
+  }
+}
+
 // LSQ backward of the learnable clip: one wave per (channel, tile).
 struct ClipBwdArgs {
   void* dw; int64_t lddw;
@@ -197,6 +249,20 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
     const bool vec = aligned16(w) && (ld % D::EPV == 0);
     if (cdiv(N * tl.n_tiles, 4) > 0x7fffffff) return AHL_ERR_ARG;
     const dim3 grid((unsigned)cdiv(N * tl.n_tiles, 4));
+    // one pass for "abs-max + per-channel noise, no quantiser" on 16-byte aligned tiles
+    if (!cfg->wmax_given && w_eff && cfg->quant_type == AHL_QUANT_NONE &&
+        noise == AHL_NOISE_ADD_NORMAL_PER_CHANNEL && vec && tl.extra == 0 && tl.base % 8 == 0 &&
+        aligned16(w_eff) && ld_eff % D::EPV == 0) {
+      ModArgs a;
+      a.w = w; a.N = N; a.K = K; a.ld = ld; a.tl = tl; a.wmax = nullptr; a.tile_max = nullptr;
+      a.tile_min = nullptr; a.w_eff = w_eff; a.ld_eff = ld_eff; a.quant_type = AHL_QUANT_NONE;
+      a.noise_type = noise; a.n_states = 1.0f; a.maxq = 1.0f; a.std_dev = cfg->std_dev;
+      a.seed = cfg->seed; a.offset = cfg->offset;
+      hipLaunchKernelGGL((k_weight_prep_rows<D>), grid, dim3(256), 0, s, a, wmax);
+      if (!cfg->skip_tile_stats)
+        hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
+      return check_launch("ahl_weight_prep(one pass)");
+    }
     if (cfg->wmax_given) {
       // wmax holds the learnable clip: nothing to reduce
     } else if (vec) {

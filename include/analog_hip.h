@@ -98,6 +98,8 @@ typedef struct AhlModifierCfg {
   int32_t wmax_given; /* != 0: wmax[T, N] is an input (clip.type LEARNABLE_PER_CHANNEL: the
                          learnable_weight_clip takes the place of the per-tile abs-max,
                          torch_utils/torch_linear.py:222-244) instead of being computed            */
+  int32_t skip_tile_stats; /* != 0: the caller does not need tile_max / tile_min (every consumer
+                              scales per channel); ahl_weight_prep may then leave them unwritten  */
   uint64_t seed;
   uint64_t offset;
 } AhlModifierCfg;

@@ -254,3 +254,24 @@ def test_reduction_bound_pipeline_one_matrix():
         batches.append(b)
         ops().running_absmax(b.cuda(), sizes, cache)
     assert torch.equal(cache.cpu(), om.calibrate_max(batches, sizes))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("k_in,max_size", [(1024, 512), (2304, 1152), (640, 128)])
+def test_one_pass_weight_prep_matches_two_pass(k_in, max_size, dtype):
+    """Abs-max + per-channel weight noise in one kernel (aligned rows) must give the bits of the
+    separate abs-max and modifier kernels (taken for a row stride that is not a multiple of 8)."""
+    from aihwkit_lightning.nn.modules.hip_utils import library as L
+
+    sizes = om.split_sizes(k_in, max_size)
+    w = (0.05 * torch.randn(96, k_in, generator=torch.Generator().manual_seed(6))).to(dtype).cuda()
+    padded = torch.zeros(96, k_in + 3, dtype=dtype, device="cuda")
+    padded[:, :k_in] = w
+    args = (sizes, L.AHL_QUANT_NONE, L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.05, 77, 1, True)
+    one = ops().weight_prep(w, *args)
+    two = ops().weight_prep(padded[:, :k_in], *args)
+    for a, b, what in zip(one, two, ("wmax", "tile_max", "tile_min", "w_eff")):
+        assert torch.equal(a, b), what
+    assert not torch.equal(one[3], w), "the noise must change the weights"
+    skipped = ops().weight_prep(w, *args, True)
+    assert torch.equal(skipped[0], one[0]) and torch.equal(skipped[3], one[3])
