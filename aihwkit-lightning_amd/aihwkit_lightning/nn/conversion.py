@@ -1,11 +1,10 @@
 """Swap the digital layers of a model for their analog counterparts and back (reference
 ``nn/conversion.py:37-300``): ``Linear`` and ``Conv1d/2d/3d`` map onto the layers built on the HIP
-operator, ``Sequential`` onto ``AnalogSequential``; the recurrent layers of the reference are not
-part of this build and stay digital."""
+operator, ``Sequential`` onto ``AnalogSequential``, ``RNN`` / ``LSTM`` / ``GRU`` onto ``AnalogRNN``."""
 from copy import deepcopy
 from typing import Callable, Dict, List, Optional, Set, Union
 
-from torch.nn import Conv1d, Conv2d, Conv3d, Linear, Module, Sequential
+from torch.nn import GRU, LSTM, RNN, Conv1d, Conv2d, Conv3d, Linear, Module, Sequential
 
 from ..exceptions import ArgumentError
 from ..simulator.configs import TorchInferenceRPUConfig
@@ -13,6 +12,7 @@ from .modules.base import AnalogLayerBase
 from .modules.container import AnalogSequential, AnalogWrapper
 from .modules.conv import AnalogConv1d, AnalogConv2d, AnalogConv3d
 from .modules.linear import AnalogLinear
+from .modules.rnn.rnn import AnalogRNN
 
 _DEFAULT_CONVERSION_MAP = {
     Linear: AnalogLinear,
@@ -20,6 +20,9 @@ _DEFAULT_CONVERSION_MAP = {
     Conv2d: AnalogConv2d,
     Conv3d: AnalogConv3d,
     Sequential: AnalogSequential,
+    LSTM: AnalogRNN,
+    GRU: AnalogRNN,
+    RNN: AnalogRNN,
 }
 _DEFAULT_DIGITAL_CONVERSION_SET = {*_DEFAULT_CONVERSION_MAP.values()}
 

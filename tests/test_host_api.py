@@ -195,9 +195,9 @@ def test_convert_to_analog_and_back():
     assert isinstance(analog, AnalogWrapper)
     assert isinstance(analog.conv1, AnalogConv1d) and isinstance(analog.conv2, AnalogConv2d)
     assert isinstance(analog.seq, AnalogSequential) and isinstance(analog.seq[0], AnalogLinear)
-    assert isinstance(analog.rnn, torch.nn.GRU), "recurrent layers stay digital in this build"
+    assert isinstance(analog.rnn, _rnn_classes()[0])
     assert isinstance(model.conv1, torch.nn.Conv1d), "without inplace the model is copied"
-    assert len(list(analog.analog_layers())) == 4
+    assert len(list(analog.analog_layers())) == 6
     assert analog.conv1.rpu_config is not analog.conv2.rpu_config
 
     untouched = convert_to_analog(model, _cfg(), conversion_map={})
@@ -239,3 +239,118 @@ def test_tile_stride_rule():
     assert tile_stride(768, 2, torch.bfloat16) == 512         # tiles of 384
     assert tile_stride(1003, 4, torch.bfloat16) == 256
     assert tile_stride(11008, 22, torch.float32) == 0
+
+
+# ---------------------------------------------------------------------------- recurrent layers
+def _rnn_classes():
+    from aihwkit_lightning.nn import (AnalogGRUCell, AnalogLSTMCell, AnalogLSTMCellCombinedWeight,
+                                      AnalogRNN, AnalogVanillaRNNCell)
+    return AnalogRNN, AnalogVanillaRNNCell, AnalogLSTMCell, AnalogGRUCell, AnalogLSTMCellCombinedWeight
+
+
+def test_rnn_module_tree_and_projection_shapes():
+    """reference nn/modules/rnn/rnn.py:169-214, cells.py: the tree is
+    rnn.layers[i](.directions[d]).cell.weight_ih / weight_hh with gate_count * hidden rows."""
+    AnalogRNN, Vanilla, Lstm, Gru, Combined = _rnn_classes()
+    for cell, gates in ((Vanilla, 1), (Lstm, 4), (Gru, 3)):
+        net = AnalogRNN(cell, 10, 20, num_layers=2, bidir=True, rpu_config=_cfg(max_input_size=16))
+        first = net.rnn.layers[0].directions[1].cell
+        second = net.rnn.layers[1].directions[0].cell
+        assert isinstance(first, cell)
+        assert first.weight_ih.weight.shape == (gates * 20, 10)
+        assert first.weight_hh.weight.shape == (gates * 20, 20)
+        assert second.weight_ih.weight.shape == (gates * 20, 40)
+        assert first.weight_hh.in_sizes == [10, 10]
+        assert len(list(net.analog_layers())) == 8
+        # torch's initialisation range
+        assert float(first.weight_ih.weight.detach().abs().max()) <= 1 / 20 ** 0.5
+    net = AnalogRNN(Combined, 10, 20, rpu_config=_cfg())
+    assert net.rnn.layers[0].cell.weight.weight.shape == (80, 30)
+    state = net.get_zero_state(3)[0]
+    assert state.hx.shape == (3, 20) and state.cx.shape == (3, 20)
+    assert AnalogRNN(Gru, 4, 5, rpu_config=_cfg()).get_zero_state(2)[0].cx is None
+
+
+def test_rnn_rejects_what_the_reference_rejects():
+    AnalogRNN, _, Lstm, _, _ = _rnn_classes()
+    with pytest.raises(RuntimeError, match="batch_first"):
+        AnalogRNN(Lstm, 4, 5, batch_first=True, rpu_config=_cfg())
+    with pytest.raises(RuntimeError, match="proj_size"):
+        AnalogRNN(Lstm, 4, 5, proj_size=2, rpu_config=_cfg())
+    with pytest.warns(UserWarning, match="dropout"):
+        AnalogRNN(Lstm, 4, 5, dropout=0.5, rpu_config=_cfg())
+    net = AnalogRNN(Lstm, 4, 5, num_layers=2, rpu_config=_cfg())
+    with pytest.raises(RuntimeError, match="2D or 3D"):
+        net(torch.zeros(4))
+    with pytest.raises(RuntimeError, match="Expecting 2 states"):
+        net(torch.zeros(3, 2, 4), net.get_zero_state(2)[:1])
+    with pytest.raises(RuntimeError, match="input_size"):
+        net(torch.zeros(3, 2, 7))
+    with pytest.raises(RuntimeError, match="Expected hidden size"):
+        net(torch.zeros(3, 2, 4), net.get_zero_state(3))
+    with pytest.raises(RuntimeError, match="should be 2-D"):
+        bad = [type(s)(s.hx[0], s.cx[0]) for s in net.get_zero_state(2)]
+        net(torch.zeros(3, 2, 4), bad)
+
+
+@pytest.mark.parametrize("kind", ["RNN", "LSTM", "GRU"])
+@pytest.mark.parametrize("bidir", [False, True])
+def test_rnn_state_dict_uses_torchs_flat_names(kind, bidir):
+    """reference rnn.py:359-392: the state dict carries torch's names and loads from either."""
+    AnalogRNN = _rnn_classes()[0]
+    digital = getattr(torch.nn, kind)(6, 8, 2, bidirectional=bidir)
+    analog = AnalogRNN.from_digital(digital, _cfg(max_input_size=4))
+    state = analog.state_dict()
+    for key, value in digital.state_dict().items():
+        assert torch.equal(state[key], value), key
+    extra = set(state) - set(digital.state_dict())
+    assert "input_range_ih_l0" in extra and "input_range_update_idx_hh_l1" in extra
+    if bidir:
+        assert "input_range_hh_l1_reverse" in extra
+    assert not [k for k in state if k.startswith("rnn.")]
+    # loads its own state dict and a plain torch one
+    other = AnalogRNN.from_digital(getattr(torch.nn, kind)(6, 8, 2, bidirectional=bidir),
+                                   _cfg(max_input_size=4))
+    assert not any(other.load_state_dict(state))
+    for (_, _, a), (_, _, b) in zip(analog.cells(), other.cells()):
+        assert torch.equal(a.weight_hh.weight, b.weight_hh.weight)
+    report = other.load_state_dict(digital.state_dict(), strict=False)
+    assert not report.unexpected_keys
+    # nested in a model the prefix is kept
+    nest = torch.nn.Sequential(analog)
+    assert "0.weight_ih_l0" in nest.state_dict()
+    assert not any(torch.nn.Sequential(other).load_state_dict(nest.state_dict()))
+    back = AnalogRNN.to_digital(analog)
+    assert type(back) is type(digital)
+    for key, value in digital.state_dict().items():
+        assert torch.equal(back.state_dict()[key], value), key
+
+
+class _SeqNet(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.gru1 = torch.nn.GRU(10, 10, 1)
+        self.lstm1 = torch.nn.LSTM(10, 20, 3, bidirectional=True)
+        self.lstm2 = torch.nn.LSTM(40, 20, 3, bias=False, bidirectional=True)
+        self.rnn1 = torch.nn.RNN(40, 20, 3, dropout=0.1)
+        self.head = torch.nn.Linear(20, 4)
+
+
+def test_convert_recurrent_layers_to_analog_and_back():
+    """reference tests/test_conversion.py:95-150."""
+    from aihwkit_lightning.nn.conversion import convert_to_analog, convert_to_digital
+    AnalogRNN, Vanilla, Lstm, Gru, _ = _rnn_classes()
+    model = _SeqNet()
+    analog = convert_to_analog(model, _cfg(), ensure_analog_root=False)
+    assert isinstance(analog.gru1, AnalogRNN) and isinstance(analog.gru1.rnn.layers[0].cell, Gru)
+    assert isinstance(analog.lstm1.rnn.layers[2].directions[1].cell, Lstm)
+    assert analog.lstm2.rnn.layers[0].directions[0].cell.weight_ih.bias is None
+    assert isinstance(analog.rnn1.rnn.layers[0].cell, Vanilla)
+    assert analog.rnn1.rnn.dropout_layer.p == 0.1
+    assert isinstance(analog.head, AnalogLinear)
+    digital = convert_to_digital(analog)
+    for name in ("gru1", "lstm1", "lstm2", "rnn1"):
+        assert type(getattr(digital, name)) is type(getattr(model, name))
+    for key, value in model.state_dict().items():
+        assert torch.equal(digital.state_dict()[key], value), key
+    assert isinstance(convert_to_analog(model, _cfg()), AnalogWrapper)
