@@ -5,6 +5,7 @@ Loading is lazy and failure is loud: there is no software fallback for any entry
 """
 import ctypes
 import os
+from functools import lru_cache
 from ctypes import (
     c_void_p, c_int32, c_int64, c_float, c_double, c_uint64, c_char_p, POINTER, Structure,
 )
@@ -232,10 +233,16 @@ def check(status: int, where: str) -> None:
     raise HipBackendError(f"{where}: {text}")
 
 
-def tile_ends_array(in_sizes):
-    """Cumulative tile ends as a host int32 array (the reference's ``upper_end_of_slices``)."""
+@lru_cache(maxsize=4096)
+def _tile_ends(in_sizes: tuple):
     ends, acc = [], 0
     for size in in_sizes:
         acc += int(size)
         ends.append(acc)
     return (c_int32 * len(ends))(*ends)
+
+
+def tile_ends_array(in_sizes):
+    """Cumulative tile ends as a host int32 array (the reference's ``upper_end_of_slices``); the
+    library only reads it, so one array per split is shared by all calls."""
+    return _tile_ends(tuple(in_sizes))

@@ -31,7 +31,8 @@ def _ptr(tensor: Optional[Tensor]):
 
 
 def _stream():
-    return c_void_p(torch.cuda.current_stream().cuda_stream)
+    # the raw handle of torch's current stream, without building a Stream object per launch
+    return c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))  # pylint: disable=protected-access
 
 
 def _rows2d(tensor: Tensor, name: str) -> Tensor:

@@ -69,6 +69,74 @@ class ModularRNN(Module):
         return inp, last_states
 
 
+class GraphedRNN:
+    """``net(inp, states)`` in evaluation mode for one input shape, recorded once as a HIP graph
+    and replayed per call. A recurrent step is a handful of small launches (two analog products,
+    ten element-wise kernels), so an eager sequence is bound by the host's launch rate; the graph
+    removes the host from the loop. Nothing in the analog operator allocates, synchronises or
+    clears memory outside kernels, so every launch of the sequence is recorded as a kernel node.
+
+    The graph reads the parameters where they were when it was recorded: in-place updates are
+    seen by later calls, re-assigned parameter tensors are not (record a new graph then). Calls
+    return copies, so results survive the next call.
+    """
+
+    def __init__(self, net: "AnalogRNN", example_inp: Tensor, states: Optional[List] = None):
+        if net.training:
+            raise RuntimeError("GraphedRNN records the evaluation-mode forward; call net.eval()")
+        if not example_inp.is_cuda:
+            raise RuntimeError("GraphedRNN needs an input on the GPU")
+        self.net = net
+        self.inp = example_inp.detach().clone()
+        batch = self.inp.size(1) if self.inp.dim() == 3 else 1
+        self.states = self._clone_states(states if states is not None
+                                         else net.get_zero_state(batch))
+        self.given_states = states is not None
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.no_grad(), torch.cuda.stream(side):
+            net(self.inp, self.states)  # loads the library and fills the host-side caches
+        torch.cuda.current_stream().wait_stream(side)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(self.graph):
+            self.out, self.last = net(self.inp, self.states)
+
+    @staticmethod
+    def _map_states(fn, states):
+        """``fn`` applied to every tensor of a nested list / tuple / ``LSTMState`` structure."""
+        if states is None:
+            return None
+        if isinstance(states, Tensor):
+            return fn(states)
+        mapped = [GraphedRNN._map_states(fn, s) for s in states]
+        if hasattr(states, "_fields"):
+            return type(states)(*mapped)
+        return type(states)(mapped)
+
+    @classmethod
+    def _clone_states(cls, states):
+        return cls._map_states(lambda t: t.detach().clone(), states)
+
+    def __call__(self, inp: Tensor, states: Optional[List] = None) -> Tuple[Tensor, List]:
+        if inp.shape != self.inp.shape or inp.dtype != self.inp.dtype:
+            raise RuntimeError(
+                f"recorded for input {tuple(self.inp.shape)} {self.inp.dtype}, "
+                f"got {tuple(inp.shape)} {inp.dtype}"
+            )
+        if (states is not None) != self.given_states:
+            raise RuntimeError("recorded with" + ("" if self.given_states else "out")
+                               + " initial states; call it the same way")
+        self.inp.copy_(inp)
+        if states is not None:
+            flat_new, flat_own = [], []
+            self._map_states(lambda t: flat_new.append(t) or t, states)
+            self._map_states(lambda t: flat_own.append(t) or t, self.states)
+            for own, new in zip(flat_own, flat_new):
+                own.copy_(new)
+        self.graph.replay()
+        return self.out.clone(), self._map_states(lambda t: t.clone(), self.last)
+
+
 class AnalogRNN(AnalogContainerBase, Module):
     """Recurrent network of ``cell`` (``AnalogVanillaRNNCell``, ``AnalogLSTMCell``,
     ``AnalogGRUCell`` or ``AnalogLSTMCellCombinedWeight``) with time-major input.
@@ -208,6 +276,11 @@ class AnalogRNN(AnalogContainerBase, Module):
         self.check_hidden_size(hidden.hx, (batch_size, self.hidden_size))
         if hidden.cx is not None:
             self.check_hidden_size(hidden.cx, (batch_size, self.hidden_size))
+
+    def graphed(self, example_inp: Tensor, states: Optional[List] = None) -> GraphedRNN:
+        """A callable with the signature of ``forward`` that replays the evaluation-mode forward
+        for inputs of ``example_inp``'s shape as one HIP graph (see :class:`GraphedRNN`)."""
+        return GraphedRNN(self, example_inp, states)
 
     # ------------------------------------------------------------------ cells and state dicts
     def cells(self) -> Iterator[Tuple[int, bool, Module]]:

@@ -189,3 +189,42 @@ def test_plain_network_is_torchs_lstm_on_the_gpu():
         assert torch.allclose(cx, c_n[i], rtol=1e-5, atol=1e-6)
     back = AnalogRNN.to_digital(analog)
     assert torch.equal(back(x)[0], want)
+
+
+@pytest.mark.parametrize("cell", ["lstm", "gru"])
+def test_graph_replays_equal_the_eager_forward(cell):
+    """The recorded sequence is replayed several times with new inputs and with eager work and
+    synchronisations in between; every replay must equal the eager result bit for bit."""
+    print(f"case graph {cell}", flush=True)
+    case = rnn_case("graph", cell, 9, 4, 40, 32, layers=2, bidir=True, max_input_size=24,
+                    dtype="bf16", ir_mode="static", ir_init=2.0, clip="channel", clip_sigma=2.5,
+                    w_scale=0.2, inp_res=254, out_res=254, out_bound=10.0, training=False, seed=74)
+    net, _ = build_network(case)
+    gen = torch.Generator().manual_seed(3)
+    example = torch.randn(9, 4, 40, generator=gen).bfloat16().cuda()
+    replay = net.graphed(example)
+    for trial in range(4):
+        x = (torch.randn(9, 4, 40, generator=gen) * (1 + trial)).bfloat16().cuda()
+        with torch.no_grad():
+            want, want_states = net(x)
+        scratch = torch.randn(256, 256, device="cuda") @ torch.randn(256, 256, device="cuda")
+        torch.cuda.synchronize()
+        got, got_states = replay(x)
+        assert torch.equal(got, want), trial
+        for pair_g, pair_w in zip(got_states, want_states):
+            for s_g, s_w in zip(pair_g, pair_w):
+                assert torch.equal(s_g[0], s_w[0]), trial
+                if s_w[1] is not None:
+                    assert torch.equal(s_g[1], s_w[1]), trial
+        del scratch
+    # in-place weight updates are seen by the graph
+    with torch.no_grad():
+        for _, _, c in net.cells():
+            c.weight_hh.weight.mul_(0.5)
+        want, _ = net(x)
+    assert torch.equal(replay(x)[0], want)
+    with pytest.raises(RuntimeError, match="recorded for input"):
+        replay(x[:5])
+    net.train()
+    with pytest.raises(RuntimeError, match="evaluation-mode"):
+        net.graphed(example)
