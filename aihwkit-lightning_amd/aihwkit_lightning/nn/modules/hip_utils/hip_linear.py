@@ -11,7 +11,8 @@ from torch import Tensor
 from torch.autograd import Function
 
 from . import library as L
-from .ops import OPS, tile_stride
+from . import ops as _impl
+from .ops import tile_stride
 from ....exceptions import ConfigError, HipBackendError
 from ....simulator.configs import (
     TorchInferenceRPUConfig,
@@ -47,6 +48,16 @@ def check_supported(rpu_config: TorchInferenceRPUConfig) -> None:
         ), "You can't learn weight ranges per column but quantize per tensor"
 
 
+def _ops_for(tensor: Tensor):
+    """Where HipLinear takes its operator calls from. It is an autograd node of its own, so
+    inside it the dispatcher adds nothing but time (about 10 us per call, three to six calls per
+    layer call): for a tensor on the current device the implementations are called directly. For
+    a tensor elsewhere the registered ops are used, whose dispatch switches the device."""
+    if tensor.device.index == torch.cuda.current_device():
+        return _impl
+    return _impl.OPS
+
+
 class HipLinear(Function):
     """y = analog_mvm(x, W) + b with DAC/ADC, noise and tiling, on MI355X."""
 
@@ -73,6 +84,7 @@ class HipLinear(Function):
                 "AnalogLinear runs only on a ROCm device (got a CPU tensor); there is no CPU path"
             )
         check_supported(rpu_config)
+        ops = _ops_for(inp)
         fwd, modifier = rpu_config.forward, rpu_config.modifier
         ir_params = rpu_config.pre_post.input_range
         k_in, n_out = weights.size(1), weights.size(0)
@@ -83,6 +95,11 @@ class HipLinear(Function):
         weights_c = weights if weights.stride(1) == 1 else weights.contiguous()
         if weights.dtype != inp.dtype:
             raise HipBackendError("input and weight dtypes differ")
+        if weights.device != inp.device or (bias is not None and bias.device != inp.device):
+            raise HipBackendError(
+                f"input on {inp.device} but parameters on {weights.device}: move the layer to the "
+                "input's device"
+            )
         m_rows = x2.size(0)
 
         apply_out_quantization = fwd.out_res > 0
@@ -137,14 +154,14 @@ class HipLinear(Function):
             wmax = learnable_weight_clip.detach()
             if not wmax.is_contiguous():
                 wmax = wmax.contiguous()
-            tile_max, tile_min, w_eff = OPS.weight_prep_clip(
+            tile_max, tile_min, w_eff = ops.weight_prep_clip(
                 weights_c, wmax, in_sizes, clip_quant,
                 NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE,
                 float(modifier.res) if w_quant else 1.0, float(modifier.std_dev), seed, 1,
             )
         elif m_rows > 0 and need_wmax:
             res = float(modifier.res) if w_quant else 1.0
-            wmax, tile_max, _, eff = OPS.weight_prep(
+            wmax, tile_max, _, eff = ops.weight_prep(
                 weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
                 NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE, res,
                 float(modifier.std_dev), seed, 1, w_noise or w_quant,
@@ -188,17 +205,17 @@ class HipLinear(Function):
         # clamp + DAC are fused into the matrix kernel's A-tile staging.
         split_dac = stride > 0 or (inp.dtype == torch.bfloat16 and dense_fwd_ok)
         if stride > 0:
-            w_eff = OPS.pad_tiles(w_eff, in_sizes, stride)
+            w_eff = ops.pad_tiles(w_eff, in_sizes, stride)
         ir_dev = xq = None
         if ir_mode == L.AHL_IR_STATIC:
             if training and init_active and fast:
-                OPS.ir_fast_update(
+                ops.ir_fast_update(
                     x2, in_sizes, input_range.data, input_range_update_idx, x_min, x_max,
                     float(ir_params.init_from_data), float(ir_params.act_range_momentum),
                 )
             elif training and init_active:
-                std = OPS.sliced_std(x2, in_sizes)
-                OPS.ir_init_update(
+                std = ops.sliced_std(x2, in_sizes)
+                ops.ir_init_update(
                     input_range.data, input_range_update_idx, std, float(ir_params.init_from_data),
                     float(ir_params.init_std_alpha),
                 )
@@ -206,14 +223,14 @@ class HipLinear(Function):
             if not ir_dev.is_contiguous():
                 ir_dev = ir_dev.contiguous()
         if split_dac:
-            xq, ir_dyn = OPS.dac(x2, ir_dev, in_sizes, icfg, fcfg)
+            xq, ir_dyn = ops.dac(x2, ir_dev, in_sizes, icfg, fcfg)
             if ir_mode == L.AHL_IR_DYNAMIC:
                 ir_dev = ir_dyn
         elif ir_mode == L.AHL_IR_DYNAMIC:
-            ir_dev = OPS.sliced_absmax(x2, in_sizes, False)[0]
+            ir_dev = ops.sliced_absmax(x2, in_sizes, False)[0]
 
         want_keep = fwd.out_bound > 0 and (need_dx or need_dw)
-        y, keep, flag = OPS.linear_fwd(
+        y, keep, flag = ops.linear_fwd(
             None if split_dac else x2, xq, w_eff, bias, ir_dev, wmax, tile_max, in_sizes, icfg, fcfg,
             want_keep,
         )
@@ -244,8 +261,9 @@ class HipLinear(Function):
         if g2.stride(-1) != 1 or (g2.size(0) > 1 and g2.stride(0) != n_out):
             g2 = g2.contiguous()
         grad_inp = grad_w = grad_b = grad_ir = grad_clip = None
+        ops = _ops_for(g2)
         if ctx.need_dx:
-            dx, ir_grad = OPS.linear_bwd_dx(
+            dx, ir_grad = ops.linear_bwd_dx(
                 g2, keep, flag, w_eff, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
                 ctx.in_sizes, ctx.icfg, ctx.fcfg,
             )
@@ -256,7 +274,7 @@ class HipLinear(Function):
         want_bias = ctx.has_bias and ctx.needs_input_grad[2]
         if ctx.need_dw:
             # the weight-gradient kernel streams all of g and sums its columns on the way
-            grad_w, dbias = OPS.linear_bwd_dw(
+            grad_w, dbias = ops.linear_bwd_dw(
                 g2, keep, flag, x2 if xq is None else None, xq, ir_dev, ctx.in_sizes, ctx.icfg,
                 ctx.fcfg, want_bias,
             )
@@ -264,11 +282,11 @@ class HipLinear(Function):
                 grad_b = dbias
             if ctx.learned_clip:
                 # gradient w.r.t. the clipped weights -> weights (in place) and clip (LSQ rule)
-                grad_clip = OPS.learned_clip_bwd(
+                grad_clip = ops.learned_clip_bwd(
                     grad_w, w_plain, clip, clip_tile_min, ctx.in_sizes, ctx.clip_quant, ctx.clip_res
                 )
         elif want_bias:
-            grad_b = OPS.col_sum(g2)
+            grad_b = ops.col_sum(g2)
         if not ctx.needs_input_grad[1]:
             grad_w = None
         return (grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None, None, None,

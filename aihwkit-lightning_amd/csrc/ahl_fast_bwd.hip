@@ -53,10 +53,10 @@ struct BwdArgs {
   int32_t dense_base, dense_extra;     // DX: dense_base > 0: x and dx are dense with the split
                                        // (base, extra) of any widths; the epilogue then works
                                        // element by element instead of in 16-byte vectors
-  int32_t slices;                      // DW: the contraction (rows m) is cut into this many
-                                       // slices, one block each; > 1 when N x K alone gives
-                                       // too few blocks to fill the chip
-  float* split;                        // slices > 1: fp32 partial results [slices][N][K]
+  int32_t slices;                      // the contraction (DW: rows m; DX: channels n) is cut
+                                       // into this many slices, one block each; > 1 when the
+                                       // output tiles alone are too few to fill the chip
+  float* split;                        // slices > 1: fp32 partial results [slices][rows][K]
 };
 
 AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
@@ -293,10 +293,10 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     else main_loop(std::false_type{}, std::false_type{});
   }
 
-  if (MODE == MODE_DW && a.slices > 1) {
+  if (a.slices > 1) {
     // partial result of this slice, fp32, straight from the accumulators: for fixed (bi, bj, v)
     // the 32 lanes of a half wave write 128 contiguous bytes of one row
-    float* sp = a.split + ((int64_t)slice * a.N) * a.K;
+    float* sp = a.split + ((int64_t)slice * R) * a.K;
 #pragma unroll
     for (int bi = 0; bi < 4; ++bi)
 #pragma unroll
@@ -460,6 +460,70 @@ __global__ __launch_bounds__(256) void k_split_reduce(const float* __restrict__ 
   *(u32x2*)(out + r * ldo + c) = pk;
 }
 
+// Sliced input gradient: sums the slices' partial results in order, rounds once, and applies the
+// epilogue of the unsliced kernel (input-range mask and partial sums, column mapping onto a dense
+// dx). One block: 16 rows x 256 columns; partial sums go to partial[(row block, column block)].
+__global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
+  __shared__ float red[8][3];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t nkb = a.K / 256;
+  const int64_t rb = blockIdx.x / nkb, bcol = blockIdx.x % nkb;
+  const int64_t c0 = bcol * 256;
+  const int t = (int)(c0 / a.tile);
+  const int vcol = tid & 31, vrow = tid >> 5;
+  const int64_t row = rb * 16 + vrow;
+  int64_t ocol = c0 + vcol * 8;
+  bool ovalid = true;
+  if (a.dense_tile > 0) {
+    const int64_t in_tile = ocol - (int64_t)t * a.tile;
+    ovalid = in_tile < a.dense_tile;
+    ocol = ovalid ? (int64_t)t * a.dense_tile + in_tile : 0;
+  }
+  const bool do_ir = a.ir_static != 0;
+  const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
+  float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
+  if (row < a.M && ovalid) {
+    f32x4 lo4 = {0.f, 0.f, 0.f, 0.f}, hi4 = {0.f, 0.f, 0.f, 0.f};
+    const float* sp = a.split + row * a.K + c0 + vcol * 8;
+    for (int sl = 0; sl < a.slices; ++sl) {
+      lo4 += *(const f32x4*)(sp + (int64_t)sl * a.M * a.K);
+      hi4 += *(const f32x4*)(sp + (int64_t)sl * a.M * a.K + 4);
+    }
+    float d[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) d[i] = bf16_bits_to_f32(f32_to_bf16_bits(d[i]));
+    if (do_ir) {
+      float xv[8];
+      BF16::unpack(ld16(a.x + row * a.ldx + ocol), xv);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
+          const bool up = xv[i] >= ir_t, lo = xv[i] <= -ir_t;
+          if (up) s_up += fminf(d[i], 0.0f);
+          if (lo) s_lo += fmaxf(d[i], 0.0f);
+          if (up || lo) cnt += 1.0f;
+        } else {
+          if (xv[i] > ir_t) s_up += d[i];
+          if (xv[i] < -ir_t) s_lo += d[i];
+        }
+        if (fabsf(xv[i]) > ir_t) d[i] = 0.0f;
+      }
+    }
+    st16(a.out + row * a.ldo + ocol, BF16::pack(d));
+  }
+  if (do_ir) {
+    s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
+    if (lane == 0) { red[wave][0] = s_up; red[wave][1] = s_lo; red[wave][2] = cnt; }
+    __syncthreads();
+    if (tid == 0) {
+      float u = 0.f, l = 0.f, c = 0.f;
+      for (int w = 0; w < 8; ++w) { u += red[w][0]; l += red[w][1]; c += red[w][2]; }
+      float* p = a.partial + (rb * nkb + bcol) * 4;
+      p[0] = u; p[1] = l; p[2] = c; p[3] = 0.0f;
+    }
+  }
+}
+
 // dbias[n] = bf16(sum of the partial rows): 16 columns per block, 16 threads per column that
 // each add every 16th row, combined in a fixed order (the partial rows can be hundreds when the
 // weight gradient is sliced)
@@ -490,12 +554,44 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
   return K % 256 == 0 && N % 8 == 0 && N >= 8 && M >= 1;
 }
 
+// Slices of the contraction for the input gradient: with few rows (a recurrent step, a small
+// batch) the M x K / 65536 output tiles are a handful of blocks that each walk all N channels;
+// the channels are cut until there are about 256 blocks, each with at least 4 chunks of 64.
+int fast_dx_slices(int64_t M, int64_t K, int64_t N) {
+  const int64_t tiles = cdiv(M, 256) * (K / 256);
+  if (tiles >= 128) return 1;
+  int64_t s = cdiv(256, tiles);
+  const int64_t chunks = cdiv(N, 64), most = chunks / 4;
+  if (s > most) s = most;
+  if (s <= 1) return 1;
+  return (int)cdiv(chunks, cdiv(chunks, s));
+}
+
+// Rows of the input-range partial sums [rows][K / 256][4] that launch_fast_dx writes: one per
+// 256 output rows, or one per 16 when the contraction is sliced.
+int64_t fast_dx_row_blocks(int64_t M, int64_t K, int64_t N, bool element_mode) {
+  return !element_mode && fast_dx_slices(M, K, N) > 1 ? cdiv(M, 16) : cdiv(M, 256);
+}
+
+static int64_t fast_dx_partial_bytes(int64_t M, int64_t K, int64_t N) {
+  return (fast_dx_row_blocks(M, K, N, false) * (K / 256) * 16 + 255) / 256 * 256;
+}
+
+// Workspace of launch_fast_dx: [input-range partial sums | slices > 1: slices x M x K floats]
+int64_t fast_dx_ws_bytes(int64_t M, int64_t K, int64_t N) {
+  const int64_t slices = fast_dx_slices(M, K, N);
+  return fast_dx_partial_bytes(M, K, N) + (slices > 1 ? slices * M * K * 4 : 0);
+}
+
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
-                   void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
+                   void* dx, int64_t lddx, void* ws, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
                    hipStream_t s) {
   BwdArgs a;
+  float* partial = (float*)ws;
+  // the element-wise epilogue for arbitrary dense splits is not part of the reduction kernel
+  const int slices = dense ? 1 : fast_dx_slices(M, K, N);
   a.dense_tile = dense_tile;
   a.dense_base = dense ? dense->base : 0;
   a.dense_extra = dense ? dense->extra : 0;
@@ -503,8 +599,9 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
   a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = ir_static;
-  a.slices = 1; a.split = nullptr;
-  const int64_t nb = cdiv(M, 256) * (K / 256);
+  a.slices = slices;
+  a.split = slices > 1 ? (float*)((char*)ws + fast_dx_partial_bytes(M, K, N)) : nullptr;
+  const int64_t nb = cdiv(M, 256) * (K / 256) * slices;
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   if (N % 64 == 0) {
     hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
@@ -513,6 +610,8 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
     hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
     hipLaunchKernelGGL((k_bwd_fast<MODE_DX, true>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
   }
+  if (slices > 1)
+    hipLaunchKernelGGL(k_dx_split_reduce, dim3((unsigned)(cdiv(M, 16) * (K / 256))), dim3(512), 0, s, a);
   return check_launch("ahl_linear_bwd_dx(fast)");
 }
 

@@ -698,9 +698,11 @@ __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N);
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
-                   void* dx, int64_t lddx, float* partial, int64_t M, int64_t K, int64_t N,
+                   void* dx, int64_t lddx, void* ws, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
                    hipStream_t s);
+int64_t fast_dx_ws_bytes(int64_t M, int64_t K, int64_t N);
+int64_t fast_dx_row_blocks(int64_t M, int64_t K, int64_t N, bool element_mode);
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
@@ -822,11 +824,15 @@ int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
                                    int64_t tile_stride) {
   if (n_tiles <= 0 || K <= 0 || M <= 0 || N <= 0) return 0;
   const int64_t es = dtype == AHL_BF16 ? 2 : 4;
-  if (tile_stride > 0) {  // only the input-range partial sums; x and dx are used in place
+  if (tile_stride > 0) {  // the MFMA kernel's workspace; x and dx are used in place
     const int64_t padded = (int64_t)n_tiles * tile_stride;
-    return dx_padded_partial_bytes(M, padded);
+    const int64_t fast = align256(fast_dx_ws_bytes(M, padded, N));
+    return fast > dx_padded_partial_bytes(M, padded) ? fast : dx_padded_partial_bytes(M, padded);
   }
-  return dx_partial_bytes(M, K, n_tiles) + align256(K * N * es);  // partials + transposed weights
+  // general kernels: partials + transposed weights; MFMA kernel: its own layout in the same space
+  const int64_t generic = dx_partial_bytes(M, K, n_tiles) + align256(K * N * es);
+  const int64_t fast = K % 256 == 0 ? align256(fast_dx_ws_bytes(M, K, N)) : 0;
+  return generic > fast ? generic : fast;
 }
 
 int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
@@ -861,13 +867,14 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     // the element-wise epilogue addresses x and dx with one offset and aligns its vectors on dx
     if (!vectors && (!aligned16(dx) || (is_static && (!aligned16(x) || ldx != lddx))))
       return AHL_ERR_UNSUPPORTED;
-    const int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial,
+    const int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, ws,
                                   M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0,
                                   vectors ? tl.base : 0, vectors ? nullptr : &tl, s);
     if (rc != AHL_OK) return rc;
     if (is_static)
       hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
-                         (const float*)partial, cdiv(M, 256), (int32_t)(padded / 256), per_tile,
+                         (const float*)partial, fast_dx_row_blocks(M, padded, N, !vectors),
+                         (int32_t)(padded / 256), per_tile,
                          per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
                          cfg->ir_grad_rule);
     return check_launch("ahl_linear_bwd_dx(fast, padded weights)");
@@ -878,13 +885,14 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
                     (!keep || aligned16(keep)) &&
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
-    int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, partial, M, K,
+    int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, ws, M, K,
                             N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, nullptr, s);
     if (rc != AHL_OK) return rc;
     if (is_static) {
       const int32_t per_tile = tl.base / 256;
       hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
-                         (const float*)partial, cdiv(M, 256), (int32_t)(K / 256), per_tile, per_tile,
+                         (const float*)partial, fast_dx_row_blocks(M, K, N, false),
+                         (int32_t)(K / 256), per_tile, per_tile,
                          tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
                          cfg->ir_grad_rule);
     }

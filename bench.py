@@ -100,6 +100,10 @@ OTHER_WORKLOADS = {
                         "per-tile input range, 8-bit DAC/ADC, out_noise 0.04, forward only",
     "mlp_3072_8192": "LLaMA-style MLP block, hidden 3072, intermediate 8192, SiLU gating, three "
                      "AnalogLinear layers, bf16, 4096 tokens, tiles of 512, fwd+bwd",
+    "lstm_1024": "AnalogRNN, 2 LSTM layers 1024->1024 bf16, 64 steps x 64 sequences, tiles of 512, "
+                 "fwd+bwd through time",
+    "lstm_1024_eval": "AnalogRNN, 2 LSTM layers 1024->1024 bf16, 64 steps x 64 sequences, tiles of "
+                      "512, evaluation-mode forward replayed as one HIP graph",
 }
 
 
@@ -142,6 +146,29 @@ def build_other(name):
         x = torch.randn(4096, 3072, generator=gen).to(torch.bfloat16)
         g = torch.randn(4096, 3072, generator=gen).to(torch.bfloat16)
         flops = 3 * 3 * 2.0 * 4096 * 3072 * 8192
+    elif name in ("lstm_1024", "lstm_1024_eval"):
+        from aihwkit_lightning.nn import AnalogLSTMCell, AnalogRNN
+
+        class Outputs(torch.nn.Module):
+            """The network's outputs without the states."""
+
+            def __init__(self):
+                super().__init__()
+                self.net = AnalogRNN(AnalogLSTMCell, 1024, 1024, 2, dtype=torch.bfloat16,
+                                     rpu_config=_analog_cfg(512, noise=name == "lstm_1024"))
+
+            def forward(self, inp):
+                return self.net(inp)[0]
+
+        layer = Outputs()
+        x = torch.randn(64, 64, 1024, generator=gen).to(torch.bfloat16)
+        g = torch.randn(64, 64, 1024, generator=gen).to(torch.bfloat16)
+        # two projections of 1024 -> 4096 per cell step, 64 steps, 2 layers
+        flops = 2 * 64 * 2 * 2.0 * 64 * 1024 * 4096
+        if name == "lstm_1024_eval":
+            replay = layer.cuda().eval().net.graphed(x.cuda())
+            return (lambda inp: replay(inp)[0]), x.cuda(), None, flops
+        flops *= 3
     else:
         raise ValueError(name)
     with torch.no_grad():

@@ -128,6 +128,23 @@ SHAPES = [
     case("tail_pad_bf16_384", dtype="bf16", M=130, K=768, N=24, max_input_size=384, ir_mode="static",
          inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_values=[1.5, 2.5], w_scale=0.1,
          seed=45),
+    # few rows and many channels (a recurrent step, a small batch): the input-gradient kernel
+    # cuts the channels into slices and a second kernel sums them and applies the epilogue
+    case("sliced_dx_bf16_clamped", dtype="bf16", M=48, K=512, N=1024, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
+         w_scale=0.1, seed=46),
+    case("sliced_dx_pad_bf16_384", dtype="bf16", M=70, K=768, N=640, max_input_size=384,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01,
+         ir_values=[1.5, 2.5], w_scale=0.1, seed=47),
+    case("sliced_dx_tail_bf16_dynamic", dtype="bf16", M=33, K=512, N=1000, max_input_size=256,
+         ir_mode="dynamic", inp_res=254, out_res=254, out_bound=0.3, w_scale=0.1, seed=48),
+    case("sliced_dx_fast_mode", dtype="bf16", M=16, K=512, N=2048, max_input_size=256, ir_mode="fast",
+         ir_values=[0.8, 2.5], inp_res=254, out_res=254, out_bound=1.5, clip="channel",
+         clip_sigma=2.5, w_scale=0.05, seed=49),
+    # uneven split: the element-wise epilogue stays unsliced
+    case("pad_bf16_uneven_wide", dtype="bf16", M=40, K=1000, N=1024, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
+         w_scale=0.1, seed=50),
     case("pad_bf16_lsq", dtype="bf16", M=64, K=200, N=64, max_input_size=100, ir_mode="static",
          clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30,
          w_scale=0.3, inp_res=254, out_res=254, out_bound=10.0, seed=36),
