@@ -101,11 +101,21 @@ class TiledAnalogLayer(AnalogLayerBase):
     def analog_mvm(self, rows: Tensor) -> Tensor:
         """``rows[..., in] @ weight_matrix^T + bias`` through the analog tile model."""
         init_active = self.training and self._init_phase_active()
+        weight, bias = self.weight_matrix(), self.bias
+        input_range, weight_clip = self.input_range, self.learnable_weight_clip
+        if not torch.is_grad_enabled():
+            # Nothing will be differentiated. The operator decides from its arguments'
+            # requires_grad what to keep for a backward pass (the clamp mask, the quantised
+            # input, the padded operands), and that flag ignores the grad mode.
+            rows, weight, bias, input_range, weight_clip = (
+                None if t is None else t.detach()
+                for t in (rows, weight, bias, input_range, weight_clip)
+            )
         out = HipLinear.apply(
             rows,
-            self.weight_matrix(),
-            self.bias,
-            self.input_range,
+            weight,
+            bias,
+            input_range,
             self.input_range_update_idx,
             self.in_sizes,
             self.rpu_config,
@@ -113,7 +123,7 @@ class TiledAnalogLayer(AnalogLayerBase):
             init_active,
             self.x_min,
             self.x_max,
-            self.learnable_weight_clip,
+            weight_clip,
         )
         if init_active:
             self._ir_init_calls += 1

@@ -512,9 +512,12 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   if (clamp_flag) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);
   // 128 x 128 blocks (NBJ = 2). Measured alternatives: 128 x 64 blocks (NBJ = 1, three to four
   // blocks per CU) are ~10 % slower, 256 x 128 blocks (one block of 8 waves per CU) ~15 % slower.
-  if (cfg->ir_mode == AHL_IR_NONE) launch_fast<0, 2>(a, noise, adc, s);
-  else if (cfg->ir_mode == AHL_IR_STATIC) launch_fast<1, 2>(a, noise, adc, s);
-  else launch_fast<2, 2>(a, noise, adc, s);
+  // When those are too few to give every CU a block (few rows: a recurrent step, a small batch),
+  // the 128 x 64 blocks double the count.
+  const bool few = cdiv(M, 128) * cdiv(N, 128) < 200;
+  if (cfg->ir_mode == AHL_IR_NONE) few ? launch_fast<0, 1>(a, noise, adc, s) : launch_fast<0, 2>(a, noise, adc, s);
+  else if (cfg->ir_mode == AHL_IR_STATIC) few ? launch_fast<1, 1>(a, noise, adc, s) : launch_fast<1, 2>(a, noise, adc, s);
+  else few ? launch_fast<2, 1>(a, noise, adc, s) : launch_fast<2, 2>(a, noise, adc, s);
   return check_launch("ahl_linear_fwd(fast)");
 }
 

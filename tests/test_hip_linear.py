@@ -178,6 +178,36 @@ def test_leading_dims_and_1d_input():
     assert empty.shape == (0, 48)
 
 
+@pytest.mark.parametrize("name", ["sliced_dx_bf16_clamped", "pad_bf16_384_static_clamped",
+                                  "pad_bf16_uneven_clamped"])
+def test_no_grad_forward_equals_the_differentiable_forward(name):
+    """Under no_grad the layer keeps nothing for a backward pass (and may take another operand
+    layout); the output is the same, and the parameters' in-place state is untouched."""
+    from hip_helpers import make_layer
+
+    c = [s for s in SHAPES if s["name"] == name][0]
+    x, w, b, _ = make_inputs(c)
+    layer = make_layer(c, inputs=(x, w, b, None))
+    layer.eval()
+    want = layer(x.cuda().requires_grad_(True))
+    assert want.requires_grad
+    with torch.no_grad():
+        got = layer(x.cuda())
+    assert not got.requires_grad
+    assert torch.equal(got, want.detach())
+
+
+def test_parameters_on_another_device_are_rejected():
+    from hip_helpers import rpu_config
+    from aihwkit_lightning.nn import AnalogLinear
+    from aihwkit_lightning.exceptions import HipBackendError
+
+    c = case("cpu", M=4, K=16, N=8)
+    layer = AnalogLinear(16, 8, rpu_config=rpu_config(c))  # parameters on the CPU
+    with pytest.raises(HipBackendError, match="move the layer"):
+        layer(torch.randn(4, 16).cuda())
+
+
 def test_cpu_tensor_is_rejected():
     from hip_helpers import rpu_config
     from aihwkit_lightning.nn import AnalogLinear
