@@ -48,6 +48,11 @@ def check_supported(rpu_config: TorchInferenceRPUConfig) -> None:
         ), "You can't learn weight ranges per column but quantize per tensor"
 
 
+# bf16 products of at least this many multiply-adds get their output channels padded to a
+# multiple of 8 (see HipLinear.forward); below it the general kernels are as fast
+PAD_CHANNELS_MIN_WORK = 1 << 22
+
+
 def _ops_for(tensor: Tensor):
     """Where HipLinear takes its operator calls from. It is an autograd node of its own, so
     inside it the dispatcher adds nothing but time (about 10 us per call, three to six calls per
@@ -176,10 +181,28 @@ class HipLinear(Function):
         # the quantised input and the effective weights are kept in a padded tile layout instead
         # (stride > 0), unless the padding would blow the work up more than the slower general
         # kernels do, or the shape does not fit the fast backward at all
+        # bf16 layers whose output width is not a multiple of 8 (a 50257-word vocabulary): the
+        # MFMA kernels handle channels in whole 16-byte vectors, so the weight-side operands get
+        # zero channels up to the next multiple of 8 and the extra output columns are dropped.
+        # (Their per-channel abs-max is set to 1 so that their ADC step is not 0; nothing of them
+        # reaches the result.) Small problems stay on the general kernels: the copies would cost
+        # more than they save.
+        pad_n = 0
+        bias_k = bias
+        if (inp.dtype == torch.bfloat16 and n_out % 8 != 0 and not learned_clip
+                and m_rows * k_in * n_out >= PAD_CHANNELS_MIN_WORK):
+            pad_n = 8 - n_out % 8
+            w_eff = torch.nn.functional.pad(w_eff.detach(), (0, 0, 0, pad_n))
+            if wmax is not None:
+                wmax = torch.nn.functional.pad(wmax, (0, pad_n), value=1.0)
+            if bias is not None:
+                bias_k = torch.nn.functional.pad(bias.detach(), (0, pad_n))
+        n_k = n_out + pad_n
+
         stride = 0
         dense_fwd_ok = len(set(in_sizes)) == 1 and in_sizes[0] % 64 == 0
-        if (inp.dtype == torch.bfloat16 and m_rows > 0 and n_out % 8 == 0
-                and weights_c.data_ptr() % 16 == 0):
+        if (inp.dtype == torch.bfloat16 and m_rows > 0 and n_k % 8 == 0
+                and w_eff.data_ptr() % 16 == 0):
             stride = tile_stride(k_in, len(in_sizes), inp.dtype)
             if stride * len(in_sizes) > 4 * k_in or (dense_fwd_ok and not (need_dx or need_dw)):
                 stride = 0
@@ -203,7 +226,7 @@ class HipLinear(Function):
         # bf16 with equal tiles of a multiple of 64 inputs: clamp + DAC (+ dynamic abs-max) run as
         # one memory-bound pass and the matrix kernel streams the quantised input; otherwise the
         # clamp + DAC are fused into the matrix kernel's A-tile staging.
-        split_dac = stride > 0 or (inp.dtype == torch.bfloat16 and dense_fwd_ok)
+        split_dac = stride > 0 or (inp.dtype == torch.bfloat16 and dense_fwd_ok and n_k % 8 == 0)
         if stride > 0:
             w_eff = ops.pad_tiles(w_eff, in_sizes, stride)
         ir_dev = xq = None
@@ -231,9 +254,15 @@ class HipLinear(Function):
 
         want_keep = fwd.out_bound > 0 and (need_dx or need_dw)
         y, keep, flag = ops.linear_fwd(
-            None if split_dac else x2, xq, w_eff, bias, ir_dev, wmax, tile_max, in_sizes, icfg, fcfg,
+            # x goes along with xq: should the MFMA kernel not apply after all (a misaligned
+            # view), the general kernel starts from x
+            x2 if (stride == 0 or not split_dac) else None, xq, w_eff, bias_k, ir_dev, wmax, tile_max,
+            in_sizes, icfg, fcfg,
             want_keep,
         )
+        if pad_n:
+            y = y[:, :n_out]
+        ctx.pad_n = pad_n
 
         ctx.in_sizes, ctx.icfg, ctx.fcfg = in_sizes, icfg, fcfg
         ctx.inp_shape, ctx.ir_mode, ctx.has_bias = inp.shape, ir_mode, bias is not None
@@ -262,6 +291,9 @@ class HipLinear(Function):
             g2 = g2.contiguous()
         grad_inp = grad_w = grad_b = grad_ir = grad_clip = None
         ops = _ops_for(g2)
+        g_plain = g2
+        if ctx.pad_n and (ctx.need_dx or ctx.need_dw):
+            g2 = torch.nn.functional.pad(g2, (0, ctx.pad_n))  # zero gradient for the extra channels
         if ctx.need_dx:
             dx, ir_grad = ops.linear_bwd_dx(
                 g2, keep, flag, w_eff, x2 if ctx.ir_mode == L.AHL_IR_STATIC else None, ir_dev,
@@ -278,6 +310,9 @@ class HipLinear(Function):
                 g2, keep, flag, x2 if xq is None else None, xq, ir_dev, ctx.in_sizes, ctx.icfg,
                 ctx.fcfg, want_bias,
             )
+            if ctx.pad_n:
+                grad_w = grad_w[:n_out]
+                dbias = dbias[:n_out] if want_bias else dbias
             if want_bias:
                 grad_b = dbias
             if ctx.learned_clip:
@@ -286,7 +321,7 @@ class HipLinear(Function):
                     grad_w, w_plain, clip, clip_tile_min, ctx.in_sizes, ctx.clip_quant, ctx.clip_res
                 )
         elif want_bias:
-            grad_b = ops.col_sum(g2)
+            grad_b = ops.col_sum(g_plain)
         if not ctx.needs_input_grad[1]:
             grad_w = None
         return (grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None, None, None,

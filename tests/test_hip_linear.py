@@ -145,6 +145,19 @@ SHAPES = [
     case("pad_bf16_uneven_wide", dtype="bf16", M=40, K=1000, N=1024, max_input_size=256,
          ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
          w_scale=0.1, seed=50),
+    # equal tiles of a multiple of 64 but an output width that is not a multiple of 8, too small
+    # for channel padding: the general kernels
+    case("bf16_aligned_tiles_odd_width", dtype="bf16", M=64, K=512, N=10, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=10.0, w_scale=0.1, seed=55),
+    # output widths that are not a multiple of 8: zero channels are appended for the MFMA kernels
+    case("padn_bf16_static_clamped", dtype="bf16", M=256, K=512, N=100, max_input_size=256,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
+         w_scale=0.1, seed=51),
+    case("padn_bf16_384_dynamic", dtype="bf16", M=130, K=768, N=75, max_input_size=384,
+         ir_mode="dynamic", inp_res=254, out_res=254, out_bound=0.3, w_scale=0.1, seed=52),
+    case("padn_bf16_pertensor_nobias", dtype="bf16", M=96, K=1000, N=61, max_input_size=256,
+         bias=False, ir_mode="static", ir_init=2.0, inp_res=1 / 254, out_res=1 / 254, out_bound=2.0,
+         w_scale=0.1, ir_decay=0.0, seed=53),
     case("pad_bf16_lsq", dtype="bf16", M=64, K=200, N=64, max_input_size=100, ir_mode="static",
          clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30,
          w_scale=0.3, inp_res=254, out_res=254, out_bound=10.0, seed=36),
@@ -195,6 +208,28 @@ def test_no_grad_forward_equals_the_differentiable_forward(name):
         got = layer(x.cuda())
     assert not got.requires_grad
     assert torch.equal(got, want.detach())
+
+
+def test_padded_channels_with_noise_stay_finite():
+    """Output noise scaled by the whole tile also lands on the appended channels; nothing of it
+    may leak into the result."""
+    from hip_helpers import make_layer
+
+    c = case("padn_noise", dtype="bf16", M=256, K=512, N=100, max_input_size=256, ir_mode="static",
+             inp_res=254, out_res=254, out_bound=10.0, out_noise=0.1, clip="channel", clip_sigma=2.5,
+             weight_noise="add_normal_per_channel", modifier_std=0.02, w_scale=0.1, seed=54)
+    x, w, b, g = make_inputs(c)
+    layer = make_layer(c, inputs=(x, w, b, None))
+    xin = x.cuda().requires_grad_(True)
+    out = layer(xin)
+    assert out.shape == (256, 100) and torch.isfinite(out).all()
+    out.backward(g.cuda())
+    assert layer.weight.grad.shape == (100, 512) and torch.isfinite(layer.weight.grad).all()
+    assert torch.isfinite(xin.grad).all() and torch.isfinite(layer.bias.grad).all()
+    quiet = dict(c, out_noise=0.0, weight_noise="none")
+    ref = make_layer(quiet, inputs=(x, w, b, None))(x.cuda())
+    err = (out.float() - ref.float()).std() / ref.float().std()
+    assert 0.0 < err < 0.2  # the noise is there, and it is noise-sized
 
 
 def test_parameters_on_another_device_are_rejected():
