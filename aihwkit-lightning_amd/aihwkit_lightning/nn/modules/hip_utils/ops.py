@@ -405,7 +405,11 @@ def _modifier_cfg(dtype, quant_type, noise_type, res, std_dev, seed, offset) -> 
     cfg = L.AhlModifierCfg()
     cfg.dtype = dtype_id(dtype)
     cfg.quant_type, cfg.noise_type = quant_type, noise_type
-    cfg.res, cfg.std_dev = res, std_dev
+    # The reference derives the number of states as max(res, 1 / res) in Python (double) and only
+    # then enters tensor arithmetic; the library would do the same in float, where 1 / (1 / 30) is
+    # 29.999998. The number of states itself is passed (a value >= 1 is taken as it is).
+    cfg.res = max(res, 1.0 / res) if res > 0 else res
+    cfg.std_dev = std_dev
     cfg.seed, cfg.offset = seed, offset
     return cfg
 

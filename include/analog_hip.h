@@ -93,7 +93,9 @@ typedef struct AhlModifierCfg {
   int32_t dtype;
   int32_t quant_type; /* AHL_QUANT_*                                                            */
   int32_t noise_type; /* AHL_NOISE_* (ignored by ahl_quantize_weights)                          */
-  float res;          /* modifier.res (number of states, or its inverse)                        */
+  float res;          /* modifier.res (number of states, or its inverse). The number of states
+                         is max(res, 1 / res) in float: callers that hold the inverse in double
+                         should pass the number of states (1 / (1 / 30) is not 30 in float)   */
   float std_dev;      /* modifier.std_dev                                                       */
   int32_t wmax_given; /* != 0: wmax[T, N] is an input (clip.type LEARNABLE_PER_CHANNEL: the
                          learnable_weight_clip takes the place of the per-tile abs-max,

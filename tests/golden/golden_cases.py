@@ -118,6 +118,13 @@ CASES = [
          w_scale=0.3, seed=20, **_ADC8),
     case("f32_lsq_clip_big", M=6, K=16, N=8, max_input_size=8, clip="learnable", lwc_scale=0.6,
          w_scale=4.0, seed=21),
+    # the clip at its initial value (the per-channel abs-max: every channel has a weight exactly on
+    # the boundary) and the resolution given as an inverse: the number of states is
+    # max(res, 1 / res) in Python's double arithmetic (exactly 30), and whether the boundary weight
+    # counts as clipped hangs on the last bit of w / (2 clip / 30)
+    case("f32_lsq_quant_boundary", M=1, K=512, N=8, max_input_size=512, ir_mode="static", ir_init=1.0,
+         ir_decay=0.0, clip="learnable", lwc_scale=1.0, weight_quant="discretize_per_channel",
+         modifier_res=1 / 30, w_scale=0.1, seed=156, **_ADC8),
     # optimizer-step clipping
     case("f32_clip_layer", kind="clip", M=4, K=40, N=24, clip="layer", clip_sigma=2.0, w_scale=1.0,
          seed=13),
