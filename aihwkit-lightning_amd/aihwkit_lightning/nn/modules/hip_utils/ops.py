@@ -45,6 +45,15 @@ def _rows2d(tensor: Tensor, name: str) -> Tensor:
     return tensor
 
 
+def _vector_aligned(tensor: Tensor) -> Tensor:
+    """``tensor`` itself if its rows start on 16-byte boundaries, else a fresh contiguous copy (the
+    MFMA kernels load whole 16-byte vectors; with operands in the padded tile layout there is no
+    other kernel to fall back to)."""
+    if tensor.data_ptr() % 16 == 0 and (_ld(tensor) * tensor.element_size()) % 16 == 0:
+        return tensor
+    return tensor.clone(memory_format=torch.contiguous_format)
+
+
 def _ld(tensor: Tensor) -> int:
     return tensor.stride(0) if tensor.size(0) > 1 else max(tensor.size(1), tensor.stride(0))
 
@@ -578,6 +587,8 @@ def linear_bwd_dx(
     k_in = sum(in_sizes)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(g.dtype, icfg, fcfg)
+    if cfg.tile_stride > 0:
+        g = _vector_aligned(g)
     static = cfg.ir_mode == L.AHL_IR_STATIC
     dx = torch.empty((m_rows, k_in), dtype=g.dtype, device=g.device)
     ir_grad = torch.empty((n_tiles,) if static else (0,), dtype=g.dtype, device=g.device)
@@ -618,6 +629,8 @@ def linear_bwd_dw(
     k_in = sum(in_sizes)
     n_tiles = len(in_sizes)
     cfg = _linear_cfg(g.dtype, icfg, fcfg)
+    if cfg.tile_stride > 0:
+        g = _vector_aligned(g)
     dw = torch.empty((n_out, k_in), dtype=g.dtype, device=g.device)
     dbias = torch.empty((n_out,) if want_bias else (0,), dtype=g.dtype, device=g.device)
     ws_bytes = lib.ahl_linear_bwd_dw_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype,

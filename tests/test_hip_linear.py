@@ -210,6 +210,30 @@ def test_no_grad_forward_equals_the_differentiable_forward(name):
     assert torch.equal(got, want.detach())
 
 
+@pytest.mark.parametrize("name", ["pad_bf16_uneven_clamped", "pad_bf16_384_static_clamped"])
+def test_misaligned_gradient_with_padded_layout(name):
+    """A gradient that starts 2 bytes off a 16-byte boundary (a slice of a larger buffer): with the
+    operands in the padded tile layout the host copies it, as no other kernel reads that layout."""
+    from hip_helpers import make_layer
+
+    c = [s for s in SHAPES if s["name"] == name][0]
+    x, w, b, g = make_inputs(c)
+    ref = oracle_fwd_bwd(c)
+    layer = make_layer(c, inputs=(x, w, b, g))
+    buf = torch.zeros(g.numel() + 1, dtype=g.dtype, device="cuda")
+    buf[1:] = g.cuda().reshape(-1)
+    g_off = buf[1:].view(g.shape)
+    assert g_off.data_ptr() % 16 != 0
+    xin = x.cuda().requires_grad_(True)
+    out = layer(xin)
+    out.backward(g_off)
+    res = dict(out=out.detach().cpu(), dx=xin.grad.cpu(), dw=layer.weight.grad.cpu(),
+               db=layer.bias.grad.cpu() if layer.bias is not None else None,
+               dir=None if layer.input_range is None or layer.input_range.grad is None
+               else layer.input_range.grad.cpu())
+    check_against(res, ref, c, name + " misaligned gradient")
+
+
 def test_padded_channels_with_noise_stay_finite():
     """Output noise scaled by the whole tile also lands on the appended channels; nothing of it
     may leak into the result."""
