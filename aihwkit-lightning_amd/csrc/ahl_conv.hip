@@ -57,6 +57,22 @@ static bool make_geom(const AhlConvGeom* a, ConvGeom* g) {
   return true;
 }
 
+// Quotient and remainder of a small non-negative int by a run-time divisor through the fp32
+// reciprocal (exact for a < 2^22 after one correction step): a handful of instructions instead
+// of the ~40 of an integer division, which otherwise dominate the address arithmetic of these kernels.
+struct SmallDiv {
+  int32_t d;
+  float inv;
+  AHL_DEV int32_t quot(int32_t a) const {
+    int32_t q = (int32_t)((float)a * inv);
+    const int32_t r = a - q * d;
+    if (r >= d) ++q;
+    if (r < 0) --q;
+    return q;
+  }
+};
+static SmallDiv make_small_div(int32_t d) { return SmallDiv{d, 1.0f / (float)d}; }
+
 // One thread gathers VEC consecutive patch entries (consecutive kernel offsets, carrying into
 // the next kernel row / plane / channel) and writes them with one store. Threads of a wave walk
 // along the patch, so the writes are contiguous; the reads of neighbouring offsets touch
@@ -128,62 +144,86 @@ __global__ __launch_bounds__(256) void k_im2col(const E* __restrict__ x, E* __re
 template <class E>
 __global__ __launch_bounds__(256) void k_im2col_tiled(const E* __restrict__ x, E* __restrict__ cols,
                                                       int64_t ldc, ConvGeom g, int64_t M,
-                                                      int32_t k_tiles) {
+                                                      int32_t k_tiles, SmallDiv by_ow, SmallDiv by_oh) {
   constexpr int KT = 128 / (int)sizeof(E);  // patch entries per tile: 64 bf16 or 32 fp32
   constexpr int EPV = 16 / (int)sizeof(E);  // entries per 16-byte vector
   constexpr int VPR = KT / EPV;             // vectors per tile row: 8
   __shared__ uint32_t tile[64 * 33];
+  __shared__ int64_t first[2];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t m0 = (int64_t)(blockIdx.x / k_tiles) * 64;
   const int32_t k0 = (int32_t)(blockIdx.x % k_tiles) * KT;
-  // this lane's patch
-  const int64_t m = m0 + lane;
-  const bool mvalid = m < M;
-  const int64_t mm = mvalid ? m : M - 1;
-  const int64_t b = mm / g.L;
-  int32_t l = (int32_t)(mm - b * g.L);
-  const int32_t ow = l % g.out[2];
-  l /= g.out[2];
-  const int32_t oh = l % g.out[1];
-  const int32_t od = l / g.out[1];
+  // (image, position) of the block's first patch: one 64-bit division per block; the lanes step
+  // on from there with 32-bit arithmetic (positions per image < 2^22: checked by the launcher)
+  if (tid == 0) {
+    const int64_t b0 = m0 / g.L;
+    first[0] = b0;
+    first[1] = m0 - b0 * g.L;
+  }
+  __syncthreads();
+  const bool mvalid = m0 + lane < M;
+  int64_t b = first[0];
+  int32_t l = (int32_t)first[1] + (mvalid ? lane : 0);
+  const int32_t per_image = (int32_t)g.L;
+  while (l >= per_image) { l -= per_image; b += 1; }
+  const int32_t row = by_ow.quot(l);          // od * out[1] + oh
+  const int32_t ow = l - row * g.out[2];
+  const int32_t od = by_oh.quot(row);
+  const int32_t oh = row - od * g.out[1];
   const int32_t id0 = od * g.str[0] - g.pad[0];
   const int32_t ih0 = oh * g.str[1] - g.pad[1];
   const int32_t iw0 = ow * g.str[2] - g.pad[2];
   const int64_t plane = (int64_t)g.in[1] * g.in[2];
   const E* xb = x + b * g.C * g.in[0] * plane;
+  // element offset of this lane's patch origin inside its image (negative inside the padding);
+  // the launcher has checked that one image has fewer than 2^31 elements
+  const int32_t lane_off = (id0 * g.in[1] + ih0) * g.in[2] + iw0;
   E* trow = (E*)tile;
   constexpr int RS = 33 * 4 / (int)sizeof(E);  // tile row stride in entries
-  // (channel, kd * dil, kh * dil, kw * dil) of the tile's patch entries, decomposed once per
-  // block instead of once per load (three integer divisions each); channel < 0: beyond K
+  // Per patch entry of the tile: its element offset inside an image relative to the patch origin
+  // and its (kd, kh, kw) * dilation, decomposed once per block instead of once per load (three
+  // integer divisions each); offset < 0 marks entries beyond K. The entry is the same for all
+  // lanes of a wave, so the loop below reads it into scalar registers and the per-lane work is
+  // one 32-bit add for the address and three range checks.
   __shared__ int32_t entry[KT][4];
   if (tid < KT) {
     const int32_t k = k0 + tid;
-    int32_t c = -1, kd = 0, kh = 0, kw = 0;
+    int32_t off = -1, kd = 0, kh = 0, kw = 0;
     if (k < g.K) {
-      c = k / g.kvol;
+      const int32_t c = k / g.kvol;
       int32_t r = k - c * g.kvol;
-      kw = r % g.ker[2];
+      kw = (r % g.ker[2]) * g.dil[2];
       r /= g.ker[2];
-      kh = r % g.ker[1];
-      kd = r / g.ker[1];
+      kh = (r % g.ker[1]) * g.dil[1];
+      kd = (r / g.ker[1]) * g.dil[0];
+      off = ((c * g.in[0] + kd) * g.in[1] + kh) * g.in[2] + kw;
     }
-    entry[tid][0] = c;
-    entry[tid][1] = kd * g.dil[0];
-    entry[tid][2] = kh * g.dil[1];
-    entry[tid][3] = kw * g.dil[2];
+    entry[tid][0] = off;
+    entry[tid][1] = kd;
+    entry[tid][2] = kh;
+    entry[tid][3] = kw;
   }
   __syncthreads();
-#pragma unroll 4
-  for (int kk = wave; kk < KT; kk += 4) {
-    const int32_t c = entry[kk][0];  // uniform over the wave
-    E val = (E)0;
-    if (c >= 0) {
-      const int32_t id = id0 + entry[kk][1], ih = ih0 + entry[kk][2], iw = iw0 + entry[kk][3];
-      if (id >= 0 && id < g.in[0] && ih >= 0 && ih < g.in[1] && iw >= 0 && iw < g.in[2])
-        val = xb[((int64_t)c * g.in[0] + id) * plane + (int64_t)ih * g.in[2] + iw];
-    }
-    trow[lane * RS + kk] = val;
+  const uint32_t in0 = (uint32_t)g.in[0], in1 = (uint32_t)g.in[1], in2 = (uint32_t)g.in[2];
+  // All loads of a wave are issued before the first value is used: entries outside the image
+  // (or beyond K) read the image's first element instead and are zeroed afterwards, so there is
+  // no branch that would make every load wait for the one before it.
+  E vals[KT / 4];
+#pragma unroll
+  for (int i = 0; i < KT / 4; ++i) {
+    const int kk = wave + 4 * i;
+    const int32_t off = __builtin_amdgcn_readfirstlane(entry[kk][0]);
+    const int32_t kd = __builtin_amdgcn_readfirstlane(entry[kk][1]);
+    const int32_t kh = __builtin_amdgcn_readfirstlane(entry[kk][2]);
+    const int32_t kw = __builtin_amdgcn_readfirstlane(entry[kk][3]);
+    // unsigned compares fold the two-sided range checks into one each
+    const bool ok = off >= 0 && (uint32_t)(id0 + kd) < in0 && (uint32_t)(ih0 + kh) < in1 &&
+                    (uint32_t)(iw0 + kw) < in2;
+    const E v = xb[ok ? lane_off + off : 0];
+    vals[i] = ok ? v : (E)0;
   }
+#pragma unroll
+  for (int i = 0; i < KT / 4; ++i) trow[lane * RS + wave + 4 * i] = vals[i];
   __syncthreads();
   const int vcol = tid % VPR, vrow = tid / VPR;  // 32 rows per pass
 #pragma unroll
@@ -239,22 +279,6 @@ __global__ __launch_bounds__(256) void k_col2im(const void* __restrict__ dcols, 
   }
   D::store(dx, idx, acc);
 }
-
-// Quotient and remainder of a small non-negative int by a run-time divisor through the fp32
-// reciprocal (exact for a < 2^22 after one correction step): a handful of instructions instead
-// of the ~40 of an integer division, which otherwise dominate the address arithmetic below.
-struct SmallDiv {
-  int32_t d;
-  float inv;
-  AHL_DEV int32_t quot(int32_t a) const {
-    int32_t q = (int32_t)((float)a * inv);
-    const int32_t r = a - q * d;
-    if (r >= d) ++q;
-    if (r < 0) --q;
-    return q;
-  }
-};
-static SmallDiv make_small_div(int32_t d) { return SmallDiv{d, 1.0f / (float)d}; }
 
 // Tiled variant: a block computes a patch of rpb rows x cpb columns (rpb * cpb = 64; cpb is the
 // smallest power of two that covers the image width, at most 64, so narrow images still fill
@@ -417,7 +441,8 @@ static int launch_im2col_tiled(const void* x, void* cols, int64_t ldc, const Con
   const int64_t blocks = cdiv(M, 64) * k_tiles;
   if (blocks > 0x7fffffff) return AHL_ERR_UNSUPPORTED;
   hipLaunchKernelGGL((k_im2col_tiled<E>), dim3((unsigned)blocks), dim3(256), 0, st, (const E*)x,
-                     (E*)cols, ldc, g, M, (int32_t)k_tiles);
+                     (E*)cols, ldc, g, M, (int32_t)k_tiles, make_small_div(g.out[2]),
+                     make_small_div(g.out[1]));
   return check_launch("k_im2col_tiled");
 }
 
@@ -426,13 +451,16 @@ extern "C" int ahl_im2col(const void* x, const AhlConvGeom* geom, int32_t dtype,
   ConvGeom g;
   if (x == nullptr || cols == nullptr || !make_geom(geom, &g) || ldc < g.K) return AHL_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
+  // the tiled kernel addresses the elements of one image with 32-bit offsets
+  // and the positions of one image with the fp32-reciprocal division
+  const bool small_image = (int64_t)g.C * g.in[0] * g.in[1] * g.in[2] <= 0x3fffffff && g.L < (1 << 22);
   if (dtype == AHL_F32) {
-    if (g.K % 4 == 0 && ldc % 4 == 0 && aligned16(cols))
+    if (g.K % 4 == 0 && ldc % 4 == 0 && aligned16(cols) && small_image)
       return launch_im2col_tiled<uint32_t>(x, cols, ldc, g, st);
     return launch_im2col<uint32_t, 1>(x, cols, ldc, g, st);
   }
   if (dtype == AHL_BF16) {
-    if (g.K % 8 == 0 && ldc % 8 == 0 && aligned16(cols))
+    if (g.K % 8 == 0 && ldc % 8 == 0 && aligned16(cols) && small_image)
       return launch_im2col_tiled<uint16_t>(x, cols, ldc, g, st);
     return launch_im2col<uint16_t, 1>(x, cols, ldc, g, st);
   }
