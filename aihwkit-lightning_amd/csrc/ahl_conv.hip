@@ -379,6 +379,109 @@ __global__ __launch_bounds__(512) void k_col2im_tiled(const void* __restrict__ d
   D::store(dx, (((b * g.C + cg * 8 + cl) * g.in[0] + d) * plane) + (int64_t)h * g.in[2] + w, acc);
 }
 
+// Wide variant: the image patch of a block has 256 pixels (rpb * cpb = 256) and a thread owns one
+// pixel for all 8 channels of the group, so the index arithmetic of a kernel offset (which output
+// position, whether it exists, where its staged row lies) is done once for 8 sums, and the halo
+// of staged output rows is shared by four times as many image rows. Same staging layout, same
+// ascending kernel-offset order and fp32 sums as above: the same bits.
+template <class D>
+__global__ __launch_bounds__(256) void k_col2im_wide(const void* __restrict__ dcols, int64_t ldc,
+                                                     ConvGeom g, FoldPlan fp,
+                                                     void* __restrict__ dx) {
+  typedef typename D::elem E;
+  constexpr int EPV = D::EPV;
+  extern __shared__ __attribute__((aligned(16))) char fold_lds[];
+  const int tid = threadIdx.x;
+  int64_t r = blockIdx.x;
+  const int32_t wt = (int32_t)(r % fp.w_tiles);
+  r /= fp.w_tiles;
+  const int32_t ht = (int32_t)(r % fp.h_tiles);
+  r /= fp.h_tiles;
+  const int32_t d = (int32_t)(r % g.in[0]);
+  r /= g.in[0];
+  const int32_t cg = (int32_t)(r % (g.C / 8));
+  const int64_t b = r / (g.C / 8);
+  const int32_t w0 = wt * fp.cpb, h0 = ht * fp.rpb;
+  const int32_t w_last = (w0 + fp.cpb - 1 < g.in[2] ? w0 + fp.cpb - 1 : g.in[2] - 1);
+  const int32_t h_last = (h0 + fp.rpb - 1 < g.in[1] ? h0 + fp.rpb - 1 : g.in[1] - 1);
+  int32_t ow_min = w0 + g.pad[2] - (g.ker[2] - 1) * g.dil[2];
+  ow_min = ow_min <= 0 ? 0 : (ow_min + g.str[2] - 1) / g.str[2];
+  int32_t ow_max = (w_last + g.pad[2]) / g.str[2];
+  if (ow_max > g.out[2] - 1) ow_max = g.out[2] - 1;
+  int32_t oh_min = h0 + g.pad[1] - (g.ker[1] - 1) * g.dil[1];
+  oh_min = oh_min <= 0 ? 0 : (oh_min + g.str[1] - 1) / g.str[1];
+  int32_t oh_max = (h_last + g.pad[1]) / g.str[1];
+  if (oh_max > g.out[1] - 1) oh_max = g.out[1] - 1;
+  const int32_t wspan = ow_max - ow_min + 1, hspan = oh_max - oh_min + 1;  // <= the plan's spans
+  const int32_t row_bytes = fp.row_vecs * 16;
+  const int32_t kbase = cg * 8 * g.kvol;
+  // ---- stage. Four vectors per thread and round, all loaded before the first is stored: slots
+  // without data load the image's first patch row instead and are dropped, so no load waits
+  // behind a branch ----
+  const int32_t vec_total = g.ker[0] * fp.oh_span * fp.ow_span * fp.row_vecs;
+  constexpr int kStageUnroll = 4;
+  const E* img = (const E*)dcols + b * g.L * ldc + kbase;
+  for (int32_t v0 = tid; v0 < vec_total; v0 += 256 * kStageUnroll) {
+    u32x4 val[kStageUnroll];
+    int32_t dst[kStageUnroll];
+#pragma unroll
+    for (int u = 0; u < kStageUnroll; ++u) {
+      const int32_t v = v0 + 256 * u;
+      const int32_t q = fp.by_row_vecs.quot(v);
+      const int32_t vc = v - q * fp.row_vecs;
+      const int32_t q2 = fp.by_ow_span.quot(q);
+      const int32_t oi = q - q2 * fp.ow_span;
+      const int32_t kd = fp.by_oh_span.quot(q2);
+      const int32_t hi = q2 - kd * fp.oh_span;
+      const int32_t td = d + g.pad[0] - kd * g.dil[0];
+      const int32_t od = td >= 0 ? fp.by_str[0].quot(td) : -1;
+      const bool ok = v < vec_total && oi < wspan && hi < hspan && od >= 0 &&
+                      od * g.str[0] == td && od < g.out[0];
+      const int64_t l = ok ? ((int64_t)od * g.out[1] + oh_min + hi) * g.out[2] + ow_min + oi : 0;
+      val[u] = ld16(img + l * ldc + (ok ? vc : 0) * EPV);
+      dst[u] = ok ? (((kd * fp.oh_span + hi) * fp.ow_span + oi) * row_bytes + vc * 16) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kStageUnroll; ++u)
+      if (dst[u] >= 0) *(u32x4*)(fold_lds + dst[u]) = val[u];
+  }
+  __syncthreads();
+  // ---- sum: thread = pixel tid of the patch, 8 channels ----
+  const int32_t prow = fp.by_cpb.quot(tid);
+  const int32_t w = w0 + tid - prow * fp.cpb, h = h0 + prow;
+  if (w >= g.in[2] || h >= g.in[1]) return;
+  float acc[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c) acc[c] = 0.f;
+  for (int32_t kd = 0; kd < g.ker[0]; ++kd) {
+    const int32_t td = d + g.pad[0] - kd * g.dil[0];
+    if (td < 0) continue;
+    const int32_t od = fp.by_str[0].quot(td);
+    if (od * g.str[0] != td || od >= g.out[0]) continue;
+    for (int32_t kh = 0; kh < g.ker[1]; ++kh) {
+      const int32_t th = h + g.pad[1] - kh * g.dil[1];
+      if (th < 0) continue;
+      const int32_t oh = fp.by_str[1].quot(th);
+      if (oh * g.str[1] != th || oh >= g.out[1]) continue;
+      const char* rows = fold_lds + ((kd * fp.oh_span + (oh - oh_min)) * fp.ow_span) * row_bytes;
+      for (int32_t kw = 0; kw < g.ker[2]; ++kw) {
+        const int32_t tw = w + g.pad[2] - kw * g.dil[2];
+        if (tw < 0) continue;
+        const int32_t ow = fp.by_str[2].quot(tw);
+        if (ow * g.str[2] != tw || ow >= g.out[2]) continue;
+        const char* row = rows + (ow - ow_min) * row_bytes;
+        const int32_t k = (kd * g.ker[1] + kh) * g.ker[2] + kw;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) acc[c] += D::load(row, c * g.kvol + k);
+      }
+    }
+  }
+  const int64_t plane = (int64_t)g.in[1] * g.in[2];
+  const int64_t o = (((b * g.C + cg * 8) * g.in[0] + d) * plane) + (int64_t)h * g.in[2] + w;
+#pragma unroll
+  for (int c = 0; c < 8; ++c) D::store(dx, o + c * g.in[0] * plane, acc[c]);
+}
+
 // dst[b][c][r] = src[b][r][c]; 32 x 32 tiles through LDS (padded against bank conflicts) so that
 // both the reads and the writes are contiguous.
 template <class E>
@@ -472,21 +575,25 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
   ConvGeom g;
   if (dcols == nullptr || dx == nullptr || !make_geom(geom, &g) || ldc < g.K) return AHL_ERR_ARG;
   const int64_t total = (int64_t)g.B * g.C * g.in[0] * g.in[1] * g.in[2];
-  // tiled kernel: channel groups of 8 whose 8 * kvol patch entries are whole 16-byte vectors
-  {
+  // tiled kernels: channel groups of 8 whose 8 * kvol patch entries are whole 16-byte vectors;
+  // first the plan with 256 pixels per block, then (if its staging area does not fit) 64
+  for (int pixels = 256; pixels >= 64; pixels /= 4) {
     const int epv = dtype == AHL_BF16 ? 8 : 4;
     const int64_t row_entries = 8 * (int64_t)g.kvol;
     int32_t cpb = 64;
     while (cpb > 8 && cpb / 2 >= g.in[2]) cpb /= 2;
-    const int32_t rpb = 64 / cpb;
+    const int32_t rpb = pixels / cpb;
     // widest window of output columns / rows that one block's image patch can reach
-    const int64_t ow_span = (cpb - 1 + (int64_t)(g.ker[2] - 1) * g.dil[2]) / g.str[2] + 2;
-    const int64_t oh_span = (rpb - 1 + (int64_t)(g.ker[1] - 1) * g.dil[1]) / g.str[1] + 2;
+    int64_t ow_span = (cpb - 1 + (int64_t)(g.ker[2] - 1) * g.dil[2]) / g.str[2] + 2;
+    int64_t oh_span = (rpb - 1 + (int64_t)(g.ker[1] - 1) * g.dil[1]) / g.str[1] + 2;
+    if (ow_span > g.out[2]) ow_span = g.out[2];
+    if (oh_span > g.out[1]) oh_span = g.out[1];
+    const int64_t lds_limit = pixels == 256 ? 64 * 1024 : 96 * 1024;
     const int64_t lds_bytes = (int64_t)g.ker[0] * oh_span * ow_span * row_entries * (dtype == AHL_BF16 ? 2 : 4);
     const int64_t w_tiles = cdiv(g.in[2], cpb), h_tiles = cdiv(g.in[1], rpb);
     const int64_t tblocks = (int64_t)g.B * (g.C / 8) * g.in[0] * h_tiles * w_tiles;
     if ((dtype == AHL_BF16 || dtype == AHL_F32) && g.C % 8 == 0 && row_entries % epv == 0 &&
-        ldc % epv == 0 && aligned16(dcols) && lds_bytes <= 96 * 1024 && tblocks <= 0x7fffffff &&
+        ldc % epv == 0 && aligned16(dcols) && lds_bytes <= lds_limit && tblocks <= 0x7fffffff &&
         g.in[0] + g.pad[0] < (1 << 22) && g.in[1] + g.pad[1] < (1 << 22) &&
         g.in[2] + g.pad[2] < (1 << 22)) {
       FoldPlan fp{cpb, rpb, (int32_t)ow_span, (int32_t)oh_span, (int32_t)(row_entries / epv),
@@ -495,10 +602,17 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
                   make_small_div((int32_t)oh_span), make_small_div(cpb),
                   {make_small_div(g.str[0]), make_small_div(g.str[1]), make_small_div(g.str[2])}};
       AHL_DISPATCH_DTYPE(dtype, {
-        hipFuncSetAttribute((const void*)k_col2im_tiled<D>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        hipLaunchKernelGGL((k_col2im_tiled<D>), dim3((unsigned)tblocks), dim3(512), (size_t)lds_bytes,
-                           (hipStream_t)stream, dcols, ldc, g, fp, dx);
+        if (pixels == 256) {
+          hipFuncSetAttribute((const void*)k_col2im_wide<D>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+          hipLaunchKernelGGL((k_col2im_wide<D>), dim3((unsigned)tblocks), dim3(256), (size_t)lds_bytes,
+                             (hipStream_t)stream, dcols, ldc, g, fp, dx);
+        } else {
+          hipFuncSetAttribute((const void*)k_col2im_tiled<D>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+          hipLaunchKernelGGL((k_col2im_tiled<D>), dim3((unsigned)tblocks), dim3(512), (size_t)lds_bytes,
+                             (hipStream_t)stream, dcols, ldc, g, fp, dx);
+        }
       });
       return check_launch("k_col2im_tiled");
     }

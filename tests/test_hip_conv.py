@@ -39,6 +39,11 @@ GEOMS = [
     (2, 8, (1, 9, 7), (1, 3, 3), (1, 2, 1), (0, 1, 1), (1, 1, 1)),     # narrow image: 8 x 8 pixel patches
     (1, 8, (2, 30, 28), (2, 5, 3), (1, 3, 2), (0, 2, 1), (1, 1, 1)),   # 2 x 32 patches, strides, 3-d
     (2, 16, (1, 14, 14), (1, 3, 3), (1, 1, 1), (0, 1, 1), (1, 2, 2)),  # 4 x 16 patches, dilation
+    # 5 x 5 kernel on a 40-wide image: the 256-pixel fold kernel's staging area does not fit,
+    # the 64-pixel one's does
+    (2, 8, (1, 12, 40), (1, 5, 5), (1, 1, 1), (0, 2, 2), (1, 1, 1)),
+    (1, 16, (1, 28, 28), (1, 3, 3), (1, 1, 1), (0, 1, 1), (1, 1, 1)),  # 8 x 32 patches of the 256-pixel kernel
+    (1, 8, (3, 10, 18), (2, 3, 3), (2, 2, 1), (1, 0, 1), (1, 1, 1)),   # 3-d, strides, 256 pixels
 ]
 
 
