@@ -83,6 +83,7 @@ class HipLinear(Function):
         x_min: Optional[Tensor] = None,
         x_max: Optional[Tensor] = None,
         learnable_weight_clip: Optional[Tensor] = None,
+        weight_cache: Optional[dict] = None,
     ) -> Tensor:
         if not inp.is_cuda:
             raise HipBackendError(
@@ -166,21 +167,28 @@ class HipLinear(Function):
             )
         elif m_rows > 0 and need_wmax:
             res = float(modifier.res) if w_quant else 1.0
-            wmax, tile_max, _, eff = ops.weight_prep(
-                weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
-                NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE, res,
-                float(modifier.std_dev), seed, 1, w_noise or w_quant,
-                # per-tile maxima are only read when the ADC bound or the output noise scale with
-                # the whole tile instead of the channel
-                (not bound_on or per_channel_bound) and (not noise_on or fwd.out_noise_per_channel),
-            )
-            if w_noise or w_quant:
-                w_eff = eff
+            # per-tile maxima are only read when the ADC bound or the output noise scale with
+            # the whole tile instead of the channel
+            skip_tile_stats = ((not bound_on or per_channel_bound)
+                               and (not noise_on or fwd.out_noise_per_channel))
+            # A caller that promises unchanged weights over several calls (the steps of a
+            # recurrent sequence) passes a dict: what depends on the weights alone is computed
+            # by the first call and reused. A modifier draws new weights per call: no reuse.
+            reuse = weight_cache if not (w_noise or w_quant) else None
+            stats_key = ("stats", skip_tile_stats)
+            if reuse is not None and stats_key in reuse:
+                wmax, tile_max = reuse[stats_key]
+            else:
+                wmax, tile_max, _, eff = ops.weight_prep(
+                    weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
+                    NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE, res,
+                    float(modifier.std_dev), seed, 1, w_noise or w_quant, skip_tile_stats,
+                )
+                if w_noise or w_quant:
+                    w_eff = eff
+                if reuse is not None:
+                    reuse[stats_key] = (wmax, tile_max)
 
-        # bf16 splits whose tiles do not start on the MFMA kernels' 256-column block boundaries:
-        # the quantised input and the effective weights are kept in a padded tile layout instead
-        # (stride > 0), unless the padding would blow the work up more than the slower general
-        # kernels do, or the shape does not fit the fast backward at all
         # bf16 layers whose output width is not a multiple of 8 (a 50257-word vocabulary): the
         # MFMA kernels handle channels in whole 16-byte vectors, so the weight-side operands get
         # zero channels up to the next multiple of 8 and the extra output columns are dropped.
@@ -192,13 +200,24 @@ class HipLinear(Function):
         if (inp.dtype == torch.bfloat16 and n_out % 8 != 0 and not learned_clip
                 and m_rows * k_in * n_out >= PAD_CHANNELS_MIN_WORK):
             pad_n = 8 - n_out % 8
-            w_eff = torch.nn.functional.pad(w_eff.detach(), (0, 0, 0, pad_n))
-            if wmax is not None:
-                wmax = torch.nn.functional.pad(wmax, (0, pad_n), value=1.0)
-            if bias is not None:
-                bias_k = torch.nn.functional.pad(bias.detach(), (0, pad_n))
+            frozen = weight_cache if w_eff is weights_c else None  # no per-call modifier
+            if frozen is not None and ("channels", pad_n) in frozen:
+                w_eff, wmax, bias_k = frozen[("channels", pad_n)]
+            else:
+                w_eff = torch.nn.functional.pad(w_eff.detach(), (0, 0, 0, pad_n))
+                if wmax is not None:
+                    wmax = torch.nn.functional.pad(wmax, (0, pad_n), value=1.0)
+                if bias is not None:
+                    bias_k = torch.nn.functional.pad(bias.detach(), (0, pad_n))
+                if frozen is not None:
+                    frozen[("channels", pad_n)] = (w_eff, wmax, bias_k)
         n_k = n_out + pad_n
+        weights_frozen = weight_cache is not None and not (w_noise or w_quant or learned_clip)
 
+        # bf16 splits whose tiles do not start on the MFMA kernels' 256-column block boundaries:
+        # the quantised input and the effective weights are kept in a padded tile layout instead
+        # (stride > 0), unless the padding would blow the work up more than the slower general
+        # kernels do, or the shape does not fit the fast backward at all
         stride = 0
         dense_fwd_ok = len(set(in_sizes)) == 1 and in_sizes[0] % 64 == 0
         if (inp.dtype == torch.bfloat16 and m_rows > 0 and n_k % 8 == 0
@@ -228,7 +247,13 @@ class HipLinear(Function):
         # clamp + DAC are fused into the matrix kernel's A-tile staging.
         split_dac = stride > 0 or (inp.dtype == torch.bfloat16 and dense_fwd_ok and n_k % 8 == 0)
         if stride > 0:
-            w_eff = ops.pad_tiles(w_eff, in_sizes, stride)
+            tiles_key = ("tiles", stride, pad_n)
+            if weights_frozen and tiles_key in weight_cache:
+                w_eff = weight_cache[tiles_key]
+            else:
+                w_eff = ops.pad_tiles(w_eff, in_sizes, stride)
+                if weights_frozen:
+                    weight_cache[tiles_key] = w_eff
         ir_dev = xq = None
         if ir_mode == L.AHL_IR_STATIC:
             if training and init_active and fast:
@@ -325,4 +350,4 @@ class HipLinear(Function):
         if not ctx.needs_input_grad[1]:
             grad_w = None
         return (grad_inp, grad_w, grad_b, grad_ir, None, None, None, None, None, None, None,
-                grad_clip)
+                grad_clip, None)

@@ -8,11 +8,14 @@ the GPU where ``batch`` rows per step do not. The result is the same, row for ro
 In training mode every step calls the cell as the reference does, so that noise draws and
 input-range updates happen once per step.
 """
+from contextlib import ExitStack
 from typing import Any, List, Tuple, Type
 
 import torch
 from torch import Tensor
 from torch.nn import Module, ModuleList
+
+from ..tiled import TiledAnalogLayer
 
 
 class AnalogRNNLayer(Module):
@@ -38,14 +41,19 @@ class AnalogRNNLayer(Module):
         steps = input_.size(0)
         order = range(steps - 1, -1, -1) if self.time_reversed else range(steps)
         outputs: List[Tensor] = [None] * steps  # type: ignore[list-item]
-        if self._project_ahead() and steps > 0:
-            igates = self.cell.project_input(input_.reshape(steps * input_.size(1), -1))
-            igates = igates.view(steps, input_.size(1), -1)
-            for t in order:
-                outputs[t], state = self.cell.recur(igates[t], state)
-        else:
-            for t in order:
-                outputs[t], state = self.cell(input_[t], state)
+        with ExitStack() as stack:
+            # the weights do not change between the steps of one sequence
+            for module in self.cell.modules():
+                if isinstance(module, TiledAnalogLayer):
+                    stack.enter_context(module.frozen_weights())
+            if self._project_ahead() and steps > 0:
+                igates = self.cell.project_input(input_.reshape(steps * input_.size(1), -1))
+                igates = igates.view(steps, input_.size(1), -1)
+                for t in order:
+                    outputs[t], state = self.cell.recur(igates[t], state)
+            else:
+                for t in order:
+                    outputs[t], state = self.cell(input_[t], state)
         return torch.stack(outputs), state
 
 

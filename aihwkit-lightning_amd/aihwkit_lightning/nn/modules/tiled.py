@@ -3,6 +3,7 @@ input dimension: ``AnalogLinear`` directly, the convolution layers through their
 ``weight.view(out_channels, -1)``. Tile split, input-range state, the call into the HIP
 operator, weight clipping and post-training quantisation follow the reference
 (``nn/modules/linear.py:53-317``, ``nn/modules/conv.py:121-367``)."""
+from contextlib import contextmanager
 from copy import deepcopy
 from typing import List, Optional, Tuple
 
@@ -98,6 +99,23 @@ class TiledAnalogLayer(AnalogLayerBase):
             self._ir_init_calls = int(idx_min) if self._ir_init_active else 0
         return bool(self._ir_init_active)
 
+    #: set by :meth:`frozen_weights`; None means "the weights may change between calls"
+    _weight_cache = None
+
+    @contextmanager
+    def frozen_weights(self):
+        """Promise that the weights do not change inside the block: what a call computes from the
+        weights alone (per-tile abs-max, padded operand copies) is computed once and reused by
+        the following calls. For callers that apply one layer many times in a row, like the steps
+        of a recurrent sequence. Nothing is reused while a weight modifier is active."""
+        outer = self._weight_cache
+        if outer is None:
+            self._weight_cache = {}
+        try:
+            yield self
+        finally:
+            self._weight_cache = outer
+
     def analog_mvm(self, rows: Tensor) -> Tensor:
         """``rows[..., in] @ weight_matrix^T + bias`` through the analog tile model."""
         init_active = self.training and self._init_phase_active()
@@ -124,6 +142,7 @@ class TiledAnalogLayer(AnalogLayerBase):
             self.x_min,
             self.x_max,
             weight_clip,
+            self._weight_cache,
         )
         if init_active:
             self._ir_init_calls += 1

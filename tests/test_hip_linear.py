@@ -234,6 +234,37 @@ def test_misaligned_gradient_with_padded_layout(name):
     check_against(res, ref, c, name + " misaligned gradient")
 
 
+@pytest.mark.parametrize("name", ["sliced_dx_bf16_clamped", "pad_bf16_uneven_clamped",
+                                  "padn_bf16_static_clamped", "edge_f32"])
+def test_frozen_weights_reuse_what_depends_on_the_weights(name):
+    """Inside ``frozen_weights()`` the per-tile abs-max and the padded operand copies are computed
+    by the first call only; results and gradients are those of ordinary calls, and a weight change
+    after the block is seen again."""
+    from hip_helpers import make_layer
+
+    c = [s for s in SHAPES if s["name"] == name][0]
+    x, w, b, g = make_inputs(c)
+    layer = make_layer(c, inputs=(x, w, b, None))
+    xin = x.cuda().requires_grad_(True)
+    want = layer(xin)
+    want.backward(g.cuda())
+    want_dx, want_dw = xin.grad.clone(), layer.weight.grad.clone()
+    xin.grad = None
+    layer.zero_grad(set_to_none=True)
+    with layer.frozen_weights():
+        first = layer(xin)
+        assert layer._weight_cache, "nothing was kept for the next call"
+        second = layer(xin)
+        second.backward(g.cuda())
+    assert layer._weight_cache is None
+    assert torch.equal(first, want) and torch.equal(second, want)
+    assert torch.equal(xin.grad, want_dx) and torch.equal(layer.weight.grad, want_dw)
+    with torch.no_grad():
+        layer.weight.mul_(0.5)
+        changed = layer(x.cuda())
+    assert not torch.equal(changed, want)
+
+
 def test_padded_channels_with_noise_stay_finite():
     """Output noise scaled by the whole tile also lands on the appended channels; nothing of it
     may leak into the result."""
