@@ -14,7 +14,7 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
@@ -179,6 +179,14 @@ SIGNATURES = {
     "ahl_sliced_quantile_ws_bytes": (c_int64, [c_int64, c_int32]),
     "ahl_ir_moving_update": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_double,
                                        c_int32, c_void_p]),
+    "ahl_lstm_gates_fwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p,
+                                     c_void_p, c_void_p, c_void_p]),
+    "ahl_lstm_gates_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64,
+                                     c_int64, c_void_p, c_void_p, c_void_p]),
+    "ahl_gru_gates_fwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p,
+                                    c_void_p, c_void_p]),
+    "ahl_gru_gates_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int64,
+                                    c_void_p, c_void_p, c_void_p, c_void_p]),
     "ahl_pad_tiles": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int64, _I32P, c_int32, c_int64,
                                 c_void_p, c_int64, c_void_p]),
     "ahl_unpad_tiles": (c_int32, [c_void_p, c_int64, c_int32, c_int64, c_int64, _I32P, c_int32,

@@ -648,6 +648,83 @@ def linear_bwd_dw(
     return dw, dbias
 
 
+# ---------------------------------------------------------------------------------------------
+# Gate arithmetic of the recurrent cells (called from the cells' autograd functions directly; no
+# dispatcher entry: they are internal to those functions)
+def gates_supported(*tensors: Tensor) -> bool:
+    """Whether the fused gate kernels can take these operands: on the GPU, float32 / bfloat16,
+    hidden size (last dimension of the last tensor) in whole 16-byte vectors."""
+    ref = tensors[-1]
+    if not ref.is_cuda or ref.dtype not in _DTYPES or ref.dim() != 2:
+        return False
+    return ref.size(1) % (16 // ref.element_size()) == 0 and ref.size(0) > 0
+
+
+def dense(tensor: Optional[Tensor]) -> Optional[Tensor]:
+    """``tensor`` as a dense, 16-byte aligned matrix (itself if it already is one)."""
+    if tensor is None:
+        return None
+    if not tensor.is_contiguous() or tensor.data_ptr() % 16 != 0:
+        tensor = tensor.clone(memory_format=torch.contiguous_format)
+    return tensor
+
+
+def lstm_gates_fwd(igates: Tensor, hgates: Optional[Tensor], c_x: Tensor,
+                   want_act: bool) -> Tuple[Tensor, Tensor, Optional[Tensor]]:
+    """``(h_y, c_y, activated gates or None)`` of an LSTM step."""
+    lib = L.load()
+    igates, hgates, c_x = dense(igates), dense(hgates), dense(c_x)
+    rows, hidden = c_x.shape
+    h_y, c_y = torch.empty_like(c_x), torch.empty_like(c_x)
+    act = torch.empty_like(igates) if want_act else None
+    L.check(lib.ahl_lstm_gates_fwd(_ptr(igates), _ptr(hgates), _ptr(c_x), dtype_id(c_x.dtype), rows,
+                                   hidden, _ptr(h_y), _ptr(c_y), _ptr(act), _stream()),
+            "ahl_lstm_gates_fwd")
+    return h_y, c_y, act
+
+
+def lstm_gates_bwd(dh_y: Tensor, dc_y: Optional[Tensor], act: Tensor, c_x: Tensor,
+                   c_y: Tensor) -> Tuple[Tensor, Tensor]:
+    """``(dgates [rows, 4H], dc_x)``."""
+    lib = L.load()
+    dh_y, dc_y = dense(dh_y), dense(dc_y)
+    rows, hidden = c_x.shape
+    dgates, dc_x = torch.empty_like(act), torch.empty_like(c_x)
+    L.check(lib.ahl_lstm_gates_bwd(_ptr(dh_y), _ptr(dc_y), _ptr(act), _ptr(c_x), _ptr(c_y),
+                                   dtype_id(c_x.dtype), rows, hidden, _ptr(dgates), _ptr(dc_x),
+                                   _stream()),
+            "ahl_lstm_gates_bwd")
+    return dgates, dc_x
+
+
+def gru_gates_fwd(igates: Tensor, hgates: Tensor, h_x: Tensor,
+                  want_act: bool) -> Tuple[Tensor, Optional[Tensor]]:
+    """``(h_y, (reset, update, new) or None)`` of a GRU step."""
+    lib = L.load()
+    igates, hgates, h_x = dense(igates), dense(hgates), dense(h_x)
+    rows, hidden = h_x.shape
+    h_y = torch.empty_like(h_x)
+    act = torch.empty_like(igates) if want_act else None
+    L.check(lib.ahl_gru_gates_fwd(_ptr(igates), _ptr(hgates), _ptr(h_x), dtype_id(h_x.dtype), rows,
+                                  hidden, _ptr(h_y), _ptr(act), _stream()),
+            "ahl_gru_gates_fwd")
+    return h_y, act
+
+
+def gru_gates_bwd(dh_y: Tensor, act: Tensor, hgates: Tensor,
+                  h_x: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
+    """``(digates, dhgates [rows, 3H], dh_x)``."""
+    lib = L.load()
+    dh_y = dense(dh_y)
+    rows, hidden = h_x.shape
+    digates, dhgates, dh_x = torch.empty_like(act), torch.empty_like(act), torch.empty_like(h_x)
+    L.check(lib.ahl_gru_gates_bwd(_ptr(dh_y), _ptr(act), _ptr(hgates), _ptr(h_x),
+                                  dtype_id(h_x.dtype), rows, hidden, _ptr(digates), _ptr(dhgates),
+                                  _ptr(dh_x), _stream()),
+            "ahl_gru_gates_bwd")
+    return digates, dhgates, dh_x
+
+
 for _name, _fn in [
     ("sliced_absmax", sliced_absmax), ("sliced_std", sliced_std),
     ("row_nonzero", row_nonzero), ("sliced_std_kept", sliced_std_kept), ("sliced_quantile", sliced_quantile),

@@ -12,20 +12,85 @@ from typing import Optional, Tuple
 
 import torch
 from torch import Tensor
+from torch.autograd import Function
 from torch.nn import Module
 
+from ..hip_utils import ops as gate_ops
 from ..linear import AnalogLinear
 from ....simulator.configs import TorchInferenceRPUConfig
 
 LSTMState = namedtuple("LSTMState", ["hx", "cx"])
 
 
-def lstm_pointwise(gates: Tensor, c_x: Tensor) -> Tuple[Tensor, Tensor]:
-    """``(h_y, c_y)`` from the summed pre-activations ``[B, 4H]`` in the order input, forget,
-    cell, output (reference cells.py:176-186)."""
+class _LstmGates(Function):
+    """LSTM gate arithmetic of one step as one kernel per pass."""
+
+    # pylint: disable=abstract-method, arguments-differ
+
+    @staticmethod
+    def forward(ctx, igates: Tensor, hgates: Optional[Tensor], c_x: Tensor):
+        needs = any(ctx.needs_input_grad)
+        c_x = gate_ops.dense(c_x)  # the backward pass reads it again
+        h_y, c_y, act = gate_ops.lstm_gates_fwd(igates, hgates, c_x, needs)
+        if needs:
+            ctx.save_for_backward(act, c_x, c_y)
+        ctx.two_products = hgates is not None
+        ctx.set_materialize_grads(False)
+        return h_y, c_y
+
+    @staticmethod
+    def backward(ctx, dh_y: Optional[Tensor], dc_y: Optional[Tensor]):
+        act, c_x, c_y = ctx.saved_tensors
+        if dh_y is None:
+            dh_y = torch.zeros_like(c_y)
+        dgates, dc_x = gate_ops.lstm_gates_bwd(dh_y, dc_y, act, c_x, c_y)
+        return dgates, dgates if ctx.two_products else None, dc_x
+
+
+class _GruGates(Function):
+    """GRU gate arithmetic of one step as one kernel per pass."""
+
+    # pylint: disable=abstract-method, arguments-differ
+
+    @staticmethod
+    def forward(ctx, igates: Tensor, hgates: Tensor, h_x: Tensor):
+        needs = any(ctx.needs_input_grad)
+        hgates, h_x = gate_ops.dense(hgates), gate_ops.dense(h_x)  # the backward pass reads them again
+        h_y, act = gate_ops.gru_gates_fwd(igates, hgates, h_x, needs)
+        if needs:
+            ctx.save_for_backward(act, hgates, h_x)
+        return h_y
+
+    @staticmethod
+    def backward(ctx, dh_y: Tensor):
+        act, hgates, h_x = ctx.saved_tensors
+        return gate_ops.gru_gates_bwd(dh_y, act, hgates, h_x)
+
+
+def lstm_pointwise(igates: Tensor, hgates: Optional[Tensor], c_x: Tensor) -> Tuple[Tensor, Tensor]:
+    """``(h_y, c_y)`` from the pre-activations ``[B, 4H]`` of the input product and (if there are
+    two products) the hidden product, gate blocks in the order input, forget, cell, output
+    (reference cells.py:176-186). One fused kernel where the operands allow it."""
+    if gate_ops.gates_supported(igates, c_x):
+        return _LstmGates.apply(igates, hgates, c_x)
+    gates = igates if hgates is None else igates + hgates
     in_gate, forget_gate, cell_gate, out_gate = gates.chunk(4, 1)
     c_y = torch.sigmoid(forget_gate) * c_x + torch.sigmoid(in_gate) * torch.tanh(cell_gate)
     return torch.sigmoid(out_gate) * torch.tanh(c_y), c_y
+
+
+def gru_pointwise(igates: Tensor, hgates: Tensor, h_x: Tensor) -> Tensor:
+    """New hidden state from the pre-activations ``[B, 3H]`` of the two products, gate blocks in
+    the order reset, update, new; the reset gate scales the hidden part of the candidate after
+    the product (reference cells.py:321-343). One fused kernel where the operands allow it."""
+    if gate_ops.gates_supported(igates, h_x):
+        return _GruGates.apply(igates, hgates, h_x)
+    i_r, i_z, i_n = igates.chunk(3, 1)
+    h_r, h_z, h_n = hgates.chunk(3, 1)
+    reset = torch.sigmoid(i_r + h_r)
+    update = torch.sigmoid(i_z + h_z)
+    cand = torch.tanh(i_n + reset * h_n)
+    return cand + update * (h_x - cand)
 
 
 class _AnalogCell(Module):
@@ -92,7 +157,7 @@ class AnalogLSTMCell(_AnalogCell):
 
     def recur(self, igates, state):
         h_x, c_x = state
-        h_y, c_y = lstm_pointwise(igates + self.weight_hh(h_x), c_x)
+        h_y, c_y = lstm_pointwise(igates, self.weight_hh(h_x), c_x)
         return h_y, (h_y, c_y)
 
 
@@ -104,12 +169,7 @@ class AnalogGRUCell(_AnalogCell):
 
     def recur(self, igates, state):
         h_x, _ = state
-        i_r, i_z, i_n = igates.chunk(3, 1)
-        h_r, h_z, h_n = self.weight_hh(h_x).chunk(3, 1)
-        reset = torch.sigmoid(i_r + h_r)
-        update = torch.sigmoid(i_z + h_z)
-        cand = torch.tanh(i_n + reset * h_n)
-        h_y = cand + update * (h_x - cand)
+        h_y = gru_pointwise(igates, self.weight_hh(h_x), h_x)
         return h_y, (h_y, None)
 
 
@@ -144,5 +204,5 @@ class AnalogLSTMCellCombinedWeight(Module):
     def forward(self, input_: Tensor, state) -> Tuple[Tensor, Tuple[Tensor, Tensor]]:
         """One time step."""
         h_x, c_x = state
-        h_y, c_y = lstm_pointwise(self.weight(torch.cat((input_, h_x), 1)), c_x)
+        h_y, c_y = lstm_pointwise(self.weight(torch.cat((input_, h_x), 1)), None, c_x)
         return h_y, (h_y, c_y)

@@ -24,7 +24,9 @@ __global__ __launch_bounds__(256) void k_sliced_absmax(const void* __restrict__ 
   if (lane == 0) D::store(out, (int64_t)t * rows + r, m);
 }
 
-// tile_max[t] = max_r v[t, r], tile_min[t] = min_r v[t, r]; one block per tile.
+// tile_max[t] = max_r v[t, r], tile_min[t] = min_r v[t, r]; one block per tile. The loads of a
+// thread do not depend on each other: eight are in flight at a time (the kernel is a handful of
+// blocks, so its duration is the latency of a thread's chain of loads).
 template <class D>
 __global__ __launch_bounds__(256) void k_tile_minmax(const void* __restrict__ v, int64_t rows,
                                                      float* __restrict__ tile_max,
@@ -32,10 +34,18 @@ __global__ __launch_bounds__(256) void k_tile_minmax(const void* __restrict__ v,
   __shared__ float smax[4], smin[4];
   const int t = blockIdx.x;
   float mx = 0.0f, mn = __builtin_inff();
-  for (int64_t r = threadIdx.x; r < rows; r += 256) {
-    const float a = D::load(v, (int64_t)t * rows + r);
-    mx = fmaxf(mx, a);
-    mn = fminf(mn, a);
+  for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 256 * 8) {
+    float a[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t r = r0 + 256 * u;
+      a[u] = D::load(v, (int64_t)t * rows + (r < rows ? r : r0));  // r0 again: no effect on max / min
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      mx = fmaxf(mx, a[u]);
+      mn = fminf(mn, a[u]);
+    }
   }
   mx = wave_max(mx);
   mn = wave_min(mn);

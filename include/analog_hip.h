@@ -191,6 +191,32 @@ int64_t ahl_sliced_quantile_ws_bytes(int64_t rows, int32_t n_tiles);
 int ahl_ir_moving_update(void* ir, int32_t* idx, const float* val, int32_t dtype, int32_t n_tiles,
                          double alpha, int32_t val_in_dtype, void* stream);
 
+/* Gate arithmetic of the recurrent cells in one pass per direction: everything between the two
+ * analog products of a step and the new state. Replaces the element-wise torch operations of
+ * nn/modules/rnn/cells.py:176-186 (LSTM: gates = igates + hgates; i, f, g, o = sigmoid / tanh of
+ * the four blocks; c' = f c + i g; h' = o tanh(c')) and :321-343 (GRU: r = sigmoid(i_r + h_r);
+ * z = sigmoid(i_z + h_z); n = tanh(i_n + r h_n); h' = n + z (h - n)) and what autograd derives
+ * from them, with the dtype rounding after every operation that the torch chain has.
+ * All matrices dense row-major, 16-byte aligned; gates [rows, 4 hidden] / [rows, 3 hidden], states
+ * [rows, hidden]; hidden a multiple of 8 (bf16) or 4 (fp32).
+ * lstm fwd: hgates may be null (one product over [x, h], cells.py:244-267); act [rows, 4 hidden]
+ *   receives the activated gates for the backward pass (null: not wanted).
+ * lstm bwd: dcy may be null (c' unused downstream); dgates is the gradient of both products'
+ *   outputs; dcx that of the previous cell state.
+ * gru fwd: act [rows, 3 hidden] receives r, z, n (null: not wanted).
+ * gru bwd: digates / dhgates are the gradients of the input / hidden product's outputs, dhx the
+ *   direct path from the previous hidden state.                                              */
+int ahl_lstm_gates_fwd(const void* igates, const void* hgates, const void* cx, int32_t dtype,
+                       int64_t rows, int64_t hidden, void* hy, void* cy, void* act, void* stream);
+int ahl_lstm_gates_bwd(const void* dhy, const void* dcy, const void* act, const void* cx,
+                       const void* cy, int32_t dtype, int64_t rows, int64_t hidden, void* dgates,
+                       void* dcx, void* stream);
+int ahl_gru_gates_fwd(const void* igates, const void* hgates, const void* hx, int32_t dtype,
+                      int64_t rows, int64_t hidden, void* hy, void* act, void* stream);
+int ahl_gru_gates_bwd(const void* dhy, const void* act, const void* hgates, const void* hx,
+                      int32_t dtype, int64_t rows, int64_t hidden, void* digates, void* dhgates,
+                      void* dhx, void* stream);
+
 /* Input-range initialisation from data, all tiles, no host sync:
  *   if idx[t] < init_from_data: if std[t] > 0 { ir[t] = (ir[t]*idx[t] + alpha*std[t])/(idx[t]+1);
  *   idx[t] += 1 }  ir[t] = |ir[t]|.   ir and idx are dtype [n_tiles], updated in place.

@@ -228,3 +228,83 @@ def test_graph_replays_equal_the_eager_forward(cell):
     net.train()
     with pytest.raises(RuntimeError, match="evaluation-mode"):
         net.graphed(example)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("rows,hidden", [(3, 8), (64, 1024), (17, 40)])
+def test_fused_gates_match_the_chain_of_torch_operations(dtype, rows, hidden):
+    """ahl_lstm_gates_* / ahl_gru_gates_* against the element-wise torch operations they replace,
+    on the same device: the forward bit for bit in fp32 up to the last place of exp / tanh and
+    exactly in bf16 (both round an fp32 activation once), the gradients to the dtype's rounding."""
+    from aihwkit_lightning.nn.modules.rnn import cells
+
+    print(f"case gates {dtype} {rows}x{hidden}", flush=True)
+    gen = torch.Generator().manual_seed(9)
+    mk = lambda *shape: (torch.randn(*shape, generator=gen) * 1.5).to(dtype).cuda().requires_grad_(True)  # noqa: E731
+    # bf16 gradients: one rounding that falls the other way (torch's kernels contract a * b + c,
+    # this library does not) is one step of the larger operand where two terms cancel, so the
+    # element-wise bound is a step at the operands' magnitude (~4) and the norm is checked too
+    tol = dict(rtol=2e-6, atol=2e-6) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=3.2e-2)
+
+    def close(a, b):
+        a, b = a.float(), b.float()
+        return torch.allclose(a, b, **tol) and float((a - b).norm()) <= 5e-3 * float(b.norm())
+
+    def chain_lstm(ig, hg, c_x):
+        i, f, g, o = (ig + hg).chunk(4, 1)
+        c_y = torch.sigmoid(f) * c_x + torch.sigmoid(i) * torch.tanh(g)
+        return torch.sigmoid(o) * torch.tanh(c_y), c_y
+
+    def chain_gru(ig, hg, h_x):
+        i_r, i_z, i_n = ig.chunk(3, 1)
+        h_r, h_z, h_n = hg.chunk(3, 1)
+        r, z = torch.sigmoid(i_r + h_r), torch.sigmoid(i_z + h_z)
+        n = torch.tanh(i_n + r * h_n)
+        return n + z * (h_x - n)
+
+    # LSTM, both outputs used
+    ig, hg, c_x = mk(rows, 4 * hidden), mk(rows, 4 * hidden), mk(rows, hidden)
+    g_h, g_c = mk(rows, hidden).detach(), mk(rows, hidden).detach()
+    assert cells.gate_ops.gates_supported(ig, c_x)
+    h_y, c_y = cells.lstm_pointwise(ig, hg, c_x)
+    ((h_y * g_h).sum() + (c_y * g_c).sum()).backward()
+    got = [t.grad.clone() for t in (ig, hg, c_x)]
+    for t in (ig, hg, c_x):
+        t.grad = None
+    want_h, want_c = chain_lstm(ig, hg, c_x)
+    ((want_h * g_h).sum() + (want_c * g_c).sum()).backward()
+    if dtype == torch.bfloat16:
+        assert torch.equal(h_y, want_h) and torch.equal(c_y, want_c)
+    else:
+        assert torch.allclose(h_y, want_h, **tol) and torch.allclose(c_y, want_c, **tol)
+    for a, t in zip(got, (ig, hg, c_x)):
+        assert close(a, t.grad)
+    # LSTM, only the hidden state used (the cell state's gradient is absent)
+    for t in (ig, hg, c_x):
+        t.grad = None
+    h_y, _ = cells.lstm_pointwise(ig, hg, c_x)
+    (h_y * g_h).sum().backward()
+    got = [t.grad.clone() for t in (ig, hg, c_x)]
+    for t in (ig, hg, c_x):
+        t.grad = None
+    (chain_lstm(ig, hg, c_x)[0] * g_h).sum().backward()
+    for a, t in zip(got, (ig, hg, c_x)):
+        assert close(a, t.grad)
+    # GRU
+    ig, hg, h_x = mk(rows, 3 * hidden), mk(rows, 3 * hidden), mk(rows, hidden)
+    h_y = cells.gru_pointwise(ig, hg, h_x)
+    (h_y * g_h).sum().backward()
+    got = [t.grad.clone() for t in (ig, hg, h_x)]
+    for t in (ig, hg, h_x):
+        t.grad = None
+    want = chain_gru(ig, hg, h_x)
+    (want * g_h).sum().backward()
+    if dtype == torch.bfloat16:
+        assert torch.equal(h_y, want)
+    else:
+        assert torch.allclose(h_y, want, **tol)
+    for a, t in zip(got, (ig, hg, h_x)):
+        assert close(a, t.grad)
+    # a hidden size that is not a whole number of vectors takes the torch chain
+    odd = mk(rows, 6)
+    assert not cells.gate_ops.gates_supported(mk(rows, 24), odd)
