@@ -1,5 +1,12 @@
 """Pretty printing shared by the parameter dataclasses."""
-from dataclasses import fields, is_dataclass
+from dataclasses import field, fields, is_dataclass
+from typing import Any
+
+
+def shown(default: Any):
+    """A dataclass field with an immutable default that printing never leaves out (the reference
+    marks such fields with the ``always_show`` metadata key)."""
+    return field(default=default, metadata={"always_show": True})
 
 
 class _PrintableMixin:

@@ -1,31 +1,22 @@
 """Weight modifier and clip settings (reference ``inference.py:29-90``)."""
-from dataclasses import dataclass, field
-from .helpers import _PrintableMixin
-from .enums import (
-    WeightModifierType,
-    WeightNoiseInjectionType,
-    WeightQuantizationType,
-    WeightClipType,
-)
+from dataclasses import dataclass
+
+from . import enums
+from .helpers import _PrintableMixin, shown
 
 
 @dataclass
 class WeightModifierParameter(_PrintableMixin):
-    """Noise (``std_dev``, relative to max|W|) and quantisation (``res``) of the weights
-    used in the training forward. ``type`` and ``enable_during_test`` are legacy fields."""
+    """Noise (``std_dev``, relative to max|W|) and quantisation (``res``: a number of states or
+    its inverse) of the weights used in the training forward. ``type`` and
+    ``enable_during_test`` are legacy fields kept for configs written for older versions."""
 
     std_dev: float = 0.0
     res: float = 0.0
     enable_during_test: bool = False
-    type: WeightModifierType = field(
-        default_factory=lambda: WeightModifierType.NONE, metadata={"always_show": True}
-    )
-    noise_type: WeightNoiseInjectionType = field(
-        default_factory=lambda: WeightNoiseInjectionType.NONE, metadata={"always_show": True}
-    )
-    quantization_type: WeightQuantizationType = field(
-        default_factory=lambda: WeightQuantizationType.NONE, metadata={"always_show": True}
-    )
+    type: enums.WeightModifierType = shown(enums.WeightModifierType.NONE)
+    noise_type: enums.WeightNoiseInjectionType = shown(enums.WeightNoiseInjectionType.NONE)
+    quantization_type: enums.WeightQuantizationType = shown(enums.WeightQuantizationType.NONE)
 
 
 @dataclass
@@ -33,6 +24,4 @@ class WeightClipParameter(_PrintableMixin):
     """Clip bound ``sigma`` (in standard deviations); inactive while ``type`` is NONE."""
 
     sigma: float = -1.0
-    type: WeightClipType = field(
-        default_factory=lambda: WeightClipType.NONE, metadata={"always_show": True}
-    )
+    type: enums.WeightClipType = shown(enums.WeightClipType.NONE)
