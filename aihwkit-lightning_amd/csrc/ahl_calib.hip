@@ -186,6 +186,10 @@ __global__ void k_ir_moving_update(void* ir, int32_t* idx, const float* __restri
   // the statistic as the Python float the reference holds: alpha * std (std in the tensor dtype)
   // or the fp32 quantile
   const float stat = val_in_dtype ? D::rd(val[t]) : val[t];
+  // No statistic (NaN: no row of the batch was kept, e.g. the all-zero hidden state of a
+  // recurrent layer's first step): the batch is passed over. The reference would average the
+  // NaN in and lose the range for good.
+  if (stat != stat) return;
   const float v = (float)(alpha * (double)stat);
   const float num = old * (float)i + v;
   D::store(ir, t, __fdiv_rn(num, (float)(i + 1)));

@@ -187,7 +187,8 @@ int64_t ahl_sliced_quantile_ws_bytes(int64_t rows, int32_t n_tiles);
 /* Moving average of the calibrated range (calibration.py:144-147), on the device:
  *   ir[t] = dtype((float(ir[t]) * idx[t] + float(alpha * val[t])) / (idx[t] + 1)); idx[t] += 1
  * ir dtype [T], idx int32 [T], val float [T]; val_in_dtype != 0 rounds val to dtype first (a std
- * that torch returns in the tensor dtype).                                                     */
+ * that torch returns in the tensor dtype). A tile whose val is NaN (no kept row in the batch) is
+ * left as it is, idx included.                                                                 */
 int ahl_ir_moving_update(void* ir, int32_t* idx, const float* val, int32_t dtype, int32_t n_tiles,
                          double alpha, int32_t val_in_dtype, void* stream);
 

@@ -446,6 +446,12 @@ def calibrate_moving(batches: Sequence[Tensor], in_sizes: Sequence[int], kind: s
     for x in batches:
         trace.append(ir.float().clone())
         rows = kept_rows(x)
+        if rows.size(0) == 0:
+            # A batch of all-zero rows (the hidden state of a recurrent layer's first step): the
+            # reference's statistic of the empty selection is NaN (std) or an error (quantile,
+            # max), which ruins the range for good. Stated here as what the product does
+            # instead: such a batch is passed over.
+            continue
         for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
             part = rows[:, lo:hi]
             if kind == "MovingStd":

@@ -123,6 +123,37 @@ def test_moving_update_bit_exact(dtype):
         assert torch.equal(ir_d.cpu(), ir) and torch.equal(idx_d.cpu(), idx)
 
 
+@pytest.mark.parametrize("kind", ["MOVING_STD", "MOVING_QUANTILE", "MAX", "CACHE_QUANTILE"])
+def test_a_batch_of_all_zero_rows_is_passed_over(kind):
+    """The hidden projection of a recurrent layer sees an all-zero batch at the first step. The
+    reference's statistics of the empty row selection are NaN or an error; here such a batch
+    leaves the calibration state alone (the same as the oracle's statement of it)."""
+    from aihwkit_lightning.inference.calibration import (InputRangeCalibrationType,
+                                                         calibrate_input_ranges)
+    from aihwkit_lightning.nn import AnalogLinear
+    from aihwkit_lightning.simulator.configs import TorchInferenceRPUConfig
+
+    cfg = TorchInferenceRPUConfig()
+    cfg.mapping.max_input_size = 16
+    layer = AnalogLinear(40, 8, rpu_config=cfg).cuda().eval()
+    gen = torch.Generator().manual_seed(11)
+    data = [torch.randn(32, 40, generator=gen) for _ in range(3)]
+    batches = [torch.zeros(32, 40), data[0], torch.zeros(32, 40), data[1], data[2]]
+    calibrate_input_ranges(layer, InputRangeCalibrationType[kind],
+                           (((b.cuda(),), {}) for b in batches), quantile=0.99, max_samples=64,
+                           std_alpha=3.0, verbose=False)
+    got = layer.input_range.detach().cpu()
+    assert torch.isfinite(got).all() and (got > 0).all()
+    sizes = [14, 13, 13]
+    if kind in ("MOVING_STD", "MOVING_QUANTILE"):
+        want, _ = om.calibrate_moving(batches, sizes, InputRangeCalibrationType[kind].value,
+                                      torch.float32, alpha=3.0, q=0.99)
+        assert torch.allclose(got, want, rtol=1e-6)
+        assert int(layer.input_range_update_idx.isinf().sum()) == 3  # marked as finished
+    elif kind == "MAX":
+        assert torch.equal(got, om.calibrate_max(data, sizes))
+
+
 def build_layer(case):
     from aihwkit_lightning.nn import AnalogConv2d, AnalogLinear
     from aihwkit_lightning.simulator.configs import TorchInferenceRPUConfig
