@@ -46,6 +46,16 @@ class AnalogWrapper(AnalogContainerBase):
     def __init__(self, module: Module):  # pylint: disable=super-init-not-called
         self.__dict__.update(module.__dict__)
 
+    @classmethod
+    def _rebuild(cls, wrapped_class: Type) -> "AnalogWrapper":
+        """An empty instance of the wrapper class of ``wrapped_class`` (for unpickling)."""
+        return cls.__new__(cls, wrapped_class.__new__(wrapped_class))
+
+    def __reduce__(self):
+        # the dynamic class cannot be looked up by name: pickle the wrapped class (which can)
+        # and the state, and build the wrapper class again when loading
+        return (AnalogWrapper._rebuild, (type(self).__bases__[1],), self.__dict__)
+
     # pylint: disable=unused-argument
     @classmethod
     def from_digital(cls, module: Module, *args: Any, **kwargs: Any) -> "AnalogWrapper":

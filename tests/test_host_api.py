@@ -354,3 +354,24 @@ def test_convert_recurrent_layers_to_analog_and_back():
     for key, value in model.state_dict().items():
         assert torch.equal(digital.state_dict()[key], value), key
     assert isinstance(convert_to_analog(model, _cfg()), AnalogWrapper)
+
+
+def test_wrapped_model_can_be_pickled():
+    """``torch.save(model)`` of a converted model: the wrapper's dynamic class is rebuilt on load
+    (in the reference this fails with a PicklingError)."""
+    import io
+    import pickle
+
+    from aihwkit_lightning.nn.conversion import convert_to_analog
+
+    model = convert_to_analog(_Net(), _cfg())
+    assert isinstance(model, AnalogWrapper)
+    clone = pickle.loads(pickle.dumps(model))
+    assert type(clone) is type(model) and isinstance(clone, _Net)
+    for (name, a), (_, b) in zip(model.state_dict().items(), clone.state_dict().items()):
+        assert torch.equal(a, b), name
+    buffer = io.BytesIO()
+    torch.save(model, buffer)
+    buffer.seek(0)
+    again = torch.load(buffer, weights_only=False)
+    assert len(list(again.analog_layers())) == len(list(model.analog_layers()))
