@@ -145,3 +145,39 @@ def test_post_training_calibration_then_8_bit_inference(strategy):
     rel = float((got - want).norm() / want.norm())
     assert rel < 0.1, rel
     assert float((got.argmax(1) == want.argmax(1)).float().mean()) > 0.9
+
+
+def test_tiny_llama_converts_trains_and_generates():
+    """The reference's main use: a Hugging Face decoder converted layer by layer and fine-tuned in
+    bf16. Covers tiles of 256 inputs, an intermediate size that is no multiple of the tile, a
+    vocabulary that is no multiple of 8, and ``generate`` (one row per call)."""
+    transformers = pytest.importorskip("transformers")
+    from aihwkit_lightning.nn.conversion import convert_to_analog, convert_to_digital
+    from aihwkit_lightning.optim import AnalogOptimizer
+
+    conf = transformers.LlamaConfig(vocab_size=1003, hidden_size=256, intermediate_size=688,
+                                    num_hidden_layers=2, num_attention_heads=4,
+                                    num_key_value_heads=4, max_position_embeddings=128)
+    torch.manual_seed(0)
+    llm = transformers.LlamaForCausalLM(conf).to("cuda", torch.bfloat16)
+    cfg = _config()
+    cfg.mapping.max_input_size = 256
+    model = convert_to_analog(llm, cfg)
+    assert len(list(model.analog_layers())) == 2 * 7 + 1  # q, k, v, o, gate, up, down; lm_head
+    ids = torch.randint(0, 1003, (4, 64), generator=torch.Generator().manual_seed(2)).cuda()
+    optim = AnalogOptimizer(torch.optim.AdamW, model.analog_layers, model.parameters(), lr=1e-3)
+    model.train()
+    losses = []
+    for _ in range(12):
+        optim.zero_grad()
+        loss = model(input_ids=ids, labels=ids).loss
+        loss.backward()
+        optim.step()
+        losses.append(float(loss.detach()))
+    assert all(v == v for v in losses) and losses[-1] < 0.8 * losses[0], losses
+    model.eval()
+    with torch.no_grad():
+        generated = model.generate(ids[:, :8], attention_mask=torch.ones_like(ids[:, :8]),
+                                   max_new_tokens=8, do_sample=False, pad_token_id=0)
+    assert generated.shape == (4, 16)
+    assert type(convert_to_digital(model)).__name__ == "LlamaForCausalLM"
