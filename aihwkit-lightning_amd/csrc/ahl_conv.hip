@@ -511,6 +511,53 @@ __global__ __launch_bounds__(256) void k_transpose_batched(const E* __restrict__
   }
 }
 
+// Vector variant for matrices whose rows and columns come in whole 16-byte vectors: 64 x 64
+// tiles, 16-byte loads along the source rows into LDS, and every thread gathers the V elements
+// of one destination vector (V consecutive source rows of one column) from LDS, so that both
+// sides of HBM see 16-byte accesses, 128 contiguous bytes per 8 (bf16) or 16 (fp32) lanes.
+template <class E>
+__global__ __launch_bounds__(256) void k_transpose_vec(const E* __restrict__ src, int64_t ld_src,
+                                                       int64_t rows, int64_t cols,
+                                                       E* __restrict__ dst, int64_t ld_dst,
+                                                       int64_t tiles_c, int64_t tiles_per_mat) {
+  constexpr int V = 16 / (int)sizeof(E);   // elements per vector
+  constexpr int T = 64;                    // tile edge
+  constexpr int VPR = T / V;               // vectors per tile row
+  constexpr int RS = T + V;                // LDS row stride in elements (a multiple of 16 bytes)
+  __shared__ __attribute__((aligned(16))) E tile[T * RS];
+  const int64_t bid = blockIdx.x;
+  const int64_t b = bid / tiles_per_mat;
+  const int64_t t = bid - b * tiles_per_mat;
+  const int64_t r0 = (t / tiles_c) * T, c0 = (t % tiles_c) * T;
+  const E* s = src + b * rows * ld_src;
+  E* d = dst + b * cols * ld_dst;
+  const int tid = threadIdx.x;
+  u32x4 raw[T * VPR / 256];
+#pragma unroll
+  for (int i = 0; i < T * VPR / 256; ++i) {
+    const int v = tid + 256 * i;
+    const int r = v / VPR, cv = v % VPR;
+    raw[i] = u32x4{0u, 0u, 0u, 0u};
+    if (r0 + r < rows && c0 + cv * V < cols) raw[i] = ld16(s + (r0 + r) * ld_src + c0 + cv * V);
+  }
+#pragma unroll
+  for (int i = 0; i < T * VPR / 256; ++i) {
+    const int v = tid + 256 * i;
+    *(u32x4*)(tile + (v / VPR) * RS + (v % VPR) * V) = raw[i];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < T * VPR / 256; ++i) {
+    const int v = tid + 256 * i;
+    const int c = v / VPR, rv = v % VPR;     // destination row c, vector rv of its 64 elements
+    if (c0 + c >= cols || r0 + rv * V >= rows) continue;
+    E out[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) out[e] = tile[(rv * V + e) * RS + c];
+    st16(d + (c0 + c) * ld_dst + r0 + rv * V, *(const u32x4*)out);
+  }
+}
+
 template <class E, int VEC>
 static int launch_im2col(const void* x, void* cols, int64_t ldc, const ConvGeom& g,
                          hipStream_t st) {
@@ -632,11 +679,30 @@ extern "C" int ahl_transpose_batched(const void* src, int64_t ld_src, int32_t dt
   if (src == nullptr || dst == nullptr || batch <= 0 || rows <= 0 || cols <= 0 || ld_src < cols ||
       ld_dst < rows)
     return AHL_ERR_ARG;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype != AHL_F32 && dtype != AHL_BF16) return AHL_ERR_ARG;
+  {
+    // whole 16-byte vectors on both sides: the vector kernel
+    const int64_t v = dtype == AHL_BF16 ? 8 : 4;
+    const int64_t tiles_c = cdiv(cols, 64), per_mat = tiles_c * cdiv(rows, 64);
+    if (rows % v == 0 && cols % v == 0 && ld_src % v == 0 && ld_dst % v == 0 && aligned16(src) &&
+        aligned16(dst) && per_mat <= 0x7fffffff && batch <= 0x7fffffff / per_mat) {
+      const dim3 vgrid((unsigned)(per_mat * batch));
+      if (dtype == AHL_F32)
+        hipLaunchKernelGGL((k_transpose_vec<uint32_t>), vgrid, dim3(256), 0, st,
+                           (const uint32_t*)src, ld_src, rows, cols, (uint32_t*)dst, ld_dst,
+                           tiles_c, per_mat);
+      else
+        hipLaunchKernelGGL((k_transpose_vec<uint16_t>), vgrid, dim3(256), 0, st,
+                           (const uint16_t*)src, ld_src, rows, cols, (uint16_t*)dst, ld_dst,
+                           tiles_c, per_mat);
+      return check_launch("k_transpose_vec");
+    }
+  }
   const int64_t tiles_c = cdiv(cols, 32), tiles_r = cdiv(rows, 32);
   const int64_t per_mat = tiles_c * tiles_r;
   if (per_mat > 0x7fffffff || batch > 0x7fffffff / per_mat) return AHL_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)(per_mat * batch));
-  hipStream_t st = (hipStream_t)stream;
   if (dtype == AHL_F32) {
     hipLaunchKernelGGL((k_transpose_batched<uint32_t>), grid, dim3(256), 0, st,
                        (const uint32_t*)src, ld_src, rows, cols, (uint32_t*)dst, ld_dst, tiles_c,

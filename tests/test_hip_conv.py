@@ -71,7 +71,10 @@ def test_patch_kernels_bit_exact(geom, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 33, 65), (2, 64, 32), (5, 7, 130), (1, 300, 17)])
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 33, 65), (2, 64, 32), (5, 7, 130), (1, 300, 17),
+                                   # whole 16-byte vectors on both sides: the vector kernel,
+                                   # full and partial 64 x 64 tiles
+                                   (3, 784, 256), (2, 72, 200), (1, 8, 8), (4, 136, 24)])
 def test_transpose_batched_bit_exact(shape, dtype):
     from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
 
