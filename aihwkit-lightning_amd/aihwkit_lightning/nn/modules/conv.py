@@ -16,6 +16,7 @@ from torch.nn.modules.conv import _ConvNd
 from torch.nn.modules.utils import _pair, _single, _triple
 
 from .hip_utils.ops import OPS, conv_out_size
+from .linear import is_at_least_volta_gpu  # noqa: F401  (re-exported)
 from .tiled import TiledAnalogLayer
 from ...exceptions import HipBackendError
 from ...simulator.configs import TorchInferenceRPUConfig
@@ -50,6 +51,35 @@ class SwapLastTwo(Function):
     @staticmethod
     def backward(ctx, grad: Tensor):
         return OPS.transpose_batched(grad)
+
+
+def unfold3d(
+    inp: Tensor,
+    kernel_size: Tuple[int, int, int],
+    padding: Tuple[int, int, int] = (0, 0, 0),
+    stride: Tuple[int, int, int] = (1, 1, 1),
+) -> Tensor:
+    """Patches of a volume in ``torch.nn.functional.unfold``'s layout:
+    ``[B, C, D, H, W] -> [B, C * kD * kH * kW, L]`` (``[C, D, H, W] -> [C * kD * kH * kW, L]``
+    without a batch), dilation 1 (reference ``nn/modules/conv.py``: ``unfold3d``). One patch
+    kernel launch and one transpose; differentiable."""
+    unbatched = inp.dim() == 4
+    if unbatched:
+        inp = inp.unsqueeze(0)
+    if inp.dim() != 5:
+        raise ValueError("expected a 4-D or 5-D input")
+    if not inp.is_cuda:
+        raise HipBackendError("patch extraction runs on a ROCm device; there is no CPU path")
+    geom = (
+        [int(inp.shape[0]), int(inp.shape[1])]
+        + [int(v) for v in inp.shape[2:]]
+        + [int(v) for v in _triple(kernel_size)]
+        + [int(v) for v in _triple(stride)]
+        + [int(v) for v in _triple(padding)]
+        + [1, 1, 1]
+    )
+    cols = SwapLastTwo.apply(PatchRows.apply(inp.contiguous(), geom))
+    return cols.squeeze(0) if unbatched else cols
 
 
 def _three(values: Tuple[int, ...], fill: int) -> List[int]:

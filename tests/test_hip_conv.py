@@ -83,6 +83,34 @@ def test_transpose_batched_bit_exact(shape, dtype):
     assert got.is_contiguous() and torch.equal(got.cpu(), src.transpose(1, 2).contiguous())
 
 
+@pytest.mark.gpu
+def test_unfold3d_is_the_unfold_of_a_volume():
+    """Two anchors that do not go through the oracle: a volume of depth 1 with a depth-1 kernel
+    is ``torch.nn.functional.unfold``'s 2-D case bit for bit, and for a real volume
+    ``weight.view(O, -1) @ unfold3d(x)`` is ``conv3d(x, weight)``; the gradient is the adjoint."""
+    from aihwkit_lightning.nn.modules.conv import unfold3d
+
+    gen = torch.Generator().manual_seed(31)
+    flat = torch.randn(2, 3, 1, 9, 11, generator=gen)
+    got = unfold3d(flat.cuda(), (1, 3, 2), padding=(0, 1, 2), stride=(1, 2, 1))
+    want = torch.nn.functional.unfold(flat[:, :, 0], (3, 2), padding=(1, 2), stride=(2, 1))
+    assert torch.equal(got.cpu(), want)
+    assert torch.equal(unfold3d(flat[0].cuda(), (1, 3, 2), (0, 1, 2), (1, 2, 1)).cpu(), want[0])
+
+    vol = torch.randn(2, 4, 6, 7, 5, generator=gen, dtype=torch.float64).float()
+    weight = torch.randn(5, 4, 3, 2, 3, generator=gen)
+    x = vol.cuda().requires_grad_()
+    cols = unfold3d(x, (3, 2, 3), padding=(1, 0, 2), stride=(2, 1, 1))
+    ref_in = vol.clone().requires_grad_()
+    ref = torch.nn.functional.conv3d(ref_in, weight, padding=(1, 0, 2), stride=(2, 1, 1))
+    out = (weight.view(5, -1).cuda() @ cols).view(ref.shape)
+    assert torch.allclose(out.cpu(), ref, rtol=1e-5, atol=1e-5)
+    g = torch.randn(ref.shape, generator=gen)
+    out.backward(g.cuda())
+    ref.backward(g)
+    assert torch.allclose(x.grad.cpu(), ref_in.grad, rtol=1e-5, atol=1e-5)
+
+
 def make_conv_layer(c, w, b):
     from hip_helpers import rpu_config
     from aihwkit_lightning.nn import AnalogConv1d, AnalogConv2d, AnalogConv3d

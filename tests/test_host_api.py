@@ -375,3 +375,18 @@ def test_wrapped_model_can_be_pickled():
     buffer.seek(0)
     again = torch.load(buffer, weights_only=False)
     assert len(list(again.analog_layers())) == len(list(model.analog_layers()))
+
+
+def test_module_level_helpers_of_the_reference_exist():
+    """``is_at_least_volta_gpu`` and ``unfold3d`` are module-level names of the reference's
+    ``linear.py`` / ``conv.py``; without a device the first says no and the second refuses."""
+    from aihwkit_lightning.exceptions import HipBackendError
+    from aihwkit_lightning.nn.modules import conv, linear
+
+    assert linear.is_at_least_volta_gpu is conv.is_at_least_volta_gpu
+    if not torch.cuda.is_available():
+        assert linear.is_at_least_volta_gpu() is False
+        with pytest.raises(HipBackendError):
+            conv.unfold3d(torch.zeros(1, 1, 2, 2, 2), (1, 1, 1))
+    with pytest.raises(ValueError):
+        conv.unfold3d(torch.zeros(2, 2), (1, 1, 1))
