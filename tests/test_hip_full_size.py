@@ -151,3 +151,86 @@ def test_llama_mlp_block_matches_oracle():
     down_on_ref = layers["down"](act_r.detach().cuda())
     assert_close_lsb(down_on_ref.detach().float().cpu(), o_out.float(), 1e-2, lsb, max_frac=1e-4,
                      what="down out on the oracle's activations")
+
+
+def _tail_reproduces(layer, x, g_shape, tail, chunk, what):
+    """Rows (images) are independent of each other: the last `tail` of a large batch must come out
+    bit for bit as they do on their own (a wrong 64-bit offset anywhere moves them), and the
+    weight / bias gradients must be the sum of the gradients of the batch's chunks."""
+    gen = torch.Generator(device="cuda").manual_seed(9)
+    xs = x[-tail:].clone().requires_grad_()
+    x.requires_grad_()
+    y = layer(x)
+    assert tuple(y.shape) == tuple(g_shape)
+    g = torch.randn(g_shape, device="cuda", generator=gen, dtype=x.dtype)
+    y.backward(g)
+    dw, db = layer.weight.grad.float(), layer.bias.grad.float()
+    layer.zero_grad(set_to_none=True)
+    ys = layer(xs)
+    ys.backward(g[-tail:].clone())
+    assert torch.equal(y[-tail:], ys), f"{what}: output of the last rows"
+    assert torch.equal(x.grad[-tail:], xs.grad), f"{what}: input gradient of the last rows"
+    acc_w, acc_b = torch.zeros_like(dw), torch.zeros_like(db)
+    for r0 in range(0, x.shape[0], chunk):
+        layer.zero_grad(set_to_none=True)
+        layer(x.detach()[r0:r0 + chunk]).backward(g[r0:r0 + chunk])
+        acc_w += layer.weight.grad.float()
+        acc_b += layer.bias.grad.float()
+    # every chunk's gradient is rounded to bf16 (2^-9 relative, 2.3e-3 in the mean); rows that
+    # went missing or were read from a wrapped offset would show as 2e-2 and more
+    assert float((dw - acc_w).norm() / acc_w.norm()) < 5e-3, f"{what}: weight gradient"
+    assert float((db - acc_b).norm() / acc_b.norm()) < 5e-3, f"{what}: bias gradient"
+
+
+def _big_case(K, N):
+    return case("big_index", dtype="bf16", M=1, K=K, N=N, max_input_size=512, ir_mode="static",
+                inp_res=254, out_res=254, out_bound=0.9, clip="channel", clip_sigma=2.5,
+                ir_decay=0.01, ir_init=3.0, w_scale=0.02, seed=5)
+
+
+@pytest.mark.parametrize("shape", [(2 ** 19 + 192, 4096, 4096, 512, 2112),
+                                   (2 ** 22 + 40, 520, 520, 260, 200)],
+                         ids=["4096x4096", "520x520_padded_tiles"])
+def test_more_than_2_31_elements_per_tensor(shape):
+    """Activations, gradients and clamp masks with more than 2^31 elements: the MFMA kernels, the
+    DAC pass and the mask addressing in 64-bit offsets."""
+    from hip_helpers import rpu_config
+    from aihwkit_lightning.nn import AnalogLinear
+
+    rows, k_in, n_out, tile, tail = shape
+    assert rows * min(k_in, n_out) > 2 ** 31
+    c = _big_case(k_in, n_out)
+    c["max_input_size"] = tile
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    layer = AnalogLinear(k_in, n_out, bias=True, dtype=torch.bfloat16, rpu_config=rpu_config(c)).cuda()
+    with torch.no_grad():
+        layer.weight.copy_(0.02 * torch.randn(n_out, k_in, device="cuda", generator=gen))
+        layer.bias.copy_(0.1 * torch.randn(n_out, device="cuda", generator=gen))
+    layer.train()
+    x = torch.randn(rows, k_in, device="cuda", generator=gen, dtype=torch.bfloat16)
+    _tail_reproduces(layer, x, (rows, n_out), tail, 65536, f"{rows} x {k_in} -> {n_out}")
+
+
+@pytest.mark.parametrize("geom", [(3700, 64, 64, 96, 2, 2, 0), (520, 64, 64, 96, 3, 1, 1)],
+                         ids=["input_2e9", "patches_2.7e9"])
+def test_convolution_with_more_than_2_31_elements(geom):
+    """Patch extraction, its adjoint and the layout change at more than 2^31 elements: once in the
+    input itself (non-overlapping 2x2 patches), once in the patch matrix only (3x3, pad 1)."""
+    from hip_helpers import rpu_config
+    from aihwkit_lightning.nn import AnalogConv2d
+
+    batch, chan, n_out, size, kernel, stride, pad = geom
+    out = (size + 2 * pad - kernel) // stride + 1
+    assert batch * out * out * chan * kernel * kernel > 2 ** 31
+    c = _big_case(chan * kernel * kernel, n_out)
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    layer = AnalogConv2d(chan, n_out, kernel, stride=stride, padding=pad, bias=True,
+                         dtype=torch.bfloat16, rpu_config=rpu_config(c)).cuda()
+    with torch.no_grad():
+        layer.weight.copy_(0.05 * torch.randn(layer.weight.shape, device="cuda", generator=gen))
+        layer.bias.copy_(0.1 * torch.randn(n_out, device="cuda", generator=gen))
+    layer.train()
+    x = torch.randn(batch, chan, size, size, device="cuda", generator=gen, dtype=torch.bfloat16)
+    _tail_reproduces(layer, x, (batch, n_out, out, out), 16, max(16, batch // 8), f"conv {geom}")
+    del x
+    torch.cuda.empty_cache()
