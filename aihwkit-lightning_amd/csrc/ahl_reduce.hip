@@ -274,6 +274,60 @@ __global__ __launch_bounds__(256) void k_clip_rows(void* w, int64_t rows, int32_
   clamp_row<D, VEC>(row, cols, lane, bound);
 }
 
+// Per channel, rows of at most 64 * R 16-byte vectors: the wave keeps its row in registers
+// between the sums and the clamp, so the matrix is read once. All R loads are issued before the
+// first value is used (vectors beyond the row re-read its first vector and count as zeros); sums
+// in the order of k_clip_rows, so both kernels give the same bound bit for bit.
+template <class D, int R>
+__global__ __launch_bounds__(256) void k_clip_rows_held(void* w, int64_t rows, int32_t cols,
+                                                        int64_t ld, float sigma) {
+  constexpr int E = D::EPV;
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  typename D::elem* row = (typename D::elem*)w + r * ld;
+  const int32_t nv = cols / E;
+  u32x4 held[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int32_t v = lane + 64 * i;
+    held[i] = ld16(row + (int64_t)(v < nv ? v : 0) * E);
+  }
+  double s = 0.0, s2 = 0.0;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    if (lane + 64 * i >= nv) {
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+      held[i] = zero;
+    }
+    float e[E];
+    D::unpack(held[i], e);
+#pragma unroll
+    for (int j = 0; j < E; ++j) {
+      s += (double)e[j];
+      s2 += (double)e[j] * (double)e[j];
+    }
+  }
+  s = wave_sum(s);
+  s2 = wave_sum(s2);
+  const float bound = clip_bound<D>(s, s2, (double)cols, sigma);
+  if (bound != bound) return;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int32_t v = lane + 64 * i;
+    float e[E];
+    D::unpack(held[i], e);
+    bool changed = false;
+#pragma unroll
+    for (int j = 0; j < E; ++j) {
+      const float c = fminf(fmaxf(e[j], -bound), bound);
+      changed |= (c != e[j]);
+      e[j] = c;
+    }
+    if (changed && v < nv) st16(row + (int64_t)v * E, D::pack(e));
+  }
+}
+
 // Whole-matrix variant, stage 1: per-block (sum, sum of squares) over kStdRows rows.
 template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_matrix_sums(const void* __restrict__ w, int64_t rows,
@@ -521,7 +575,16 @@ int ahl_clip_weights(void* w, int32_t dtype, int64_t rows, int64_t cols, int64_t
     const bool vec = aligned16(w) && (ld % D::EPV == 0);
     if (clip_kind == AHL_CLIP_PER_CHANNEL) {
       const dim3 grid((unsigned)cdiv(rows, 4));
-      if (vec) hipLaunchKernelGGL((k_clip_rows<D, true>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
+      const int64_t per_lane = cols % D::EPV == 0 ? cdiv(cols / D::EPV, 64) : 0;
+      if (vec && per_lane >= 1 && per_lane <= 4)
+        hipLaunchKernelGGL((k_clip_rows_held<D, 4>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
+      else if (vec && per_lane > 4 && per_lane <= 8)
+        hipLaunchKernelGGL((k_clip_rows_held<D, 8>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
+      else if (vec && per_lane > 8 && per_lane <= 16)
+        hipLaunchKernelGGL((k_clip_rows_held<D, 16>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
+      else if (vec && per_lane > 16 && per_lane <= 32)
+        hipLaunchKernelGGL((k_clip_rows_held<D, 32>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
+      else if (vec) hipLaunchKernelGGL((k_clip_rows<D, true>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
       else hipLaunchKernelGGL((k_clip_rows<D, false>), grid, dim3(256), 0, s, w, rows, (int32_t)cols, ld, sigma);
     } else {
       const int64_t nb = cdiv(rows, kStdRows);

@@ -180,6 +180,105 @@ def build_other(name):
     return layer.cuda().train(), x.cuda().requires_grad_(True), g.cuda(), flops
 
 
+POST_TRAINING = ("post-training weight processing and calibration, fp32: 64 weight matrices "
+                 "8192 x 3072 (N(0, 0.02) + 0.1 % outliers x 20, 6 tiles of 512 inputs) clipped at 3 "
+                 "sigma per channel and quantised to 254 states per channel and tile; running "
+                 "abs-max calibration over 256 batches of 2048 x 3072 Laplace(0, 1) activations")
+# per matrix: one read for abs-max and sums, read + write for clip-and-quantise; per batch one read
+POST_TRAINING_BYTES = 64 * 3 * 8192 * 3072 * 4 + 256 * 2048 * 3072 * 4
+
+
+def _post_training_cfg():
+    from aihwkit_lightning.simulator.configs import (TorchInferenceRPUConfig, WeightClipType,
+                                                     WeightQuantizationType)
+    cfg = TorchInferenceRPUConfig()
+    cfg.mapping.max_input_size = 512
+    cfg.clip.type = WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL
+    cfg.clip.sigma = 3.0
+    cfg.modifier.quantization_type = WeightQuantizationType.DISCRETIZE_PER_CHANNEL
+    cfg.modifier.res = 254
+    return cfg
+
+
+def time_post_training(with_cpu):
+    """The reduction-bound configuration: `clip_weights` + `quantize_weights` of 64 layers through
+    the layer methods, then the running abs-max of the MAX calibration over 256 activation
+    batches (the kernel the calibration hook calls; 16 distinct batches, 403 MB, visited in turn).
+    One timed pass over fresh matrices, wall clock around it."""
+    from aihwkit_lightning.nn import AnalogLinear
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+
+    n, k, m, n_mat, n_batch = 8192, 3072, 2048, 64, 256
+    gen = torch.Generator(device="cuda").manual_seed(4)
+
+    def fresh(layer):
+        with torch.no_grad():
+            w = layer.weight
+            w.normal_(0.0, 0.02, generator=gen)
+            w.mul_(1.0 + 19.0 * (torch.rand(w.shape, device="cuda", generator=gen) < 1e-3))
+
+    layers = [AnalogLinear(k, n, bias=False, device="cuda", rpu_config=_post_training_cfg())
+              for _ in range(n_mat + 2)]
+    for layer in layers:
+        fresh(layer)
+    lap = torch.distributions.Laplace(0.0, 1.0)
+    batches = [lap.sample((m, k)).cuda() for _ in range(16)]
+    in_sizes = layers[0].in_sizes
+    for layer in layers[n_mat:]:  # warm-up on the two spare matrices
+        layer.clip_weights()
+        layer.quantize_weights()
+    stat = torch.full((len(in_sizes),), float("-inf"), dtype=torch.float32, device="cuda")
+    OPS.running_absmax(batches[0], in_sizes, stat)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for layer in layers[:n_mat]:
+        layer.clip_weights()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for layer in layers[:n_mat]:
+        layer.quantize_weights()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for i in range(n_batch):
+        OPS.running_absmax(batches[i % 16], in_sizes, stat)
+    torch.cuda.synchronize()
+    t3 = time.perf_counter()
+    total = t3 - t0
+    gbs = POST_TRAINING_BYTES / total / 1e9
+    line = {
+        "metric": "GB/s of algorithmic bytes, post-training weight processing + calibration",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": 1, "warmup": 0,
+        "ms_per_step": round(total * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": POST_TRAINING, "ms": {"clip_weights x64": round((t1 - t0) * 1e3, 3),
+                                                    "quantize_weights x64": round((t2 - t1) * 1e3, 3),
+                                                    "running_absmax x256": round((t3 - t2) * 1e3, 3)}},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None},
+    }
+    if with_cpu:
+        from oracle import torch_mode as om
+
+        threads = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(threads)
+        cgen = torch.Generator().manual_seed(4)
+        mats = []
+        for _ in range(16):
+            w = 0.02 * torch.randn(n, k, generator=cgen)
+            mats.append(w * (1.0 + 19.0 * (torch.rand(n, k, generator=cgen) < 1e-3)))
+        cb = [lap.sample((m, k)) for _ in range(64)]
+        t0 = time.perf_counter()
+        for w in mats:
+            om.quantize_weights(om.clip_weights(w, 3.0, True), in_sizes, "discretize_per_channel", 254.0)
+        om.calibrate_max(cb, in_sizes)
+        dt = (time.perf_counter() - t0) * 4.0
+        line["cpu_baseline"] = {
+            "value": POST_TRAINING_BYTES / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"16 of 64 matrices and 64 of 256 batches, time scaled by 4 ({dt:.1f} s for the "
+                      "whole configuration)"}
+    return line
+
+
 def time_other(name, steps, warmup):
     """ms per fwd+bwd step and TFLOP/s of one of OTHER_WORKLOADS (wall clock around K steps)."""
     layer, x, g, flops = build_other(name)
@@ -359,7 +458,7 @@ def main():
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--kernels-only", action="store_true",
                         help="only launch the individual kernels (for rocprofv3 runs)")
-    parser.add_argument("--workload", default="linear", choices=["linear", *OTHER_WORKLOADS],
+    parser.add_argument("--workload", default="linear", choices=["linear", "post_training", *OTHER_WORKLOADS],
                         help="'linear' is the headline workload; the others print their own line")
     ns = parser.parse_args()
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -370,6 +469,9 @@ def main():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
 
+    if ns.workload == "post_training":
+        print(json.dumps(time_post_training(not ns.no_cpu)))
+        return
     if ns.workload != "linear":
         torch.manual_seed(0)
         res = time_other(ns.workload, ns.steps, ns.warmup)

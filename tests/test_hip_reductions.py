@@ -134,6 +134,30 @@ def test_clip_weights_closed_form(dtype, per_channel):
         assert mism < 2e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("vectors", [1, 63, 256, 257, 768, 1024, 2048, 2049],
+                         ids=lambda v: f"{v}_vectors")
+def test_clip_weights_per_channel_row_lengths(vectors, dtype):
+    """Rows of 1 .. 2049 16-byte vectors: the kernels that keep a row in registers (up to 4, 8, 16,
+    32 vectors per lane, with full and partly filled last rounds) and the one that reads it twice
+    (2049 vectors); a clamped row's values may only be the row's own values or +-bound."""
+    cols = vectors * (4 if dtype == torch.float32 else 8)
+    gen = torch.Generator().manual_seed(vectors)
+    w = torch.randn(37, cols, generator=gen)
+    w = (w * (1.0 + 4.0 * (torch.rand(37, cols, generator=gen) < 0.02))).to(dtype)
+    dev = w.cuda().clone()
+    ops().clip_weights(dev, 2.0, 1)
+    got, ref = dev.cpu(), om.clip_weights(w, 2.0, True)
+    if dtype == torch.float32:
+        assert torch.allclose(got, ref, rtol=2e-6, atol=0)
+    else:
+        assert float((got != ref).float().mean()) < 2e-3
+    changed = got != w
+    assert bool(changed.any()) or cols < 64
+    bound = got.abs().amax(dim=1, keepdim=True)
+    assert torch.equal(got[changed].abs(), bound.expand_as(got)[changed])
+
+
 @pytest.mark.parametrize("name", ["f32_quantize_channel", "f32_quantize_odd", "bf16_quantize_tensor"])
 def test_quantize_weights_matches_reference(name):
     from hip_helpers import make_layer
