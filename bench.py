@@ -395,8 +395,8 @@ def hbm_kernel_rooflines(reps):
         "sliced_absmax(W)": (lambda: OPS.sliced_absmax(nxt(ws), in_sizes, True), wb),
         "sliced_std(x)": (lambda: OPS.sliced_std(nxt(xs), in_sizes), xbytes),
         "running_absmax(x)": (lambda: OPS.running_absmax(nxt(xs), in_sizes, cache), xbytes),
-        # std pass + clamp pass; the clamp pass re-reads W and writes only changed vectors
-        "clip_weights(W, per channel)": (lambda: OPS.clip_weights(nxt(ws), 3.0, L.AHL_CLIP_PER_CHANNEL), 2 * wb),
+        # sums and clamp from one read of W (a row stays in registers); writes only changed vectors
+        "clip_weights(W, per channel)": (lambda: OPS.clip_weights(nxt(ws), 3.0, L.AHL_CLIP_PER_CHANNEL), wb),
         # abs-max pass + quantise pass (read + write)
         "quantize_weights(W)": (lambda: OPS.quantize_weights(
             nxt(ws), in_sizes, L.AHL_QUANT_DISCRETIZE_PER_CHANNEL, 254.0), 3 * wb),
