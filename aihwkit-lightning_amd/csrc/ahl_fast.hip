@@ -132,8 +132,12 @@ AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
   return BF16::rd((B + B) * a.out_res);
 }
 
-template <int IRMODE, bool NOISE, bool ADC, int NBJ>
+// QM, what happens to a tile's outputs after the noise: 0 nothing, 1 clamp at the bound, 2 ADC
+// quantisation and clamp, 3 the same without the rounding step (skip_rounding). Compile-time, so
+// that the per-group epilogue has no branches apart from the rare "something left the range".
+template <int IRMODE, bool NOISE, int QM, int NBJ>
 __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs a) {
+  constexpr bool ADC = QM >= 2, CLAMP = QM >= 1, ROUND = QM != 3;
   constexpr int BN = 64 * NBJ;   // block columns
   constexpr int WN = 32 * NBJ;   // wave columns
   constexpr int NB = 2 * NBJ;    // B vectors per thread and chunk
@@ -152,7 +156,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
   int64_t bm, bn;
   block_to_tile(blockIdx.x, nb, cdiv_dev(a.M, 128), nbn, 8, bm, bn);
   const int64_t m0 = bm * 128, n0 = bn * BN;
-  const bool bound_on = ADC || a.clamp_on;
+  constexpr bool bound_on = CLAMP;
 
   f32x16 acc[2][NBJ];
   uint32_t totp[2][NBJ][8];   // running total, bf16 pairs: [g*2 + (c>>1)] = rows c, c+1 of group g
@@ -349,7 +353,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
               for (int c = 0; c < 4; ++c) y[c] *= rcpv[c];
               rd2(y[0], y[1]); rd2(y[2], y[3]);
-              if (!a.skip_rounding) {
+              if (ROUND) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) y[c] = rintf(y[c]);
               }
@@ -357,11 +361,11 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
               for (int c = 0; c < 4; ++c) y[c] *= rv[c];
               rd2(y[0], y[1]); rd2(y[2], y[3]);
             }
-            if (a.clamp_on) {
+            if (CLAMP) {
               bool over = false;
 #pragma unroll
               for (int c = 0; c < 4; ++c) over |= !(fabsf(y[c]) <= Bv[c]);
-              if (__any(over)) {  // rare: some output of this group left the ADC range
+              if (__builtin_expect(__any(over), 0)) {  // rare: an output of this group left the range
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
                   const bool cl = !(fabsf(y[c]) <= Bv[c]);
@@ -385,7 +389,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
         }
       }
     }
-    if (a.keep != nullptr && a.clamp_on) {
+    if (CLAMP && a.keep != nullptr) {
       // the clamp-mask words of this tile: per 32-column block, the 64 rows of the wave are
       // 256 contiguous bytes
       uint32_t* plane = a.keep + (int64_t)t * clamp_plane_words(a.M, a.N);
@@ -454,16 +458,18 @@ static int significant_bits(float v) {
 }
 
 template <int IRMODE, int NBJ>
-static void launch_fast(const FastFwdArgs& a, bool noise, bool adc, hipStream_t s) {
+static void launch_fast(const FastFwdArgs& a, bool noise, int qm, hipStream_t s) {
   constexpr int lds_bytes = (128 + 64 * NBJ) * kLdsStrideF + 2 * 384 * (int)sizeof(float);
   const dim3 block(256), grid((unsigned)(cdiv(a.M, 128) * cdiv(a.N, 64 * NBJ)));
+#define AHL_FWD(NZ, Q) hipLaunchKernelGGL((k_fwd_fast<IRMODE, NZ, Q, NBJ>), grid, block, lds_bytes, s, a)
   if (noise) {
-    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, true, NBJ>), grid, block, lds_bytes, s, a);
-    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, true, false, NBJ>), grid, block, lds_bytes, s, a);
+    if (qm == 0) AHL_FWD(true, 0); else if (qm == 1) AHL_FWD(true, 1);
+    else if (qm == 2) AHL_FWD(true, 2); else AHL_FWD(true, 3);
   } else {
-    if (adc) hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, true, NBJ>), grid, block, lds_bytes, s, a);
-    else hipLaunchKernelGGL((k_fwd_fast<IRMODE, false, false, NBJ>), grid, block, lds_bytes, s, a);
+    if (qm == 0) AHL_FWD(false, 0); else if (qm == 1) AHL_FWD(false, 1);
+    else if (qm == 2) AHL_FWD(false, 2); else AHL_FWD(false, 3);
   }
+#undef AHL_FWD
 }
 
 namespace ahl {
@@ -472,6 +478,7 @@ namespace ahl {
 bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, const void* w,
                        int64_t ldw, int64_t K, const Tiling& tl) {
   if (cfg->dtype != AHL_BF16 || xq == nullptr) return false;
+  if (cfg->out_res > 0.0f && !(cfg->out_bound > 0.0f)) return false;  // an ADC needs its bound
   if (!aligned16(xq) || !aligned16(w) || ldxq % 8 != 0 || ldw % 8 != 0) return false;
   if (cfg->tile_stride > 0) {  // padded tile layout: any split
     const int64_t padded = (int64_t)tl.n_tiles * cfg->tile_stride;
@@ -515,9 +522,10 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   // When those are too few to give every CU a block (few rows: a recurrent step, a small batch),
   // the 128 x 64 blocks double the count.
   const bool few = cdiv(M, 128) * cdiv(N, 128) < 200;
-  if (cfg->ir_mode == AHL_IR_NONE) few ? launch_fast<0, 1>(a, noise, adc, s) : launch_fast<0, 2>(a, noise, adc, s);
-  else if (cfg->ir_mode == AHL_IR_STATIC) few ? launch_fast<1, 1>(a, noise, adc, s) : launch_fast<1, 2>(a, noise, adc, s);
-  else few ? launch_fast<2, 1>(a, noise, adc, s) : launch_fast<2, 2>(a, noise, adc, s);
+  const int qm = adc ? (cfg->skip_rounding ? 3 : 2) : (a.clamp_on ? 1 : 0);
+  if (cfg->ir_mode == AHL_IR_NONE) few ? launch_fast<0, 1>(a, noise, qm, s) : launch_fast<0, 2>(a, noise, qm, s);
+  else if (cfg->ir_mode == AHL_IR_STATIC) few ? launch_fast<1, 1>(a, noise, qm, s) : launch_fast<1, 2>(a, noise, qm, s);
+  else few ? launch_fast<2, 1>(a, noise, qm, s) : launch_fast<2, 2>(a, noise, qm, s);
   return check_launch("ahl_linear_fwd(fast)");
 }
 
