@@ -105,9 +105,9 @@ struct FastFwdArgs {
   int32_t tile;                  // columns of a tile that hold data, rounded up to 64
   int32_t tile_stride;           // columns from one tile start to the next (>= tile)
   int32_t n_tiles;
-  float out_bound, out_res, two_inv_res;
+  float out_bound, out_res, step_factor;
   float noise_scale;
-  int32_t noise_per_channel, bound_per_channel, skip_rounding, clamp_on, res_is_states, res_mul_exact;
+  int32_t noise_per_channel, bound_per_channel, skip_rounding, clamp_on, step_by_division;
   uint64_t seed, offset;
 };
 
@@ -122,14 +122,14 @@ AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// step of an ADC with bound B (bf16 value held in fp32)
+// step of an ADC with bound B (bf16 value held in fp32): rd(rd(2B) / n) for n states, rd(2B * res)
+// for a relative resolution. 2B is exact, so the second form is one product with the factor
+// 2 * res; for n with <= 8 significant bits the product with fl(2 / n) rounds to the same bf16 as
+// the quotient (see BF16::div). Only other n need the division; that case is a branch on a
+// launch constant, so the common one carries no division code.
 AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
-  if (a.res_is_states) {
-    // rd(rd(2B) / n): 2B is exact; for n with <= 8 significant bits the product with fl(2/n)
-    // rounds to the same bf16 as the quotient (see BF16::div), otherwise divide
-    return a.res_mul_exact ? BF16::rd(B * a.two_inv_res) : BF16::rd(__fdiv_rn(B + B, a.out_res));
-  }
-  return BF16::rd((B + B) * a.out_res);
+  if (__builtin_expect(a.step_by_division != 0, 0)) return BF16::rd(__fdiv_rn(B + B, a.out_res));
+  return BF16::rd(B * a.step_factor);
 }
 
 // QM, what happens to a tile's outputs after the noise: 0 nothing, 1 clamp at the bound, 2 ADC
@@ -334,11 +334,16 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
               if (bound_on) {
                 rd2(Bv[0], Bv[1]); rd2(Bv[2], Bv[3]);
                 if (ADC) {
+                  if (__builtin_expect(a.step_by_division != 0, 0)) {
 #pragma unroll
-                  for (int c = 0; c < 4; ++c) {
-                    rv[c] = adc_step(Bv[c], a);
-                    rcpv[c] = __builtin_amdgcn_rcpf(fmaxf(rv[c], kTinyF32));
+                    for (int c = 0; c < 4; ++c) rv[c] = adc_step(Bv[c], a);
+                  } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) rv[c] = Bv[c] * a.step_factor;
+                    rd2(rv[0], rv[1]); rd2(rv[2], rv[3]);
                   }
+#pragma unroll
+                  for (int c = 0; c < 4; ++c) rcpv[c] = __builtin_amdgcn_rcpf(fmaxf(rv[c], kTinyF32));
                 }
               }
             }
@@ -511,9 +516,9 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   a.noise_scale = noise ? (float)((double)cfg->out_noise / sqrt((double)tl.n_tiles)) : 0.0f;
   a.noise_per_channel = cfg->out_noise_per_channel; a.bound_per_channel = cfg->bound_per_channel;
   a.skip_rounding = cfg->skip_rounding; a.clamp_on = cfg->out_bound > 0.0f ? 1 : 0;
-  a.res_is_states = cfg->out_res > 1.0f ? 1 : 0;
-  a.res_mul_exact = (adc && a.res_is_states && significant_bits(cfg->out_res) <= 8) ? 1 : 0;
-  a.two_inv_res = adc ? 2.0f / cfg->out_res : 0.0f;
+  const bool states = cfg->out_res > 1.0f;
+  a.step_by_division = (adc && states && significant_bits(cfg->out_res) > 8) ? 1 : 0;
+  a.step_factor = !adc ? 0.0f : states ? 2.0f / cfg->out_res : 2.0f * cfg->out_res;
   a.seed = cfg->seed; a.offset = cfg->offset;
   if (cdiv(M, 128) * cdiv(N, 64) > 0x7fffffff) return AHL_ERR_ARG;
   if (clamp_flag) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);

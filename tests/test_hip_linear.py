@@ -158,6 +158,16 @@ SHAPES = [
     case("padn_bf16_pertensor_nobias", dtype="bf16", M=96, K=1000, N=61, max_input_size=256,
          bias=False, ir_mode="static", ir_init=2.0, inp_res=1 / 254, out_res=1 / 254, out_bound=2.0,
          w_scale=0.1, ir_decay=0.0, seed=53),
+    # converter resolutions with more than 8 significant bits: the quantiser steps come from a
+    # division (the product with 2 / n is only exact for n of up to 8 bits)
+    case("bf16_10bit_static", dtype="bf16", M=200, K=512, N=136, max_input_size=256,
+         ir_mode="static", inp_res=1022, out_res=1022, out_bound=0.6, ir_decay=0.01, ir_init=2.0,
+         w_scale=0.1, seed=56),
+    case("bf16_16bit_dynamic", dtype="bf16", M=130, K=512, N=72, max_input_size=256,
+         ir_mode="dynamic", inp_res=65534, out_res=65534, out_bound=0.3, w_scale=0.1, seed=57),
+    case("bf16_odd_states_static", dtype="bf16", M=96, K=768, N=64, max_input_size=384,
+         ir_mode="static", inp_res=1001, out_res=1001, out_bound=0.6, ir_values=[1.5, 2.5],
+         w_scale=0.1, seed=58),
     case("pad_bf16_lsq", dtype="bf16", M=64, K=200, N=64, max_input_size=100, ir_mode="static",
          clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30,
          w_scale=0.3, inp_res=254, out_res=254, out_bound=10.0, seed=36),
