@@ -30,8 +30,8 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 # rocprofv3 FETCH_SIZE and WRITE_SIZE runs of `bench.py --kernels-only`, each scaled by what the
 # same counter reads for the 256 MiB copy below (profiles/*_hbm_traffic.txt holds the table).
 MEASURED_TRAFFIC_BYTES = {
-    "linear_fwd": int((708.4 + 96.2) * 2 ** 20),
-    "linear_bwd_dx(+ir_grad)": int((480.4 + 64.0) * 2 ** 20),
+    "linear_fwd": int((707.6 + 96.2) * 2 ** 20),
+    "linear_bwd_dx(+ir_grad)": int((480.5 + 64.0) * 2 ** 20),
     "linear_bwd_dw(+bias_grad)": int((416.2 + 32.2) * 2 ** 20),
 }
 
