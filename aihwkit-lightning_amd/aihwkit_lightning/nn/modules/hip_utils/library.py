@@ -14,7 +14,7 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
@@ -147,11 +147,12 @@ SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int64, _I32P, c_int32,
          POINTER(AhlLinearCfg), c_void_p],
     ),
+    "ahl_linear_fwd_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32]),
     "ahl_linear_fwd": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
          c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, _I32P,
-         c_int32, POINTER(AhlLinearCfg), c_void_p],
+         c_int32, POINTER(AhlLinearCfg), c_void_p, c_void_p],
     ),
     "ahl_linear_bwd_dx": (
         c_int32,

@@ -540,6 +540,11 @@ def dac(x: Tensor, ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
     return xq, ir_dyn
 
 
+# Hand the forward a workspace for calls of few rows (one K-tile per block, summed in tile order
+# afterwards). The result is the same bit for bit either way; the switch exists for comparisons.
+SPLIT_FEW_ROW_FORWARD = True
+
+
 def linear_fwd(
     x: Optional[Tensor], xq: Optional[Tensor], w_eff: Tensor, bias: Optional[Tensor],
     ir: Optional[Tensor], wmax: Optional[Tensor], tile_max: Optional[Tensor], in_sizes: List[int],
@@ -563,12 +568,16 @@ def linear_fwd(
     keep = torch.empty((n_tiles, (n_out + 31) // 32, (m_rows + 63) // 64 * 64) if want_keep else (0,),
                        dtype=torch.int32, device=ref.device)
     flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
+    ws_bytes = 0
+    if xq is not None and SPLIT_FEW_ROW_FORWARD:
+        ws_bytes = lib.ahl_linear_fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype)
+    ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=ref.device) if ws_bytes else None
     L.check(
         lib.ahl_linear_fwd(
             _ptr(x), _ld(x) if x is not None else 0, _ptr(xq), _ld(xq) if xq is not None else 0,
             _ptr(w_eff), _ld(w_eff), _ptr(bias), _ptr(y), n_out, _ptr(keep) if want_keep else None,
             _ptr(flag) if want_keep else None, _ptr(ir), _ptr(wmax), _ptr(tile_max), m_rows, k_in,
-            n_out, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _stream(),
+            n_out, L.tile_ends_array(in_sizes), n_tiles, byref(cfg), _ptr(ws), _stream(),
         ),
         "ahl_linear_fwd",
     )

@@ -109,6 +109,8 @@ struct FastFwdArgs {
   float noise_scale;
   int32_t noise_per_channel, bound_per_channel, skip_rounding, clamp_on, step_by_division;
   uint64_t seed, offset;
+  uint16_t* part;                // null, or [T, M, N]: every block takes ONE K-tile and leaves its
+                                 // result there; k_tile_sum adds the tiles in order (few rows)
 };
 
 AHL_DEV void mma_bf16_zero(const u32x4& a, const u32x4& b, f32x16& c) {
@@ -152,9 +154,11 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
   const int h = lane >> 5;
 
   const int64_t nbn = cdiv_dev(a.N, BN);
-  const int64_t nb = gridDim.x;
+  const bool one_tile = a.part != nullptr;
+  const int64_t nb = one_tile ? gridDim.x / a.n_tiles : gridDim.x;   // output blocks
+  const int t_first = one_tile ? (int)(blockIdx.x / nb) : 0;
   int64_t bm, bn;
-  block_to_tile(blockIdx.x, nb, cdiv_dev(a.M, 128), nbn, 8, bm, bn);
+  block_to_tile(blockIdx.x % nb, nb, cdiv_dev(a.M, 128), nbn, 8, bm, bn);
   const int64_t m0 = bm * 128, n0 = bn * BN;
   constexpr bool bound_on = CLAMP;
 
@@ -200,13 +204,14 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
     for (int j = 0; j < NB; ++j)
       rawB[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsB, voB[j], kc * 2, 0));
   };
-  load(0);
-  const int cpt = a.tile / 64, nchunks = a.n_tiles * cpt;
+  const int32_t k_first = t_first * a.tile_stride;
+  load(k_first);
+  const int cpt = a.tile / 64, nchunks = (one_tile ? 1 : a.n_tiles) * cpt;
   // k offset of the chunk after the one being loaded: next 64 columns, or the next tile's start
-  int32_t knext = 64;
+  int32_t knext = k_first + 64;
   int lcin = 1;  // position inside its tile of the chunk at knext
-  if (lcin == cpt) { lcin = 0; knext = a.tile_stride; }
-  int t = 0, cin = 0;
+  if (lcin == cpt) { lcin = 0; knext = k_first + a.tile_stride; }
+  int t = t_first, cin = 0;
   // registers -> LDS for the chunk held in rawA/rawB; `tt` is its K-tile, `first` whether it
   // opens that tile (then the dynamic-mode per-row constants of the tile are written too)
   auto stage = [&](int tt, bool first) {
@@ -419,13 +424,14 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
     for (int bj = 0; bj < NBJ; ++bj) {
       const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
-      const float b = (a.bias && n < a.N) ? BF16::load(a.bias, n) : 0.0f;
+      const bool add_bias = a.bias != nullptr && !one_tile;
+      const float b = (add_bias && n < a.N) ? BF16::load(a.bias, n) : 0.0f;
 #pragma unroll
       for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
         for (int pr = 0; pr < 8; ++pr) {
           uint32_t tp = totp[bi][bj][pr];
-          if (a.bias) tp = pack_bf16x2(unpack_lo(tp) + b, unpack_hi(tp) + b);
+          if (add_bias) tp = pack_bf16x2(unpack_lo(tp) + b, unpack_hi(tp) + b);
           const int ro = bi * 32 + 8 * (pr >> 1) + 2 * (pr & 1);
           *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)tp;
           *(uint16_t*)(obase + (ro + 1) * kOutStride + bj * 64) = (uint16_t)(tp >> 16);
@@ -436,14 +442,41 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
     constexpr int RPP = 256 / VPR;       // rows per pass
     const int vcol = tid % VPR, vrow = tid / VPR;
     const int64_t n = n0 + vcol * 8;
+    uint16_t* yout = one_tile ? a.part + (int64_t)t_first * a.M * a.N : (uint16_t*)a.y;
+    const int64_t ldy = one_tile ? a.N : a.ldy;
 #pragma unroll
     for (int j = 0; j < 128 / RPP; ++j) {
       const int row = vrow + RPP * j;
       const int64_t m = m0 + row;
       if (m < a.M && n < a.N)
-        st16((uint16_t*)a.y + m * a.ldy + n, *(const u32x4*)(lds + row * kOutStride + vcol * 16));
+        st16(yout + m * ldy + n, *(const u32x4*)(lds + row * kOutStride + vcol * 16));
     }
   }
+}
+
+// y[m, n] = rd(...rd(rd(0 + part[0]) + part[1])... ) (+ bias): the running total of k_fwd_fast over
+// the tiles, for results that were computed one tile per block. One 16-byte vector per thread.
+__global__ __launch_bounds__(256) void k_tile_sum(const uint16_t* __restrict__ part, int32_t n_tiles,
+                                                  int64_t M, int64_t N, const uint16_t* __restrict__ bias,
+                                                  uint16_t* __restrict__ y, int64_t ldy) {
+  const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t nv = N / 8;
+  if (v >= M * nv) return;
+  const int64_t m = v / nv, n = (v - m * nv) * 8;
+  float tot[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < n_tiles; ++t) {
+    float e[8];
+    BF16::unpack(ld16(part + ((int64_t)t * M + m) * N + n), e);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) tot[i] = BF16::rd(tot[i] + e[i]);
+  }
+  if (bias != nullptr) {
+    float b[8];
+    BF16::unpack(ld16(bias + n), b);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) tot[i] = BF16::rd(tot[i] + b[i]);
+  }
+  st16(y + m * ldy + n, BF16::pack(tot));
 }
 
 __global__ void k_zero_u32(uint32_t* p) { *p = 0u; }
@@ -465,7 +498,7 @@ static int significant_bits(float v) {
 template <int IRMODE, int NBJ>
 static void launch_fast(const FastFwdArgs& a, bool noise, int qm, hipStream_t s) {
   constexpr int lds_bytes = (128 + 64 * NBJ) * kLdsStrideF + 2 * 384 * (int)sizeof(float);
-  const dim3 block(256), grid((unsigned)(cdiv(a.M, 128) * cdiv(a.N, 64 * NBJ)));
+  const dim3 block(256), grid((unsigned)(cdiv(a.M, 128) * cdiv(a.N, 64 * NBJ) * (a.part ? a.n_tiles : 1)));
 #define AHL_FWD(NZ, Q) hipLaunchKernelGGL((k_fwd_fast<IRMODE, NZ, Q, NBJ>), grid, block, lds_bytes, s, a)
   if (noise) {
     if (qm == 0) AHL_FWD(true, 0); else if (qm == 1) AHL_FWD(true, 1);
@@ -478,6 +511,17 @@ static void launch_fast(const FastFwdArgs& a, bool noise, int qm, hipStream_t s)
 }
 
 namespace ahl {
+
+// Few rows (a recurrent step, a decoding step): the 128 x 64 output blocks alone leave most CUs
+// idle and every block walks the whole contraction with one chunk in flight. With a workspace
+// the K-tiles of an output block go to different blocks as well.
+bool fast_fwd_split(int64_t M, int64_t N, int32_t n_tiles) {
+  return n_tiles > 1 && cdiv(M, 128) * cdiv(N, 64) <= 256;
+}
+
+int64_t fast_fwd_ws_bytes(int64_t M, int64_t N, int32_t n_tiles) {
+  return fast_fwd_split(M, N, n_tiles) ? (int64_t)n_tiles * M * N * 2 : 0;
+}
 
 // Whether ahl_linear_fwd can take the bf16 fast path for these arguments.
 bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, const void* w,
@@ -497,7 +541,7 @@ bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, co
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
                     void* y, int64_t ldy, uint32_t* keep, uint32_t* clamp_flag, const void* ir,
                     const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
-                    const Tiling& tl, const AhlLinearCfg* cfg, hipStream_t s) {
+                    const Tiling& tl, const AhlLinearCfg* cfg, void* ws, hipStream_t s) {
   FastFwdArgs a;
   a.xq = xq; a.ldx = ldxq; a.w = w_eff; a.ldw = ldw; a.bias = bias; a.y = y; a.ldy = ldy;
   a.keep = keep; a.clamp_flag = clamp_flag; a.ir = ir; a.wmax = wmax; a.tile_max = tile_max;
@@ -527,10 +571,16 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   // When those are too few to give every CU a block (few rows: a recurrent step, a small batch),
   // the 128 x 64 blocks double the count.
   const bool few = cdiv(M, 128) * cdiv(N, 128) < 200;
+  const bool split = ws != nullptr && aligned16(ws) && (!bias || aligned16(bias)) &&
+                     fast_fwd_split(M, N, tl.n_tiles);
+  a.part = split ? (uint16_t*)ws : nullptr;
   const int qm = adc ? (cfg->skip_rounding ? 3 : 2) : (a.clamp_on ? 1 : 0);
   if (cfg->ir_mode == AHL_IR_NONE) few ? launch_fast<0, 1>(a, noise, qm, s) : launch_fast<0, 2>(a, noise, qm, s);
   else if (cfg->ir_mode == AHL_IR_STATIC) few ? launch_fast<1, 1>(a, noise, qm, s) : launch_fast<1, 2>(a, noise, qm, s);
   else few ? launch_fast<2, 1>(a, noise, qm, s) : launch_fast<2, 2>(a, noise, qm, s);
+  if (split)
+    hipLaunchKernelGGL(k_tile_sum, dim3((unsigned)cdiv(M * (N / 8), 256)), dim3(256), 0, s, a.part,
+                       tl.n_tiles, M, N, (const uint16_t*)bias, (uint16_t*)y, ldy);
   return check_launch("ahl_linear_fwd(fast)");
 }
 

@@ -693,7 +693,8 @@ bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, co
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
                     void* y, int64_t ldy, uint32_t* keep, uint32_t* clamp_flag, const void* ir,
                     const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
-                    const Tiling& tl, const AhlLinearCfg* cfg, hipStream_t s);
+                    const Tiling& tl, const AhlLinearCfg* cfg, void* ws, hipStream_t s);
+int64_t fast_fwd_ws_bytes(int64_t M, int64_t N, int32_t n_tiles);
 __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N);
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
@@ -751,11 +752,17 @@ static void launch_dx(const DxArgs& a, bool is_static, dim3 grid, hipStream_t s)
 
 extern "C" {
 
+int64_t ahl_linear_fwd_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype) {
+  (void)K;
+  if (dtype != AHL_BF16 || M <= 0 || N <= 0 || n_tiles <= 0) return 0;
+  return fast_fwd_ws_bytes(M, N, n_tiles);
+}
+
 int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* w_eff,
                    int64_t ldw, const void* bias, void* y, int64_t ldy, uint32_t* keep,
                    uint32_t* clamp_flag, const void* ir, const void* wmax, const float* tile_max,
                    int64_t M, int64_t K, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
-                   const AhlLinearCfg* cfg, void* stream) {
+                   const AhlLinearCfg* cfg, void* ws, void* stream) {
   if (!cfg_ok(cfg) || (!x && !xq) || !w_eff || !y || M <= 0 || K <= 0 || N <= 0) return AHL_ERR_ARG;
   if ((x && ldx < K) || (xq && ldxq < K) || ldw < K || ldy < N) return AHL_ERR_ARG;
   Tiling tl;
@@ -770,7 +777,7 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
   if (fast_fwd_eligible(cfg, xq, ldxq, w_eff, ldw, K, tl) && N % 8 == 0 && ldy % 8 == 0 &&
       aligned16(y) && (!keep || (((uintptr_t)keep) & 3u) == 0))
     return launch_fast_fwd(xq, ldxq, w_eff, ldw, bias, y, ldy, keep, clamp_flag, ir, wmax, tile_max,
-                           M, K, N, tl, cfg, (hipStream_t)stream);
+                           M, K, N, tl, cfg, ws, (hipStream_t)stream);
   // only the fast path can start from xq alone or read the padded tile layout
   if (!x || cfg->tile_stride > 0) return AHL_ERR_UNSUPPORTED;
   FwdArgs a;

@@ -316,12 +316,18 @@ int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_i
  *            consumed by the two backward entry points.
  *   clamp_flag  uint32 [1] or NULL: receives non-zero if any tile output was clamped (or if the
  *            kernel does not track it); the backward entry points skip the mask when it is zero.
+ *   ws       NULL, or ahl_linear_fwd_ws_bytes(...) bytes, 16-byte aligned. With it, calls of few
+ *            rows (a recurrent or decoding step) give every K-tile of an output block to a block
+ *            of its own and add the per-tile results in tile order afterwards: the same
+ *            arithmetic and the same result bit for bit, on more of the chip. The size function
+ *            returns 0 where that does not apply.
  * Slot of TritonLinear.forward, triton_utils/triton_linear.py:446-690.                   */
+int64_t ahl_linear_fwd_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype);
 int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, const void* w_eff,
                    int64_t ldw, const void* bias, void* y, int64_t ldy, uint32_t* clamp_mask,
                    uint32_t* clamp_flag, const void* ir, const void* wmax, const float* tile_max,
                    int64_t M, int64_t K, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
-                   const AhlLinearCfg* cfg, void* stream);
+                   const AhlLinearCfg* cfg, void* ws, void* stream);
 
 /* Input gradient and input-range gradient (torch_utils/torch_linear.py:29-108 backward):
  *   d[:, tile t] = (g * !clamped_t) @ w_eff[:, tile t]      w_eff [N, K] as used by the forward

@@ -424,3 +424,35 @@ def test_misaligned_input_with_padded_layout():
     res = dict(out=out.detach().cpu(), dx=xin.grad.cpu(), dw=layer.weight.grad.cpu(),
                db=layer.bias.grad.cpu(), dir=layer.input_range.grad.cpu())
     check_against(res, ref, c, "misaligned x")
+
+
+@pytest.mark.parametrize("rows", [1, 48, 130])
+@pytest.mark.parametrize("ir_mode", ["static", "dynamic"])
+def test_few_row_forward_with_one_tile_per_block_is_bit_identical(rows, ir_mode):
+    """Few rows: every K-tile of an output block goes to a block of its own and the per-tile
+    results are added in tile order by a second kernel. Output (noise on: the normals are keyed
+    by tile, row and column, not by block), clamp mask and gradients equal the one-block-per-
+    output-block forward bit for bit."""
+    from hip_helpers import make_layer
+    from aihwkit_lightning.nn.modules.hip_utils import ops
+
+    c = case(f"few_rows_{rows}_{ir_mode}", dtype="bf16", M=rows, K=1536, N=1024, max_input_size=512,
+             ir_mode=ir_mode, inp_res=254, out_res=254, out_bound=0.4, out_noise=0.05,
+             ir_decay=0.01, ir_init=2.0, w_scale=0.1, training=True, seed=61)
+    x, w, b, g = make_inputs(c)
+    results = []
+    for split in (True, False):
+        ops.SPLIT_FEW_ROW_FORWARD = split
+        try:
+            layer = make_layer(c, inputs=(x, w, b, g))
+            torch.manual_seed(11)   # the Philox seed of the call comes from torch's generator
+            inp = x.cuda().requires_grad_()
+            out = layer(inp)
+            out.backward(g.cuda())
+            results.append((out.detach().clone(), inp.grad.clone(), layer.weight.grad.clone(),
+                            layer.bias.grad.clone()))
+        finally:
+            ops.SPLIT_FEW_ROW_FORWARD = True
+    for got, want, what in zip(results[0], results[1], ("out", "dx", "dw", "db")):
+        assert torch.equal(got, want), what
+    assert results[0][0].abs().max() > 0
