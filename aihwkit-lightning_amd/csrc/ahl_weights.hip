@@ -182,6 +182,67 @@ __global__ __launch_bounds__(256) void k_weight_prep_rows(ModArgs a, void* __res
   }
 }
 
+// Abs-max and the per-channel quantiser in one pass over W: one wave per (channel, tile) reduces
+// the maximum of its segment, writes wmax[t, n] and quantises the segment with its own scale --
+// from registers for segments of up to 1024 inputs, else from a second (cache-resident) read.
+// The reference's resolution convention switches to "number of states" when EVERY scale of the
+// tile exceeds one; a wave whose own scale does not knows the switch is off. The others leave
+// their segment to the second launch (DEFERRED), which runs after the tile minima are known and
+// returns at once for every other segment. Same arithmetic as k_weight_modify; in place or not.
+template <class D, bool DEFERRED>
+__global__ __launch_bounds__(256) void k_quantize_rows(ModArgs a, void* __restrict__ wmax_io) {
+  constexpr int E = D::EPV;
+  constexpr int VPG = 8 / E;
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t n = wave / a.tl.n_tiles;
+  const int32_t t = (int32_t)(wave % a.tl.n_tiles);
+  if (n >= a.N) return;
+  const int32_t g0 = a.tl.start(t) >> 3, g1 = a.tl.start(t + 1) >> 3;
+  const typename D::elem* row = (const typename D::elem*)a.w + n * a.ld;
+  typename D::elem* dst = (typename D::elem*)a.w_eff + n * a.ld_eff;
+  float keep[2][8];
+  float mx = 0.0f;
+  bool all_gt1 = false;
+  if (DEFERRED) {
+    mx = D::load(wmax_io, (int64_t)t * a.N + n);
+    if (!(D::rd(__fdiv_rn(mx, a.n_states)) > 1.0f)) return;   // done by the first launch
+    all_gt1 = D::rd(__fdiv_rn(a.tile_min[t], a.n_states)) > 1.0f;
+  } else {
+    int it = 0;
+    for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
+      float v[8];
+#pragma unroll
+      for (int q = 0; q < VPG; ++q) D::unpack(ld16(row + (int64_t)g * 8 + q * E), v + q * E);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
+      if (it < 2) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) keep[it][e] = v[e];
+      }
+    }
+    mx = wave_max(mx);
+    if (lane == 0) D::store(wmax_io, (int64_t)t * a.N + n, mx);
+    if (D::rd(__fdiv_rn(D::rd(mx), a.n_states)) > 1.0f) return;  // needs the tile minimum: deferred
+  }
+  const WQuant q = make_wquant<D>(D::rd(mx), a.n_states, all_gt1);
+  int it = 0;
+  for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
+    float v[8];
+    if (!DEFERRED && it < 2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = keep[it][e];
+    } else {
+#pragma unroll
+      for (int qv = 0; qv < VPG; ++qv) D::unpack(ld16(row + (int64_t)g * 8 + qv * E), v + qv * E);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = wquant_apply<D>(v[e], q, a.maxq);
+#pragma unroll
+    for (int qv = 0; qv < VPG; ++qv) st16(dst + (int64_t)g * 8 + qv * E, D::pack(v + qv * E));
+  }
+}
+
 // LSQ backward of the learnable clip: one wave per (channel, tile).
 struct ClipBwdArgs {
   void* dw; int64_t lddw;
@@ -262,6 +323,21 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       if (!cfg->skip_tile_stats)
         hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
       return check_launch("ahl_weight_prep(one pass)");
+    }
+    // one pass for "abs-max + per-channel quantiser, no noise" on 16-byte aligned tiles
+    if (!cfg->wmax_given && w_eff && cfg->quant_type == AHL_QUANT_DISCRETIZE_PER_CHANNEL &&
+        noise == AHL_NOISE_NONE && vec && tl.extra == 0 && tl.base % 8 == 0 && aligned16(w_eff) &&
+        ld_eff % D::EPV == 0) {
+      ModArgs a;
+      a.w = w; a.N = N; a.K = K; a.ld = ld; a.tl = tl; a.wmax = nullptr; a.tile_max = tile_max;
+      a.tile_min = tile_min; a.w_eff = w_eff; a.ld_eff = ld_eff; a.quant_type = cfg->quant_type;
+      a.noise_type = noise; a.n_states = fmaxf(cfg->res, 1.0f / cfg->res);
+      a.maxq = D::kIsBf16 ? host_round_bf16(a.n_states / 2.0f) : a.n_states / 2.0f;
+      a.std_dev = 0.0f; a.seed = 0; a.offset = 0;
+      hipLaunchKernelGGL((k_quantize_rows<D, false>), grid, dim3(256), 0, s, a, wmax);
+      hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
+      hipLaunchKernelGGL((k_quantize_rows<D, true>), grid, dim3(256), 0, s, a, wmax);
+      return check_launch("ahl_weight_prep(one-pass quantiser)");
     }
     if (cfg->wmax_given) {
       // wmax holds the learnable clip: nothing to reduce

@@ -187,6 +187,37 @@ def test_quantize_weights_matches_reference(name):
     assert torch.allclose(before, after, rtol=tol, atol=tol * float(ref_out.abs().mean()))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("scales", ["small", "all_large", "mixed"])
+@pytest.mark.parametrize("cols,tile", [(512, 256), (2560, 1280), (300, 100)],
+                         ids=["held", "long_segments", "unaligned_tiles"])
+def test_quantize_weights_per_channel_scale_switch(cols, tile, scales, dtype):
+    """The per-channel quantiser against the oracle where the reference's resolution convention
+    matters: it reads the scales as numbers of states only if EVERY scale of a tile exceeds one.
+    `small`: none does (the one-pass kernel alone); `all_large`: all do; `mixed`: some channels do,
+    so the switch stays off but their segments wait for the tile minimum. Segments held in
+    registers, segments longer than that, and a split the one-pass kernel does not take."""
+    from aihwkit_lightning.nn.modules.hip_utils import library as L
+
+    gen = torch.Generator().manual_seed(cols + len(scales))
+    w = torch.randn(24, cols, generator=gen)
+    if scales == "all_large":
+        w = w * 400.0
+    elif scales == "mixed":
+        w[::3] = w[::3] * 400.0
+    w = w.to(dtype)
+    sizes = om.split_sizes(cols, tile)
+    dev = w.cuda().clone()
+    ops().quantize_weights(dev, sizes, L.AHL_QUANT_DISCRETIZE_PER_CHANNEL, 30.0)
+    ref = om.quantize_weights(w, sizes, om.DISCRETIZE_PER_CHANNEL, 30.0)
+    got = dev.cpu()
+    if dtype == torch.bfloat16:
+        assert torch.equal(got, ref)
+    else:
+        assert torch.allclose(got, ref, rtol=1e-6, atol=1e-9)
+    assert not torch.equal(got, w)
+
+
 @pytest.mark.parametrize("in_size", [10, 255, 257])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_calibration_max(in_size, dtype):
