@@ -397,9 +397,9 @@ def hbm_kernel_rooflines(reps):
         "running_absmax(x)": (lambda: OPS.running_absmax(nxt(xs), in_sizes, cache), xbytes),
         # sums and clamp from one read of W (a row stays in registers); writes only changed vectors
         "clip_weights(W, per channel)": (lambda: OPS.clip_weights(nxt(ws), 3.0, L.AHL_CLIP_PER_CHANNEL), wb),
-        # abs-max pass + quantise pass (read + write)
+        # abs-max and quantisation from one read, one write
         "quantize_weights(W)": (lambda: OPS.quantize_weights(
-            nxt(ws), in_sizes, L.AHL_QUANT_DISCRETIZE_PER_CHANNEL, 254.0), 3 * wb),
+            nxt(ws), in_sizes, L.AHL_QUANT_DISCRETIZE_PER_CHANNEL, 254.0), 2 * wb),
         "dac(x bf16 8192x3072)": (lambda: OPS.dac(nxt(xbs), irb, in_sizes, icfg, fcfg),
                                   2 * xbs[0].numel() * 2),
         # calibration statistics: row filter + sums (2 reads); row filter + 4 digit histograms +
