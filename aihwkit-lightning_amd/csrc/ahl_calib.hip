@@ -63,7 +63,7 @@ __global__ void k_select_init(SelState* st, uint32_t* hist, const uint32_t* n_ke
 // Histogram of digit `pass` (0 = most significant byte) over the kept elements of every tile
 // whose higher digits equal the tile's prefix. One wave per (group of rows, tile); per-wave
 // histogram in LDS, then one integer atomic per non-empty bin.
-template <class D>
+template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x, int64_t rows,
                                                      int64_t ld, const uint8_t* __restrict__ kept,
                                                      Tiling tl, int rpw, int pass,
@@ -88,13 +88,12 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
       if (r >= rows) break;
       if (!kept[r]) continue;
       const typename D::elem* row = (const typename D::elem*)x + r * ld;
-      for (int32_t c = tl.start(t) + lane; c < tl.start(t + 1); c += 64) {
-        const float v = D::load(row, c);
+      wave_row_foreach2<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
         nan |= (v != v);
         const uint32_t key = f32_key(v);
         // digits above this pass must match the prefix found so far
         if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1u);
-      }
+      });
     }
     if (pass == 0 && __builtin_amdgcn_ballot_w64(nan) != 0ull && lane == 0) atomicOr(&st[t].has_nan, 1u);
     for (int i = lane; i < 256; i += 64) {
@@ -130,7 +129,7 @@ __global__ void k_select_pick(SelState* st, uint32_t* hist, int pass) {
 }
 
 // next_key[t] = smallest key above the selected one
-template <class D>
+template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_select_next(const void* __restrict__ x, int64_t rows,
                                                      int64_t ld, const uint8_t* __restrict__ kept,
                                                      Tiling tl, int rpw, SelState* __restrict__ st) {
@@ -147,10 +146,10 @@ __global__ __launch_bounds__(256) void k_select_next(const void* __restrict__ x,
     if (r >= rows) break;
     if (!kept[r]) continue;
     const typename D::elem* row = (const typename D::elem*)x + r * ld;
-    for (int32_t c = tl.start(t) + lane; c < tl.start(t + 1); c += 64) {
-      const uint32_t key = f32_key(D::load(row, c));
+    wave_row_foreach2<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
+      const uint32_t key = f32_key(v);
       if (key > sel && key < best) best = key;
-    }
+    });
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
@@ -238,10 +237,12 @@ int ahl_sliced_quantile(const void* x, int32_t dtype, int64_t rows, int64_t cols
     else hipLaunchKernelGGL((k_row_nonzero<D, false>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
     hipLaunchKernelGGL(k_select_init, dim3(n_tiles), dim3(256), 0, s, st, hist, (const uint32_t*)n_kept, tl, q);
     for (int pass = 0; pass < 4; ++pass) {
-      hipLaunchKernelGGL((k_select_hist<D>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist);
+      if (vec) hipLaunchKernelGGL((k_select_hist<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist);
+      else hipLaunchKernelGGL((k_select_hist<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist);
       hipLaunchKernelGGL(k_select_pick, dim3(n_tiles), dim3(256), 0, s, st, hist, pass);
     }
-    hipLaunchKernelGGL((k_select_next<D>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, st);
+    if (vec) hipLaunchKernelGGL((k_select_next<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, st);
+    else hipLaunchKernelGGL((k_select_next<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, st);
   });
   hipLaunchKernelGGL(k_select_final, dim3((unsigned)cdiv(n_tiles, 64)), dim3(64), 0, s, (const SelState*)st, n_tiles, out);
   return check_launch("ahl_sliced_quantile");
