@@ -5,6 +5,7 @@ device pointers, sizes and the current HIP stream to one C entry point, and retu
 registered for the CUDA (= ROCm/HIP) dispatch key only: calling them on CPU tensors raises.
 """
 from ctypes import byref, c_void_p
+from functools import lru_cache
 from typing import List, Optional, Tuple
 
 import torch
@@ -540,6 +541,12 @@ def dac(x: Tensor, ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
     return xq, ir_dyn
 
 
+@lru_cache(maxsize=4096)
+def _fwd_ws_bytes(m_rows: int, k_in: int, n_out: int, n_tiles: int, dtype: int) -> int:
+    """The library's answer per shape (host arithmetic there; asked once per shape here)."""
+    return int(L.load().ahl_linear_fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, dtype))
+
+
 # Hand the forward a workspace for calls of few rows (one K-tile per block, summed in tile order
 # afterwards). The result is the same bit for bit either way; the switch exists for comparisons.
 SPLIT_FEW_ROW_FORWARD = True
@@ -570,7 +577,7 @@ def linear_fwd(
     flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
     ws_bytes = 0
     if xq is not None and SPLIT_FEW_ROW_FORWARD:
-        ws_bytes = lib.ahl_linear_fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype)
+        ws_bytes = _fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=ref.device) if ws_bytes else None
     L.check(
         lib.ahl_linear_fwd(
