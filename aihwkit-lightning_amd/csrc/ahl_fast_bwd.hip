@@ -455,7 +455,16 @@ __global__ __launch_bounds__(256) void k_split_reduce(const float* __restrict__ 
   if (idx >= R * K) return;
   const int64_t r = idx / K, c = idx - r * K;  // K is a multiple of 256: the 4 share a row
   f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < slices; ++s) sum += *(const f32x4*)(split + (int64_t)s * R * K + idx);
+  // four slices' loads in flight at a time; the sums stay in slice order
+  for (int s = 0; s < slices; s += 4) {
+    f32x4 part[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      part[u] = *(const f32x4*)(split + (int64_t)(s + u < slices ? s + u : slices - 1) * R * K + idx);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (s + u < slices) sum += part[u];
+  }
   u32x2 pk = {pack_bf16x2(sum.x, sum.y), pack_bf16x2(sum.z, sum.w)};
   *(u32x2*)(out + r * ldo + c) = pk;
 }
@@ -485,9 +494,18 @@ __global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
   if (row < a.M && ovalid) {
     f32x4 lo4 = {0.f, 0.f, 0.f, 0.f}, hi4 = {0.f, 0.f, 0.f, 0.f};
     const float* sp = a.split + row * a.K + c0 + vcol * 8;
-    for (int sl = 0; sl < a.slices; ++sl) {
-      lo4 += *(const f32x4*)(sp + (int64_t)sl * a.M * a.K);
-      hi4 += *(const f32x4*)(sp + (int64_t)sl * a.M * a.K + 4);
+    // four slices' loads in flight at a time; the sums stay in slice order
+    for (int sl = 0; sl < a.slices; sl += 4) {
+      f32x4 l[4], h[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t si = sl + u < a.slices ? sl + u : a.slices - 1;
+        l[u] = *(const f32x4*)(sp + si * a.M * a.K);
+        h[u] = *(const f32x4*)(sp + si * a.M * a.K + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (sl + u < a.slices) { lo4 += l[u]; hi4 += h[u]; }
     }
     float d[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
 #pragma unroll
