@@ -106,26 +106,35 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
 }
 
 // The bin that holds rank k_rem: extend the prefix, rebase the rank, clear the histogram.
-__global__ void k_select_pick(SelState* st, uint32_t* hist, int pass) {
-  const int t = blockIdx.x;
-  if (threadIdx.x == 0) {
-    SelState s = st[t];
-    if (s.n != 0) {
-      uint32_t cum = 0u;
-      int b = 0;
-      for (; b < 255; ++b) {
-        const uint32_t c = hist[t * 256 + b];
-        if (cum + c > s.k_rem) break;
-        cum += c;
-      }
-      s.prefix = (s.prefix << 8) | (uint32_t)b;
-      s.k_rem -= cum;
-      if (pass == 3) s.n_le = (s.lo - s.k_rem) + hist[t * 256 + b];  // below + equal
-      st[t] = s;
-    }
-  }
+// 256 threads, one bin each: inclusive prefix sums through LDS, then the first bin (of 0..254)
+// whose running count exceeds the rank, bin 255 otherwise.
+__global__ __launch_bounds__(256) void k_select_pick(SelState* st, uint32_t* hist, int pass) {
+  __shared__ uint32_t cum[2][256];
+  __shared__ int pick;
+  const int t = blockIdx.x, b = threadIdx.x;
+  const uint32_t c = hist[t * 256 + b];
+  const SelState s0 = st[t];
+  if (b == 0) pick = 255;
+  cum[0][b] = c;
   __syncthreads();
-  for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[t * 256 + i] = 0u;
+  int cur = 0;
+#pragma unroll
+  for (int off = 1; off < 256; off <<= 1) {
+    cum[cur ^ 1][b] = cum[cur][b] + (b >= off ? cum[cur][b - off] : 0u);
+    cur ^= 1;
+    __syncthreads();
+  }
+  const uint32_t incl = cum[cur][b], excl = incl - c;
+  if (b < 255 && excl <= s0.k_rem && incl > s0.k_rem) pick = b;   // at most one bin qualifies
+  __syncthreads();
+  if (b == pick && s0.n != 0) {
+    SelState s = s0;
+    s.prefix = (s.prefix << 8) | (uint32_t)b;
+    s.k_rem -= excl;
+    if (pass == 3) s.n_le = (s.lo - s.k_rem) + c;  // below + equal
+    st[t] = s;
+  }
+  hist[t * 256 + b] = 0u;
 }
 
 // next_key[t] = smallest key above the selected one
@@ -156,7 +165,8 @@ __global__ __launch_bounds__(256) void k_select_next(const void* __restrict__ x,
     const uint32_t o = (uint32_t)__shfl_xor((int)best, off, 64);
     best = o < best ? o : best;
   }
-  if (lane == 0 && best != 0xffffffffu) atomicMin(&st[t].next_key, best);
+  if (lane == 0 && best < __hip_atomic_load(&st[t].next_key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+    atomicMin(&st[t].next_key, best);
 }
 
 // out[t] = lerp(x_(lo), x_(lo+1), weight) with torch's two-sided lerp formula
@@ -195,9 +205,12 @@ __global__ void k_ir_moving_update(void* ir, int32_t* idx, const float* __restri
   idx[t] = i + 1;
 }
 
+// Rows per wave of the selection passes: every wave ends with one atomic per non-empty bin of
+// its tile's histogram, and atomics on one address are served one after the other, so a few
+// hundred waves per tile is the budget (the leading digit of real data fills a handful of bins).
 static int select_rpw(int64_t rows) {
-  const int64_t r = rows / 4096;
-  return (int)(r < 1 ? 1 : (r > 16 ? 16 : r));
+  const int64_t r = rows / 256;
+  return (int)(r < 1 ? 1 : (r > 32 ? 32 : r));
 }
 
 }  // namespace ahl

@@ -307,10 +307,11 @@ AHL_DEV void wave_row_foreach(const void* row, int32_t c0, int32_t c1, int lane,
   }
 }
 
-// The same walk with two 16-byte loads in flight per lane: for kernels whose per-element work
-// (LDS atomics, compares) the compiler will not move a load across.
-template <class D, bool VEC, class F>
-AHL_DEV void wave_row_foreach2(const void* row, int32_t c0, int32_t c1, int lane, F f) {
+// The same walk with U 16-byte loads in flight per lane: for kernels whose per-element work
+// (LDS atomics, compares) the compiler will not move a load across, and for rows walked by a
+// single wave.
+template <class D, bool VEC, int U, class F>
+AHL_DEV void wave_row_foreach_n(const void* row, int32_t c0, int32_t c1, int lane, F f) {
   if (VEC) {
     constexpr int E = D::EPV;
     int32_t a0 = (c0 + E - 1) / E * E;
@@ -319,24 +320,29 @@ AHL_DEV void wave_row_foreach2(const void* row, int32_t c0, int32_t c1, int lane
     for (int32_t c = c0 + lane; c < a0; c += 64) f(D::load(row, c));
     const typename D::elem* base = (const typename D::elem*)row;
     const int32_t v1 = a1 / E;
-    for (int32_t v = a0 / E + lane; v < v1; v += 128) {
-      const bool two = v + 64 < v1;
-      const u32x4 x0 = ld16(base + (int64_t)v * E);
-      const u32x4 x1 = ld16(base + (int64_t)(two ? v + 64 : v) * E);
-      float e[E];
-      D::unpack(x0, e);
+    for (int32_t v = a0 / E + lane; v < v1; v += 64 * U) {
+      u32x4 x[U];
 #pragma unroll
-      for (int i = 0; i < E; ++i) f(e[i]);
-      if (two) {
-        D::unpack(x1, e);
+      for (int u = 0; u < U; ++u) x[u] = ld16(base + (int64_t)(v + 64 * u < v1 ? v + 64 * u : v) * E);
 #pragma unroll
-        for (int i = 0; i < E; ++i) f(e[i]);
+      for (int u = 0; u < U; ++u) {
+        if (v + 64 * u < v1) {
+          float e[E];
+          D::unpack(x[u], e);
+#pragma unroll
+          for (int i = 0; i < E; ++i) f(e[i]);
+        }
       }
     }
     for (int32_t c = a1 + lane; c < c1; c += 64) f(D::load(row, c));
   } else {
     for (int32_t c = c0 + lane; c < c1; c += 64) f(D::load(row, c));
   }
+}
+
+template <class D, bool VEC, class F>
+AHL_DEV void wave_row_foreach2(const void* row, int32_t c0, int32_t c1, int lane, F f) {
+  wave_row_foreach_n<D, VEC, 2>(row, c0, c1, lane, f);
 }
 
 }  // namespace ahl

@@ -414,7 +414,11 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
     t += 1;
   }
 
-  if (a.clamp_flag != nullptr && __any(any_clamp != 0u) && lane == 0) atomicOr(a.clamp_flag, 1u);
+  // most waves find the flag already set and skip the atomic (atomics on one address are served
+  // one after the other)
+  if (a.clamp_flag != nullptr && __any(any_clamp != 0u) && lane == 0 &&
+      __hip_atomic_load(a.clamp_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u)
+    atomicOr(a.clamp_flag, 1u);
 
   // ---- store y = total (+ bias): transposed through LDS, 16-byte row-contiguous stores ----
   {

@@ -64,22 +64,29 @@ static __global__ void k_fill_u32(uint32_t* p, uint32_t v, int n) {
 }
 
 // kept[r] = 1 unless every element of row r is zero (-0.0 counts as zero, NaN does not);
-// *n_kept += number of kept rows. One wave per row.
+// *n_kept += number of kept rows. One wave per row, one atomic per block (atomics on one
+// address are served one after the other: a per-row atomic cost more than reading the rows).
 template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_row_nonzero(const void* __restrict__ x, int64_t rows,
                                                      int64_t cols, int64_t ld,
                                                      uint8_t* __restrict__ kept,
                                                      uint32_t* __restrict__ n_kept) {
-  const int lane = threadIdx.x & 63;
-  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (r >= rows) return;
-  const typename D::elem* row = (const typename D::elem*)x + r * ld;
-  bool any = false;
-  wave_row_foreach<D, VEC>(row, 0, (int32_t)cols, lane, [&](float v) { any |= (v != 0.0f); });
-  const bool keep = __builtin_amdgcn_ballot_w64(any) != 0ull;
-  if (lane == 0) {
-    kept[r] = keep ? 1 : 0;
-    if (keep) atomicAdd(n_kept, 1u);
+  __shared__ uint32_t wave_kept[4];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t r = (int64_t)blockIdx.x * 4 + wave;
+  bool keep = false;
+  if (r < rows) {
+    const typename D::elem* row = (const typename D::elem*)x + r * ld;
+    bool any = false;
+    wave_row_foreach_n<D, VEC, 4>(row, 0, (int32_t)cols, lane, [&](float v) { any |= (v != 0.0f); });
+    keep = __builtin_amdgcn_ballot_w64(any) != 0ull;
+    if (lane == 0) kept[r] = keep ? 1 : 0;
+  }
+  if (lane == 0) wave_kept[wave] = keep ? 1u : 0u;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const uint32_t n = wave_kept[0] + wave_kept[1] + wave_kept[2] + wave_kept[3];
+    if (n) atomicAdd(n_kept, n);
   }
 }
 
