@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
       if (r >= rows) break;
       if (!kept[r]) continue;
       const typename D::elem* row = (const typename D::elem*)x + r * ld;
-      wave_row_foreach2<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
+      wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
         nan |= (v != v);
         const uint32_t key = f32_key(v);
         // digits above this pass must match the prefix found so far
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void k_select_next(const void* __restrict__ x,
     if (r >= rows) break;
     if (!kept[r]) continue;
     const typename D::elem* row = (const typename D::elem*)x + r * ld;
-    wave_row_foreach2<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
+    wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
       const uint32_t key = f32_key(v);
       if (key > sel && key < best) best = key;
     });

@@ -286,30 +286,10 @@ AHL_DEV float dac_apply(float x, const Dac& d, bool skip_rounding) {
 // Iterates one wave over the columns [c0, c1) of a row; f(value) is called once per element.
 // VEC: the row base (p + row*ld) is 16-byte aligned, so whole `vec`s can be loaded for the
 // aligned middle part; head and tail are done element-wise.
-template <class D, bool VEC, class F>
-AHL_DEV void wave_row_foreach(const void* row, int32_t c0, int32_t c1, int lane, F f) {
-  if (VEC) {
-    constexpr int E = D::EPV;
-    int32_t a0 = (c0 + E - 1) / E * E;
-    int32_t a1 = c1 / E * E;
-    if (a0 > a1) { a0 = c1; a1 = c1; }
-    for (int32_t c = c0 + lane; c < a0; c += 64) f(D::load(row, c));
-    const typename D::elem* base = (const typename D::elem*)row;
-    for (int32_t v = a0 / E + lane; v < a1 / E; v += 64) {
-      float e[E];
-      D::unpack(ld16(base + (int64_t)v * E), e);
-#pragma unroll
-      for (int i = 0; i < E; ++i) f(e[i]);
-    }
-    for (int32_t c = a1 + lane; c < c1; c += 64) f(D::load(row, c));
-  } else {
-    for (int32_t c = c0 + lane; c < c1; c += 64) f(D::load(row, c));
-  }
-}
-
-// The same walk with U 16-byte loads in flight per lane: for kernels whose per-element work
-// (LDS atomics, compares) the compiler will not move a load across, and for rows walked by a
-// single wave.
+// U 16-byte loads are in flight per lane before the first value is used (a lane's elements still
+// arrive in ascending column order, so sums do not depend on U): the compiler does not move a
+// load across per-element work such as LDS atomics, and a wave that walks its row with one load
+// in flight is bound by that load's latency.
 template <class D, bool VEC, int U, class F>
 AHL_DEV void wave_row_foreach_n(const void* row, int32_t c0, int32_t c1, int lane, F f) {
   if (VEC) {
@@ -341,7 +321,7 @@ AHL_DEV void wave_row_foreach_n(const void* row, int32_t c0, int32_t c1, int lan
 }
 
 template <class D, bool VEC, class F>
-AHL_DEV void wave_row_foreach2(const void* row, int32_t c0, int32_t c1, int lane, F f) {
+AHL_DEV void wave_row_foreach(const void* row, int32_t c0, int32_t c1, int lane, F f) {
   wave_row_foreach_n<D, VEC, 2>(row, c0, c1, lane, f);
 }
 
