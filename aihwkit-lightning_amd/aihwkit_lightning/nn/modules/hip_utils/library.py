@@ -14,7 +14,8 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 11
+ABI_VERSION = 12
+STATIC_DX_SCRATCH_BYTES = 16 * 1024 * 1024
 
 AHL_F32, AHL_BF16 = 0, 1
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
@@ -159,6 +160,12 @@ SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
          c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32,
          POINTER(AhlLinearCfg), c_void_p, c_void_p],
+    ),
+    "ahl_linear_bwd_dx_static": (
+        c_int32,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
+         c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, _I32P, c_int32,
+         POINTER(AhlLinearCfg), c_void_p],
     ),
     "ahl_linear_bwd_dx_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int64]),
     "ahl_linear_bwd_dw": (

@@ -18,6 +18,7 @@
 //   C[8 * (v / 4) + 4 * (l / 32) + (v % 4)][l % 32].
 #include "ahl_host.h"
 #include <math.h>
+#include <mutex>
 
 namespace ahl {
 
@@ -929,6 +930,61 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     });
   }
   return check_launch("ahl_linear_bwd_dx");
+}
+
+
+// ---- allocation-free variant of ahl_linear_bwd_dx -------------------------------------------
+// The workspace of the input gradient (input-range partial sums, slice partial results, the
+// transposed weights of the general kernels) lives in a file-scope device array instead of a
+// caller buffer. Each GPU holds its own copy of the array at its own address; the address is
+// looked up once per device and used for every launch (the array's name is only a host-side
+// handle, never a device address).
+static constexpr int64_t kStaticDxScratchBytes = AHL_STATIC_DX_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticDxScratchBytes];
+
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of `scratch` on the current device (cached per device); null + recorded error
+// if the lookup fails.
+static void* static_scratch_ptr() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) { record_hip_error(e, "ahl_linear_bwd_dx_static(hipGetDevice)"); return nullptr; }
+  if (dev < 0 || dev >= kMaxDevices) {
+    record_hip_error(hipErrorInvalidDevice, "ahl_linear_bwd_dx_static(device index)");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      record_hip_error(e, "ahl_linear_bwd_dx_static(hipGetSymbolAddress)");
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+int ahl_linear_bwd_dx_static(const void* g, int64_t ldg, const uint32_t* keep,
+                             const uint32_t* clamp_flag, const void* w_eff, int64_t ldw,
+                             const void* x, int64_t ldx, const void* ir, void* dx, int64_t lddx,
+                             void* ir_grad, int64_t M, int64_t K, int64_t N,
+                             const int32_t* tile_ends_host, int32_t n_tiles,
+                             const AhlLinearCfg* cfg, void* stream) {
+  if (!cfg_ok(cfg) || M <= 0 || K <= 0 || N <= 0 || n_tiles <= 0) return AHL_ERR_ARG;
+  const int64_t need = ahl_linear_bwd_dx_ws_bytes(M, K, N, n_tiles, cfg->dtype, cfg->tile_stride);
+  // larger shapes are for ahl_linear_bwd_dx with a caller workspace
+  if (need > kStaticDxScratchBytes) return AHL_ERR_WORKSPACE;
+  void* ptr = static_scratch_ptr();
+  if (ptr == nullptr) return AHL_ERR_LAUNCH;
+  // every slot of the workspace is written by this call's kernels before it is read: nothing
+  // has to start at zero, whatever the previous call left behind
+  return ahl_linear_bwd_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, ir_grad, M,
+                           K, N, tile_ends_host, n_tiles, cfg, ptr, stream);
 }
 
 

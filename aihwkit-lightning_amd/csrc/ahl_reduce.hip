@@ -425,7 +425,7 @@ using namespace ahl;
 // ============================================================================================
 extern "C" {
 
-int ahl_abi_version(void) { return 11; }
+int ahl_abi_version(void) { return 12; }
 const char* ahl_last_hip_error(void) { return ahl::g_err; }
 
 int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,

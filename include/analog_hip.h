@@ -347,6 +347,23 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* clamp_mask, co
 int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
                                    int64_t tile_stride);
 
+/* ahl_linear_bwd_dx without a workspace argument, for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). It has no
+ * counterpart in the reference. Same arguments, kernels and results as ahl_linear_bwd_dx; the
+ * workspace is a static device array of AHL_STATIC_DX_SCRATCH_BYTES that every GPU the library
+ * runs on holds until the process ends. Shapes whose ahl_linear_bwd_dx_ws_bytes(...) exceeds that
+ * size return AHL_ERR_WORKSPACE (nothing is launched). The call itself allocates and frees
+ * nothing. All calls on one GPU share that GPU's array: calls that overlap on one GPU (different
+ * streams or threads) race; calls on one stream, or ordered by events, are safe. Nothing in the
+ * array has to be cleared between calls (every slot is written before it is read).            */
+#define AHL_STATIC_DX_SCRATCH_BYTES (16 * 1024 * 1024)
+int ahl_linear_bwd_dx_static(const void* g, int64_t ldg, const uint32_t* clamp_mask,
+                             const uint32_t* clamp_flag, const void* w_eff, int64_t ldw,
+                             const void* x, int64_t ldx, const void* ir, void* dx, int64_t lddx,
+                             void* ir_grad, int64_t M, int64_t K, int64_t N,
+                             const int32_t* tile_ends_host, int32_t n_tiles,
+                             const AhlLinearCfg* cfg, void* stream);
+
 /* Backward of the learnable weight clip (UniformQuantize.backward with learn_res,
  * torch_utils/quant_utils.py:123-153, as called from clip_and_quantize :184-233).
  *   dw    dtype [N, K], in/out: on entry the gradient w.r.t. the clipped (and quantised) weights,
