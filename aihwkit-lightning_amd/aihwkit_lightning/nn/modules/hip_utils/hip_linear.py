@@ -151,7 +151,23 @@ class HipLinear(Function):
         need_dx = ctx.needs_input_grad[0] or (ctx.needs_input_grad[3] and ir_needs_grad)
         need_dw = ctx.needs_input_grad[1] or clip_needs_grad
 
-        seed = draw_seed() if (noise_on or w_noise) else 0
+        # One Philox seed per call from the host generator -- or, while the stream is being
+        # captured into a HIP graph, the device-resident noise state advanced by one recorded
+        # launch per call, so that every replay draws new noise.
+        seed, state_ptr = 0, 0
+        if (noise_on or w_noise) and m_rows > 0:
+            if torch.cuda.is_current_stream_capturing():
+                state = _impl.noise_state(inp.device, create=False)
+                if state is None:
+                    raise HipBackendError(
+                        "a noisy layer is being captured into a graph before the device noise "
+                        "state exists: call aihwkit_lightning.nn.graphs.prepare_noise_state(device) "
+                        "(or use graphed_module) before the capture"
+                    )
+                _impl.seed_advance(state, 2)
+                state_ptr = state.data_ptr()
+            else:
+                seed = draw_seed()
         wmax = tile_max = tile_min = None
         w_eff = weights_c
         clip_quant = L.AHL_QUANT_DISCRETIZE_PER_CHANNEL if w_quant else L.AHL_QUANT_CLIP_LEARNED
@@ -163,7 +179,7 @@ class HipLinear(Function):
             tile_max, tile_min, w_eff = ops.weight_prep_clip(
                 weights_c, wmax, in_sizes, clip_quant,
                 NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE,
-                float(modifier.res) if w_quant else 1.0, float(modifier.std_dev), seed, 1,
+                float(modifier.res) if w_quant else 1.0, float(modifier.std_dev), seed, 1, state_ptr,
             )
         elif m_rows > 0 and need_wmax:
             res = float(modifier.res) if w_quant else 1.0
@@ -182,7 +198,7 @@ class HipLinear(Function):
                 wmax, tile_max, _, eff = ops.weight_prep(
                     weights_c, in_sizes, QUANT_IDS[modifier.quantization_type],
                     NOISE_IDS[modifier.noise_type] if w_noise else L.AHL_NOISE_NONE, res,
-                    float(modifier.std_dev), seed, 1, w_noise or w_quant, skip_tile_stats,
+                    float(modifier.std_dev), seed, 1, w_noise or w_quant, skip_tile_stats, state_ptr,
                 )
                 if w_noise or w_quant:
                     w_eff = eff
@@ -233,6 +249,7 @@ class HipLinear(Function):
             # fast_mode clamps with torch.clamp: its autograd rule instead of the learned-range one
             L.AHL_IR_GRAD_CLAMP if fast else L.AHL_IR_GRAD_LEARNED,
             stride,
+            state_ptr,
         ]
         fcfg = [
             float(fwd.inp_res), float(fwd.out_res), float(fwd.out_bound),

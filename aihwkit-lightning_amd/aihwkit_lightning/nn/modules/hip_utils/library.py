@@ -54,6 +54,7 @@ class AhlLinearCfg(Structure):
         ("tile_stride", c_int32),
         ("seed", c_uint64),
         ("offset", c_uint64),
+        ("seed_state", c_void_p),
     ]
 
 
@@ -70,6 +71,7 @@ class AhlModifierCfg(Structure):
         ("skip_tile_stats", c_int32),
         ("seed", c_uint64),
         ("offset", c_uint64),
+        ("seed_state", c_void_p),
     ]
 
 
@@ -92,6 +94,7 @@ _I32P = POINTER(c_int32)
 # name -> (restype, argtypes); every exported symbol of include/analog_hip.h
 SIGNATURES = {
     "ahl_abi_version": (c_int32, []),
+    "ahl_seed_advance": (c_int32, [c_void_p, c_uint64, c_void_p]),
     "ahl_conv_out_size": (c_int32, [POINTER(AhlConvGeom), _I32P]),
     "ahl_im2col": (c_int32, [c_void_p, POINTER(AhlConvGeom), c_int32, c_void_p, c_int64, c_void_p]),
     "ahl_col2im": (c_int32, [c_void_p, c_int64, POINTER(AhlConvGeom), c_int32, c_void_p, c_void_p]),

@@ -66,6 +66,8 @@ def _linear_cfg(dtype: torch.dtype, icfg: List[int], fcfg: List[float]) -> L.Ahl
      cfg.skip_rounding, seed, offset) = icfg[:7]
     cfg.ir_grad_rule = icfg[7] if len(icfg) > 7 else L.AHL_IR_GRAD_LEARNED
     cfg.tile_stride = icfg[8] if len(icfg) > 8 else 0
+    # device address of the noise state {key, call counter} (0: the seed comes by value)
+    cfg.seed_state = (icfg[9] or None) if len(icfg) > 9 else None
     (cfg.inp_res, cfg.out_res, cfg.out_bound, cfg.out_noise, cfg.ir_decay,
      cfg.ir_input_min_percentage) = fcfg
     cfg.seed, cfg.offset = seed, offset
@@ -95,13 +97,13 @@ LIB.define("clip_weights(Tensor(a!) w, float sigma, int kind) -> ()")
 LIB.define("col_sum(Tensor x) -> Tensor")
 LIB.define(
     "weight_prep(Tensor w, int[] in_sizes, int quant_type, int noise_type, float res, "
-    "float std_dev, int seed, int offset, bool want_eff, bool skip_tile_stats=False) "
-    "-> (Tensor, Tensor, Tensor, Tensor)"
+    "float std_dev, int seed, int offset, bool want_eff, bool skip_tile_stats=False, "
+    "int seed_state=0) -> (Tensor, Tensor, Tensor, Tensor)"
 )
 LIB.define("quantize_weights(Tensor(a!) w, int[] in_sizes, int quant_type, float res) -> ()")
 LIB.define(
     "weight_prep_clip(Tensor w, Tensor clip, int[] in_sizes, int quant_type, int noise_type, "
-    "float res, float std_dev, int seed, int offset) -> (Tensor, Tensor, Tensor)"
+    "float res, float std_dev, int seed, int offset, int seed_state=0) -> (Tensor, Tensor, Tensor)"
 )
 LIB.define(
     "learned_clip_bwd(Tensor(a!) dw, Tensor w, Tensor clip, Tensor tile_min, int[] in_sizes, "
@@ -128,6 +130,31 @@ LIB.define("unpad_tiles(Tensor x, int[] in_sizes, int stride) -> Tensor")
 LIB.define("im2col(Tensor x, int[] geom) -> Tensor")
 LIB.define("col2im(Tensor dcols, int[] geom) -> Tensor")
 LIB.define("transpose_batched(Tensor src) -> Tensor")
+
+
+_NOISE_STATES = {}
+
+
+def noise_state(device: torch.device, create: bool = True) -> Optional[Tensor]:
+    """The device-resident noise state of ``device``: int64 ``[2]`` = (Philox key, call counter).
+
+    Launches that are replayed from a HIP graph cannot carry their seed by value (every replay
+    would draw the same noise): under stream capture the layers point their kernels at this
+    state and record one :func:`seed_advance` per call. The key is drawn from torch's CPU
+    generator when the state is created, so ``torch.manual_seed`` makes graphed runs reproducible.
+    It has to exist before a capture starts (creating it copies from the host)."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    state = _NOISE_STATES.get(index)
+    if state is None and create:
+        key = int(torch.randint(0, 2**62, (1,)).item())
+        state = torch.tensor([key, 0], dtype=torch.int64, device=torch.device("cuda", index))
+        _NOISE_STATES[index] = state
+    return state
+
+
+def seed_advance(state: Tensor, delta: int) -> None:
+    """``state[1] += delta`` on the device (one small launch on the current stream)."""
+    L.check(L.load().ahl_seed_advance(_ptr(state), int(delta), _stream()), "ahl_seed_advance")
 
 
 def tile_stride(k_in: int, n_tiles: int, dtype: torch.dtype) -> int:
@@ -411,7 +438,8 @@ def col_sum(x: Tensor) -> Tensor:
     return out
 
 
-def _modifier_cfg(dtype, quant_type, noise_type, res, std_dev, seed, offset) -> L.AhlModifierCfg:
+def _modifier_cfg(dtype, quant_type, noise_type, res, std_dev, seed, offset,
+                  seed_state: int = 0) -> L.AhlModifierCfg:
     cfg = L.AhlModifierCfg()
     cfg.dtype = dtype_id(dtype)
     cfg.quant_type, cfg.noise_type = quant_type, noise_type
@@ -421,12 +449,13 @@ def _modifier_cfg(dtype, quant_type, noise_type, res, std_dev, seed, offset) -> 
     cfg.res = max(res, 1.0 / res) if res > 0 else res
     cfg.std_dev = std_dev
     cfg.seed, cfg.offset = seed, offset
+    cfg.seed_state = seed_state or None
     return cfg
 
 
 def weight_prep(
     w: Tensor, in_sizes: List[int], quant_type: int, noise_type: int, res: float, std_dev: float,
-    seed: int, offset: int, want_eff: bool, skip_tile_stats: bool = False,
+    seed: int, offset: int, want_eff: bool, skip_tile_stats: bool = False, seed_state: int = 0,
 ) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     """wmax ``[T, N]``, tile max/min ``[T]`` and, if wanted, the modified copy ``[N, K]``.
     ``skip_tile_stats``: the caller does not use tile max/min (they may come back unwritten)."""
@@ -440,7 +469,7 @@ def weight_prep(
     tile_max = torch.empty((n_tiles,), dtype=torch.float32, device=dev)
     tile_min = torch.empty((n_tiles,), dtype=torch.float32, device=dev)
     w_eff = torch.empty((n_out, n_in) if want_eff else (0,), dtype=w.dtype, device=dev)
-    cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset)
+    cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset, seed_state)
     cfg.skip_tile_stats = int(skip_tile_stats)
     L.check(
         lib.ahl_weight_prep(
@@ -454,7 +483,7 @@ def weight_prep(
 
 def weight_prep_clip(
     w: Tensor, clip: Tensor, in_sizes: List[int], quant_type: int, noise_type: int, res: float,
-    std_dev: float, seed: int, offset: int,
+    std_dev: float, seed: int, offset: int, seed_state: int = 0,
 ) -> Tuple[Tensor, Tensor, Tensor]:
     """Weights under a learnable per-channel clip ``clip [T, N]`` (which also takes the place of
     the per-tile abs-max): tile max/min of the clip and the clipped (+ quantised, + noisy) copy."""
@@ -468,7 +497,7 @@ def weight_prep_clip(
     tile_max = torch.empty((n_tiles,), dtype=torch.float32, device=w.device)
     tile_min = torch.empty((n_tiles,), dtype=torch.float32, device=w.device)
     w_eff = torch.empty((n_out, n_in), dtype=w.dtype, device=w.device)
-    cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset)
+    cfg = _modifier_cfg(w.dtype, quant_type, noise_type, res, std_dev, seed, offset, seed_state)
     cfg.wmax_given = 1
     L.check(
         lib.ahl_weight_prep(

@@ -25,7 +25,7 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("AHL_EXTRA_FLAGS", "").split()
 
 
 def _newest_dep() -> float:

@@ -185,6 +185,17 @@ AHL_DEV void box_muller16(uint32_t w, float& n0, float& n1) {
   n1 = r * __builtin_amdgcn_sinf(rev);
 }
 
+// Philox key and counter offset of a call. They come by value, or -- for launches that are
+// replayed from a HIP graph, where a value baked into the launch would repeat the same noise on
+// every replay -- from device memory: state[0] = key, state[1] = a running call counter that
+// ahl_seed_advance moves; the by-value offset is added to it.
+struct NoiseKey { uint64_t seed, offset; };
+AHL_DEV NoiseKey noise_key(uint64_t seed, uint64_t offset, const uint64_t* state) {
+  NoiseKey k = {seed, offset};
+  if (state != nullptr) { k.seed = state[0]; k.offset = state[1] + offset; }
+  return k;
+}
+
 AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, uint32_t c0,
                      uint32_t c1, float* out8) {
   u32x4 c = {c0, c1, stream_and_tile, (uint32_t)offset};

@@ -14,20 +14,12 @@
 // blocks fit on a CU and the VALU epilogue of one can overlap the MFMA phase of the other. With
 // this wave tile the kernel reads 64 KB of MFMA fragments from LDS and writes 32 KB into it per
 // 512 MFMA cycles of a SIMD: LDS bandwidth, not the MFMA pipe, bounds the plain product.
-#include "ahl_host.h"
-#include <math.h>
+#include "ahl_fwd_common.h"
 
 namespace ahl {
 
 static constexpr int kLdsStrideF = 144;            // bytes; 128 data + 16 pad
 static constexpr int kChunkLdsF = 128 * kLdsStrideF;
-
-// round two fp32 values to bf16 precision, keeping them in fp32 registers (3 instructions)
-AHL_DEV void rd2(float& a, float& b) {
-  const uint32_t p = pack_bf16x2(a, b);
-  a = unpack_lo(p);
-  b = unpack_hi(p);
-}
 
 // -------------------------------------------------------------------------------------------
 // DAC pre-pass, one wave per row: xq[m, k] = DAC(clamp(x[m, k])) with the input range of k's
@@ -90,50 +82,6 @@ __global__ __launch_bounds__(256) void k_dac_rows(const void* __restrict__ x, in
   }
 }
 
-// -------------------------------------------------------------------------------------------
-struct FastFwdArgs {
-  const void* xq; int64_t ldx;   // pre-quantised input, bf16 [M, K]
-  const void* w; int64_t ldw;    // effective weights, bf16 [N, K]
-  const void* bias;
-  void* y; int64_t ldy;
-  uint32_t* keep;                // clamp mask [T, ceil(N/32), M] or null
-  uint32_t* clamp_flag;          // set to non-zero if any tile output was clamped; may be null
-  const void* ir;                // [T] static, [T, M] dynamic
-  const void* wmax;              // [T, N]
-  const float* tile_max;         // [T]
-  int64_t M, N;
-  int32_t tile;                  // columns of a tile that hold data, rounded up to 64
-  int32_t tile_stride;           // columns from one tile start to the next (>= tile)
-  int32_t n_tiles;
-  float out_bound, out_res, step_factor;
-  float noise_scale;
-  int32_t noise_per_channel, bound_per_channel, skip_rounding, clamp_on, step_by_division;
-  uint64_t seed, offset;
-  uint16_t* part;                // null, or [T, M, N]: every block takes ONE K-tile and leaves its
-                                 // result there; k_tile_sum adds the tiles in order (few rows)
-};
-
-AHL_DEV void mma_bf16_zero(const u32x4& a, const u32x4& b, f32x16& c) {
-  const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                              __builtin_bit_cast(bf16x8, b), z, 0, 0, 0);
-}
-
-AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
-  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                              __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
-
-// step of an ADC with bound B (bf16 value held in fp32): rd(rd(2B) / n) for n states, rd(2B * res)
-// for a relative resolution. 2B is exact, so the second form is one product with the factor
-// 2 * res; for n with <= 8 significant bits the product with fl(2 / n) rounds to the same bf16 as
-// the quotient (see BF16::div). Only other n need the division; that case is a branch on a
-// launch constant, so the common one carries no division code.
-AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
-  if (__builtin_expect(a.step_by_division != 0, 0)) return BF16::rd(__fdiv_rn(B + B, a.out_res));
-  return BF16::rd(B * a.step_factor);
-}
-
 // QM, what happens to a tile's outputs after the noise: 0 nothing, 1 clamp at the bound, 2 ADC
 // quantisation and clamp, 3 the same without the rounding step (skip_rounding). Compile-time, so
 // that the per-group epilogue has no branches apart from the rare "something left the range".
@@ -162,6 +110,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
   const int64_t m0 = bm * 128, n0 = bn * BN;
   constexpr bool bound_on = CLAMP;
 
+  const NoiseKey nk = noise_key(a.seed, a.offset, a.seed_state);
   f32x16 acc[2][NBJ];
   uint32_t totp[2][NBJ][8];   // running total, bf16 pairs: [g*2 + (c>>1)] = rows c, c+1 of group g
   uint32_t cwords[NBJ];       // lane L: clamp-mask word of row wm * 64 + L for the current tile
@@ -310,7 +259,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
           float xi[8];
           if (NOISE) {
             const uint32_t mrow = (uint32_t)(m0 + rbase + 16 * gp);
-            normal8(a.seed, a.offset, (uint32_t)t, (uint32_t)n, (mrow >> 4) * 2 + ((mrow >> 2) & 1), xi);
+            normal8(nk.seed, nk.offset, (uint32_t)t, (uint32_t)n, (mrow >> 4) * 2 + ((mrow >> 2) & 1), xi);
           }
 #pragma unroll
           for (int gg = 0; gg < 2; ++gg) {
@@ -567,7 +516,7 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   const bool states = cfg->out_res > 1.0f;
   a.step_by_division = (adc && states && significant_bits(cfg->out_res) > 8) ? 1 : 0;
   a.step_factor = !adc ? 0.0f : states ? 2.0f / cfg->out_res : 2.0f * cfg->out_res;
-  a.seed = cfg->seed; a.offset = cfg->offset;
+  a.seed = cfg->seed; a.offset = cfg->offset; a.seed_state = cfg->seed_state;
   if (cdiv(M, 128) * cdiv(N, 64) > 0x7fffffff) return AHL_ERR_ARG;
   if (clamp_flag) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);
   // 128 x 128 blocks (NBJ = 2). Measured alternatives: 128 x 64 blocks (NBJ = 1, three to four

@@ -1,0 +1,60 @@
+// Shared by the bf16 forward kernels (ahl_fast.hip, ahl_fwd_pipe.hip): launch arguments and the
+// small device helpers of the per-K-tile epilogue.
+#pragma once
+#include "ahl_host.h"
+#include <math.h>
+
+namespace ahl {
+
+// round two fp32 values to bf16 precision, keeping them in fp32 registers (3 instructions)
+AHL_DEV void rd2(float& a, float& b) {
+  const uint32_t p = pack_bf16x2(a, b);
+  a = unpack_lo(p);
+  b = unpack_hi(p);
+}
+
+struct FastFwdArgs {
+  const void* xq; int64_t ldx;   // pre-quantised input, bf16 [M, K]
+  const void* w; int64_t ldw;    // effective weights, bf16 [N, K]
+  const void* bias;
+  void* y; int64_t ldy;
+  uint32_t* keep;                // clamp mask [T, ceil(N/32), M] or null
+  uint32_t* clamp_flag;          // set to non-zero if any tile output was clamped; may be null
+  const void* ir;                // [T] static, [T, M] dynamic
+  const void* wmax;              // [T, N]
+  const float* tile_max;         // [T]
+  int64_t M, N;
+  int32_t tile;                  // columns of a tile that hold data, rounded up to 64
+  int32_t tile_stride;           // columns from one tile start to the next (>= tile)
+  int32_t n_tiles;
+  float out_bound, out_res, step_factor;
+  float noise_scale;
+  int32_t noise_per_channel, bound_per_channel, skip_rounding, clamp_on, step_by_division;
+  uint64_t seed, offset;
+  const uint64_t* seed_state;    // null, or device {key, call counter} that replaces seed / offset
+  uint16_t* part;                // null, or [T, M, N]: every block takes ONE K-tile and leaves its
+                                 // result there; k_tile_sum adds the tiles in order (few rows)
+};
+
+AHL_DEV void mma_bf16_zero(const u32x4& a, const u32x4& b, f32x16& c) {
+  const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                              __builtin_bit_cast(bf16x8, b), z, 0, 0, 0);
+}
+
+AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
+  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                              __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+// step of an ADC with bound B (bf16 value held in fp32): rd(rd(2B) / n) for n states, rd(2B * res)
+// for a relative resolution. 2B is exact, so the second form is one product with the factor
+// 2 * res; for n with <= 8 significant bits the product with fl(2 / n) rounds to the same bf16 as
+// the quotient (see BF16::div). Only other n need the division; that case is a branch on a
+// launch constant, so the common one carries no division code.
+AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
+  if (__builtin_expect(a.step_by_division != 0, 0)) return BF16::rd(__fdiv_rn(B + B, a.out_res));
+  return BF16::rd(B * a.step_factor);
+}
+
+}  // namespace ahl

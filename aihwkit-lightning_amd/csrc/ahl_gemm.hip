@@ -141,6 +141,7 @@ struct FwdArgs {
   int32_t noise_per_channel, bound_per_channel, skip_rounding;
   int32_t dac_on, adc_on, bound_on, clamp_on, noise_on;
   uint64_t seed, offset;
+  const uint64_t* seed_state;  // null, or device {key, call counter} that replaces seed / offset
 };
 
 template <class D, bool VEC, int IRMODE>
@@ -271,7 +272,8 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
             if (a.noise_on) {
               // rows m0 + rbase + 16 * gp + {0..3, 8..11}: one Philox call per lane and pair of groups
               const uint32_t mrow = (uint32_t)(m0 + rbase + 16 * gp);
-            normal8(a.seed, a.offset, (uint32_t)t, (uint32_t)n, (mrow >> 4) * 2 + ((mrow >> 2) & 1), xi);
+              const NoiseKey nk = noise_key(a.seed, a.offset, a.seed_state);
+              normal8(nk.seed, nk.offset, (uint32_t)t, (uint32_t)n, (mrow >> 4) * 2 + ((mrow >> 2) & 1), xi);
             }
 #pragma unroll
             for (int gg = 0; gg < 2; ++gg) {
@@ -793,7 +795,7 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
   a.adc_on = cfg->out_res > 0.0f ? 1 : 0;
   a.clamp_on = cfg->out_bound > 0.0f ? 1 : 0;
   a.bound_on = (a.adc_on || a.clamp_on) ? 1 : 0;
-  a.seed = cfg->seed; a.offset = cfg->offset;
+  a.seed = cfg->seed; a.offset = cfg->offset; a.seed_state = cfg->seed_state;
   if (cfg->ir_mode == AHL_IR_NONE && (a.dac_on || a.bound_on || a.noise_on)) return AHL_ERR_ARG;
   if (cfg->ir_mode != AHL_IR_NONE && !ir) return AHL_ERR_ARG;
   if ((a.noise_on || a.bound_on) && (!wmax || !tile_max)) return AHL_ERR_ARG;

@@ -7,6 +7,8 @@
 
 namespace ahl {
 
+__global__ void k_seed_advance(uint64_t* state, uint64_t delta) { state[1] += delta; }
+
 static thread_local char g_err[256] = {0};
 int record_hip_error(hipError_t e, const char* where) {
   snprintf(g_err, sizeof(g_err), "%s: %s", where, hipGetErrorString(e));
@@ -426,6 +428,12 @@ using namespace ahl;
 extern "C" {
 
 int ahl_abi_version(void) { return 12; }
+
+int ahl_seed_advance(uint64_t* state, uint64_t delta, void* stream) {
+  if (!state) return AHL_ERR_ARG;
+  hipLaunchKernelGGL(k_seed_advance, dim3(1), dim3(1), 0, (hipStream_t)stream, state, delta);
+  return check_launch("ahl_seed_advance");
+}
 const char* ahl_last_hip_error(void) { return ahl::g_err; }
 
 int ahl_sliced_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,

@@ -57,6 +57,7 @@ struct ModArgs {
   int32_t quant_type, noise_type;
   float n_states, maxq, std_dev;
   uint64_t seed, offset;
+  const uint64_t* seed_state;  // null, or device {key, call counter} that replaces seed / offset
 };
 
 // One thread per group of 8 consecutive inputs of one channel (one Philox call gives the 8
@@ -82,8 +83,10 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t block
 
   if (modify) {
     float xi[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (a.noise_type != AHL_NOISE_NONE)
-      normal8(a.seed, a.offset, 1u << 24, (uint32_t)(kb >> 3), (uint32_t)n, xi);
+    if (a.noise_type != AHL_NOISE_NONE) {
+      const NoiseKey nk = noise_key(a.seed, a.offset, a.seed_state);
+      normal8(nk.seed, nk.offset, 1u << 24, (uint32_t)(kb >> 3), (uint32_t)n, xi);
+    }
     // constants of a tile for this channel
     struct TileConst { WQuant q; float nstd; };
     auto tile_const = [&](int t) {
@@ -164,6 +167,7 @@ __global__ __launch_bounds__(256) void k_weight_prep_rows(ModArgs a, void* __res
   mx = wave_max(mx);
   if (lane == 0) D::store(wmax_out, (int64_t)t * a.N + n, mx);
   const float nstd = D::rd(a.std_dev * D::rd(mx));
+  const NoiseKey nk = noise_key(a.seed, a.offset, a.seed_state);
   it = 0;
   for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
     float v[8], xi[8];
@@ -174,7 +178,7 @@ __global__ __launch_bounds__(256) void k_weight_prep_rows(ModArgs a, void* __res
 #pragma unroll
       for (int q = 0; q < VPG; ++q) D::unpack(ld16(row + (int64_t)g * 8 + q * E), v + q * E);
     }
-    normal8(a.seed, a.offset, 1u << 24, (uint32_t)g, (uint32_t)n, xi);
+    normal8(nk.seed, nk.offset, 1u << 24, (uint32_t)g, (uint32_t)n, xi);
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = D::rd(v[e] + D::rd(nstd * D::rd(xi[e])));
 #pragma unroll
@@ -318,7 +322,7 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       a.w = w; a.N = N; a.K = K; a.ld = ld; a.tl = tl; a.wmax = nullptr; a.tile_max = nullptr;
       a.tile_min = nullptr; a.w_eff = w_eff; a.ld_eff = ld_eff; a.quant_type = AHL_QUANT_NONE;
       a.noise_type = noise; a.n_states = 1.0f; a.maxq = 1.0f; a.std_dev = cfg->std_dev;
-      a.seed = cfg->seed; a.offset = cfg->offset;
+      a.seed = cfg->seed; a.offset = cfg->offset; a.seed_state = cfg->seed_state;
       hipLaunchKernelGGL((k_weight_prep_rows<D>), grid, dim3(256), 0, s, a, wmax);
       if (!cfg->skip_tile_stats)
         hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
@@ -333,7 +337,7 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       a.tile_min = tile_min; a.w_eff = w_eff; a.ld_eff = ld_eff; a.quant_type = cfg->quant_type;
       a.noise_type = noise; a.n_states = fmaxf(cfg->res, 1.0f / cfg->res);
       a.maxq = D::kIsBf16 ? host_round_bf16(a.n_states / 2.0f) : a.n_states / 2.0f;
-      a.std_dev = 0.0f; a.seed = 0; a.offset = 0;
+      a.std_dev = 0.0f; a.seed = 0; a.offset = 0; a.seed_state = nullptr;
       hipLaunchKernelGGL((k_quantize_rows<D, false>), grid, dim3(256), 0, s, a, wmax);
       hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
       hipLaunchKernelGGL((k_quantize_rows<D, true>), grid, dim3(256), 0, s, a, wmax);
@@ -357,7 +361,7 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       // clamp(Tensor, Scalar, Scalar) converts its bounds to the tensor dtype first
       a.maxq = D::kIsBf16 ? host_round_bf16(a.n_states / 2.0f) : a.n_states / 2.0f;
       if (clip_only) a.maxq = 1.0f;
-      a.std_dev = cfg->std_dev; a.seed = cfg->seed; a.offset = cfg->offset;
+      a.std_dev = cfg->std_dev; a.seed = cfg->seed; a.offset = cfg->offset; a.seed_state = cfg->seed_state;
       const int64_t bpr = cdiv(cdiv(K, 8), 256);
       if (bpr * N > 0x7fffffff) return AHL_ERR_ARG;
       const bool vec_mod = vec && K % 8 == 0 && aligned16(w_eff) && ld_eff % D::EPV == 0;

@@ -456,6 +456,8 @@ def main():
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    parser.add_argument("--eager", action="store_true",
+                        help="time the eager step instead of its HIP-graph replay")
     parser.add_argument("--kernels-only", action="store_true",
                         help="only launch the individual kernels (for rocprofv3 runs)")
     parser.add_argument("--workload", default="linear", choices=["linear", "post_training", *OTHER_WORKLOADS],
@@ -499,15 +501,27 @@ def main():
         kernels, _ = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 1))
         print(json.dumps({"ms_per_launch": kernels}))
         return
-    for _ in range(ns.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(ns.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / ns.steps * 1e3
+
+    def timed(fn):
+        for _ in range(ns.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(ns.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / ns.steps * 1e3
+
+    # The step as a training loop drives it: recorded once into a HIP graph and replayed, so that
+    # its launches follow each other without the host in between (every replay draws new noise
+    # from the device-resident Philox state). The eager step (Python between the launches) is
+    # timed next to it.
+    ms_eager = timed(step)
+    if ns.eager:
+        ms_per_step = ms_eager
+    else:
+        from aihwkit_lightning.nn.graphs import CapturedStep
+        ms_per_step = timed(CapturedStep(step))
     step_flops = 3 * 2.0 * M_TOKENS * K_IN * N_OUT
     value = step_flops / (ms_per_step * 1e-3) / 1e12
 
@@ -525,6 +539,8 @@ def main():
                         "range (decay 0.01), 8-bit DAC/ADC, out_noise 0.04, weight noise 0.02 per "
                         "channel, fwd+bwd",
             "frac_of_bf16_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
+            "step": "eager" if ns.eager else "forward + backward replayed from one HIP graph",
+            "ms_per_step_eager": round(ms_eager, 4),
         },
         "roofline": {
             "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,

@@ -85,6 +85,11 @@ typedef struct AhlLinearCfg {
                                     padded tile layout with this stride (see ahl_tile_stride)    */
   uint64_t seed;                 /* Philox key for this call                                    */
   uint64_t offset;               /* Philox counter offset for this call                         */
+  const uint64_t* seed_state;    /* NULL, or a DEVICE uint64[2] = {key, call counter}: the kernels
+                                    then take the key from [0] and add [1] to `offset`. For
+                                    launches recorded into a HIP graph, whose by-value arguments
+                                    would repeat the same noise on every replay: record an
+                                    ahl_seed_advance on the state in front of them               */
 } AhlLinearCfg;
 
 /* Weight modifier of the training forward / post-training quantisation; a flattened
@@ -104,6 +109,7 @@ typedef struct AhlModifierCfg {
                               scales per channel); ahl_weight_prep may then leave them unwritten  */
   uint64_t seed;
   uint64_t offset;
+  const uint64_t* seed_state; /* as in AhlLinearCfg                                             */
 } AhlModifierCfg;
 
 /* ---- padded tile layout ------------------------------------------------------------------
@@ -137,6 +143,12 @@ int ahl_unpad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows
 int ahl_abi_version(void);
 /* Text of the last HIP error seen by a launcher on this thread ("" if none). */
 const char* ahl_last_hip_error(void);
+
+/* state[1] += delta for a device-resident noise state uint64[2] = {Philox key, call counter}
+ * (AhlLinearCfg.seed_state): one small launch, so that every replay of a recorded graph draws
+ * new noise. The reference draws one seed per call on the host (triton_utils/
+ * triton_linear.py:541,617); this is that draw for callers whose launches are replayed.        */
+int ahl_seed_advance(uint64_t* state, uint64_t delta, void* stream);
 
 /* ---- reductions (memory-bound) ------------------------------------------------------------ */
 
