@@ -151,20 +151,22 @@ AHL_DEV uint32_t xor3(uint32_t a, uint32_t b, uint32_t c) {
 }
 
 // Philox4x32-10 (Salmon et al., "Parallel random numbers: as easy as 1, 2, 3", SC'11).
+// one round: the counter is replaced, the key moves on
+AHL_DEV void philox_round(u32x4& c, uint32_t& k0, uint32_t& k1) {
+  const uint64_t p0 = (uint64_t)0xD2511F53u * c.x;
+  const uint64_t p1 = (uint64_t)0xCD9E8D57u * c.z;
+  u32x4 n;
+  n.x = xor3((uint32_t)(p1 >> 32), c.y, k0);
+  n.y = (uint32_t)p1;
+  n.z = xor3((uint32_t)(p0 >> 32), c.w, k1);
+  n.w = (uint32_t)p0;
+  c = n;
+  k0 += 0x9E3779B9u;
+  k1 += 0xBB67AE85u;
+}
 AHL_DEV u32x4 philox4x32_10(u32x4 c, uint32_t k0, uint32_t k1) {
 #pragma unroll
-  for (int r = 0; r < 10; ++r) {
-    const uint64_t p0 = (uint64_t)0xD2511F53u * c.x;
-    const uint64_t p1 = (uint64_t)0xCD9E8D57u * c.z;
-    u32x4 n;
-    n.x = xor3((uint32_t)(p1 >> 32), c.y, k0);
-    n.y = (uint32_t)p1;
-    n.z = xor3((uint32_t)(p0 >> 32), c.w, k1);
-    n.w = (uint32_t)p0;
-    c = n;
-    k0 += 0x9E3779B9u;
-    k1 += 0xBB67AE85u;
-  }
+  for (int r = 0; r < 10; ++r) philox_round(c, k0, k1);
   return c;
 }
 

@@ -1,4 +1,4 @@
-// Shared by the bf16 forward kernels (ahl_fast.hip, ahl_fwd_pipe.hip): launch arguments and the
+// Shared by the bf16 forward kernels (ahl_fast.hip): launch arguments and the
 // small device helpers of the per-K-tile epilogue.
 #pragma once
 #include "ahl_host.h"

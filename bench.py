@@ -26,14 +26,29 @@ import torch  # noqa: E402
 
 M_TOKENS, K_IN, N_OUT, TILE = 8192, 4096, 4096, 512
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
-# Bytes per launch that the L2s pull from / push to the fabric (HBM or Infinity Cache), from
-# rocprofv3 FETCH_SIZE and WRITE_SIZE runs of `bench.py --kernels-only`, each scaled by what the
-# same counter reads for the 256 MiB copy below (profiles/*_hbm_traffic.txt holds the table).
-MEASURED_TRAFFIC_BYTES = {
-    "linear_fwd": int((707.6 + 96.2) * 2 ** 20),
-    "linear_bwd_dx(+ir_grad)": int((480.5 + 64.0) * 2 ** 20),
-    "linear_bwd_dw(+bias_grad)": int((416.2 + 32.2) * 2 ** 20),
+# Bytes per launch that the L2s pull from / push to the fabric (HBM or Infinity Cache) are not
+# measured by this run: they come from rocprofv3 FETCH_SIZE and WRITE_SIZE runs of
+# `bench.py --kernels-only`, each scaled by what the same counter reads for the 256 MiB copy
+# below. The table of the last such run is read from this file (and named in the line).
+TRAFFIC_TABLE = os.path.join("profiles", "linear_fwd_bwd_4096x4096_8192tok_bf16_hbm_traffic.txt")
+TRAFFIC_ROWS = {
+    "linear_fwd": "ahl::k_fwd_fast<",
+    "linear_bwd_dx(+ir_grad)": "ahl::k_bwd_fast<0",
+    "linear_bwd_dw(+bias_grad)": "ahl::k_bwd_fast<1",
 }
+
+
+def measured_traffic_bytes(kernel):
+    """fetch + write bytes per launch of `kernel` from the committed counter table, or None."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_TABLE)) as handle:
+            for line in handle:
+                if line.startswith(TRAFFIC_ROWS[kernel]):
+                    fetch, write = line.split()[-4:-2]
+                    return int((float(fetch) + float(write)) * 2 ** 20)
+    except (OSError, ValueError, KeyError):
+        pass
+    return None
 
 
 def build_layer():
@@ -456,8 +471,8 @@ def main():
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    parser.add_argument("--eager", action="store_true",
-                        help="time the eager step instead of its HIP-graph replay")
+    parser.add_argument("--graph", action="store_true",
+                        help="report the step replayed from one HIP graph instead of the eager step")
     parser.add_argument("--kernels-only", action="store_true",
                         help="only launch the individual kernels (for rocprofv3 runs)")
     parser.add_argument("--workload", default="linear", choices=["linear", "post_training", *OTHER_WORKLOADS],
@@ -512,16 +527,14 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / ns.steps * 1e3
 
-    # The step as a training loop drives it: recorded once into a HIP graph and replayed, so that
-    # its launches follow each other without the host in between (every replay draws new noise
-    # from the device-resident Philox state). The eager step (Python between the launches) is
-    # timed next to it.
+    # The eager step (Python between the launches) is the headline; next to it the same step
+    # recorded once into a HIP graph and replayed (every replay draws new noise from the
+    # device-resident Philox state). At this size the GPU is never waiting for the host, so the
+    # two agree.
+    from aihwkit_lightning.nn.graphs import CapturedStep
     ms_eager = timed(step)
-    if ns.eager:
-        ms_per_step = ms_eager
-    else:
-        from aihwkit_lightning.nn.graphs import CapturedStep
-        ms_per_step = timed(CapturedStep(step))
+    ms_graph = timed(CapturedStep(step))
+    ms_per_step = ms_graph if ns.graph else ms_eager
     step_flops = 3 * 2.0 * M_TOKENS * K_IN * N_OUT
     value = step_flops / (ms_per_step * 1e-3) / 1e12
 
@@ -539,19 +552,39 @@ def main():
                         "range (decay 0.01), 8-bit DAC/ADC, out_noise 0.04, weight noise 0.02 per "
                         "channel, fwd+bwd",
             "frac_of_bf16_mfma_peak": round(value / PEAK_BF16_TFLOPS, 4),
-            "step": "eager" if ns.eager else "forward + backward replayed from one HIP graph",
-            "ms_per_step_eager": round(ms_eager, 4),
+            "step": "forward + backward replayed from one HIP graph" if ns.graph else "eager",
+            "ms_per_step_eager": round(ms_eager, 4), "ms_per_step_graph_replay": round(ms_graph, 4),
         },
         "roofline": {
             "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+            "traffic": measured_traffic_bytes(dom),
+            "traffic_source": TRAFFIC_TABLE + " (rocprofv3 FETCH_SIZE and WRITE_SIZE runs of "
+                              "`bench.py --kernels-only`, not this run)",
             "ms_per_launch": {k: round(v, 4) for k, v in kernels.items()},
         },
     }
     result["hbm_kernels"] = hbm_kernel_rooflines(max(ns.steps, 5))
     if not ns.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
+    # The other configurations of the benchmark set, a few steps each, after the headline's
+    # timed region: the dynamic-range forward, the MLP block, the reduction-bound post-training
+    # pass (with its own CPU baseline). `--workload NAME` prints each as a line of its own.
+    del layer, x, g
+    torch.cuda.empty_cache()
+    others = {}
+    for name in ("fwd_dynamic_4096", "mlp_3072_8192"):
+        res = time_other(name, 10, 3)
+        res["frac_of_bf16_mfma_peak"] = round(res["tflops"] / PEAK_BF16_TFLOPS, 4)
+        others[name] = res
+        torch.cuda.empty_cache()
+    post = time_post_training(not ns.no_cpu)
+    others["post_training"] = {
+        "workload": post["config"]["workload"], "ms": post["ms_per_step"], "parts_ms": post["config"]["ms"],
+        "GB/s": post["value"], "frac_hbm": post["roofline"]["frac"],
+        "cpu_baseline": post.get("cpu_baseline"),
+    }
+    result["other_configs"] = others
     print(json.dumps(result))
 
 
