@@ -27,11 +27,52 @@ def dtype_id(dtype: torch.dtype) -> int:
         ) from None
 
 
+# Shape inference ("fake" / meta kernels, what torch.compile and torch.library.opcheck ask an
+# op for) runs the op's own Python with the launches left out: inside `_shapes_only()` pointers
+# and the stream are null, every entry point returns 0 (the OK status; as a workspace size: no
+# workspace) without being called, and sizes may be symbolic.
+_SHAPES_ONLY = [0]
+
+
+class _NoLaunch:
+    """Stands in for the library while shapes are inferred: every entry point is ``lambda *a: 0``."""
+
+    def __getattr__(self, name):
+        return lambda *args: 0
+
+
+def _lib():
+    return _NoLaunch() if _SHAPES_ONLY[0] else L.load()
+
+
+def _shapes_only(fn):
+    """``fn`` as a fake kernel: same outputs (shapes, dtypes, devices), nothing launched."""
+    def fake(*args, **kwargs):
+        _SHAPES_ONLY[0] += 1
+        try:
+            return fn(*args, **kwargs)
+        finally:
+            _SHAPES_ONLY[0] -= 1
+    return fake
+
+
 def _ptr(tensor: Optional[Tensor]):
-    return None if tensor is None else c_void_p(tensor.data_ptr())
+    if tensor is None or _SHAPES_ONLY[0]:
+        return None
+    return c_void_p(tensor.data_ptr())
+
+
+def _ref(struct):
+    return None if struct is None else byref(struct)
+
+
+def _aligned16(tensor: Tensor) -> bool:
+    return bool(_SHAPES_ONLY[0]) or tensor.data_ptr() % 16 == 0
 
 
 def _stream():
+    if _SHAPES_ONLY[0]:
+        return None
     # the raw handle of torch's current stream, without building a Stream object per launch
     return c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))  # pylint: disable=protected-access
 
@@ -50,7 +91,7 @@ def _vector_aligned(tensor: Tensor) -> Tensor:
     """``tensor`` itself if its rows start on 16-byte boundaries, else a fresh contiguous copy (the
     MFMA kernels load whole 16-byte vectors; with operands in the padded tile layout there is no
     other kernel to fall back to)."""
-    if tensor.data_ptr() % 16 == 0 and (_ld(tensor) * tensor.element_size()) % 16 == 0:
+    if _aligned16(tensor) and (_ld(tensor) * tensor.element_size()) % 16 == 0:
         return tensor
     return tensor.clone(memory_format=torch.contiguous_format)
 
@@ -154,18 +195,18 @@ def noise_state(device: torch.device, create: bool = True) -> Optional[Tensor]:
 
 def seed_advance(state: Tensor, delta: int) -> None:
     """``state[1] += delta`` on the device (one small launch on the current stream)."""
-    L.check(L.load().ahl_seed_advance(_ptr(state), int(delta), _stream()), "ahl_seed_advance")
+    L.check(_lib().ahl_seed_advance(_ptr(state), int(delta), _stream()), "ahl_seed_advance")
 
 
 def tile_stride(k_in: int, n_tiles: int, dtype: torch.dtype) -> int:
     """Column stride of the padded tile layout the fast kernels want for this split, or 0 when
     the dense layout already suits them (host arithmetic in the library)."""
-    return int(L.load().ahl_tile_stride(k_in, n_tiles, dtype_id(dtype)))
+    return int(_lib().ahl_tile_stride(k_in, n_tiles, dtype_id(dtype)))
 
 
 def pad_tiles(x: Tensor, in_sizes: List[int], stride: int) -> Tensor:
     """Dense ``[rows, K]`` to the padded tile layout ``[rows, T * stride]``."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     rows, k_in = x.shape
     n_tiles = len(in_sizes)
@@ -178,7 +219,7 @@ def pad_tiles(x: Tensor, in_sizes: List[int], stride: int) -> Tensor:
 
 def unpad_tiles(x: Tensor, in_sizes: List[int], stride: int) -> Tensor:
     """Padded tile layout ``[rows, T * stride]`` back to dense ``[rows, K]``."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     rows, k_in, n_tiles = x.size(0), sum(in_sizes), len(in_sizes)
     out = torch.empty((rows, k_in), dtype=x.dtype, device=x.device)
@@ -193,6 +234,8 @@ def conv_geom(geom: List[int]) -> L.AhlConvGeom:
     geometry struct."""
     if len(geom) != 17:
         raise HipBackendError(f"a convolution geometry has 17 integers, got {len(geom)}")
+    if _SHAPES_ONLY[0]:
+        return None
     out = L.AhlConvGeom()
     out.batch, out.channels = int(geom[0]), int(geom[1])
     for i in range(3):
@@ -206,14 +249,17 @@ def conv_geom(geom: List[int]) -> L.AhlConvGeom:
 
 def conv_out_size(geom: List[int]) -> List[int]:
     """Output extents (3) of a convolution geometry; host arithmetic in the library."""
+    if _SHAPES_ONLY[0]:   # the same formula on what may be symbolic sizes
+        return [(geom[2 + i] + 2 * geom[11 + i] - geom[14 + i] * (geom[5 + i] - 1) - 1) // geom[8 + i] + 1
+                for i in range(3)]
     out = (L.c_int32 * 3)()
-    L.check(L.load().ahl_conv_out_size(byref(conv_geom(geom)), out), "ahl_conv_out_size")
+    L.check(_lib().ahl_conv_out_size(byref(conv_geom(geom)), out), "ahl_conv_out_size")
     return [int(v) for v in out]
 
 
 def im2col(x: Tensor, geom: List[int]) -> Tensor:
     """Patches ``[B, L, C * kD * kH * kW]`` of ``x [B, C, D, H, W]``."""
-    lib = L.load()
+    lib = _lib()
     x = x.contiguous()
     cgeom = conv_geom(geom)
     if x.numel() != geom[0] * geom[1] * geom[2] * geom[3] * geom[4]:
@@ -222,14 +268,14 @@ def im2col(x: Tensor, geom: List[int]) -> Tensor:
     n_pos = out_size[0] * out_size[1] * out_size[2]
     k_in = geom[1] * geom[5] * geom[6] * geom[7]
     cols = torch.empty((geom[0], n_pos, k_in), dtype=x.dtype, device=x.device)
-    L.check(lib.ahl_im2col(_ptr(x), byref(cgeom), dtype_id(x.dtype), _ptr(cols), k_in, _stream()),
+    L.check(lib.ahl_im2col(_ptr(x), _ref(cgeom), dtype_id(x.dtype), _ptr(cols), k_in, _stream()),
             "ahl_im2col")
     return cols
 
 
 def col2im(dcols: Tensor, geom: List[int]) -> Tensor:
     """Adjoint of :func:`im2col`: ``[B, L, K]`` patch gradients to ``[B, C, D, H, W]``."""
-    lib = L.load()
+    lib = _lib()
     dcols = dcols.contiguous()
     cgeom = conv_geom(geom)
     out_size = conv_out_size(geom)
@@ -238,14 +284,14 @@ def col2im(dcols: Tensor, geom: List[int]) -> Tensor:
         raise HipBackendError(f"patches of shape {tuple(dcols.shape)} do not match geometry {geom}")
     dx = torch.empty((geom[0], geom[1], geom[2], geom[3], geom[4]), dtype=dcols.dtype,
                      device=dcols.device)
-    L.check(lib.ahl_col2im(_ptr(dcols), k_in, byref(cgeom), dtype_id(dcols.dtype), _ptr(dx),
+    L.check(lib.ahl_col2im(_ptr(dcols), k_in, _ref(cgeom), dtype_id(dcols.dtype), _ptr(dx),
                            _stream()), "ahl_col2im")
     return dx
 
 
 def transpose_batched(src: Tensor) -> Tensor:
     """``dst[b, c, r] = src[b, r, c]`` as a new contiguous tensor."""
-    lib = L.load()
+    lib = _lib()
     if src.dim() != 3:
         raise HipBackendError(f"transpose_batched takes a 3-D tensor, got {tuple(src.shape)}")
     src = src.contiguous()
@@ -259,7 +305,7 @@ def transpose_batched(src: Tensor) -> Tensor:
 
 def sliced_absmax(x: Tensor, in_sizes: List[int], tile_stats: bool) -> Tuple[Tensor, Tensor, Tensor]:
     """``out[t, r] = max |x[r, tile t]|`` (+ per-tile max/min over rows)."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     n_tiles, rows = len(in_sizes), x.size(0)
     out = torch.empty((n_tiles, rows), dtype=x.dtype, device=x.device)
@@ -279,7 +325,7 @@ def sliced_absmax(x: Tensor, in_sizes: List[int], tile_stats: bool) -> Tuple[Ten
 
 def sliced_std(x: Tensor, in_sizes: List[int]) -> Tensor:
     """Unbiased std of every K-tile over all rows, float32 ``[T]``."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     n_tiles = len(in_sizes)
     out = torch.empty((n_tiles,), dtype=torch.float32, device=x.device)
@@ -297,7 +343,7 @@ def sliced_std(x: Tensor, in_sizes: List[int]) -> Tensor:
 
 def row_nonzero(x: Tensor) -> Tensor:
     """uint8 ``[rows]``: 1 for every row of ``x`` that is not all zero."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     kept = torch.empty((x.size(0),), dtype=torch.uint8, device=x.device)
     count = torch.empty((1,), dtype=torch.int32, device=x.device)
@@ -311,7 +357,7 @@ def row_nonzero(x: Tensor) -> Tensor:
 
 def sliced_std_kept(x: Tensor, in_sizes: List[int]) -> Tensor:
     """Unbiased std of every K-tile over the rows that are not all zero, float32 ``[T]``."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     n_tiles = len(in_sizes)
     out = torch.empty((n_tiles,), dtype=torch.float32, device=x.device)
@@ -330,7 +376,7 @@ def sliced_std_kept(x: Tensor, in_sizes: List[int]) -> Tensor:
 def sliced_quantile(x: Tensor, in_sizes: List[int], q: float) -> Tensor:
     """``torch.quantile(x[kept rows, tile].float().flatten(), q)`` of every K-tile, float32
     ``[T]``; kept rows are those that are not all zero."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     n_tiles = len(in_sizes)
     out = torch.empty((n_tiles,), dtype=torch.float32, device=x.device)
@@ -348,7 +394,7 @@ def sliced_quantile(x: Tensor, in_sizes: List[int], q: float) -> Tensor:
 
 def ir_moving_update(ir: Tensor, idx: Tensor, val: Tensor, alpha: float, val_in_dtype: bool) -> None:
     """In-place moving-average step of the calibrated ranges; ``idx`` is int32 ``[T]``."""
-    lib = L.load()
+    lib = _lib()
     if not (ir.is_contiguous() and idx.is_contiguous() and idx.dtype == torch.int32
             and val.dtype == torch.float32 and val.is_contiguous()):
         raise HipBackendError("ir_moving_update: contiguous ir, int32 idx and float32 val expected")
@@ -361,7 +407,7 @@ def ir_moving_update(ir: Tensor, idx: Tensor, val: Tensor, alpha: float, val_in_
 
 def ir_init_update(ir: Tensor, idx: Tensor, std: Tensor, init_from_data: float, alpha: float) -> None:
     """In-place input-range initialisation step from the per-tile std."""
-    lib = L.load()
+    lib = _lib()
     if not (ir.is_contiguous() and idx.is_contiguous() and ir.dtype == idx.dtype):
         raise HipBackendError("input_range and input_range_update_idx must be contiguous, same dtype")
     L.check(
@@ -375,7 +421,7 @@ def ir_init_update(ir: Tensor, idx: Tensor, std: Tensor, init_from_data: float, 
 
 def running_absmax(x: Tensor, in_sizes: List[int], cache: Tensor) -> None:
     """``cache[t] = max(cache[t], max |x[:, tile t]|)``; cache is float32 ``[T]`` on the device."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     if cache.dtype != torch.float32 or not cache.is_contiguous() or cache.numel() != len(in_sizes):
         raise HipBackendError("cache must be a contiguous float32 tensor with one entry per tile")
@@ -391,7 +437,7 @@ def running_absmax(x: Tensor, in_sizes: List[int], cache: Tensor) -> None:
 def ir_fast_update(x: Tensor, in_sizes: List[int], ir: Tensor, idx: Tensor, x_min: Tensor,
                    x_max: Tensor, init_from_data: float, momentum: float) -> None:
     """In-place fast_mode update of the running min / max, the step counter and the range."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     for buf in (ir, idx, x_min, x_max):
         if not (buf.is_contiguous() and buf.dtype == x.dtype and buf.numel() == len(in_sizes)):
@@ -411,7 +457,7 @@ def ir_fast_update(x: Tensor, in_sizes: List[int], ir: Tensor, idx: Tensor, x_mi
 
 def clip_weights(w: Tensor, sigma: float, kind: int) -> None:
     """In-place clamp of ``w`` at ``sigma`` standard deviations (per matrix or per row)."""
-    lib = L.load()
+    lib = _lib()
     if w.dim() != 2 or w.stride(1) != 1:
         raise HipBackendError("weight must be a row-major 2-D tensor")
     ws = torch.empty((lib.ahl_clip_weights_ws_bytes(w.size(0)),), dtype=torch.uint8, device=w.device)
@@ -425,7 +471,7 @@ def clip_weights(w: Tensor, sigma: float, kind: int) -> None:
 
 def col_sum(x: Tensor) -> Tensor:
     """Column sums of a 2-D tensor in its dtype (float accumulation)."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     out = torch.empty((x.size(1),), dtype=x.dtype, device=x.device)
     ws = torch.empty((lib.ahl_col_sum_ws_bytes(x.size(1)),), dtype=torch.uint8, device=x.device)
@@ -459,7 +505,7 @@ def weight_prep(
 ) -> Tuple[Tensor, Tensor, Tensor, Tensor]:
     """wmax ``[T, N]``, tile max/min ``[T]`` and, if wanted, the modified copy ``[N, K]``.
     ``skip_tile_stats``: the caller does not use tile max/min (they may come back unwritten)."""
-    lib = L.load()
+    lib = _lib()
     if w.dim() != 2 or w.stride(1) != 1:
         raise HipBackendError("weight must be a row-major 2-D tensor")
     n_out, n_in = w.shape
@@ -487,7 +533,7 @@ def weight_prep_clip(
 ) -> Tuple[Tensor, Tensor, Tensor]:
     """Weights under a learnable per-channel clip ``clip [T, N]`` (which also takes the place of
     the per-tile abs-max): tile max/min of the clip and the clipped (+ quantised, + noisy) copy."""
-    lib = L.load()
+    lib = _lib()
     if w.dim() != 2 or w.stride(1) != 1:
         raise HipBackendError("weight must be a row-major 2-D tensor")
     n_out, n_in = w.shape
@@ -513,7 +559,7 @@ def learned_clip_bwd(dw: Tensor, w: Tensor, clip: Tensor, tile_min: Tensor, in_s
                      quant_type: int, res: float) -> Tensor:
     """LSQ backward of the learnable clip: ``dw`` (gradient w.r.t. the clipped weights) becomes
     the gradient w.r.t. the weights in place; returns the gradient of the clip ``[T, N]``."""
-    lib = L.load()
+    lib = _lib()
     if dw.stride(1) != 1 or w.stride(1) != 1:
         raise HipBackendError("weight and its gradient must be row-major")
     n_out, n_in = w.shape
@@ -531,7 +577,7 @@ def learned_clip_bwd(dw: Tensor, w: Tensor, clip: Tensor, tile_min: Tensor, in_s
 
 def quantize_weights(w: Tensor, in_sizes: List[int], quant_type: int, res: float) -> None:
     """In-place per-tile weight quantisation with scales from each slice's own abs-max."""
-    lib = L.load()
+    lib = _lib()
     if w.dim() != 2 or w.stride(1) != 1:
         raise HipBackendError("weight must be a row-major 2-D tensor")
     n_tiles = len(in_sizes)
@@ -550,7 +596,7 @@ def quantize_weights(w: Tensor, in_sizes: List[int], quant_type: int, res: float
 def dac(x: Tensor, ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
         fcfg: List[float]) -> Tuple[Tensor, Tensor]:
     """Clamp + DAC pre-pass: returns ``xq [M, K]`` and, in dynamic mode, the ranges ``[T, M]``."""
-    lib = L.load()
+    lib = _lib()
     x = _rows2d(x, "x")
     m_rows, k_in = x.shape
     n_tiles = len(in_sizes)
@@ -573,7 +619,7 @@ def dac(x: Tensor, ir: Optional[Tensor], in_sizes: List[int], icfg: List[int],
 @lru_cache(maxsize=4096)
 def _fwd_ws_bytes(m_rows: int, k_in: int, n_out: int, n_tiles: int, dtype: int) -> int:
     """The library's answer per shape (host arithmetic there; asked once per shape here)."""
-    return int(L.load().ahl_linear_fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, dtype))
+    return int(_lib().ahl_linear_fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, dtype))
 
 
 # Hand the forward a workspace for calls of few rows (one K-tile per block, summed in tile order
@@ -588,7 +634,7 @@ def linear_fwd(
 ) -> Tuple[Tensor, Tensor, Tensor]:
     """The analog forward; returns ``y [M, N]``, the clamp mask (empty if not wanted) and the
     one-word "anything clamped" flag."""
-    lib = L.load()
+    lib = _lib()
     ref = x if x is not None else xq
     if x is not None:
         x = _rows2d(x, "x")
@@ -603,9 +649,11 @@ def linear_fwd(
     # rows padded to a multiple of 64 (the kernels never write or use the padding rows)
     keep = torch.empty((n_tiles, (n_out + 31) // 32, (m_rows + 63) // 64 * 64) if want_keep else (0,),
                        dtype=torch.int32, device=ref.device)
+    if want_keep and m_rows % 64 != 0:
+        keep[:, :, m_rows:].zero_()   # the padding rows: defined contents for whoever compares masks
     flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
     ws_bytes = 0
-    if xq is not None and SPLIT_FEW_ROW_FORWARD:
+    if xq is not None and SPLIT_FEW_ROW_FORWARD and not _SHAPES_ONLY[0]:
         ws_bytes = _fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=ref.device) if ws_bytes else None
     L.check(
@@ -626,7 +674,7 @@ def linear_bwd_dx(
     fcfg: List[float],
 ) -> Tuple[Tensor, Tensor]:
     """Input gradient ``[M, K]`` and input-range gradient ``[T]`` (empty unless static range)."""
-    lib = L.load()
+    lib = _lib()
     g = _rows2d(g, "g")
     m_rows, n_out = g.shape
     k_in = sum(in_sizes)
@@ -642,7 +690,7 @@ def linear_bwd_dx(
                      dtype=torch.uint8, device=g.device)
     if x is not None:
         x = _rows2d(x, "x")
-        if cfg.tile_stride > 0 and (x.data_ptr() % 16 != 0 or _ld(x) != k_in):
+        if cfg.tile_stride > 0 and (not _aligned16(x) or _ld(x) != k_in):
             x = x.clone(memory_format=torch.contiguous_format)  # same row stride and alignment as dx
     L.check(
         lib.ahl_linear_bwd_dx(
@@ -663,7 +711,7 @@ def linear_bwd_dw(
 ) -> Tuple[Tensor, Tensor]:
     """Weight gradient ``[N, K]`` from the raw input ``x`` or the saved quantised input ``xq``,
     and (if wanted, else empty) the bias gradient ``[N]``, the column sums of ``g``."""
-    lib = L.load()
+    lib = _lib()
     g = _rows2d(g, "g")
     ref = xq if xq is not None else x
     if x is not None:
@@ -709,7 +757,7 @@ def dense(tensor: Optional[Tensor]) -> Optional[Tensor]:
     """``tensor`` as a dense, 16-byte aligned matrix (itself if it already is one)."""
     if tensor is None:
         return None
-    if not tensor.is_contiguous() or tensor.data_ptr() % 16 != 0:
+    if not tensor.is_contiguous() or not _aligned16(tensor):
         tensor = tensor.clone(memory_format=torch.contiguous_format)
     return tensor
 
@@ -717,7 +765,7 @@ def dense(tensor: Optional[Tensor]) -> Optional[Tensor]:
 def lstm_gates_fwd(igates: Tensor, hgates: Optional[Tensor], c_x: Tensor,
                    want_act: bool) -> Tuple[Tensor, Tensor, Optional[Tensor]]:
     """``(h_y, c_y, activated gates or None)`` of an LSTM step."""
-    lib = L.load()
+    lib = _lib()
     igates, hgates, c_x = dense(igates), dense(hgates), dense(c_x)
     rows, hidden = c_x.shape
     h_y, c_y = torch.empty_like(c_x), torch.empty_like(c_x)
@@ -731,7 +779,7 @@ def lstm_gates_fwd(igates: Tensor, hgates: Optional[Tensor], c_x: Tensor,
 def lstm_gates_bwd(dh_y: Tensor, dc_y: Optional[Tensor], act: Tensor, c_x: Tensor,
                    c_y: Tensor) -> Tuple[Tensor, Tensor]:
     """``(dgates [rows, 4H], dc_x)``."""
-    lib = L.load()
+    lib = _lib()
     dh_y, dc_y = dense(dh_y), dense(dc_y)
     rows, hidden = c_x.shape
     dgates, dc_x = torch.empty_like(act), torch.empty_like(c_x)
@@ -745,7 +793,7 @@ def lstm_gates_bwd(dh_y: Tensor, dc_y: Optional[Tensor], act: Tensor, c_x: Tenso
 def gru_gates_fwd(igates: Tensor, hgates: Tensor, h_x: Tensor,
                   want_act: bool) -> Tuple[Tensor, Optional[Tensor]]:
     """``(h_y, (reset, update, new) or None)`` of a GRU step."""
-    lib = L.load()
+    lib = _lib()
     igates, hgates, h_x = dense(igates), dense(hgates), dense(h_x)
     rows, hidden = h_x.shape
     h_y = torch.empty_like(h_x)
@@ -759,7 +807,7 @@ def gru_gates_fwd(igates: Tensor, hgates: Tensor, h_x: Tensor,
 def gru_gates_bwd(dh_y: Tensor, act: Tensor, hgates: Tensor,
                   h_x: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
     """``(digates, dhgates [rows, 3H], dh_x)``."""
-    lib = L.load()
+    lib = _lib()
     dh_y = dense(dh_y)
     rows, hidden = h_x.shape
     digates, dhgates, dh_x = torch.empty_like(act), torch.empty_like(act), torch.empty_like(h_x)
@@ -783,5 +831,6 @@ for _name, _fn in [
     ("dac", dac), ("linear_fwd", linear_fwd), ("linear_bwd_dx", linear_bwd_dx), ("linear_bwd_dw", linear_bwd_dw),
 ]:
     LIB.impl(_name, _fn, "CUDA")
+    torch.library.register_fake(f"aihwkit_hip::{_name}", _shapes_only(_fn), lib=LIB)
 
 OPS = torch.ops.aihwkit_hip

@@ -116,6 +116,11 @@ class TiledAnalogLayer(AnalogLayerBase):
         finally:
             self._weight_cache = outer
 
+    # torch.compile does not trace into the operator: its host side draws seeds, keeps per-layer
+    # state and calls the library through ctypes. It runs as an opaque eager call between the
+    # compiled parts of a model (the custom ops it is made of carry fake kernels for callers
+    # that trace them directly).
+    @torch.compiler.disable
     def analog_mvm(self, rows: Tensor) -> Tensor:
         """``rows[..., in] @ weight_matrix^T + bias`` through the analog tile model."""
         init_active = self.training and self._init_phase_active()

@@ -390,3 +390,36 @@ def test_module_level_helpers_of_the_reference_exist():
             conv.unfold3d(torch.zeros(1, 1, 2, 2, 2), (1, 1, 1))
     with pytest.raises(ValueError):
         conv.unfold3d(torch.zeros(2, 2), (1, 1, 1))
+
+
+def test_fake_kernels_give_shapes_without_a_gpu():
+    """Every custom op has a fake kernel (what torch.compile and opcheck trace with): under
+    FakeTensorMode the ops return tensors of the right shape, dtype and device and launch nothing."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    from aihwkit_lightning.nn.modules.hip_utils import library as L
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+
+    in_sizes = [256, 256]
+    icfg = [L.AHL_IR_DYNAMIC, 0, 1, 0, 0, 0, 0]
+    fcfg = [254.0, 254.0, 0.5, 0.0, 0.01, 0.95]
+    with FakeTensorMode():
+        x = torch.empty(64, 512, device="cuda", dtype=torch.bfloat16)
+        w = torch.empty(96, 512, device="cuda", dtype=torch.bfloat16)
+        wmax, tile_max, tile_min, w_eff = OPS.weight_prep(w, in_sizes, 0, 2, 1.0, 0.02, 3, 0, True)
+        assert wmax.shape == (2, 96) and tile_max.shape == (2,) and tile_min.dtype == torch.float32
+        assert w_eff.shape == w.shape and w_eff.dtype == w.dtype
+        xq, ir_dyn = OPS.dac(x, None, in_sizes, icfg, fcfg)
+        assert xq.shape == x.shape and ir_dyn.shape == (2, 64)
+        y, keep, flag = OPS.linear_fwd(x, xq, w_eff, None, ir_dyn, wmax, tile_max, in_sizes, icfg, fcfg, True)
+        assert y.shape == (64, 96) and y.device.type == "cuda" and keep.shape == (2, 3, 64) and flag.shape == (1,)
+        dx, ir_grad = OPS.linear_bwd_dx(y, keep, flag, w_eff, x, ir_dyn, in_sizes, icfg, fcfg)
+        assert dx.shape == x.shape and ir_grad.numel() == 0
+        dw, db = OPS.linear_bwd_dw(y, keep, flag, x, xq, ir_dyn, in_sizes, icfg, fcfg, True)
+        assert dw.shape == w.shape and db.shape == (96,)
+        assert OPS.sliced_std(x.float(), in_sizes).shape == (2,)
+        assert OPS.sliced_quantile(x.float(), in_sizes, 0.99).shape == (2,)
+        assert OPS.pad_tiles(x, [200, 312], 512).shape == (64, 1024)
+        geom = [2, 8, 1, 12, 12, 1, 3, 3, 1, 1, 1, 0, 1, 1, 1, 1, 1]
+        cols = OPS.im2col(torch.empty(2, 8, 1, 12, 12, device="cuda"), geom)
+        assert cols.shape == (2, 144, 72) and OPS.col2im(cols, geom).shape == (2, 8, 1, 12, 12)
