@@ -42,7 +42,10 @@ def _tile_rows(mod, args: Tuple, kwargs: Dict) -> Tensor:
 def _calibration_pre_forward(mod, args: Tuple, kwargs: Dict, calibration_type, cache: Dict,
                              key: str, max_samples: int, ir_quantile: float) -> None:
     """Forward pre-hook: fold this batch into the layer's calibration state (reference
-    ``calibration.py:57-152``). Everything stays on the device; nothing synchronises."""
+    ``calibration.py:57-152``). Everything stays on the device. ``MAX`` and the two moving
+    strategies never wait for it; ``CACHE_QUANTILE`` does once per batch (the number of rows
+    that are not all zero decides a tensor shape) and keeps up to ``max_samples`` fp32 rows of
+    ``in_features`` values per layer in device memory, where the reference keeps them on the host."""
     x_input = _tile_rows(mod, args, kwargs)
     if x_input.size(0) == 0:
         return
@@ -157,7 +160,7 @@ def calibrate_input_ranges(
         weight = layer.weight
         config = saved_configs[name]
         layer.input_range_update_idx = Parameter(
-            torch.full((len(layer.in_sizes),), float("-inf"), device=weight.device),
+            torch.full((len(layer.in_sizes),), float("-inf"), device=weight.device, dtype=weight.dtype),
             requires_grad=False,
         )
         if not moving:

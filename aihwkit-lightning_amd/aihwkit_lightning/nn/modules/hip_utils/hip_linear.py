@@ -256,7 +256,13 @@ class HipLinear(Function):
             float(fwd.out_noise) if noise_on else 0.0, float(ir_params.decay),
             float(ir_params.input_min_percentage),
         ]
-        if m_rows == 0:
+        ctx.empty = m_rows == 0
+        if ctx.empty:
+            # no rows: zero gradients for everything that asks for one (the reference returns
+            # zeros here too, e.g. for a routed expert that received no token in a step)
+            ctx.zero_like = [t if (t is not None and need) else None for t, need in zip(
+                (inp, weights, bias, input_range, learnable_weight_clip),
+                (ctx.needs_input_grad[i] for i in (0, 1, 2, 3, 11)))]
             return inp.new_zeros(out_shape)
 
         # bf16 with equal tiles of a multiple of 64 inputs: clamp + DAC (+ dynamic abs-max) run as
@@ -326,6 +332,10 @@ class HipLinear(Function):
 
     @staticmethod
     def backward(ctx, grad_out: Tensor):
+        if ctx.empty:
+            d_inp, d_w, d_b, d_ir, d_clip = (None if t is None else torch.zeros_like(t)
+                                             for t in ctx.zero_like)
+            return (d_inp, d_w, d_b, d_ir, None, None, None, None, None, None, None, d_clip, None)
         x2, xq, w_eff, keep, flag, ir_dev, w_plain, clip, clip_tile_min = ctx.saved_tensors
         n_out = grad_out.size(-1)
         g2 = grad_out.reshape(-1, n_out)

@@ -744,13 +744,24 @@ def linear_bwd_dw(
 # ---------------------------------------------------------------------------------------------
 # Gate arithmetic of the recurrent cells (called from the cells' autograd functions directly; no
 # dispatcher entry: they are internal to those functions)
-def gates_supported(*tensors: Tensor) -> bool:
-    """Whether the fused gate kernels can take these operands: on the GPU, float32 / bfloat16,
-    hidden size (last dimension of the last tensor) in whole 16-byte vectors."""
-    ref = tensors[-1]
-    if not ref.is_cuda or ref.dtype not in _DTYPES or ref.dim() != 2:
+def gates_supported(igates: Tensor, hgates: Optional[Tensor], state: Tensor, n_gates: int) -> bool:
+    """Whether the fused gate kernels can take these operands: everything on one GPU in one of
+    float32 / bfloat16, ``state [rows, hidden]`` with the hidden size in whole 16-byte vectors,
+    the projections ``[rows, n_gates * hidden]``. (The kernels read raw pointers: a projection
+    in another dtype or shape than the state would be read out of bounds; such calls take the
+    torch formula, which type-promotes.)"""
+    if not state.is_cuda or state.dtype not in _DTYPES or state.dim() != 2 or state.size(0) == 0:
         return False
-    return ref.size(1) % (16 // ref.element_size()) == 0 and ref.size(0) > 0
+    rows, hidden = state.shape
+    if hidden % (16 // state.element_size()) != 0:
+        return False
+    for gates in (igates, hgates):
+        if gates is None:
+            continue
+        if (gates.device != state.device or gates.dtype != state.dtype
+                or tuple(gates.shape) != (rows, n_gates * hidden)):
+            return False
+    return True
 
 
 def dense(tensor: Optional[Tensor]) -> Optional[Tensor]:

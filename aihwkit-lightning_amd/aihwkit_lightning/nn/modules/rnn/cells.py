@@ -71,7 +71,7 @@ def lstm_pointwise(igates: Tensor, hgates: Optional[Tensor], c_x: Tensor) -> Tup
     """``(h_y, c_y)`` from the pre-activations ``[B, 4H]`` of the input product and (if there are
     two products) the hidden product, gate blocks in the order input, forget, cell, output
     (reference cells.py:176-186). One fused kernel where the operands allow it."""
-    if gate_ops.gates_supported(igates, c_x):
+    if gate_ops.gates_supported(igates, hgates, c_x, 4):
         return _LstmGates.apply(igates, hgates, c_x)
     gates = igates if hgates is None else igates + hgates
     in_gate, forget_gate, cell_gate, out_gate = gates.chunk(4, 1)
@@ -83,7 +83,7 @@ def gru_pointwise(igates: Tensor, hgates: Tensor, h_x: Tensor) -> Tensor:
     """New hidden state from the pre-activations ``[B, 3H]`` of the two products, gate blocks in
     the order reset, update, new; the reset gate scales the hidden part of the candidate after
     the product (reference cells.py:321-343). One fused kernel where the operands allow it."""
-    if gate_ops.gates_supported(igates, h_x):
+    if gate_ops.gates_supported(igates, hgates, h_x, 3):
         return _GruGates.apply(igates, hgates, h_x)
     i_r, i_z, i_n = igates.chunk(3, 1)
     h_r, h_z, h_n = hgates.chunk(3, 1)

@@ -3,6 +3,7 @@ input dimension: ``AnalogLinear`` directly, the convolution layers through their
 ``weight.view(out_channels, -1)``. Tile split, input-range state, the call into the HIP
 operator, weight clipping and post-training quantisation follow the reference
 (``nn/modules/linear.py:53-317``, ``nn/modules/conv.py:121-367``)."""
+import math
 from contextlib import contextmanager
 from copy import deepcopy
 from typing import List, Optional, Tuple
@@ -95,7 +96,9 @@ class TiledAnalogLayer(AnalogLayerBase):
             return False
         if self._ir_init_active is None or self._ir_init_calls >= ir_params.init_from_data:
             idx_min = float(self.input_range_update_idx.min().item())
-            self._ir_init_active = idx_min < ir_params.init_from_data
+            # a counter that is not finite (calibration leaves -inf, calibration.py:159) means
+            # "the ranges are set": the initialisation from data is over
+            self._ir_init_active = math.isfinite(idx_min) and idx_min < ir_params.init_from_data
             self._ir_init_calls = int(idx_min) if self._ir_init_active else 0
         return bool(self._ir_init_active)
 
@@ -220,7 +223,19 @@ class TiledAnalogLayer(AnalogLayerBase):
         ``base.py:208-212``)."""
         check_supported(self.rpu_config)
         quant_type = self.rpu_config.modifier.quantization_type
-        if quant_type != WeightQuantizationType.NONE:
+        if self.rpu_config.clip.type == WeightClipType.LEARNABLE_PER_CHANNEL:
+            # the learned clip is the clamp (no quantiser) or the quantiser's range: what the
+            # training forward applies on the fly, written back (quant_utils.py:184-233)
+            assert self.learnable_weight_clip is not None, "learnable_weight_clip should not be None"
+            self._require_device("quantize_weights")
+            quantised = QUANT_IDS[quant_type] != L.AHL_QUANT_NONE
+            w_new = OPS.weight_prep_clip(
+                self.weight_matrix().data, self.learnable_weight_clip.data, self.in_sizes,
+                L.AHL_QUANT_DISCRETIZE_PER_CHANNEL if quantised else L.AHL_QUANT_CLIP_LEARNED,
+                L.AHL_NOISE_NONE, float(self.rpu_config.modifier.res) if quantised else 1.0, 0.0, 0, 0,
+            )[2]
+            self.weight_matrix().data.copy_(w_new)
+        elif quant_type != WeightQuantizationType.NONE:
             self._require_device("quantize_weights")
             OPS.quantize_weights(
                 self.weight_matrix().data, self.in_sizes, QUANT_IDS[quant_type],

@@ -378,13 +378,19 @@ def clip_weights(weights: Tensor, sigma: float, per_channel: bool) -> Tensor:
     return torch.clamp(weights, -bound, bound)
 
 
-def quantize_weights(weights: Tensor, in_sizes: Sequence[int], kind: str, res: float) -> Tensor:
-    """Post-training per-tile quantisation with the slice's own abs-max
-    (nn/modules/linear.py:285-303). Returns a new tensor."""
+def quantize_weights(weights: Tensor, in_sizes: Sequence[int], kind: str, res: float,
+                     learnable_clip: Optional[Tensor] = None) -> Tensor:
+    """Post-training per-tile quantisation (nn/modules/linear.py:285-303 -> clip_and_quantize,
+    torch_utils/quant_utils.py:159-236): with the slice's own abs-max, or -- under a learned
+    per-channel clip ``learnable_clip [T, N]`` -- the clamp at the learned clip (no quantiser) /
+    the quantiser whose range is the learned clip. Returns a new tensor."""
     out = weights.clone()
-    for lo, hi in tile_bounds(in_sizes):
+    for t, (lo, hi) in enumerate(tile_bounds(in_sizes)):
         w_t = weights[:, lo:hi]
-        out[:, lo:hi] = quantize_weight_tile(w_t, w_t.abs().amax(dim=1, keepdim=True), kind, res)
+        if learnable_clip is not None:
+            out[:, lo:hi] = learned_clip_tile(w_t, learnable_clip[t].unsqueeze(-1), kind, res)[0]
+        else:
+            out[:, lo:hi] = quantize_weight_tile(w_t, w_t.abs().amax(dim=1, keepdim=True), kind, res)
     return out
 
 

@@ -139,6 +139,21 @@ CASES = [
          weight_quant="discretize_per_channel", modifier_res=31, w_scale=0.5, seed=14),
     case("bf16_quantize_tensor", dtype="bf16", kind="quantize", M=4, K=40, N=24, max_input_size=16,
          weight_quant="discretize", modifier_res=62, w_scale=0.5, seed=14),
+    # post-training quantisation under a learned per-channel clip: the clip alone (the weights
+    # are clamped in place), the clip as the quantiser's range, and clip values above one (the
+    # "all scales above one" switch of the resolution convention)
+    case("f32_quantize_lsq_clip", kind="quantize", M=4, K=40, N=24, max_input_size=16,
+         clip="learnable", lwc_scale=0.6, w_scale=0.5, seed=22),
+    case("bf16_quantize_lsq_clip", dtype="bf16", kind="quantize", M=4, K=40, N=24, max_input_size=16,
+         clip="learnable", lwc_scale=0.6, w_scale=0.5, seed=22),
+    case("f32_quantize_lsq_quant", kind="quantize", M=4, K=40, N=24, max_input_size=16,
+         clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30,
+         w_scale=0.5, seed=23),
+    case("bf16_quantize_lsq_quant", dtype="bf16", kind="quantize", M=4, K=40, N=24,
+         max_input_size=16, clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel",
+         modifier_res=30, w_scale=0.5, seed=23),
+    case("f32_quantize_lsq_clip_big", kind="quantize", M=4, K=32, N=8, max_input_size=16,
+         clip="learnable", lwc_scale=0.6, w_scale=6.0, seed=24),
 ]
 
 CASES_BY_NAME = {c["name"]: c for c in CASES}

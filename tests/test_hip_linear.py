@@ -199,6 +199,14 @@ def test_leading_dims_and_1d_input():
     assert torch.equal(one, flat[0])
     empty = layer(x[:0].cuda())
     assert empty.shape == (0, 48)
+    # no rows, with gradients asked for: zeros for the input and every parameter
+    x_empty = x[:0].cuda().requires_grad_(True)
+    layer.zero_grad(set_to_none=True)
+    layer(x_empty).sum().backward()
+    assert x_empty.grad.shape == x_empty.shape
+    for param in layer.parameters():
+        if param.requires_grad:
+            assert param.grad is not None and not bool(param.grad.any())
 
 
 @pytest.mark.parametrize("name", ["sliced_dx_bf16_clamped", "pad_bf16_384_static_clamped",
@@ -456,3 +464,25 @@ def test_few_row_forward_with_one_tile_per_block_is_bit_identical(rows, ir_mode)
     for got, want, what in zip(results[0], results[1], ("out", "dx", "dw", "db")):
         assert torch.equal(got, want), what
     assert results[0][0].abs().max() > 0
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_counter_left_at_minus_infinity_means_the_ranges_are_set(dtype):
+    """Calibration leaves ``input_range_update_idx`` at -inf (reference calibration.py:159). A
+    training forward of such a layer with ``init_from_data > 0`` -- e.g. after its state was
+    loaded into a fresh layer -- must treat the initialisation as finished: the ranges stay."""
+    from hip_helpers import make_layer
+
+    c = case("minus_inf", dtype=dtype, M=32, K=64, N=16, max_input_size=32, ir_mode="static",
+             init_from_data=10, inp_res=254, seed=33)
+    x, w, b, _ = make_inputs(c)
+    layer = make_layer(c, inputs=(x, w, b, None))
+    layer.input_range.data.fill_(1.5)
+    layer.input_range_update_idx.data.fill_(float("-inf"))
+    state = {k: v.clone() for k, v in layer.state_dict().items()}
+    fresh = make_layer(c, inputs=(x, w, b, None))
+    fresh.load_state_dict(state)
+    fresh.train()
+    out = fresh(x.cuda())
+    assert bool(torch.isfinite(out.float()).all())
+    assert torch.equal(fresh.input_range.data.cpu().float(), torch.full((2,), 1.5))

@@ -158,7 +158,10 @@ def test_clip_weights_per_channel_row_lengths(vectors, dtype):
     assert torch.equal(got[changed].abs(), bound.expand_as(got)[changed])
 
 
-@pytest.mark.parametrize("name", ["f32_quantize_channel", "f32_quantize_odd", "bf16_quantize_tensor"])
+@pytest.mark.parametrize("name", ["f32_quantize_channel", "f32_quantize_odd", "bf16_quantize_tensor",
+                                  "f32_quantize_lsq_clip", "bf16_quantize_lsq_clip",
+                                  "f32_quantize_lsq_quant", "bf16_quantize_lsq_quant",
+                                  "f32_quantize_lsq_clip_big"])
 def test_quantize_weights_matches_reference(name):
     from hip_helpers import make_layer
     from aihwkit_lightning.simulator.configs import WeightQuantizationType, WeightClipType

@@ -265,7 +265,7 @@ def test_fused_gates_match_the_chain_of_torch_operations(dtype, rows, hidden):
     # LSTM, both outputs used
     ig, hg, c_x = mk(rows, 4 * hidden), mk(rows, 4 * hidden), mk(rows, hidden)
     g_h, g_c = mk(rows, hidden).detach(), mk(rows, hidden).detach()
-    assert cells.gate_ops.gates_supported(ig, c_x)
+    assert cells.gate_ops.gates_supported(ig, hg, c_x, 4)
     h_y, c_y = cells.lstm_pointwise(ig, hg, c_x)
     ((h_y * g_h).sum() + (c_y * g_c).sum()).backward()
     got = [t.grad.clone() for t in (ig, hg, c_x)]
@@ -307,4 +307,14 @@ def test_fused_gates_match_the_chain_of_torch_operations(dtype, rows, hidden):
         assert close(a, t.grad)
     # a hidden size that is not a whole number of vectors takes the torch chain
     odd = mk(rows, 6)
-    assert not cells.gate_ops.gates_supported(mk(rows, 24), odd)
+    assert not cells.gate_ops.gates_supported(mk(rows, 24), None, odd, 4)
+    # a state in another dtype than the projections (a user-built state) takes the torch chain
+    # too, which type-promotes, instead of a kernel that would read the projections out of bounds
+    other = torch.float32 if dtype == torch.bfloat16 else torch.bfloat16
+    ig, hg = mk(rows, 4 * hidden).detach(), mk(rows, 4 * hidden).detach()
+    c_other = mk(rows, hidden).detach().to(other)
+    assert not cells.gate_ops.gates_supported(ig, hg, c_other, 4)
+    h_y, c_y = cells.lstm_pointwise(ig, hg, c_other)
+    want_h, want_c = chain_lstm(ig, hg, c_other)
+    assert torch.equal(h_y, want_h) and torch.equal(c_y, want_c)
+    assert not cells.gate_ops.gates_supported(ig[:, :-8], hg, mk(rows, hidden), 4)

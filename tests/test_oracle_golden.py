@@ -2,7 +2,7 @@
 import pytest
 import torch
 
-from golden_cases import CASES, DTYPES, make_inputs
+from golden_cases import CASES, DTYPES, make_inputs, make_learnable_clip
 from helpers import golden, golden_tensor, oracle_cfg, oracle_fwd_bwd, case_input_range
 from oracle import torch_mode as om
 
@@ -90,16 +90,25 @@ def test_clip_weights(name):
     assert not torch.equal(got, w), "the case must actually clip something"
 
 
-@pytest.mark.parametrize("name", ["f32_quantize_channel", "f32_quantize_odd", "bf16_quantize_tensor"])
+QUANTIZE_CASES = ["f32_quantize_channel", "f32_quantize_odd", "bf16_quantize_tensor",
+                  "f32_quantize_lsq_clip", "bf16_quantize_lsq_clip", "f32_quantize_lsq_quant",
+                  "bf16_quantize_lsq_quant", "f32_quantize_lsq_clip_big"]
+
+
+@pytest.mark.parametrize("name", QUANTIZE_CASES)
 def test_quantize_weights(name):
     case = [c for c in CASES if c["name"] == name][0]
     dtype = DTYPES[case["dtype"]]
     x, w, b, _ = make_inputs(case)
     in_sizes = om.split_sizes(case["K"], case["max_input_size"])
-    got = om.quantize_weights(w, in_sizes, case["weight_quant"], case["modifier_res"])
+    lwc = make_learnable_clip(case, w) if case["clip"] == "learnable" else None
+    got = om.quantize_weights(w, in_sizes, case["weight_quant"], case["modifier_res"], lwc)
+    if lwc is not None:
+        assert not torch.equal(got, w), "the case must actually change weights"
     _exact_or_close(got, golden_tensor(f"{name}/w_quantized"), dtype, "quantised weights")
     # the reference switches quantisation off afterwards and evaluates the layer plainly
     cfg = oracle_cfg(case)
     cfg.weight_quant = om.NONE
+    cfg.clip_learnable = cfg.bound_per_channel = False   # ... and the clipping (base.py:208-212)
     out, _ = om.linear_forward(x, got, b, cfg, None, False)
     _exact_or_close(out, golden_tensor(f"{name}/out"), dtype, "output after quantisation")
