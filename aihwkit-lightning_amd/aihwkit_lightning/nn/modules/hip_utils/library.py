@@ -17,7 +17,7 @@ LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "
 ABI_VERSION = 12
 STATIC_DX_SCRATCH_BYTES = 16 * 1024 * 1024
 
-AHL_F32, AHL_BF16 = 0, 1
+AHL_F32, AHL_BF16, AHL_F16 = 0, 1, 2
 AHL_IR_NONE, AHL_IR_STATIC, AHL_IR_DYNAMIC = 0, 1, 2
 AHL_NOISE_NONE, AHL_NOISE_ADD_NORMAL, AHL_NOISE_ADD_NORMAL_PER_CHANNEL = 0, 1, 2
 AHL_QUANT_NONE, AHL_QUANT_DISCRETIZE, AHL_QUANT_DISCRETIZE_PER_CHANNEL = 0, 1, 2

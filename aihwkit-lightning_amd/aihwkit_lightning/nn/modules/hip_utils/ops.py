@@ -14,7 +14,7 @@ from torch import Tensor
 from . import library as L
 from ....exceptions import HipBackendError
 
-_DTYPES = {torch.float32: L.AHL_F32, torch.bfloat16: L.AHL_BF16}
+_DTYPES = {torch.float32: L.AHL_F32, torch.bfloat16: L.AHL_BF16, torch.float16: L.AHL_F16}
 
 
 def dtype_id(dtype: torch.dtype) -> int:
@@ -23,7 +23,7 @@ def dtype_id(dtype: torch.dtype) -> int:
         return _DTYPES[dtype]
     except KeyError:
         raise HipBackendError(
-            f"dtype {dtype} is not supported by the HIP backend (float32 and bfloat16 are)"
+            f"dtype {dtype} is not supported by the HIP backend (float32, bfloat16 and float16 are)"
         ) from None
 
 

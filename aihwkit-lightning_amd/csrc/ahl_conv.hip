@@ -604,6 +604,7 @@ extern "C" int ahl_im2col(const void* x, const AhlConvGeom* geom, int32_t dtype,
   // the tiled kernel addresses the elements of one image with 32-bit offsets
   // and the positions of one image with the fp32-reciprocal division
   const bool small_image = (int64_t)g.C * g.in[0] * g.in[1] * g.in[2] <= 0x3fffffff && g.L < (1 << 22);
+  if (dtype == AHL_F16) dtype = AHL_BF16;   // patch extraction moves 2-byte elements, whatever they hold
   if (dtype == AHL_F32) {
     if (g.K % 4 == 0 && ldc % 4 == 0 && aligned16(cols) && small_image)
       return launch_im2col_tiled<uint32_t>(x, cols, ldc, g, st);
@@ -625,7 +626,7 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
   // tiled kernels: channel groups of 8 whose 8 * kvol patch entries are whole 16-byte vectors;
   // first the plan with 256 pixels per block, then (if its staging area does not fit) 64
   for (int pixels = 256; pixels >= 64; pixels /= 4) {
-    const int epv = dtype == AHL_BF16 ? 8 : 4;
+    const int epv = dtype == AHL_F32 ? 4 : 8;
     const int64_t row_entries = 8 * (int64_t)g.kvol;
     int32_t cpb = 64;
     while (cpb > 8 && cpb / 2 >= g.in[2]) cpb /= 2;
@@ -636,10 +637,10 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
     if (ow_span > g.out[2]) ow_span = g.out[2];
     if (oh_span > g.out[1]) oh_span = g.out[1];
     const int64_t lds_limit = pixels == 256 ? 64 * 1024 : 96 * 1024;
-    const int64_t lds_bytes = (int64_t)g.ker[0] * oh_span * ow_span * row_entries * (dtype == AHL_BF16 ? 2 : 4);
+    const int64_t lds_bytes = (int64_t)g.ker[0] * oh_span * ow_span * row_entries * dtype_bytes(dtype);
     const int64_t w_tiles = cdiv(g.in[2], cpb), h_tiles = cdiv(g.in[1], rpb);
     const int64_t tblocks = (int64_t)g.B * (g.C / 8) * g.in[0] * h_tiles * w_tiles;
-    if ((dtype == AHL_BF16 || dtype == AHL_F32) && g.C % 8 == 0 && row_entries % epv == 0 &&
+    if (dtype_known(dtype) && g.C % 8 == 0 && row_entries % epv == 0 &&
         ldc % epv == 0 && aligned16(dcols) && lds_bytes <= lds_limit && tblocks <= 0x7fffffff &&
         g.in[0] + g.pad[0] < (1 << 22) && g.in[1] + g.pad[1] < (1 << 22) &&
         g.in[2] + g.pad[2] < (1 << 22)) {
@@ -680,6 +681,7 @@ extern "C" int ahl_transpose_batched(const void* src, int64_t ld_src, int32_t dt
       ld_dst < rows)
     return AHL_ERR_ARG;
   hipStream_t st = (hipStream_t)stream;
+  if (dtype == AHL_F16) dtype = AHL_BF16;   // a transposition moves 2-byte elements, whatever they hold
   if (dtype != AHL_F32 && dtype != AHL_BF16) return AHL_ERR_ARG;
   {
     // whole 16-byte vectors on both sides: the vector kernel

@@ -87,6 +87,7 @@ struct F32 {
   static constexpr int kId = 0;
   static constexpr int EPV = 4;
   static constexpr bool kIsBf16 = false;
+  static AHL_DEV float tiny() { return 1.17549435e-38f; }   // torch.finfo(dtype).tiny
   static AHL_DEV float rd(float x) { return x; }
   static AHL_DEV elem to_elem(float x) { return x; }
   static AHL_DEV float load(const void* p, int64_t i) { return ((const float*)p)[i]; }
@@ -109,6 +110,7 @@ struct BF16 {
   static constexpr int kId = 1;
   static constexpr int EPV = 8;
   static constexpr bool kIsBf16 = true;
+  static AHL_DEV float tiny() { return 1.17549435e-38f; }
   static AHL_DEV float rd(float x) { return bf16_bits_to_f32(f32_to_bf16_bits(x)); }
   static AHL_DEV elem to_elem(float x) { return (elem)f32_to_bf16_bits(x); }
   static AHL_DEV float load(const void* p, int64_t i) {
@@ -131,6 +133,51 @@ struct BF16 {
   // x * fl32(1/d) to bf16 gives bit-identical results to rounding fl32(x / d). The caller
   // rounds the returned value with rd().
   static AHL_DEV float div(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
+};
+
+// float16: like bfloat16, every elementwise result is rounded to the tensor dtype (round to
+// nearest even; v_cvt_f16_f32 / v_cvt_f32_f16), 8 elements per 16-byte vector.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+AHL_DEV uint32_t pack_f16x2(float lo, float hi) {
+  f32x2 v = {lo, hi};
+  f16x2 h = __builtin_convertvector(v, f16x2);
+  return __builtin_bit_cast(uint32_t, h);
+}
+AHL_DEV float f16_lo(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[0]; }
+AHL_DEV float f16_hi(uint32_t w) { return (float)__builtin_bit_cast(f16x2, w)[1]; }
+
+struct F16 {
+  typedef uint16_t elem;
+  static constexpr int kId = 2;
+  static constexpr int EPV = 8;
+  static constexpr bool kIsBf16 = false;
+  static AHL_DEV float tiny() { return 6.103515625e-05f; }
+  // The two conversions are written as instructions: left to the compiler, "round the fp32
+  // result of an operation to float16" is merged with the operation into mixed-precision
+  // instructions in some kernels and not in others, and the two forms do not always round alike.
+  static AHL_DEV float rd(float x) {
+    uint32_t h;
+    float r;
+    asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(x));
+    asm("v_cvt_f32_f16 %0, %1" : "=v"(r) : "v"(h));
+    return r;
+  }
+  static AHL_DEV elem to_elem(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
+  static AHL_DEV float load(const void* p, int64_t i) { return (float)((const _Float16*)p)[i]; }
+  static AHL_DEV void store(void* p, int64_t i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
+  static AHL_DEV void unpack(const u32x4& v, float* f) {
+    f[0] = f16_lo(v.x); f[1] = f16_hi(v.x); f[2] = f16_lo(v.y); f[3] = f16_hi(v.y);
+    f[4] = f16_lo(v.z); f[5] = f16_hi(v.z); f[6] = f16_lo(v.w); f[7] = f16_hi(v.w);
+  }
+  static AHL_DEV u32x4 pack(const float* f) {
+    u32x4 v = {pack_f16x2(f[0], f[1]), pack_f16x2(f[2], f[3]), pack_f16x2(f[4], f[5]),
+               pack_f16x2(f[6], f[7])};
+    return v;
+  }
+  // 11-bit significands: the product with an approximate reciprocal can land on the other side
+  // of a rounding boundary, so the IEEE quotient is taken (the caller rounds it with rd()).
+  static AHL_DEV float div(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
 };
 
 static constexpr float kTinyF32 = 1.17549435e-38f;  // finfo(float32).tiny == finfo(bfloat16).tiny
@@ -279,7 +326,7 @@ AHL_DEV Dac make_dac(float ir, float inp_res) {
   Dac d;
   d.ir = ir;
   d.r = inp_res > 0.0f ? quant_step<D>(ir, inp_res) : 1.0f;
-  d.rc = fmaxf(d.r, kTinyF32);
+  d.rc = fmaxf(d.r, D::tiny());
   d.rcp = __fdiv_rn(1.0f, d.rc);
   return d;
 }

@@ -44,6 +44,13 @@ struct Mma<BF16> {
   }
 };
 template <>
+struct Mma<F16> {
+  static AHL_DEV void run(const u32x4& a, const u32x4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                               __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
 struct Mma<F32> {
   static AHL_DEV void run(const u32x4& a, const u32x4& b, f32x16& c) {
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
@@ -258,7 +265,7 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
             B = D::rd(D::rd(ir_t * a.out_bound) * wb);
             if (a.adc_on) {
               r = quant_step<D>(B, a.out_res);
-              rc = fmaxf(r, kTinyF32);
+              rc = fmaxf(r, D::tiny());
               rcp = __fdiv_rn(1.0f, rc);
             }
           }
@@ -291,7 +298,7 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
                     B = D::rd(D::rd(irm * a.out_bound) * wb);
                     if (a.adc_on) {
                       r = quant_step<D>(B, a.out_res);
-                      rc = fmaxf(r, kTinyF32);
+                      rc = fmaxf(r, D::tiny());
                       rcp = __fdiv_rn(1.0f, rc);
                     }
                   }
@@ -683,7 +690,7 @@ static constexpr int kGemmLds = 2 * kChunkLds + 2 * 128 * (int)sizeof(float);
 
 static bool cfg_ok(const AhlLinearCfg* c) {
   if (!c) return false;
-  if (c->dtype != AHL_F32 && c->dtype != AHL_BF16) return false;
+  if (!dtype_known(c->dtype)) return false;
   if (c->ir_mode < 0 || c->ir_mode > 2) return false;
   if (c->ir_grad_rule != AHL_IR_GRAD_LEARNED && c->ir_grad_rule != AHL_IR_GRAD_CLAMP) return false;
   if (c->tile_stride < 0 || c->tile_stride % 256 != 0) return false;
@@ -806,6 +813,7 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
   // this kernel does not track clamping: tell the backward to honour the mask
   if (clamp_flag) hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, s, clamp_flag, 1u);
   if (cfg->dtype == AHL_F32) launch_fwd<F32>(a, cfg->ir_mode, grid, s);
+  else if (cfg->dtype == AHL_F16) launch_fwd<F16>(a, cfg->ir_mode, grid, s);
   else launch_fwd<BF16>(a, cfg->ir_mode, grid, s);
   return check_launch("ahl_linear_fwd");
 }
@@ -833,7 +841,7 @@ static int64_t dx_padded_partial_bytes(int64_t M, int64_t padded) {
 int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
                                    int64_t tile_stride) {
   if (n_tiles <= 0 || K <= 0 || M <= 0 || N <= 0) return 0;
-  const int64_t es = dtype == AHL_BF16 ? 2 : 4;
+  const int64_t es = dtype_bytes(dtype);
   if (tile_stride > 0) {  // the MFMA kernel's workspace; x and dx are used in place
     const int64_t padded = (int64_t)n_tiles * tile_stride;
     const int64_t fast = align256(fast_dx_ws_bytes(M, padded, N));
@@ -923,6 +931,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     hipLaunchKernelGGL((k_transpose<uint16_t>), tgrid, dim3(256), 0, s, (const uint16_t*)w_eff, N, K, ldw, (uint16_t*)wt, N);
   const dim3 grid((unsigned)(mb * nkb));
   if (cfg->dtype == AHL_F32) launch_dx<F32>(a, is_static, grid, s);
+  else if (cfg->dtype == AHL_F16) launch_dx<F16>(a, is_static, grid, s);
   else launch_dx<BF16>(a, is_static, grid, s);
   if (is_static) {
     AHL_DISPATCH_DTYPE(cfg->dtype, {
@@ -992,7 +1001,7 @@ int ahl_linear_bwd_dx_static(const void* g, int64_t ldg, const uint32_t* keep,
 
 int64_t ahl_linear_bwd_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype,
                                    int32_t has_keep, int64_t tile_stride) {
-  const int64_t es = dtype == AHL_BF16 ? 2 : 4;
+  const int64_t es = dtype_bytes(dtype);
   (void)has_keep;
   if (tile_stride > 0) {  // [workspace of the MFMA kernel | dw in the padded tile layout]
     const int64_t padded = (int64_t)n_tiles * tile_stride;

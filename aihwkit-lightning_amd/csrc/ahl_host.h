@@ -45,6 +45,18 @@ inline float host_round_bf16(float x) {
   return x;
 }
 
+// Round-to-nearest-even of a float to float16 precision, on the host (normal range; what the
+// launchers round are small constants such as half a number of quantiser states).
+inline float host_round_f16(float x) { return (float)(_Float16)x; }
+
+// a host constant as the tensor dtype holds it
+inline float host_round_dtype(int32_t dtype, float x) {
+  return dtype == AHL_BF16 ? host_round_bf16(x) : dtype == AHL_F16 ? host_round_f16(x) : x;
+}
+
+inline bool dtype_known(int32_t dtype) { return dtype == AHL_F32 || dtype == AHL_BF16 || dtype == AHL_F16; }
+inline int64_t dtype_bytes(int32_t dtype) { return dtype == AHL_F32 ? 4 : 2; }
+
 inline bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
 inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -64,6 +76,9 @@ inline int check_launch(const char* where) {
       __VA_ARGS__                                      \
     } else if ((dtype) == AHL_BF16) {                  \
       typedef ahl::BF16 D;                             \
+      __VA_ARGS__                                      \
+    } else if ((dtype) == AHL_F16) {                   \
+      typedef ahl::F16 D;                              \
       __VA_ARGS__                                      \
     } else {                                           \
       return AHL_ERR_ARG;                              \

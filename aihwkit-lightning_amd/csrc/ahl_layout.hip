@@ -80,6 +80,7 @@ int launch_pad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t row
   const int64_t spans = cdiv(padded, kCopySpan);
   if (padded > 0x7fffffff || rows * spans > 0x7fffffff) return AHL_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)(rows * spans));
+  if (dtype == AHL_F16) dtype = AHL_BF16;   // copies of 2-byte elements
   if (dtype == AHL_F32)
     hipLaunchKernelGGL((k_pad_tiles<uint32_t>), grid, dim3(256), 0, s, (const uint32_t*)src, ld_src,
                        (uint32_t*)dst, ld_dst, tl, (int32_t)stride, (int32_t)spans);
@@ -97,6 +98,7 @@ int launch_unpad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t r
   if ((int64_t)tl.n_tiles * stride > 0x7fffffff || rows * spans > 0x7fffffff)
     return AHL_ERR_UNSUPPORTED;
   const dim3 grid((unsigned)(rows * spans));
+  if (dtype == AHL_F16) dtype = AHL_BF16;   // copies of 2-byte elements
   if (dtype == AHL_F32)
     hipLaunchKernelGGL((k_unpad_tiles<uint32_t>), grid, dim3(256), 0, s, (const uint32_t*)src,
                        ld_src, (uint32_t*)dst, ld_dst, tl, (int32_t)stride, (int32_t)K,

@@ -200,8 +200,8 @@ __global__ __launch_bounds__(256) void k_gru_gates_bwd(const void* __restrict__ 
 }
 
 static bool gate_args_ok(int32_t dtype, int64_t rows, int64_t hidden, int64_t* blocks) {
-  if (rows <= 0 || hidden <= 0 || (dtype != AHL_F32 && dtype != AHL_BF16)) return false;
-  const int epv = dtype == AHL_BF16 ? 8 : 4;
+  if (rows <= 0 || hidden <= 0 || !dtype_known(dtype)) return false;
+  const int epv = dtype == AHL_F32 ? 4 : 8;
   if (hidden % epv != 0) return false;
   *blocks = cdiv(rows * (hidden / epv), 256);
   return *blocks <= 0x7fffffff;

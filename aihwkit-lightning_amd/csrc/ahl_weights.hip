@@ -20,7 +20,7 @@ AHL_DEV WQuant make_wquant(float wm, float n_states, bool all_gt1) {
   WQuant q;
   q.step = all_gt1 ? D::rd(__fdiv_rn(2.0f, sc)) : D::rd(2.0f * sc);
   if (q.step == 0.0f) q.step = 1.0f;
-  q.rc = fmaxf(q.step, kTinyF32);
+  q.rc = fmaxf(q.step, D::tiny());
   q.rcp = __fdiv_rn(1.0f, q.rc);
   return q;
 }
@@ -40,7 +40,7 @@ AHL_DEV WQuant make_wclip(float clip, bool all_gt1) {
   WQuant q;
   q.step = all_gt1 ? D::rd(__fdiv_rn(1.0f, clip)) : clip;
   if (q.step == 0.0f) q.step = 1.0f;
-  q.rc = fmaxf(q.step, kTinyF32);
+  q.rc = fmaxf(q.step, D::tiny());
   q.rcp = __fdiv_rn(1.0f, q.rc);
   return q;
 }
@@ -336,7 +336,7 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       a.w = w; a.N = N; a.K = K; a.ld = ld; a.tl = tl; a.wmax = nullptr; a.tile_max = tile_max;
       a.tile_min = tile_min; a.w_eff = w_eff; a.ld_eff = ld_eff; a.quant_type = cfg->quant_type;
       a.noise_type = noise; a.n_states = fmaxf(cfg->res, 1.0f / cfg->res);
-      a.maxq = D::kIsBf16 ? host_round_bf16(a.n_states / 2.0f) : a.n_states / 2.0f;
+      a.maxq = host_round_dtype(D::kId, a.n_states / 2.0f);
       a.std_dev = 0.0f; a.seed = 0; a.offset = 0; a.seed_state = nullptr;
       hipLaunchKernelGGL((k_quantize_rows<D, false>), grid, dim3(256), 0, s, a, wmax);
       hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
@@ -359,7 +359,7 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       const float res = cfg->res;
       a.n_states = (cfg->quant_type != AHL_QUANT_NONE && !clip_only) ? fmaxf(res, 1.0f / res) : 1.0f;
       // clamp(Tensor, Scalar, Scalar) converts its bounds to the tensor dtype first
-      a.maxq = D::kIsBf16 ? host_round_bf16(a.n_states / 2.0f) : a.n_states / 2.0f;
+      a.maxq = host_round_dtype(D::kId, a.n_states / 2.0f);
       if (clip_only) a.maxq = 1.0f;
       a.std_dev = cfg->std_dev; a.seed = cfg->seed; a.offset = cfg->offset; a.seed_state = cfg->seed_state;
       const int64_t bpr = cdiv(cdiv(K, 8), 256);
@@ -404,7 +404,7 @@ int ahl_learned_clip_bwd(void* dw, int64_t lddw, const void* w, int64_t ldw, con
   a.dclip = dclip; a.N = N; a.tl = tl; a.quant_type = cfg->quant_type;
   a.n_states = quant ? fmaxf(cfg->res, 1.0f / cfg->res) : 1.0f;
   a.maxq_exact = quant ? a.n_states / 2.0f : 1.0f;
-  a.maxq = (cfg->dtype == AHL_BF16) ? host_round_bf16(a.maxq_exact) : a.maxq_exact;
+  a.maxq = host_round_dtype(cfg->dtype, a.maxq_exact);
   const int64_t nb = cdiv(N * n_tiles, 4);
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   AHL_DISPATCH_DTYPE(cfg->dtype, {

@@ -7,9 +7,12 @@
  *     NULL is the default stream). All data pointers are DEVICE pointers unless a parameter is
  *     named *_host. The caller owns every buffer, including scratch ("ws_*" parameters).
  *   - Matrices are row-major with an explicit leading dimension in ELEMENTS.
- *   - dtype is AHL_F32 or AHL_BF16 and applies to every pointer documented as "dtype".
- *     In AHL_BF16 every elementwise result is rounded to bfloat16 (round-to-nearest-even)
- *     exactly where the reference's torch-mode rounds when it runs on bfloat16 tensors.
+ *   - dtype is AHL_F32, AHL_BF16 or AHL_F16 and applies to every pointer documented as "dtype".
+ *     In AHL_BF16 / AHL_F16 every elementwise result is rounded to the 16-bit type
+ *     (round-to-nearest-even) exactly where the reference's torch-mode rounds when it runs on
+ *     tensors of that type. The MFMA kernels for large shapes exist for AHL_BF16 only; AHL_F16
+ *     runs on the general kernels (the reference's accelerated slot takes float32 and float16,
+ *     triton_utils/triton_linear.py:630).
  *   - K-tiles ("analog tiles" along the input dimension) are described by `tile_ends_host`,
  *     the reference's `upper_end_of_slices` (nn/modules/linear.py:76-80) as a HOST int32 array
  *     of n_tiles cumulative end offsets. It must follow the reference's split rule
@@ -38,6 +41,7 @@ extern "C" {
 /* ---- enums -------------------------------------------------------------------------------- */
 #define AHL_F32 0
 #define AHL_BF16 1
+#define AHL_F16 2
 
 #define AHL_IR_NONE 0     /* input range disabled: no clamp, no DAC                               */
 #define AHL_IR_STATIC 1   /* one scalar per tile, ir[n_tiles] (learned or calibrated)             */
@@ -68,7 +72,7 @@ extern "C" {
 /* Forward/backward behaviour of one AnalogLinear call; a flattened
  * TorchInferenceRPUConfig (simulator/configs/configs.py:27-88) plus call state.          */
 typedef struct AhlLinearCfg {
-  int32_t dtype;                 /* AHL_F32 | AHL_BF16                                          */
+  int32_t dtype;                 /* AHL_F32 | AHL_BF16 | AHL_F16                                */
   int32_t ir_mode;               /* AHL_IR_*                                                    */
   float inp_res;                 /* forward.inp_res; <= 0 switches the DAC off                  */
   float out_res;                 /* forward.out_res; <= 0 switches ADC quantisation off         */

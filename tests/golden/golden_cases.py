@@ -5,7 +5,7 @@ file holds only the reference's outputs plus input checksums.
 """
 import torch
 
-DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16}
+DTYPES = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
 
 DEFAULTS = dict(
     dtype="f32", M=8, K=16, N=8, bias=True, max_input_size=-1,
@@ -155,6 +155,11 @@ CASES = [
     case("f32_quantize_lsq_clip_big", kind="quantize", M=4, K=32, N=8, max_input_size=16,
          clip="learnable", lwc_scale=0.6, w_scale=6.0, seed=24),
 ]
+
+# float16 (the dtype of the reference's accelerated path and speed scripts): every bfloat16 case
+# once more in float16
+CASES += [dict(c, name=c["name"].replace("bf16", "f16"), dtype="f16") for c in CASES
+          if c["dtype"] == "bf16"]
 
 CASES_BY_NAME = {c["name"]: c for c in CASES}
 

@@ -38,7 +38,7 @@ def sample(rows, cols, dtype, seed, zero_rows=(), ties=True):
     return x.to(dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("rows,cols,max_size,zero_rows", [
     (1, 7, 3, ()), (12, 40, 16, (1, 4)), (130, 257, 128, (0, 129)), (64, 1024, 512, (5,)),
     (5, 33, -1, (0, 1, 2, 3, 4)),
@@ -58,7 +58,7 @@ def test_row_filter_and_std_over_kept_rows(rows, cols, max_size, zero_rows, dtyp
             assert abs(float(got[t]) - float(want)) <= 1e-6 * float(want) + 1e-12
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("q", [0.0, 0.25, 0.5, 0.99, 0.99995, 1.0])
 @pytest.mark.parametrize("rows,cols,max_size,zero_rows", [
     (1, 7, 3, ()), (12, 40, 16, (1, 4)), (130, 257, 128, (0, 129)), (300, 96, 32, (7,)),
@@ -108,7 +108,7 @@ def test_quantile_full_size_order_property():
             assert below <= lo < at_most, (t, lo, below, at_most)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 def test_moving_update_bit_exact(dtype):
     vals = [torch.tensor([0.1234567, 7.25, 1e-3]), torch.tensor([2.5, 0.3333333, 9.75]),
             torch.tensor([1.0, 1.0, 1.0])]

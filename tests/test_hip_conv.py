@@ -52,7 +52,7 @@ def _geom_list(geom):
     return [batch, chan, *size, *kernel, *stride, *padding, *dilation]
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("geom", GEOMS, ids=[f"geom{i}" for i in range(len(GEOMS))])
 def test_patch_kernels_bit_exact(geom, dtype):
     from aihwkit_lightning.nn.modules.hip_utils.ops import OPS, conv_out_size
@@ -70,7 +70,7 @@ def test_patch_kernels_bit_exact(geom, dtype):
     assert torch.equal(dx.cpu(), want_dx)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("shape", [(1, 1, 1), (3, 33, 65), (2, 64, 32), (5, 7, 130), (1, 300, 17),
                                    # whole 16-byte vectors on both sides: the vector kernel,
                                    # full and partial 64 x 64 tiles

@@ -19,7 +19,7 @@ NOISELESS = [
     c for c in CASES
     if c["kind"] == "fwd_bwd" and c["out_noise"] == 0 and c["weight_noise"] == "none"
 ]
-RTOL = {"f32": 1e-5, "bf16": 1e-2}
+RTOL = {"f32": 1e-5, "bf16": 1e-2, "f16": 1e-3}
 
 
 def adc_lsb(c, wmax_scale=None):
@@ -172,6 +172,13 @@ SHAPES = [
          clip="learnable", lwc_scale=0.7, weight_quant="discretize_per_channel", modifier_res=30,
          w_scale=0.3, inp_res=254, out_res=254, out_bound=10.0, seed=36),
 ]
+
+
+# float16 runs on the general kernels: a selection of the shapes above once more in float16
+SHAPES += [dict(c, name=c["name"].replace("bf16", "f16"), dtype="f16") for c in SHAPES if c["name"] in (
+    "edge_bf16", "vec_bf16_static", "vec_bf16_dynamic", "vec_bf16_many_tiles", "fast_bf16_clamped",
+    "fast_bf16_dynamic_clamped", "one_token_bf16", "pad_bf16_uneven_clamped", "tail_bf16_both_dynamic",
+    "bf16_10bit_static", "bf16_odd_states_static", "pad_bf16_lsq", "sliced_dw_bf16_clamped")]
 
 
 @pytest.mark.parametrize("c", SHAPES, ids=[c["name"] for c in SHAPES])

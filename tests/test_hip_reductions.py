@@ -18,7 +18,7 @@ def ops():
     return OPS
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("n", [1, 10, 25, 255, 257, 1023, 1025])
 def test_sliced_absmax_brute_force(n, dtype):
     # sizes and tile width of the reference's self-check (triton_abs_max.py:405-419); bit exact
@@ -41,7 +41,7 @@ def test_sliced_absmax_strided_rows_and_activation_shape():
     assert torch.equal(out.cpu(), om.sliced_abs_max(view.cpu(), sizes))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("shape,max_size", [((1, 63), 11), ((64, 512), 256), ((333, 1030), 128)])
 def test_sliced_std(shape, max_size, dtype):
     torch.manual_seed(1)
@@ -118,7 +118,7 @@ def test_clip_weights_via_optimizer_matches_reference(name):
 
 
 @pytest.mark.parametrize("per_channel", [False, True])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 def test_clip_weights_closed_form(dtype, per_channel):
     # the reference's test_clipping: W == W0.clamp(+-sigma * std)
     torch.manual_seed(2)
@@ -134,7 +134,7 @@ def test_clip_weights_closed_form(dtype, per_channel):
         assert mism < 2e-3
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("vectors", [1, 63, 256, 257, 768, 1024, 2048, 2049],
                          ids=lambda v: f"{v}_vectors")
 def test_clip_weights_per_channel_row_lengths(vectors, dtype):
@@ -190,7 +190,7 @@ def test_quantize_weights_matches_reference(name):
     assert torch.allclose(before, after, rtol=tol, atol=tol * float(ref_out.abs().mean()))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("scales", ["small", "all_large", "mixed"])
 @pytest.mark.parametrize("cols,tile", [(512, 256), (2560, 1280), (300, 100)],
                          ids=["held", "long_segments", "unaligned_tiles"])
@@ -222,7 +222,7 @@ def test_quantize_weights_per_channel_scale_switch(cols, tile, scales, dtype):
 
 
 @pytest.mark.parametrize("in_size", [10, 255, 257])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 def test_calibration_max(in_size, dtype):
     # tests/test_calibration.py:155-158: input_range[t] == |x[:, tile]|.max()
     from aihwkit_lightning.inference import calibrate_input_ranges, InputRangeCalibrationType
@@ -244,7 +244,7 @@ def test_calibration_max(in_size, dtype):
     assert out.shape == (2, 3, 7)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 def test_col_sum(dtype):
     torch.manual_seed(4)
     g = torch.randn(1000, 517).to(dtype)
@@ -255,7 +255,7 @@ def test_col_sum(dtype):
 
 
 @pytest.mark.parametrize("mode", ["static", "dynamic"])
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 def test_dac_prepass_bit_exact(dtype, mode):
     """The clamp + DAC (+ dynamic abs-max) pass against the oracle's quantiser, bit for bit."""
     from aihwkit_lightning.nn.modules.hip_utils import library as L
@@ -314,7 +314,7 @@ def test_reduction_bound_pipeline_one_matrix():
     assert torch.equal(cache.cpu(), om.calibrate_max(batches, sizes))
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("k_in,max_size", [(1024, 512), (2304, 1152), (640, 128)])
 def test_one_pass_weight_prep_matches_two_pass(k_in, max_size, dtype):
     """Abs-max + per-channel weight noise in one kernel (aligned rows) must give the bits of the

@@ -230,7 +230,7 @@ def test_graph_replays_equal_the_eager_forward(cell):
         net.graphed(example)
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("rows,hidden", [(3, 8), (64, 1024), (17, 40)])
 def test_fused_gates_match_the_chain_of_torch_operations(dtype, rows, hidden):
     """ahl_lstm_gates_* / ahl_gru_gates_* against the element-wise torch operations they replace,

@@ -59,6 +59,8 @@ def linear_cases(seed, count):
 
 
 LINEAR = linear_cases(0, 48) + linear_cases(1, 48)
+# the same generator once more with every case in float16
+LINEAR += [dict(c, dtype="f16", name=c["name"] + "_f16") for c in linear_cases(2, 32)]
 
 
 @pytest.fixture(autouse=True)
@@ -146,7 +148,7 @@ def test_random_convolutions(c):
     dx, dw, db, dir_ = oc.conv_backward(gb, saved)
     if not batched:
         ref_out, dx = ref_out[0], dx[0]
-    rtol = {"f32": 1e-5, "bf16": 1e-2}[c["dtype"]]
+    rtol = {"f32": 1e-5, "bf16": 1e-2, "f16": 1e-3}[c["dtype"]]
     lsb = None
     if c["ir_mode"] != "none":  # an upper bound of the ADC step: 2 * range * out_bound * max|w| / 254
         lsb = 2 * 2.0 * c["out_bound"] * float(w.abs().max()) / 254 * 1.05

@@ -10,11 +10,11 @@ FWD_BWD = [c for c in CASES if c["kind"] == "fwd_bwd"]
 
 
 def _exact_or_close(got, ref, dtype, what):
-    """bf16 results must be identical; fp32 results may differ by accumulation order only."""
+    """bf16 / f16 results must be identical; fp32 results may differ by accumulation order only."""
     got = got.float()
-    if dtype == torch.bfloat16:
+    if dtype in (torch.bfloat16, torch.float16):
         mism = int((got != ref).sum())
-        assert mism == 0, f"{what}: {mism} of {ref.numel()} bf16 elements differ"
+        assert mism == 0, f"{what}: {mism} of {ref.numel()} 16-bit elements differ"
     else:
         scale = ref.abs().mean().clamp_min(1e-30)
         err = ((got - ref).abs() / (ref.abs() + scale)).max()
