@@ -149,3 +149,51 @@ def test_capture_without_noise_state_is_refused(monkeypatch):
             layer(xin)
     finally:
         ops._NOISE_STATES.update(saved)
+
+
+def test_recurrent_training_step_in_one_graph_equals_eager_step():
+    """A two-layer LSTM's forward + backward through time recorded into one graph (hundreds of
+    launches the eager step spreads over Python): outputs and every gradient equal the eager
+    step's, replay after replay, and with output noise on the replays differ from each other."""
+    from aihwkit_lightning.nn.graphs import CapturedStep
+    from rnn_cases import rnn_case
+    from test_hip_rnn import build_network
+
+    def net_and_step(out_noise):
+        c = rnn_case("graph_lstm", "lstm", 6, 8, 64, 64, layers=2, bidir=False, max_input_size=32,
+                     dtype="bf16", ir_mode="static", ir_init=2.0, clip="channel", clip_sigma=2.5,
+                     w_scale=0.2, inp_res=254, out_res=254, out_bound=10.0, out_noise=out_noise,
+                     training=True, seed=74)
+        net, _ = build_network(c)
+        gen = torch.Generator().manual_seed(9)
+        x = torch.randn(6, 8, 64, generator=gen).bfloat16().cuda().requires_grad_(True)
+        g = torch.randn(6, 8, 64, generator=gen).bfloat16().cuda()
+
+        def step():
+            x.grad = None
+            net.zero_grad(set_to_none=True)
+            out = net(x)[0]
+            out.backward(g)
+            return out
+        return net, x, step
+
+    net_e, x_e, step_e = net_and_step(0.0)
+    out_e = step_e()
+    net_g, x_g, step_g = net_and_step(0.0)
+    replay = CapturedStep(step_g)
+    for i in range(3):
+        out = replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, out_e), f"out, replay {i}"
+        assert torch.equal(x_g.grad, x_e.grad), f"dx, replay {i}"
+        for (name, p_g), (_, p_e) in zip(net_g.named_parameters(), net_e.named_parameters()):
+            if p_e.grad is not None:
+                assert torch.equal(p_g.grad, p_e.grad), f"{name}, replay {i}"
+        _ = out.float().sum().item()
+    _, _, step_n = net_and_step(0.1)
+    noisy = CapturedStep(step_n)
+    outs = []
+    for _ in range(3):
+        outs.append(noisy().detach().float().clone())
+        torch.cuda.synchronize()
+    assert not torch.equal(outs[0], outs[1]) and not torch.equal(outs[1], outs[2])
