@@ -15,6 +15,7 @@
 // this wave tile the kernel reads 64 KB of MFMA fragments from LDS and writes 32 KB into it per
 // 512 MFMA cycles of a SIMD: LDS bandwidth, not the MFMA pipe, bounds the plain product.
 #include "ahl_fwd_common.h"
+#include <stdlib.h>
 
 namespace ahl {
 
@@ -261,6 +262,15 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
             const uint32_t mrow = (uint32_t)(m0 + rbase + 16 * gp);
             normal8(nk.seed, nk.offset, (uint32_t)t, (uint32_t)n, (mrow >> 4) * 2 + ((mrow >> 2) & 1), xi);
           }
+          // "Did an output leave the range" is decided once per eight elements, from a running
+          // maximum kept in a vector register: a compare whose result goes to scalar registers
+          // (and the scalar OR that collects it) costs the wave tens of cycles each, which eight
+          // times per unit was a quarter of the whole epilogue. The rare case redoes the sums
+          // with the clamped values. (A NaN output is no longer treated as clamped; it passes
+          // through, as it does through torch.clamp.)
+          float y8[8], B8[8];
+          uint32_t tpo[4];
+          float excess = -1.0f;   // max over the unit of |y| - bound
 #pragma unroll
           for (int gg = 0; gg < 2; ++gg) {
             const int g = 2 * gp + gg;
@@ -321,25 +331,42 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
               rd2(y[0], y[1]); rd2(y[2], y[3]);
             }
             if (CLAMP) {
-              bool over = false;
 #pragma unroll
-              for (int c = 0; c < 4; ++c) over |= !(fabsf(y[c]) <= Bv[c]);
-              if (__builtin_expect(__any(over), 0)) {  // rare: an output of this group left the range
+              for (int c = 0; c < 4; ++c) {
+                y8[4 * gg + c] = y[c];
+                B8[4 * gg + c] = Bv[c];
+              }
+              if (IRMODE == AHL_IR_DYNAMIC) {
 #pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                  const bool cl = !(fabsf(y[c]) <= Bv[c]);
-                  if (a.keep != nullptr) clamp_record(cl && nvalid, 32 * bi + 8 * g + c, cwords[bj]);
-                  y[c] = fminf(fmaxf(y[c], -Bv[c]), Bv[c]);
-                }
-                any_clamp |= over ? 1u : 0u;
+                for (int c = 0; c < 4; ++c) excess = fmaxf(excess, fabsf(y[c]) - Bv[c]);
+              } else {   // one bound for the whole unit
+                excess = fmaxf(excess, fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))) - Bv[0]);
               }
             }
             // total = rd(total + y), bf16 pairs
 #pragma unroll
             for (int pr = 0; pr < 2; ++pr) {
               const uint32_t tp = totp[bi][bj][2 * g + pr];
+              tpo[2 * gg + pr] = tp;
               totp[bi][bj][2 * g + pr] =
                   pack_bf16x2(unpack_lo(tp) + y[2 * pr], unpack_hi(tp) + y[2 * pr + 1]);
+            }
+          }
+          if (CLAMP) {
+            const bool over = excess > 0.0f;
+            if (__builtin_expect(__any(over), 0)) {
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                const bool cl = fabsf(y8[e]) > B8[e];
+                if (a.keep != nullptr)
+                  clamp_record(cl && nvalid, 32 * bi + 8 * (2 * gp + (e >> 2)) + (e & 3), cwords[bj]);
+                y8[e] = fminf(fmaxf(y8[e], -B8[e]), B8[e]);
+              }
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                totp[bi][bj][4 * gp + q] =
+                    pack_bf16x2(unpack_lo(tpo[q]) + y8[2 * q], unpack_hi(tpo[q]) + y8[2 * q + 1]);
+              any_clamp |= over ? 1u : 0u;
             }
           }
           // keep the scheduler from interleaving the 8 Philox/Box-Muller chains of a block:
@@ -465,6 +492,10 @@ static void launch_fast(const FastFwdArgs& a, bool noise, int qm, hipStream_t s)
 
 namespace ahl {
 
+// ahl_fwd_pipe.hip: the kernel for large grids
+bool pipe_fwd_eligible(const FastFwdArgs& a, int ir_mode);
+bool launch_pipe_fwd(const FastFwdArgs& a, int ir_mode, bool noise, int qm, hipStream_t s);
+
 // Few rows (a recurrent step, a decoding step): the 128 x 64 output blocks alone leave most CUs
 // idle and every block walks the whole contraction with one chunk in flight. With a workspace
 // the K-tiles of an output block go to different blocks as well.
@@ -528,6 +559,12 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
                      fast_fwd_split(M, N, tl.n_tiles);
   a.part = split ? (uint16_t*)ws : nullptr;
   const int qm = adc ? (cfg->skip_rounding ? 3 : 2) : (a.clamp_on ? 1 : 0);
+  // Large grids go to the kernel that runs a tile's epilogue inside the next tile's product loop
+  // (same results bit for bit); AHL_FORWARD_KERNEL=blocks in the environment keeps them here.
+  const char* pick = getenv("AHL_FORWARD_KERNEL");
+  if (!(pick != nullptr && strcmp(pick, "blocks") == 0) && pipe_fwd_eligible(a, cfg->ir_mode) &&
+      launch_pipe_fwd(a, cfg->ir_mode, noise, qm, s))
+    return check_launch("ahl_linear_fwd(pipe)");
   if (cfg->ir_mode == AHL_IR_NONE) few ? launch_fast<0, 1>(a, noise, qm, s) : launch_fast<0, 2>(a, noise, qm, s);
   else if (cfg->ir_mode == AHL_IR_STATIC) few ? launch_fast<1, 1>(a, noise, qm, s) : launch_fast<1, 2>(a, noise, qm, s);
   else few ? launch_fast<2, 1>(a, noise, qm, s) : launch_fast<2, 2>(a, noise, qm, s);
