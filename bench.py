@@ -32,7 +32,7 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 # below. The table of the last such run is read from this file (and named in the line).
 TRAFFIC_TABLE = os.path.join("profiles", "linear_fwd_bwd_4096x4096_8192tok_bf16_hbm_traffic.txt")
 TRAFFIC_ROWS = {
-    "linear_fwd": "ahl::k_fwd_fast<",
+    "linear_fwd": "ahl::k_fwd_pipe<",
     "linear_bwd_dx(+ir_grad)": "ahl::k_bwd_fast<0",
     "linear_bwd_dw(+bias_grad)": "ahl::k_bwd_fast<1",
 }
@@ -483,6 +483,8 @@ def main():
     parser.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     parser.add_argument("--graph", action="store_true",
                         help="report the step replayed from one HIP graph instead of the eager step")
+    parser.add_argument("--no-others", action="store_true",
+                        help="headline workload only: skip the other configurations' short runs")
     parser.add_argument("--kernels-only", action="store_true",
                         help="only launch the individual kernels (for rocprofv3 runs)")
     parser.add_argument("--workload", default="linear", choices=["linear", "post_training", *OTHER_WORKLOADS],
@@ -580,6 +582,9 @@ def main():
     # The other configurations of the benchmark set, a few steps each, after the headline's
     # timed region: the dynamic-range forward, the MLP block, the reduction-bound post-training
     # pass (with its own CPU baseline). `--workload NAME` prints each as a line of its own.
+    if ns.no_others:
+        print(json.dumps(result))
+        return
     del layer, x, g
     torch.cuda.empty_cache()
     others = {}
