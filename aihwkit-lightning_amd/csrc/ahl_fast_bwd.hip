@@ -64,6 +64,175 @@ AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// Everything after the product loop: the fp32 partial result of a slice, or the 256 x 256 result
+// written through LDS with the input-range epilogue of the input gradient.
+struct BwdPos {
+  int64_t r0, c0, R, brow, bcol, nkb;
+  int t, slice;
+};
+
+template <int MODE>
+AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2], char* lds,
+                        float (*red)[3]) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 2, wn = wave & 3;
+  const int h = lane >> 5;
+  const int64_t r0 = pos.r0, c0 = pos.c0, R = pos.R, brow = pos.brow, bcol = pos.bcol, nkb = pos.nkb;
+  const int t = pos.t, slice = pos.slice;
+  if (a.slices > 1) {
+    // partial result of this slice, fp32, straight from the accumulators: for fixed (bi, bj, v)
+    // the 32 lanes of a half wave write 128 contiguous bytes of one row
+    float* sp = a.split + ((int64_t)slice * R) * a.K;
+#pragma unroll
+    for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int64_t row = r0 + wm * 128 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        if (row >= R) continue;
+#pragma unroll
+        for (int bj = 0; bj < 2; ++bj)
+          sp[row * a.K + c0 + wn * 64 + bj * 32 + (lane & 31)] = acc[bi][bj][v];
+      }
+    return;
+  }
+
+  // ---- epilogue: the 256 x 256 result goes through LDS (the operand buffers are free after
+  // the loop's last barrier) so that global memory is touched in row-contiguous 16-byte vectors;
+  // the forward input needed by the input-range gradient is fetched the same way ----
+  float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
+  const bool do_ir = MODE == MODE_DX && a.ir_static != 0;
+  const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
+  constexpr int kOutStride = 256 * 2 + 16;
+  const int vcol = tid & 31, vrow = tid >> 5;  // 16-byte vector column, row within a pass of 16
+  // column of this thread's vectors in x / dx: the operand column itself, or, with dense x / dx
+  // next to a padded W_eff, the same offset inside the dense tile (padding columns: no vector)
+  int64_t ocol = c0 + vcol * 8;
+  bool ovalid = true;
+  if (MODE == MODE_DX && a.dense_tile > 0) {
+    const int64_t in_tile = ocol - (int64_t)t * a.tile;
+    ovalid = in_tile < a.dense_tile;
+    ocol = ovalid ? (int64_t)t * a.dense_tile + in_tile : 0;
+  }
+  uint16_t* op = a.out + (r0 + vrow) * a.ldo + ocol;
+  {
+    char* obase = lds + (wm * 128 + 4 * h) * kOutStride + (wn * 64 + (lane & 31)) * 2;
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int bi = 0; bi < 4; ++bi)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
+          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)f32_to_bf16_bits(acc[bi][bj][v]);
+        }
+  }
+  __syncthreads();
+  if (MODE == MODE_DX && a.dense_base > 0) {
+    // Dense x / dx whose tiles start at arbitrary columns. Per output row the block owns one
+    // contiguous run of dense columns; it is written as 16-byte vectors from the first 16-byte
+    // boundary of dx on (x has the same alignment: the launcher checks ldx == ldo and the base
+    // pointers), the few elements before and after as single 2-byte accesses. Sub-dword
+    // accesses for everything cost more than the padded copies they replace. A half wave
+    // handles one row per pass; wave w owns rows 32 w .. 32 w + 31.
+    const int32_t tw = a.dense_base + (t < a.dense_extra ? 1 : 0);
+    const int64_t dstart = (int64_t)t * a.dense_base + (t < a.dense_extra ? t : a.dense_extra);
+    const int64_t in0 = c0 - (int64_t)t * a.tile;  // block's first column inside the padded tile
+    const int count = (int)(tw - in0 < 256 ? tw - in0 : 256);  // columns with data (may be <= 0)
+    const int hw = lane >> 5, l32 = lane & 31;
+    auto element = [&](float d, float x1) -> float {
+      if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
+        const bool up = x1 >= ir_t, lo = x1 <= -ir_t;
+        if (up) s_up += fminf(d, 0.0f);
+        if (lo) s_lo += fmaxf(d, 0.0f);
+        if (up || lo) cnt += 1.0f;
+      } else {
+        if (x1 > ir_t) s_up += d;
+        if (x1 < -ir_t) s_lo += d;
+      }
+      return fabsf(x1) > ir_t ? 0.0f : d;
+    };
+    for (int rr = 0; rr < 32; rr += 2) {
+      const int row = wave * 32 + rr + hw;
+      if (count <= 0 || r0 + row >= R) continue;
+      const int64_t e0 = (r0 + row) * a.ldo + dstart + in0;   // first element of the run in dx (and x)
+      const int head = (int)((8 - (e0 & 7)) & 7) < count ? (int)((8 - (e0 & 7)) & 7) : count;
+      const int nv = (count - head) >> 3;
+      const int tail0 = head + 8 * nv;                        // first column of the tail
+      const char* lrow = lds + row * kOutStride;
+      if (l32 < nv) {
+        const int j = head + 8 * l32;
+        float d[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) d[i] = bf16_bits_to_f32(*(const uint16_t*)(lrow + (j + i) * 2));
+        if (do_ir) {
+          float xv[8];
+          BF16::unpack(ld16(a.x + e0 + j), xv);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) d[i] = element(d[i], xv[i]);
+        }
+        st16(a.out + e0 + j, BF16::pack(d));
+      }
+      // up to 7 elements before the first and after the last vector
+      const int j1 = l32 < head ? l32 : tail0 + (l32 - head);
+      if (l32 < head + (count - tail0)) {
+        float d = bf16_bits_to_f32(*(const uint16_t*)(lrow + j1 * 2));
+        if (do_ir) d = element(d, bf16_bits_to_f32(a.x[e0 + j1]));
+        a.out[e0 + j1] = (uint16_t)f32_to_bf16_bits(d);
+      }
+    }
+  } else
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    u32x4 xr[8];
+    if (do_ir && ovalid) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int row = vrow + 16 * (8 * half + j);
+        // rows beyond the matrix re-read the last row (the values are not used)
+        const int64_t xrow = r0 + row < R ? r0 + row : R - 1;
+        xr[j] = ld16(a.x + xrow * a.ldx + ocol);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int row = vrow + 16 * (8 * half + j);
+      u32x4 d4 = *(const u32x4*)(lds + row * kOutStride + vcol * 16);
+      if (r0 + row >= R || !ovalid) continue;
+      if (do_ir) {
+        float d[8], xv[8];
+        BF16::unpack(d4, d);
+        BF16::unpack(xr[j], xv);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
+            const bool up = xv[i] >= ir_t, lo = xv[i] <= -ir_t;
+            if (up) s_up += fminf(d[i], 0.0f);
+            if (lo) s_lo += fmaxf(d[i], 0.0f);
+            if (up || lo) cnt += 1.0f;
+          } else {
+            if (xv[i] > ir_t) s_up += d[i];
+            if (xv[i] < -ir_t) s_lo += d[i];
+          }
+          if (fabsf(xv[i]) > ir_t) d[i] = 0.0f;
+        }
+        d4 = BF16::pack(d);
+      }
+      st16(op + (int64_t)(16 * (8 * half + j)) * a.ldo, d4);
+    }
+  }
+  if (do_ir) {
+    s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
+    if (lane == 0) { red[wave][0] = s_up; red[wave][1] = s_lo; red[wave][2] = cnt; }
+    __syncthreads();
+    if (tid == 0) {
+      float u = 0.f, l = 0.f, c = 0.f;
+      for (int w = 0; w < 8; ++w) { u += red[w][0]; l += red[w][1]; c += red[w][2]; }
+      float* p = a.partial + (brow * nkb + bcol) * 4;
+      p[0] = u; p[1] = l; p[2] = c; p[3] = 0.0f;
+    }
+  }
+}
+
 // TAIL: the contraction length is not a multiple of 64 (its last chunk is loaded with
 // predicates); the TAIL = false instantiation has no trace of that in its hot loop.
 template <int MODE, bool TAIL>
@@ -293,158 +462,8 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     else main_loop(std::false_type{}, std::false_type{});
   }
 
-  if (a.slices > 1) {
-    // partial result of this slice, fp32, straight from the accumulators: for fixed (bi, bj, v)
-    // the 32 lanes of a half wave write 128 contiguous bytes of one row
-    float* sp = a.split + ((int64_t)slice * R) * a.K;
-#pragma unroll
-    for (int bi = 0; bi < 4; ++bi)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int64_t row = r0 + wm * 128 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
-        if (row >= R) continue;
-#pragma unroll
-        for (int bj = 0; bj < 2; ++bj)
-          sp[row * a.K + c0 + wn * 64 + bj * 32 + (lane & 31)] = acc[bi][bj][v];
-      }
-    return;
-  }
-
-  // ---- epilogue: the 256 x 256 result goes through LDS (the operand buffers are free after
-  // the loop's last barrier) so that global memory is touched in row-contiguous 16-byte vectors;
-  // the forward input needed by the input-range gradient is fetched the same way ----
-  float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
-  const bool do_ir = MODE == MODE_DX && a.ir_static != 0;
-  const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
-  constexpr int kOutStride = 256 * 2 + 16;
-  const int vcol = tid & 31, vrow = tid >> 5;  // 16-byte vector column, row within a pass of 16
-  // column of this thread's vectors in x / dx: the operand column itself, or, with dense x / dx
-  // next to a padded W_eff, the same offset inside the dense tile (padding columns: no vector)
-  int64_t ocol = c0 + vcol * 8;
-  bool ovalid = true;
-  if (MODE == MODE_DX && a.dense_tile > 0) {
-    const int64_t in_tile = ocol - (int64_t)t * a.tile;
-    ovalid = in_tile < a.dense_tile;
-    ocol = ovalid ? (int64_t)t * a.dense_tile + in_tile : 0;
-  }
-  uint16_t* op = a.out + (r0 + vrow) * a.ldo + ocol;
-  {
-    char* obase = lds + (wm * 128 + 4 * h) * kOutStride + (wn * 64 + (lane & 31)) * 2;
-#pragma unroll
-    for (int bj = 0; bj < 2; ++bj)
-#pragma unroll
-      for (int bi = 0; bi < 4; ++bi)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
-          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)f32_to_bf16_bits(acc[bi][bj][v]);
-        }
-  }
-  __syncthreads();
-  if (MODE == MODE_DX && a.dense_base > 0) {
-    // Dense x / dx whose tiles start at arbitrary columns. Per output row the block owns one
-    // contiguous run of dense columns; it is written as 16-byte vectors from the first 16-byte
-    // boundary of dx on (x has the same alignment: the launcher checks ldx == ldo and the base
-    // pointers), the few elements before and after as single 2-byte accesses. Sub-dword
-    // accesses for everything cost more than the padded copies they replace. A half wave
-    // handles one row per pass; wave w owns rows 32 w .. 32 w + 31.
-    const int32_t tw = a.dense_base + (t < a.dense_extra ? 1 : 0);
-    const int64_t dstart = (int64_t)t * a.dense_base + (t < a.dense_extra ? t : a.dense_extra);
-    const int64_t in0 = c0 - (int64_t)t * a.tile;  // block's first column inside the padded tile
-    const int count = (int)(tw - in0 < 256 ? tw - in0 : 256);  // columns with data (may be <= 0)
-    const int hw = lane >> 5, l32 = lane & 31;
-    auto element = [&](float d, float x1) -> float {
-      if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
-        const bool up = x1 >= ir_t, lo = x1 <= -ir_t;
-        if (up) s_up += fminf(d, 0.0f);
-        if (lo) s_lo += fmaxf(d, 0.0f);
-        if (up || lo) cnt += 1.0f;
-      } else {
-        if (x1 > ir_t) s_up += d;
-        if (x1 < -ir_t) s_lo += d;
-      }
-      return fabsf(x1) > ir_t ? 0.0f : d;
-    };
-    for (int rr = 0; rr < 32; rr += 2) {
-      const int row = wave * 32 + rr + hw;
-      if (count <= 0 || r0 + row >= R) continue;
-      const int64_t e0 = (r0 + row) * a.ldo + dstart + in0;   // first element of the run in dx (and x)
-      const int head = (int)((8 - (e0 & 7)) & 7) < count ? (int)((8 - (e0 & 7)) & 7) : count;
-      const int nv = (count - head) >> 3;
-      const int tail0 = head + 8 * nv;                        // first column of the tail
-      const char* lrow = lds + row * kOutStride;
-      if (l32 < nv) {
-        const int j = head + 8 * l32;
-        float d[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) d[i] = bf16_bits_to_f32(*(const uint16_t*)(lrow + (j + i) * 2));
-        if (do_ir) {
-          float xv[8];
-          BF16::unpack(ld16(a.x + e0 + j), xv);
-#pragma unroll
-          for (int i = 0; i < 8; ++i) d[i] = element(d[i], xv[i]);
-        }
-        st16(a.out + e0 + j, BF16::pack(d));
-      }
-      // up to 7 elements before the first and after the last vector
-      const int j1 = l32 < head ? l32 : tail0 + (l32 - head);
-      if (l32 < head + (count - tail0)) {
-        float d = bf16_bits_to_f32(*(const uint16_t*)(lrow + j1 * 2));
-        if (do_ir) d = element(d, bf16_bits_to_f32(a.x[e0 + j1]));
-        a.out[e0 + j1] = (uint16_t)f32_to_bf16_bits(d);
-      }
-    }
-  } else
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    u32x4 xr[8];
-    if (do_ir && ovalid) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int row = vrow + 16 * (8 * half + j);
-        // rows beyond the matrix re-read the last row (the values are not used)
-        const int64_t xrow = r0 + row < R ? r0 + row : R - 1;
-        xr[j] = ld16(a.x + xrow * a.ldx + ocol);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int row = vrow + 16 * (8 * half + j);
-      u32x4 d4 = *(const u32x4*)(lds + row * kOutStride + vcol * 16);
-      if (r0 + row >= R || !ovalid) continue;
-      if (do_ir) {
-        float d[8], xv[8];
-        BF16::unpack(d4, d);
-        BF16::unpack(xr[j], xv);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
-            const bool up = xv[i] >= ir_t, lo = xv[i] <= -ir_t;
-            if (up) s_up += fminf(d[i], 0.0f);
-            if (lo) s_lo += fmaxf(d[i], 0.0f);
-            if (up || lo) cnt += 1.0f;
-          } else {
-            if (xv[i] > ir_t) s_up += d[i];
-            if (xv[i] < -ir_t) s_lo += d[i];
-          }
-          if (fabsf(xv[i]) > ir_t) d[i] = 0.0f;
-        }
-        d4 = BF16::pack(d);
-      }
-      st16(op + (int64_t)(16 * (8 * half + j)) * a.ldo, d4);
-    }
-  }
-  if (do_ir) {
-    s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
-    if (lane == 0) { red[wave][0] = s_up; red[wave][1] = s_lo; red[wave][2] = cnt; }
-    __syncthreads();
-    if (tid == 0) {
-      float u = 0.f, l = 0.f, c = 0.f;
-      for (int w = 0; w < 8; ++w) { u += red[w][0]; l += red[w][1]; c += red[w][2]; }
-      float* p = a.partial + (brow * nkb + bcol) * 4;
-      p[0] = u; p[1] = l; p[2] = c; p[3] = 0.0f;
-    }
-  }
+  const BwdPos pos = {r0, c0, R, brow, bcol, nkb, t, slice};
+  bwd_finish<MODE>(a, pos, acc, lds, red);
 }
 
 // out[r, c] = bf16(sum over slices of split[s][r][c]), slices added in order

@@ -35,6 +35,7 @@
 // the dynamic input range (no gain measured there) and other tile widths: same arithmetic per
 // element, same Philox counters (tile, row group, column).
 #include "ahl_fwd_common.h"
+#include "ahl_lds_direct.h"
 #include <type_traits>
 
 namespace ahl {
@@ -48,29 +49,6 @@ static constexpr int kPRowc = kPStages * kPStage;     // dynamic range: [2][2][2
 static constexpr int kPColc = kPRowc + 2 * 2 * 256 * (int)sizeof(float);   // [8 waves][2][32][4] per-column constants
 static constexpr int kPColw = kPColc + 8 * 2 * 32 * 4 * (int)sizeof(float);  // [8 waves][2][32][2] (dynamic range)
 static constexpr int kPLdsBytes = kPColw + 8 * 2 * 32 * 2 * (int)sizeof(float);
-
-typedef __attribute__((address_space(3))) void* lds_void_ptr;
-
-// s_waitcnt immediate (gfx9 encoding): vmcnt(n), lgkmcnt(0), expcnt unconstrained
-static constexpr int vm_wait(int n) { return (n & 15) | ((n >> 4) << 14) | 0x0070; }
-
-// Workgroup barrier that orders LDS accesses and waits until at most `flying` of this wave's
-// vector memory operations are outstanding. __syncthreads() would wait for all of them, i.e.
-// drain the direct-to-LDS loads of the chunks ahead at every barrier.
-template <int FLYING>
-AHL_DEV void lds_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_waitcnt(vm_wait(FLYING));
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
-// 16 bytes per lane from global memory straight into LDS: lane L's data lands at lds_base + 16 L
-// (a device-only wrapper: the builtin inside a kernel body keeps the host pass from emitting the
-// kernel's launch stub)
-AHL_DEV void load_to_lds16(__amdgpu_buffer_rsrc_t rsrc, char* lds_base, int voffset, int soffset) {
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_void_ptr)lds_base, 16, voffset, soffset, 0, 0);
-}
 
 template <bool V> using flag = std::integral_constant<bool, V>;
 
