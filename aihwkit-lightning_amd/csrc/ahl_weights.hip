@@ -190,50 +190,29 @@ __global__ __launch_bounds__(256) void k_weight_prep_rows(ModArgs a, void* __res
 // the maximum of its segment, writes wmax[t, n] and quantises the segment with its own scale --
 // from registers for segments of up to 1024 inputs, else from a second (cache-resident) read.
 // The reference's resolution convention switches to "number of states" when EVERY scale of the
-// tile exceeds one; a wave whose own scale does not knows the switch is off. The others leave
-// their segment to the second launch (DEFERRED), which runs after the tile minima are known and
-// returns at once for every other segment. Same arithmetic as k_weight_modify; in place or not.
-template <class D, bool DEFERRED>
-__global__ __launch_bounds__(256) void k_quantize_rows(ModArgs a, void* __restrict__ wmax_io) {
+// tile exceeds one; a wave whose own scale does not knows the switch is off. The others (weights
+// beyond the number of states: rare) leave their segment to k_quantize_finish, which runs after
+// the tile minima are known. Same arithmetic as k_weight_modify; in place or not.
+template <class D>
+AHL_DEV bool quantize_deferred(float mx, float n_states) {
+  return D::rd(__fdiv_rn(mx, n_states)) > 1.0f;
+}
+
+// Quantises segment (n, t) with the scale of its abs-max mx. `keep`: the first two vectors per
+// lane if the caller still holds them, else null (they are read again).
+template <class D>
+AHL_DEV void quantize_segment(const ModArgs& a, int64_t n, int32_t t, float mx, bool all_gt1, int lane,
+                              const float (*keep)[8]) {
   constexpr int E = D::EPV;
   constexpr int VPG = 8 / E;
-  const int lane = threadIdx.x & 63;
-  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int64_t n = wave / a.tl.n_tiles;
-  const int32_t t = (int32_t)(wave % a.tl.n_tiles);
-  if (n >= a.N) return;
   const int32_t g0 = a.tl.start(t) >> 3, g1 = a.tl.start(t + 1) >> 3;
   const typename D::elem* row = (const typename D::elem*)a.w + n * a.ld;
   typename D::elem* dst = (typename D::elem*)a.w_eff + n * a.ld_eff;
-  float keep[2][8];
-  float mx = 0.0f;
-  bool all_gt1 = false;
-  if (DEFERRED) {
-    mx = D::load(wmax_io, (int64_t)t * a.N + n);
-    if (!(D::rd(__fdiv_rn(mx, a.n_states)) > 1.0f)) return;   // done by the first launch
-    all_gt1 = D::rd(__fdiv_rn(a.tile_min[t], a.n_states)) > 1.0f;
-  } else {
-    int it = 0;
-    for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
-      float v[8];
-#pragma unroll
-      for (int q = 0; q < VPG; ++q) D::unpack(ld16(row + (int64_t)g * 8 + q * E), v + q * E);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
-      if (it < 2) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) keep[it][e] = v[e];
-      }
-    }
-    mx = wave_max(mx);
-    if (lane == 0) D::store(wmax_io, (int64_t)t * a.N + n, mx);
-    if (D::rd(__fdiv_rn(D::rd(mx), a.n_states)) > 1.0f) return;  // needs the tile minimum: deferred
-  }
   const WQuant q = make_wquant<D>(D::rd(mx), a.n_states, all_gt1);
   int it = 0;
   for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
     float v[8];
-    if (!DEFERRED && it < 2) {
+    if (keep != nullptr && it < 2) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = keep[it][e];
     } else {
@@ -244,6 +223,89 @@ __global__ __launch_bounds__(256) void k_quantize_rows(ModArgs a, void* __restri
     for (int e = 0; e < 8; ++e) v[e] = wquant_apply<D>(v[e], q, a.maxq);
 #pragma unroll
     for (int qv = 0; qv < VPG; ++qv) st16(dst + (int64_t)g * 8 + qv * E, D::pack(v + qv * E));
+  }
+}
+
+template <class D>
+__global__ __launch_bounds__(256) void k_quantize_rows(ModArgs a, void* __restrict__ wmax_io) {
+  constexpr int E = D::EPV;
+  constexpr int VPG = 8 / E;
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t n = wave / a.tl.n_tiles;
+  const int32_t t = (int32_t)(wave % a.tl.n_tiles);
+  if (n >= a.N) return;
+  const int32_t g0 = a.tl.start(t) >> 3, g1 = a.tl.start(t + 1) >> 3;
+  const typename D::elem* row = (const typename D::elem*)a.w + n * a.ld;
+  float keep[2][8];
+  float mx = 0.0f;
+  int it = 0;
+  for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
+    float v[8];
+#pragma unroll
+    for (int q = 0; q < VPG; ++q) D::unpack(ld16(row + (int64_t)g * 8 + q * E), v + q * E);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
+    if (it < 2) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) keep[it][e] = v[e];
+    }
+  }
+  mx = wave_max(mx);
+  if (lane == 0) D::store(wmax_io, (int64_t)t * a.N + n, mx);
+  if (quantize_deferred<D>(D::rd(mx), a.n_states)) return;  // needs the tile minimum
+  quantize_segment<D>(a, n, t, mx, false, lane, keep);
+}
+
+// After k_quantize_rows, one block per tile: the tile's largest and smallest segment abs-max
+// (what k_tile_minmax computes), and the segments that kernel deferred, if any: with no such
+// segment (the usual case) the block is done after the reduction. With some, every wave walks a
+// quarter of the channels, 64 at a time, and quantises the deferred ones among them.
+template <class D>
+__global__ __launch_bounds__(256) void k_quantize_finish(ModArgs a, const void* __restrict__ wmax,
+                                                         float* __restrict__ tile_max,
+                                                         float* __restrict__ tile_min) {
+  __shared__ float smax[4], smin[4];
+  __shared__ int s_any;
+  const int32_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  float mx = 0.0f, mn = __builtin_inff();
+  bool mine = false;
+  if (threadIdx.x == 0) s_any = 0;
+  for (int64_t r0 = threadIdx.x; r0 < a.N; r0 += 256 * 8) {
+    float v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t r = r0 + 256 * u;
+      v[u] = D::load(wmax, (int64_t)t * a.N + (r < a.N ? r : r0));  // r0 again: no effect
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      mx = fmaxf(mx, v[u]);
+      mn = fminf(mn, v[u]);
+      mine = mine || quantize_deferred<D>(v[u], a.n_states);
+    }
+  }
+  mx = wave_max(mx);
+  mn = wave_min(mn);
+  if (lane == 0) { smax[wv] = mx; smin[wv] = mn; }
+  __syncthreads();
+  if (mine) s_any = 1;
+  __syncthreads();
+  const float tmax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
+  const float tmin = fminf(fminf(smin[0], smin[1]), fminf(smin[2], smin[3]));
+  if (threadIdx.x == 0) { tile_max[t] = tmax; tile_min[t] = tmin; }
+  if (s_any == 0) return;
+  const bool all_gt1 = quantize_deferred<D>(tmin, a.n_states);
+  for (int64_t base = (int64_t)wv * 64; base < a.N; base += 256) {
+    const int64_t nl = base + lane;
+    const float m = nl < a.N ? D::load(wmax, (int64_t)t * a.N + nl) : 0.0f;
+    uint64_t todo = __ballot(nl < a.N && quantize_deferred<D>(m, a.n_states));
+    while (todo) {
+      const int src = __builtin_ctzll(todo);
+      todo &= todo - 1;
+      quantize_segment<D>(a, base + src, t, __shfl(m, src), all_gt1, lane, nullptr);
+    }
   }
 }
 
@@ -338,9 +400,9 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       a.noise_type = noise; a.n_states = fmaxf(cfg->res, 1.0f / cfg->res);
       a.maxq = host_round_dtype(D::kId, a.n_states / 2.0f);
       a.std_dev = 0.0f; a.seed = 0; a.offset = 0; a.seed_state = nullptr;
-      hipLaunchKernelGGL((k_quantize_rows<D, false>), grid, dim3(256), 0, s, a, wmax);
-      hipLaunchKernelGGL((k_tile_minmax<D>), dim3(tl.n_tiles), dim3(256), 0, s, wmax, N, tile_max, tile_min);
-      hipLaunchKernelGGL((k_quantize_rows<D, true>), grid, dim3(256), 0, s, a, wmax);
+      hipLaunchKernelGGL((k_quantize_rows<D>), grid, dim3(256), 0, s, a, wmax);
+      hipLaunchKernelGGL((k_quantize_finish<D>), dim3(tl.n_tiles), dim3(256), 0, s, a, (const void*)wmax, tile_max,
+                         tile_min);
       return check_launch("ahl_weight_prep(one-pass quantiser)");
     }
     if (cfg->wmax_given) {

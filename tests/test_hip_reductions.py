@@ -194,16 +194,18 @@ def test_quantize_weights_matches_reference(name):
 @pytest.mark.parametrize("scales", ["small", "all_large", "mixed"])
 @pytest.mark.parametrize("cols,tile", [(512, 256), (2560, 1280), (300, 100)],
                          ids=["held", "long_segments", "unaligned_tiles"])
-def test_quantize_weights_per_channel_scale_switch(cols, tile, scales, dtype):
+@pytest.mark.parametrize("rows", [24, 700])
+def test_quantize_weights_per_channel_scale_switch(rows, cols, tile, scales, dtype):
     """The per-channel quantiser against the oracle where the reference's resolution convention
     matters: it reads the scales as numbers of states only if EVERY scale of a tile exceeds one.
     `small`: none does (the one-pass kernel alone); `all_large`: all do; `mixed`: some channels do,
     so the switch stays off but their segments wait for the tile minimum. Segments held in
-    registers, segments longer than that, and a split the one-pass kernel does not take."""
+    registers, segments longer than that, and a split the one-pass kernel does not take; a
+    handful of channels and more than one block's worth of them."""
     from aihwkit_lightning.nn.modules.hip_utils import library as L
 
     gen = torch.Generator().manual_seed(cols + len(scales))
-    w = torch.randn(24, cols, generator=gen)
+    w = torch.randn(rows, cols, generator=gen)
     if scales == "all_large":
         w = w * 400.0
     elif scales == "mixed":
