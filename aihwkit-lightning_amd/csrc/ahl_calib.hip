@@ -5,7 +5,13 @@
 // The quantile is exact: torch.quantile's linear interpolation between the two neighbouring
 // order statistics, which are found by a most-significant-digit radix selection on the
 // order-preserving integer image of the fp32 values -- four histogram passes of 8 bits over the
-// data (integer atomics only: deterministic), one pass for the successor of the selected value.
+// data (integer atomics only: deterministic). The successor of the selected value, which the
+// interpolation needs, comes out of the last pass: it is the next non-empty bin of that pass's
+// histogram, or else the smallest key whose upper 24 bits exceed the selected prefix, a minimum
+// the last pass takes on the way.
+// Seven launches: the row filter, the set-up, the four histogram passes, the interpolation;
+// "which bin holds the rank" is worked out from the previous pass's histogram by every wave of
+// the next pass for itself (a 256-bin prefix sum) rather than by a launch between.
 // No sort, no copy of the data; everything stays on the device, so a calibration run never
 // synchronises with the host.
 #include "ahl_host.h"
@@ -23,33 +29,43 @@ AHL_DEV float key_f32(uint32_t k) {
   return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
 }
 
-// per-tile selection state
+// per-tile selection state; st[p][t] is the state in front of histogram pass p (after p digits)
 struct SelState {
   uint32_t prefix;    // digits of the selected key found so far (right-aligned)
   uint32_t k_rem;     // rank of the wanted element among the elements that match the prefix
   uint32_t lo;        // rank of the lower order statistic
   uint32_t need_hi;   // the interpolation needs the next order statistic too
   float weight;       // interpolation weight of the upper order statistic
-  uint32_t n_le;      // elements <= the selected value (set by the last pick)
-  uint32_t next_key;  // smallest key above the selected one (0xffffffff: none)
-  uint32_t has_nan;
+  uint32_t n_le;      // elements <= the selected value (set with the last digit)
   uint32_t n;         // elements of the tile over the kept rows
-  uint32_t pad[3];
+  uint32_t pad;
 };
-static_assert(sizeof(SelState) == 48, "layout");
+static_assert(sizeof(SelState) == 32, "layout");
 
-// n, rank and weight per tile: rank = q * (n - 1) evaluated in fp32 as torch.quantile does for
-// an fp32 input (aten/src/ATen/native/Sorting.cpp quantile_compute)
-__global__ void k_select_init(SelState* st, uint32_t* hist, const uint32_t* n_kept, Tiling tl,
-                              float q) {
+// Set-up, one block per tile: the number of kept rows (a sum over the row flags), from it n,
+// rank and weight -- rank = q * (n - 1) evaluated in fp32 as torch.quantile does for an fp32
+// input (aten/src/ATen/native/Sorting.cpp quantile_compute) --, cleared histograms of all four
+// passes, "no successor yet" and "no NaN seen".
+__global__ __launch_bounds__(256) void k_select_init(SelState* st, uint32_t* hist, uint32_t* next_key,
+                                                     uint32_t* has_nan, const uint8_t* __restrict__ kept,
+                                                     int64_t rows, Tiling tl, float q) {
+  __shared__ uint32_t part[4];
   const int t = blockIdx.x, i = threadIdx.x;
-  hist[t * 256 + i] = 0u;
+  const int32_t n_tiles = gridDim.x;
+  for (int p = 0; p < 4; ++p) hist[((int64_t)p * n_tiles + t) * 256 + i] = 0u;
+  uint32_t cnt = 0u;
+  for (int64_t r = i; r < rows; r += 256) cnt += kept[r];
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) cnt += (uint32_t)__shfl_xor((int)cnt, off, 64);
+  if ((i & 63) == 0) part[i >> 6] = cnt;
+  __syncthreads();
   if (i != 0) return;
-  const uint64_t n64 = (uint64_t)*n_kept * (uint64_t)tl.size(t);
+  next_key[t] = 0xffffffffu;
+  has_nan[t] = 0u;
+  const uint64_t n64 = (uint64_t)(part[0] + part[1] + part[2] + part[3]) * (uint64_t)tl.size(t);
   SelState s;
   s.n = (uint32_t)n64;
-  s.prefix = 0u; s.n_le = 0u; s.next_key = 0xffffffffu; s.has_nan = 0u;
-  s.pad[0] = s.pad[1] = s.pad[2] = 0u;
+  s.prefix = 0u; s.n_le = 0u; s.pad = 0u;
   if (n64 == 0) { s.k_rem = 0u; s.lo = 0u; s.need_hi = 0u; s.weight = 0.0f; st[t] = s; return; }
   const float rank = q * (float)(n64 - 1);
   const float below = floorf(rank);
@@ -60,6 +76,43 @@ __global__ void k_select_init(SelState* st, uint32_t* hist, const uint32_t* n_ke
   st[t] = s;
 }
 
+// The state after digit `pass`, from the state in front of it and the finished histogram of
+// that pass, computed by one wave (every lane gets the result): the bin that holds rank k_rem
+// -- the first of bins 0..254 whose running count exceeds the rank, bin 255 otherwise -- extends
+// the prefix and rebases the rank. Lane l owns bins 4 l .. 4 l + 3.
+AHL_DEV SelState wave_pick(const SelState& s0, const uint32_t* __restrict__ h, int pass, int lane) {
+  if (s0.n == 0) return s0;
+  uint32_t c[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) c[j] = h[4 * lane + j];
+  const uint32_t mine = c[0] + c[1] + c[2] + c[3];
+  uint32_t incl = mine;   // inclusive sum over lanes
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const uint32_t o = (uint32_t)__shfl_up((int)incl, off, 64);
+    if (lane >= off) incl += o;
+  }
+  uint32_t excl = incl - mine, bin_excl = 0u, bin_c = 0u;
+  int bin = -1;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int b = 4 * lane + j;
+    if (bin < 0 && b < 255 && excl <= s0.k_rem && excl + c[j] > s0.k_rem) { bin = b; bin_excl = excl; bin_c = c[j]; }
+    if (b == 255 && bin < 0) { bin_excl = excl; bin_c = c[j]; }   // lane 63 keeps bin 255 at hand
+    excl += c[j];
+  }
+  const uint64_t found = __builtin_amdgcn_ballot_w64(bin >= 0);
+  const int src = found ? __builtin_ctzll(found) : 63;
+  const int pick = found ? __shfl(bin, src, 64) : 255;
+  const uint32_t p_excl = (uint32_t)__shfl((int)bin_excl, src, 64);
+  const uint32_t p_c = (uint32_t)__shfl((int)bin_c, src, 64);
+  SelState s = s0;
+  s.prefix = (s.prefix << 8) | (uint32_t)pick;
+  s.k_rem -= p_excl;
+  if (pass == 3) s.n_le = (s.lo - s.k_rem) + p_c;  // below + equal
+  return s;
+}
+
 // Histogram of digit `pass` (0 = most significant byte) over the kept elements of every tile
 // whose higher digits equal the tile's prefix. One wave per (group of rows, tile); per-wave
 // histogram in LDS, then one integer atomic per non-empty bin.
@@ -68,7 +121,9 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
                                                      int64_t ld, const uint8_t* __restrict__ kept,
                                                      Tiling tl, int rpw, int pass,
                                                      SelState* __restrict__ st,
-                                                     uint32_t* __restrict__ hist) {
+                                                     uint32_t* __restrict__ hist,
+                                                     uint32_t* __restrict__ has_nan,
+                                                     uint32_t* __restrict__ next_key) {
   // eight copies of the wave's histogram, one per lane residue: the leading digits of real data
   // fall into a handful of bins, and a single copy would serialise the LDS atomics of a wave
   __shared__ uint32_t lh[4][8][256];
@@ -80,9 +135,16 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
   const int32_t t = (int32_t)(wave % tl.n_tiles);
   const int64_t r0 = grp * rpw;
   if (r0 < rows) {  // no early return: nothing below synchronises across waves, but keep it simple
-    const uint32_t prefix = st[t].prefix;
+    SelState s = st[(int64_t)(pass > 0 ? pass - 1 : 0) * tl.n_tiles + t];
+    if (pass > 0) {
+      s = wave_pick(s, hist + ((int64_t)(pass - 1) * tl.n_tiles + t) * 256, pass - 1, lane);
+      if (grp == 0 && lane == 0) st[(int64_t)pass * tl.n_tiles + t] = s;   // for the next launch
+    }
+    const uint32_t prefix = s.prefix;
+    uint32_t* ht = hist + ((int64_t)pass * tl.n_tiles + t) * 256;
     const int shift = 24 - 8 * pass;
     bool nan = false;
+    uint32_t above = 0xffffffffu;   // last pass: smallest key whose upper 24 bits exceed the prefix
     for (int i = 0; i < rpw; ++i) {
       const int64_t r = r0 + i;
       if (r >= rows) break;
@@ -93,91 +155,57 @@ __global__ __launch_bounds__(256) void k_select_hist(const void* __restrict__ x,
         const uint32_t key = f32_key(v);
         // digits above this pass must match the prefix found so far
         if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&mine[(key >> shift) & 255u], 1u);
+        if (pass == 3 && (key >> 8) > prefix && key < above) above = key;
       });
     }
-    if (pass == 0 && __builtin_amdgcn_ballot_w64(nan) != 0ull && lane == 0) atomicOr(&st[t].has_nan, 1u);
+    if (pass == 0 && __builtin_amdgcn_ballot_w64(nan) != 0ull && lane == 0) atomicOr(&has_nan[t], 1u);
+    if (pass == 3) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)above, off, 64);
+        above = o < above ? o : above;
+      }
+      if (lane == 0 && above < __hip_atomic_load(&next_key[t], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+        atomicMin(&next_key[t], above);
+    }
     for (int i = lane; i < 256; i += 64) {
       uint32_t c = 0u;
 #pragma unroll
       for (int j = 0; j < 8; ++j) c += lh[w][j][i];
-      if (c) atomicAdd(&hist[t * 256 + i], c);
+      if (c) atomicAdd(&ht[i], c);
     }
   }
 }
 
-// The bin that holds rank k_rem: extend the prefix, rebase the rank, clear the histogram.
-// 256 threads, one bin each: inclusive prefix sums through LDS, then the first bin (of 0..254)
-// whose running count exceeds the rank, bin 255 otherwise.
-__global__ __launch_bounds__(256) void k_select_pick(SelState* st, uint32_t* hist, int pass) {
-  __shared__ uint32_t cum[2][256];
-  __shared__ int pick;
-  const int t = blockIdx.x, b = threadIdx.x;
-  const uint32_t c = hist[t * 256 + b];
-  const SelState s0 = st[t];
-  if (b == 0) pick = 255;
-  cum[0][b] = c;
-  __syncthreads();
-  int cur = 0;
+// One wave per tile: the last digit, the successor of the selected key -- the next non-empty bin
+// of the last histogram, else the smallest key beyond the prefix that the last pass left in
+// next_key -- and out[t] = lerp(x_(lo), x_(lo+1), weight) with torch's two-sided lerp formula.
+__global__ __launch_bounds__(64) void k_select_final(const SelState* st, const uint32_t* hist,
+                                                     const uint32_t* next_key, const uint32_t* has_nan,
+                                                     float* out) {
+  const int t = blockIdx.x, lane = threadIdx.x;
+  const int32_t n_tiles = gridDim.x;
+  const uint32_t* h = hist + ((int64_t)3 * n_tiles + t) * 256;
+  const SelState s = wave_pick(st[(int64_t)3 * n_tiles + t], h, 3, lane);
+  if (s.n == 0 || has_nan[t]) {
+    if (lane == 0) out[t] = __builtin_nanf("");
+    return;
+  }
+  const int digit = (int)(s.prefix & 255u);
+  int nb = 256;   // first non-empty bin above the selected digit among this lane's four
 #pragma unroll
-  for (int off = 1; off < 256; off <<= 1) {
-    cum[cur ^ 1][b] = cum[cur][b] + (b >= off ? cum[cur][b - off] : 0u);
-    cur ^= 1;
-    __syncthreads();
-  }
-  const uint32_t incl = cum[cur][b], excl = incl - c;
-  if (b < 255 && excl <= s0.k_rem && incl > s0.k_rem) pick = b;   // at most one bin qualifies
-  __syncthreads();
-  if (b == pick && s0.n != 0) {
-    SelState s = s0;
-    s.prefix = (s.prefix << 8) | (uint32_t)b;
-    s.k_rem -= excl;
-    if (pass == 3) s.n_le = (s.lo - s.k_rem) + c;  // below + equal
-    st[t] = s;
-  }
-  hist[t * 256 + b] = 0u;
-}
-
-// next_key[t] = smallest key above the selected one
-template <class D, bool VEC>
-__global__ __launch_bounds__(256) void k_select_next(const void* __restrict__ x, int64_t rows,
-                                                     int64_t ld, const uint8_t* __restrict__ kept,
-                                                     Tiling tl, int rpw, SelState* __restrict__ st) {
-  const int lane = threadIdx.x & 63;
-  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  const int64_t grp = wave / tl.n_tiles;
-  const int32_t t = (int32_t)(wave % tl.n_tiles);
-  const int64_t r0 = grp * rpw;
-  if (r0 >= rows) return;
-  const uint32_t sel = st[t].prefix;
-  uint32_t best = 0xffffffffu;
-  for (int i = 0; i < rpw; ++i) {
-    const int64_t r = r0 + i;
-    if (r >= rows) break;
-    if (!kept[r]) continue;
-    const typename D::elem* row = (const typename D::elem*)x + r * ld;
-    wave_row_foreach<D, VEC>(row, tl.start(t), tl.start(t + 1), lane, [&](float v) {
-      const uint32_t key = f32_key(v);
-      if (key > sel && key < best) best = key;
-    });
-  }
+  for (int j = 3; j >= 0; --j)
+    if (4 * lane + j > digit && h[4 * lane + j] != 0u) nb = 4 * lane + j;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
-    const uint32_t o = (uint32_t)__shfl_xor((int)best, off, 64);
-    best = o < best ? o : best;
+    const int o = __shfl_xor(nb, off, 64);
+    nb = o < nb ? o : nb;
   }
-  if (lane == 0 && best < __hip_atomic_load(&st[t].next_key, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
-    atomicMin(&st[t].next_key, best);
-}
-
-// out[t] = lerp(x_(lo), x_(lo+1), weight) with torch's two-sided lerp formula
-__global__ void k_select_final(const SelState* st, int32_t n_tiles, float* out) {
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
-  if (t >= n_tiles) return;
-  const SelState s = st[t];
-  if (s.n == 0 || s.has_nan) { out[t] = __builtin_nanf(""); return; }
+  const uint32_t succ = nb < 256 ? ((s.prefix & ~255u) | (uint32_t)nb) : next_key[t];
+  if (lane != 0) return;
   const float lo = key_f32(s.prefix);
   float hi = lo;
-  if (s.need_hi && s.n_le < s.lo + 2u && s.next_key != 0xffffffffu) hi = key_f32(s.next_key);
+  if (s.need_hi && s.n_le < s.lo + 2u && succ != 0xffffffffu) hi = key_f32(succ);
   const float w = s.weight, diff = hi - lo;
   out[t] = w < 0.5f ? lo + w * diff : hi - diff * (1.0f - w);
 }
@@ -219,11 +247,14 @@ using namespace ahl;
 
 extern "C" {
 
-// workspace: [SelState[T] | hist[T][256] | kept-row counter | kept flags, one byte per row]
+// workspace: [SelState[4][T] | hist[4][T][256] | next_key[T] | has_nan[T] | kept flags, one byte per row]
+static int64_t select_head_bytes(int32_t n_tiles) {
+  return ((int64_t)n_tiles * (int64_t)(4 * sizeof(SelState) + 4 * 1024 + 8) + 255) / 256 * 256;
+}
+
 int64_t ahl_sliced_quantile_ws_bytes(int64_t rows, int32_t n_tiles) {
   if (rows <= 0 || n_tiles <= 0) return 0;
-  const int64_t head = ((int64_t)n_tiles * (int64_t)(sizeof(SelState) + 1024) + 255) / 256 * 256;
-  return head + 256 + rows;
+  return select_head_bytes(n_tiles) + rows;
 }
 
 int ahl_sliced_quantile(const void* x, int32_t dtype, int64_t rows, int64_t cols, int64_t ld,
@@ -236,28 +267,26 @@ int ahl_sliced_quantile(const void* x, int32_t dtype, int64_t rows, int64_t cols
   if (rows * (int64_t)widest_tile(tl) > 0xffffffffll) return AHL_ERR_UNSUPPORTED;
   hipStream_t s = (hipStream_t)stream;
   SelState* st = (SelState*)ws;
-  uint32_t* hist = (uint32_t*)(st + n_tiles);
-  const int64_t head = ((int64_t)n_tiles * (int64_t)(sizeof(SelState) + 1024) + 255) / 256 * 256;
-  uint32_t* n_kept = (uint32_t*)((char*)ws + head);
-  uint8_t* kept = (uint8_t*)n_kept + 256;
+  uint32_t* hist = (uint32_t*)(st + 4 * (int64_t)n_tiles);
+  uint32_t* next_key = hist + 4 * (int64_t)n_tiles * 256;
+  uint32_t* has_nan = next_key + n_tiles;
+  uint8_t* kept = (uint8_t*)ws + select_head_bytes(n_tiles);
   const int rpw = select_rpw(rows);
   const int64_t nb = cdiv(cdiv(rows, rpw) * n_tiles, 4);
   if (nb > 0x7fffffff || cdiv(rows, 4) > 0x7fffffff) return AHL_ERR_ARG;
-  hipLaunchKernelGGL(k_fill_u32, dim3(1), dim3(64), 0, s, n_kept, 0u, 1);
+  uint32_t* no_count = nullptr;   // the set-up kernel counts the kept rows from the flags
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(x) && (ld % D::EPV == 0);
-    if (vec) hipLaunchKernelGGL((k_row_nonzero<D, true>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
-    else hipLaunchKernelGGL((k_row_nonzero<D, false>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, n_kept);
-    hipLaunchKernelGGL(k_select_init, dim3(n_tiles), dim3(256), 0, s, st, hist, (const uint32_t*)n_kept, tl, q);
+    if (vec) hipLaunchKernelGGL((k_row_nonzero<D, true>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, no_count);
+    else hipLaunchKernelGGL((k_row_nonzero<D, false>), dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, s, x, rows, cols, ld, kept, no_count);
+    hipLaunchKernelGGL(k_select_init, dim3(n_tiles), dim3(256), 0, s, st, hist, next_key, has_nan, (const uint8_t*)kept, rows, tl, q);
     for (int pass = 0; pass < 4; ++pass) {
-      if (vec) hipLaunchKernelGGL((k_select_hist<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist);
-      else hipLaunchKernelGGL((k_select_hist<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist);
-      hipLaunchKernelGGL(k_select_pick, dim3(n_tiles), dim3(256), 0, s, st, hist, pass);
+      if (vec) hipLaunchKernelGGL((k_select_hist<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist, has_nan, next_key);
+      else hipLaunchKernelGGL((k_select_hist<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, pass, st, hist, has_nan, next_key);
     }
-    if (vec) hipLaunchKernelGGL((k_select_next<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, st);
-    else hipLaunchKernelGGL((k_select_next<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, (const uint8_t*)kept, tl, rpw, st);
   });
-  hipLaunchKernelGGL(k_select_final, dim3((unsigned)cdiv(n_tiles, 64)), dim3(64), 0, s, (const SelState*)st, n_tiles, out);
+  hipLaunchKernelGGL(k_select_final, dim3((unsigned)n_tiles), dim3(64), 0, s, (const SelState*)st,
+                     (const uint32_t*)hist, (const uint32_t*)next_key, (const uint32_t*)has_nan, out);
   return check_launch("ahl_sliced_quantile");
 }
 

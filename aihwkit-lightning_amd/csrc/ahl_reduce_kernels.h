@@ -64,8 +64,9 @@ static __global__ void k_fill_u32(uint32_t* p, uint32_t v, int n) {
 }
 
 // kept[r] = 1 unless every element of row r is zero (-0.0 counts as zero, NaN does not);
-// *n_kept += number of kept rows. One wave per row, one atomic per block (atomics on one
-// address are served one after the other: a per-row atomic cost more than reading the rows).
+// *n_kept += number of kept rows (n_kept may be null: flags only). One wave per row, one atomic
+// per block (atomics on one address are served one after the other: a per-row atomic cost more
+// than reading the rows).
 template <class D, bool VEC>
 __global__ __launch_bounds__(256) void k_row_nonzero(const void* __restrict__ x, int64_t rows,
                                                      int64_t cols, int64_t ld,
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(256) void k_row_nonzero(const void* __restrict__ x,
   __syncthreads();
   if (threadIdx.x == 0) {
     const uint32_t n = wave_kept[0] + wave_kept[1] + wave_kept[2] + wave_kept[3];
-    if (n) atomicAdd(n_kept, n);
+    if (n && n_kept != nullptr) atomicAdd(n_kept, n);
   }
 }
 

@@ -81,7 +81,7 @@ def build_layer():
     return layer, x, g
 
 
-def _analog_cfg(tile, noise=True):
+def _analog_cfg(tile, noise=True, out_noise=0.04):
     from aihwkit_lightning.simulator.configs import (
         TorchInferenceRPUConfig, WeightClipType, WeightNoiseInjectionType,
     )
@@ -91,7 +91,7 @@ def _analog_cfg(tile, noise=True):
     cfg.forward.inp_res = 254
     cfg.forward.out_res = 254
     cfg.forward.out_bound = 10.0
-    cfg.forward.out_noise = 0.04 if noise else 0.0
+    cfg.forward.out_noise = out_noise if noise else 0.0
     cfg.clip.type = WeightClipType.LAYER_GAUSSIAN_PER_CHANNEL
     cfg.clip.sigma = 2.5
     if noise:
@@ -114,7 +114,8 @@ OTHER_WORKLOADS = {
     "fwd_dynamic_4096": "AnalogLinear 4096->4096 bf16, 8192 tokens, 8 tiles x 512, dynamic per-token "
                         "per-tile input range, 8-bit DAC/ADC, out_noise 0.04, forward only",
     "mlp_3072_8192": "LLaMA-style MLP block, hidden 3072, intermediate 8192, SiLU gating, three "
-                     "AnalogLinear layers, bf16, 4096 tokens, tiles of 512, fwd+bwd",
+                     "AnalogLinear layers, bf16, 4096 tokens, tiles of 512, learned input range, 8-bit "
+                     "DAC/ADC, out_noise 0.067, fwd+bwd",
     "lstm_1024": "AnalogRNN, 2 LSTM layers 1024->1024 bf16, 64 steps x 64 sequences, tiles of 512, "
                  "fwd+bwd through time",
     "lstm_1024_eval": "AnalogRNN, 2 LSTM layers 1024->1024 bf16, 64 steps x 64 sequences, tiles of "
@@ -150,8 +151,11 @@ def build_other(name):
         class Mlp(torch.nn.Module):
             def __init__(self):
                 super().__init__()
-                mk = lambda k, n: AnalogLinear(k, n, bias=False, dtype=torch.bfloat16,  # noqa: E731
-                                               rpu_config=_analog_cfg(512))
+                def mk(k, n):   # learned range, 8-bit DAC/ADC, out_noise 0.067, no weight noise
+                    cfg = _analog_cfg(512, noise=False)
+                    cfg.forward.out_noise = 0.067
+                    return AnalogLinear(k, n, bias=False, dtype=torch.bfloat16, rpu_config=cfg)
+
                 self.gate, self.up, self.down = mk(3072, 8192), mk(3072, 8192), mk(8192, 3072)
 
             def forward(self, inp):
@@ -456,11 +460,11 @@ def hbm_kernel_rooflines(reps):
             nxt(ws), in_sizes, L.AHL_QUANT_DISCRETIZE_PER_CHANNEL, 254.0), 2 * wb),
         "dac(x bf16 8192x3072)": (lambda: OPS.dac(nxt(xbs), irb, in_sizes, icfg, fcfg),
                                   2 * xbs[0].numel() * 2),
-        # calibration statistics: row filter + sums (2 reads); row filter + 4 digit histograms +
-        # successor pass of the radix selection (6 reads)
+        # calibration statistics: row filter + sums (2 reads); row filter + 4 digit histograms of
+        # the radix selection (5 reads)
         "sliced_std_kept(x)": (lambda: OPS.sliced_std_kept(nxt(xs), in_sizes), 2 * xbytes),
         "sliced_quantile(x, 0.99995)": (lambda: OPS.sliced_quantile(nxt(xs), in_sizes, 0.99995),
-                                        6 * xbytes),
+                                        5 * xbytes),
         # patch extraction and fold of a 3x3 convolution, 64 x 256 x 28 x 28 bf16 (231 MB of patches)
         "im2col(3x3, 256 ch)": (lambda: OPS.im2col(nxt(imgs), geom), patch_bytes + img_bytes),
         "col2im(3x3, 256 ch)": (lambda: OPS.col2im(nxt(patches), geom), patch_bytes + img_bytes),
