@@ -3,6 +3,7 @@
 ``nn/modules/linear.py:120-135`` / ``triton_utils/triton_linear.py:446-764``), with the
 semantics of the reference's torch-mode (``torch_utils/torch_linear.py:116-314``).
 """
+import itertools
 import os
 from typing import List, Optional
 
@@ -61,6 +62,14 @@ def _ops_for(tensor: Tensor):
     if tensor.device.index == torch.cuda.current_device():
         return _impl
     return _impl.OPS
+
+
+_FLAG_TOKENS = itertools.count(1)
+
+
+def next_flag_token() -> int:
+    """A non-zero 32-bit value that differs from call to call (``AhlLinearCfg.flag_token``)."""
+    return next(_FLAG_TOKENS) % 0xFFFFFFFF + 1
 
 
 class HipLinear(Function):
@@ -250,6 +259,9 @@ class HipLinear(Function):
             L.AHL_IR_GRAD_CLAMP if fast else L.AHL_IR_GRAD_LEARNED,
             stride,
             state_ptr,
+            # what "something was clamped" looks like in this call's one-word flag: a value of
+            # its own per call, so that the forward need not clear the word first
+            next_flag_token(),
         ]
         fcfg = [
             float(fwd.inp_res), float(fwd.out_res), float(fwd.out_bound),

@@ -7,14 +7,14 @@ import ctypes
 import os
 from functools import lru_cache
 from ctypes import (
-    c_void_p, c_int32, c_int64, c_float, c_double, c_uint64, c_char_p, POINTER, Structure,
+    c_void_p, c_int32, c_uint32, c_int64, c_float, c_double, c_uint64, c_char_p, POINTER, Structure,
 )
 
 from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 12
+ABI_VERSION = 13
 STATIC_DX_SCRATCH_BYTES = 16 * 1024 * 1024
 
 AHL_F32, AHL_BF16, AHL_F16 = 0, 1, 2
@@ -52,6 +52,7 @@ class AhlLinearCfg(Structure):
         ("ir_input_min_percentage", c_float),
         ("ir_grad_rule", c_int32),
         ("tile_stride", c_int32),
+        ("flag_token", c_uint32),
         ("seed", c_uint64),
         ("offset", c_uint64),
         ("seed_state", c_void_p),

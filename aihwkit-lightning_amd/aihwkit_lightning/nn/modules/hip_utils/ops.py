@@ -109,6 +109,9 @@ def _linear_cfg(dtype: torch.dtype, icfg: List[int], fcfg: List[float]) -> L.Ahl
     cfg.tile_stride = icfg[8] if len(icfg) > 8 else 0
     # device address of the noise state {key, call counter} (0: the seed comes by value)
     cfg.seed_state = (icfg[9] or None) if len(icfg) > 9 else None
+    # what "something was clamped" looks like in the forward's one-word flag (0: the library
+    # clears the word itself with a launch of its own and uses "non-zero")
+    cfg.flag_token = icfg[10] if len(icfg) > 10 else 0
     (cfg.inp_res, cfg.out_res, cfg.out_bound, cfg.out_noise, cfg.ir_decay,
      cfg.ir_input_min_percentage) = fcfg
     cfg.seed, cfg.offset = seed, offset

@@ -65,6 +65,13 @@ AHL_DEV void block_to_tile(int64_t bid, int64_t nb, int64_t nbm, int64_t nbn, in
 AHL_DEV int64_t clamp_rows(int64_t M) { return (M + 63) & ~(int64_t)63; }
 AHL_DEV int64_t clamp_plane_words(int64_t M, int64_t N) { return ((N + 31) >> 5) * clamp_rows(M); }
 AHL_DEV int64_t clamp_word(int64_t m, int64_t n, int64_t M) { return (n >> 5) * clamp_rows(M) + m; }
+// Whether the forward's one-word flag says that some output was clamped (no flag: assume so).
+// token 0: the forward cleared the word and set it non-zero; otherwise it stored the token.
+AHL_DEV bool clamp_flag_says_clamped(const uint32_t* flag, uint32_t token) {
+  if (flag == nullptr) return true;
+  const uint32_t v = *flag;
+  return token ? v == token : v != 0u;
+}
 
 // ---------------------------------------------------------------------------------------------
 // bf16 <-> f32

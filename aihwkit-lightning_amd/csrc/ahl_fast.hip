@@ -393,8 +393,8 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
   // most waves find the flag already set and skip the atomic (atomics on one address are served
   // one after the other)
   if (a.clamp_flag != nullptr && __any(any_clamp != 0u) && lane == 0 &&
-      __hip_atomic_load(a.clamp_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u)
-    atomicOr(a.clamp_flag, 1u);
+      __hip_atomic_load(a.clamp_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != a.flag_value)
+    __hip_atomic_store(a.clamp_flag, a.flag_value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   // ---- store y = total (+ bias): transposed through LDS, 16-byte row-contiguous stores ----
   {
@@ -549,7 +549,10 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   a.step_factor = !adc ? 0.0f : states ? 2.0f / cfg->out_res : 2.0f * cfg->out_res;
   a.seed = cfg->seed; a.offset = cfg->offset; a.seed_state = cfg->seed_state;
   if (cdiv(M, 128) * cdiv(N, 64) > 0x7fffffff) return AHL_ERR_ARG;
-  if (clamp_flag) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);
+  // the caller's token needs no cleared word: whatever the word holds, it is not the token
+  // (or it is by accident, and the backward then applies a mask that clamps nothing)
+  a.flag_value = cfg->flag_token ? cfg->flag_token : 1u;
+  if (clamp_flag && !cfg->flag_token) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(1), 0, s, clamp_flag);
   // 128 x 128 blocks (NBJ = 2). Measured alternatives: 128 x 64 blocks (NBJ = 1, three to four
   // blocks per CU) are ~10 % slower, 256 x 128 blocks (one block of 8 waves per CU) ~15 % slower.
   // When those are too few to give every CU a block (few rows: a recurrent step, a small batch),

@@ -38,6 +38,7 @@ struct BwdArgs {
   const uint16_t* g; int64_t ldg;      // [M, N]
   const uint32_t* keep;                // clamp mask [T, ceil(N/32), M] or null
   const uint32_t* clamp_flag;          // null or the forward's flag
+  uint32_t flag_token;                 // 0: "clamped" reads non-zero; else: reads this value
   const uint16_t* b; int64_t ldb;      // DX: W_eff [N, K]; DW: xq [M, K]
   const uint16_t* x; int64_t ldx;      // DX static range: the forward input [M, K]
   const uint16_t* ir;                  // DX static range: [T]
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   const int t = (int)(c0 / a.tile);
   const int64_t R = MODE == MODE_DX ? a.M : a.N;      // output rows
   const int64_t L = MODE == MODE_DX ? a.N : a.M;      // contraction length
-  const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
+  const bool use_keep = a.keep != nullptr && clamp_flag_says_clamped(a.clamp_flag, a.flag_token);
   const uint32_t* plane = use_keep ? a.keep + (int64_t)t * clamp_plane_words(a.M, a.N) : nullptr;
 
   f32x16 acc[4][2];
@@ -621,7 +622,7 @@ int64_t fast_dx_ws_bytes(int64_t M, int64_t K, int64_t N) {
 }
 
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
-                   const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
+                   uint32_t flag_token, const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, void* ws, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
                    hipStream_t s) {
@@ -632,7 +633,7 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   a.dense_tile = dense_tile;
   a.dense_base = dense ? dense->base : 0;
   a.dense_extra = dense ? dense->extra : 0;
-  a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
+  a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = flag_token;
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
   a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = ir_static;
@@ -675,13 +676,13 @@ int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N) {
 }
 
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
-                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
+                   uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
                    hipStream_t s) {
   BwdArgs a;
   const int slices = fast_dw_slices(M, K, N);
   float* bias_partial = (float*)ws;
-  a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag;
+  a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = flag_token;
   a.b = (const uint16_t*)xq; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;
   a.out = (uint16_t*)dw; a.ldo = lddw; a.partial = nullptr;
   a.bias_partial = dbias ? bias_partial : nullptr;

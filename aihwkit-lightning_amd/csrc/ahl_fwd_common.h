@@ -19,7 +19,8 @@ struct FastFwdArgs {
   const void* bias;
   void* y; int64_t ldy;
   uint32_t* keep;                // clamp mask [T, ceil(N/32), M] or null
-  uint32_t* clamp_flag;          // set to non-zero if any tile output was clamped; may be null
+  uint32_t* clamp_flag;          // receives flag_value if any tile output was clamped; may be null
+  uint32_t flag_value;           // the caller's token, or 1 for a word the launcher cleared
   const void* ir;                // [T] static, [T, M] dynamic
   const void* wmax;              // [T, N]
   const float* tile_max;         // [T]

@@ -475,8 +475,8 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
 
   // most waves find the flag already set and skip the atomic
   if (a.clamp_flag != nullptr && __any(any_clamp != 0u) && lane == 0 &&
-      __hip_atomic_load(a.clamp_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u)
-    atomicOr(a.clamp_flag, 1u);
+      __hip_atomic_load(a.clamp_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != a.flag_value)
+    __hip_atomic_store(a.clamp_flag, a.flag_value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 
   // ---- store y = total (+ bias): transposed through LDS, 16-byte row-contiguous stores ----
   {

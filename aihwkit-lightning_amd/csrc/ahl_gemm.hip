@@ -363,6 +363,7 @@ struct DxArgs {
   const void* g; int64_t ldg;
   const uint32_t* keep;
   const uint32_t* clamp_flag;
+  uint32_t flag_token;
   const void* wt;  // w_eff_t [K, N]
   const void* x; int64_t ldx;
   const void* ir;
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dx(DxArgs a) {
   const int64_t m0 = (logical / nkb) * kBM;
   int t; int32_t c0, c1;
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
-  const bool use_keep = a.keep != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
+  const bool use_keep = a.keep != nullptr && clamp_flag_says_clamped(a.clamp_flag, a.flag_token);
   const uint32_t* plane =
       use_keep ? a.keep + (int64_t)t * clamp_plane_words(a.M, a.N) : nullptr;
 
@@ -550,6 +551,7 @@ struct DwArgs {
   const void* gt;       // [N, M]
   const uint32_t* keept; // the clamp mask in its native layout, or null
   const uint32_t* clamp_flag;
+  uint32_t flag_token;
   const void* xqt;      // [K, M]
   void* dw; int64_t lddw;
   int64_t M, N, K;
@@ -572,7 +574,7 @@ __global__ __launch_bounds__(256) void k_linear_bwd_dw(DwArgs a) {
   const int64_t n0 = (logical / nkb) * kBM;
   int t; int32_t c0, c1;
   decode_kblock(a.tl, a.kb_big, a.kb_small, (int32_t)(logical % nkb), t, c0, c1);
-  const bool use_keep = a.keept != nullptr && (a.clamp_flag == nullptr || *a.clamp_flag != 0u);
+  const bool use_keep = a.keept != nullptr && clamp_flag_says_clamped(a.clamp_flag, a.flag_token);
   const uint32_t* plane =
       use_keep ? a.keept + (int64_t)t * clamp_plane_words(a.M, a.N) : nullptr;
 
@@ -708,14 +710,14 @@ int64_t fast_fwd_ws_bytes(int64_t M, int64_t N, int32_t n_tiles);
 __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N);
 int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
-                   const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
+                   uint32_t flag_token, const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, void* ws, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
                    hipStream_t s);
 int64_t fast_dx_ws_bytes(int64_t M, int64_t K, int64_t N);
 int64_t fast_dx_row_blocks(int64_t M, int64_t K, int64_t N, bool element_mode);
 int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
-                   const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
+                   uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
                    hipStream_t s);
 int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N);
@@ -811,7 +813,8 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   const dim3 grid((unsigned)nb);
   // this kernel does not track clamping: tell the backward to honour the mask
-  if (clamp_flag) hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, s, clamp_flag, 1u);
+  if (clamp_flag)
+    hipLaunchKernelGGL(k_set_u32, dim3(1), dim3(1), 0, s, clamp_flag, cfg->flag_token ? cfg->flag_token : 1u);
   if (cfg->dtype == AHL_F32) launch_fwd<F32>(a, cfg->ir_mode, grid, s);
   else if (cfg->dtype == AHL_F16) launch_fwd<F16>(a, cfg->ir_mode, grid, s);
   else launch_fwd<BF16>(a, cfg->ir_mode, grid, s);
@@ -885,7 +888,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     // the element-wise epilogue addresses x and dx with one offset and aligns its vectors on dx
     if (!vectors && (!aligned16(dx) || (is_static && (!aligned16(x) || ldx != lddx))))
       return AHL_ERR_UNSUPPORTED;
-    const int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, ws,
+    const int rc = launch_fast_dx(g, ldg, keep, clamp_flag, cfg->flag_token, w_eff, ldw, x, ldx, ir, dx, lddx, ws,
                                   M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0,
                                   vectors ? tl.base : 0, vectors ? nullptr : &tl, s);
     if (rc != AHL_OK) return rc;
@@ -903,7 +906,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
                     (!keep || aligned16(keep)) &&
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
-    int rc = launch_fast_dx(g, ldg, keep, clamp_flag, w_eff, ldw, x, ldx, ir, dx, lddx, ws, M, K,
+    int rc = launch_fast_dx(g, ldg, keep, clamp_flag, cfg->flag_token, w_eff, ldw, x, ldx, ir, dx, lddx, ws, M, K,
                             N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, nullptr, s);
     if (rc != AHL_OK) return rc;
     if (is_static) {
@@ -917,7 +920,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     return check_launch("ahl_linear_bwd_dx(fast)");
   }
   DxArgs a;
-  a.g = g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.wt = wt; a.x = x; a.ldx = ldx;
+  a.g = g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = cfg->flag_token; a.wt = wt; a.x = x; a.ldx = ldx;
   a.ir = ir; a.dx = dx; a.lddx = lddx; a.partial = partial; a.M = M; a.N = N; a.K = K; a.tl = tl;
   a.ir_rule = cfg->ir_grad_rule;
   kblocks(tl, &a.kb_big, &a.kb_small);
@@ -1034,14 +1037,14 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
       return AHL_ERR_UNSUPPORTED;
     void* dwp = (char*)ws + align256(fast_dw_ws_bytes(M, padded, N));
     const Tiling ptl{n_tiles, (int32_t)stride, 0};
-    const int rc = launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dwp, padded, dbias, ws, M,
+    const int rc = launch_fast_dw(g, ldg, keep, clamp_flag, cfg->flag_token, xq, ldxq, dwp, padded, dbias, ws, M,
                                   padded, N, ptl, s);
     if (rc != AHL_OK) return rc;
     return launch_unpad_tiles(dwp, padded, AHL_BF16, N, K, tl, stride, dw, lddw, s);
   }
   if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
       ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && aligned16(dw) && (!keep || aligned16(keep)))
-    return launch_fast_dw(g, ldg, keep, clamp_flag, xq, ldxq, dw, lddw, dbias, ws, M, K, N, tl, s);
+    return launch_fast_dw(g, ldg, keep, clamp_flag, cfg->flag_token, xq, ldxq, dw, lddw, dbias, ws, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
   DwArgs a;
   a.M = M; a.N = N; a.K = K; a.tl = tl; a.dw = dw; a.lddw = lddw;
@@ -1066,7 +1069,7 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
       hipLaunchKernelGGL((k_dac_transpose<D, 1>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
     else
       hipLaunchKernelGGL((k_dac_transpose<D, 2>), tgrid_x, dim3(256), 0, s, x, M, K, ldx, ir, tl, cfg->inp_res, dac_on, cfg->skip_rounding, (void*)xqt);
-    a.gt = gt; a.keept = keept; a.xqt = xqt; a.clamp_flag = clamp_flag;
+    a.gt = gt; a.keept = keept; a.xqt = xqt; a.clamp_flag = clamp_flag; a.flag_token = cfg->flag_token;
     const bool vec = M % D::EPV == 0;
     const dim3 grid((unsigned)(nbn * nkb)), block(256);
     if (vec) hipLaunchKernelGGL((k_linear_bwd_dw<D, true>), grid, block, kGemmLds, s, a);

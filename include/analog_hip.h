@@ -87,6 +87,14 @@ typedef struct AhlLinearCfg {
   int32_t ir_grad_rule;          /* AHL_IR_GRAD_*: which backward the static range clamp has     */
   int32_t tile_stride;           /* 0: xq and w_eff are dense [rows, K]. > 0: they are in the
                                     padded tile layout with this stride (see ahl_tile_stride)    */
+  uint32_t flag_token;           /* what "something was clamped" looks like in the one-word
+                                    clamp_flag. 0: ahl_linear_fwd clears the word (one small
+                                    launch) and sets it non-zero; the backward entry points read
+                                    "non-zero". != 0: the forward stores this value and clears
+                                    nothing, the backward reads "equal to this value" -- pass the
+                                    same cfg to both, and a value that differs from call to call:
+                                    a stale or accidental match only makes the backward apply a
+                                    mask that clamps nothing                                     */
   uint64_t seed;                 /* Philox key for this call                                    */
   uint64_t offset;               /* Philox counter offset for this call                         */
   const uint64_t* seed_state;    /* NULL, or a DEVICE uint64[2] = {key, call counter}: the kernels

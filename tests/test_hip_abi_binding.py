@@ -15,7 +15,7 @@ reference's slot it returns the output without bias.
 """
 import ctypes
 import os
-from ctypes import POINTER, byref, c_float, c_int32, c_int64, c_uint64, c_void_p
+from ctypes import POINTER, byref, c_float, c_int32, c_int64, c_uint32, c_uint64, c_void_p
 
 import pytest
 import torch
@@ -33,8 +33,8 @@ class AhlLinearCfg(ctypes.Structure):          # struct AhlLinearCfg of include/
                 ("out_noise_per_channel", c_int32), ("bound_per_channel", c_int32),
                 ("training", c_int32), ("skip_rounding", c_int32), ("ir_decay", c_float),
                 ("ir_input_min_percentage", c_float), ("ir_grad_rule", c_int32),
-                ("tile_stride", c_int32), ("seed", c_uint64), ("offset", c_uint64),
-                ("seed_state", c_void_p)]
+                ("tile_stride", c_int32), ("flag_token", c_uint32), ("seed", c_uint64),
+                ("offset", c_uint64), ("seed_state", c_void_p)]
 
 
 class AhlModifierCfg(ctypes.Structure):        # struct AhlModifierCfg
@@ -115,7 +115,7 @@ class HipSlotLinear(torch.autograd.Function):
         cfg = AhlLinearCfg(dt, ir_mode, fwd.inp_res, fwd.out_res, fwd.out_bound,
                            fwd.out_noise if training else 0.0, int(fwd.out_noise_per_channel),
                            int(per_channel), int(training), 0, irp.decay, irp.input_min_percentage,
-                           0, 0, seed, 0, None)
+                           0, 0, seed % 0xFFFFFFFF + 1, seed, 0, None)   # flag_token: new per call
         # input: clamp to the range + DAC in one pass (the dynamic ranges come out of it)
         xq = new(m_rows, k_in)
         ir = input_range.detach().contiguous() if ir_mode == AHL_IR_STATIC else None

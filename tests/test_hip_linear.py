@@ -493,3 +493,49 @@ def test_counter_left_at_minus_infinity_means_the_ranges_are_set(dtype):
     out = fresh(x.cuda())
     assert bool(torch.isfinite(out.float()).all())
     assert torch.equal(fresh.input_range.data.cpu().float(), torch.full((2,), 1.5))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("clamps", [False, True], ids=["nothing_clamped", "some_clamped"])
+def test_clamp_flag_token_and_a_stale_match(dtype, clamps):
+    """The forward's one-word "something was clamped" flag in its two forms: cleared by the
+    library and set non-zero (token 0), or the caller's per-call token stored into a word that
+    nobody cleared. Both give the backward the same answer; and a word that holds the token
+    although nothing was clamped (a stale value in reused memory) only makes the backward apply
+    a mask without bits: the same gradients, bit for bit."""
+    from aihwkit_lightning.nn.modules.hip_utils import library as L
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+
+    gen = torch.Generator().manual_seed(21)
+    m_rows, k_in, n_out, tile = 256, 512, 256, 256
+    in_sizes = [tile] * (k_in // tile)
+    x = torch.randn(m_rows, k_in, generator=gen).to(dtype).cuda()
+    w = (0.05 * torch.randn(n_out, k_in, generator=gen)).to(dtype).cuda()
+    g = torch.randn(m_rows, n_out, generator=gen).to(dtype).cuda()
+    ir = torch.full((len(in_sizes),), 3.0).to(dtype).cuda()
+    out_bound = 1.0 if clamps else 1000.0
+    fcfg = [254.0, 254.0, out_bound, 0.0, 0.01, 0.95]
+    wmax, tile_max, _, _ = OPS.weight_prep(w, in_sizes, 0, 0, 1.0, 0.0, 0, 0, False, False)
+
+    def run(token, overwrite_flag=None):
+        icfg = [L.AHL_IR_STATIC, 0, 1, 1, 0, 0, 0, L.AHL_IR_GRAD_LEARNED, 0, 0, token]
+        xq, _ = OPS.dac(x, ir, in_sizes, icfg, fcfg)
+        y, keep, flag = OPS.linear_fwd(x, xq, w, None, ir, wmax, tile_max, in_sizes, icfg, fcfg, True)
+        if overwrite_flag is not None:
+            flag.fill_(overwrite_flag)
+        dx, ir_grad = OPS.linear_bwd_dx(g, keep, flag, w, x, ir, in_sizes, icfg, fcfg)
+        dw, dbias = OPS.linear_bwd_dw(g, keep, flag, None, xq, ir, in_sizes, icfg, fcfg, True)
+        return y, keep, int(flag.item()), dx, ir_grad, dw, dbias
+
+    classic = run(0)
+    token = 0x5EED1234
+    tokened = run(token)
+    if dtype == torch.bfloat16:   # the MFMA kernels of the bf16 path track clamping; the general
+        assert (classic[2] != 0) == clamps   # kernels always tell the backward to honour the mask
+    assert (tokened[2] == token) or not clamps
+    if clamps:
+        assert bool((classic[1] != 0).any())
+    stale = run(token, overwrite_flag=token)   # the word says "clamped" whatever happened
+    for a, b, c in zip(classic, tokened, stale):
+        if isinstance(a, torch.Tensor):
+            assert torch.equal(a, b) and torch.equal(a, c)
