@@ -162,6 +162,9 @@ def build_other(name):
                 return self.down(torch.nn.functional.silu(self.gate(inp)) * self.up(inp))
 
         layer = Mlp()
+        for lin in (layer.gate, layer.up, layer.down):   # W ~ N(0, 0.02^2) like the other workloads
+            lin.set_weights_and_biases(
+                (0.02 * torch.randn(lin.out_features, lin.in_features, generator=gen)).to(torch.bfloat16), None)
         x = torch.randn(4096, 3072, generator=gen).to(torch.bfloat16)
         g = torch.randn(4096, 3072, generator=gen).to(torch.bfloat16)
         flops = 3 * 3 * 2.0 * 4096 * 3072 * 8192
