@@ -64,6 +64,9 @@ def _ops_for(tensor: Tensor):
     return _impl.OPS
 
 
+# dtypes with MFMA kernels of their own (two-byte elements); float32 runs on the general kernels
+MFMA16_DTYPES = (torch.bfloat16, torch.float16)
+
 _FLAG_TOKENS = itertools.count(1)
 
 
@@ -214,7 +217,7 @@ class HipLinear(Function):
                 if reuse is not None:
                     reuse[stats_key] = (wmax, tile_max)
 
-        # bf16 layers whose output width is not a multiple of 8 (a 50257-word vocabulary): the
+        # 16-bit layers whose output width is not a multiple of 8 (a 50257-word vocabulary): the
         # MFMA kernels handle channels in whole 16-byte vectors, so the weight-side operands get
         # zero channels up to the next multiple of 8 and the extra output columns are dropped.
         # (Their per-channel abs-max is set to 1 so that their ADC step is not 0; nothing of them
@@ -222,7 +225,7 @@ class HipLinear(Function):
         # more than they save.
         pad_n = 0
         bias_k = bias
-        if (inp.dtype == torch.bfloat16 and n_out % 8 != 0 and not learned_clip
+        if (inp.dtype in MFMA16_DTYPES and n_out % 8 != 0 and not learned_clip
                 and m_rows * k_in * n_out >= PAD_CHANNELS_MIN_WORK):
             pad_n = 8 - n_out % 8
             frozen = weight_cache if w_eff is weights_c else None  # no per-call modifier
@@ -239,13 +242,13 @@ class HipLinear(Function):
         n_k = n_out + pad_n
         weights_frozen = weight_cache is not None and not (w_noise or w_quant or learned_clip)
 
-        # bf16 splits whose tiles do not start on the MFMA kernels' 256-column block boundaries:
+        # 16-bit splits whose tiles do not start on the MFMA kernels' 256-column block boundaries:
         # the quantised input and the effective weights are kept in a padded tile layout instead
         # (stride > 0), unless the padding would blow the work up more than the slower general
         # kernels do, or the shape does not fit the fast backward at all
         stride = 0
         dense_fwd_ok = len(set(in_sizes)) == 1 and in_sizes[0] % 64 == 0
-        if (inp.dtype == torch.bfloat16 and m_rows > 0 and n_k % 8 == 0
+        if (inp.dtype in MFMA16_DTYPES and m_rows > 0 and n_k % 8 == 0
                 and w_eff.data_ptr() % 16 == 0):
             stride = tile_stride(k_in, len(in_sizes), inp.dtype)
             if stride * len(in_sizes) > 4 * k_in or (dense_fwd_ok and not (need_dx or need_dw)):
@@ -277,10 +280,10 @@ class HipLinear(Function):
                 (ctx.needs_input_grad[i] for i in (0, 1, 2, 3, 11)))]
             return inp.new_zeros(out_shape)
 
-        # bf16 with equal tiles of a multiple of 64 inputs: clamp + DAC (+ dynamic abs-max) run as
+        # 16-bit dtypes with equal tiles of a multiple of 64 inputs: clamp + DAC (+ dynamic abs-max) run as
         # one memory-bound pass and the matrix kernel streams the quantised input; otherwise the
         # clamp + DAC are fused into the matrix kernel's A-tile staging.
-        split_dac = stride > 0 or (inp.dtype == torch.bfloat16 and dense_fwd_ok and n_k % 8 == 0)
+        split_dac = stride > 0 or (inp.dtype in MFMA16_DTYPES and dense_fwd_ok and n_k % 8 == 0)
         if stride > 0:
             tiles_key = ("tiles", stride, pad_n)
             if weights_frozen and tiles_key in weight_cache:

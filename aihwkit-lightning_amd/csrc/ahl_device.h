@@ -140,6 +140,13 @@ struct BF16 {
   // x * fl32(1/d) to bf16 gives bit-identical results to rounding fl32(x / d). The caller
   // rounds the returned value with rd().
   static AHL_DEV float div(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
+  // two values as one register of 16-bit halves (rounded to nearest even), and back
+  static AHL_DEV uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+  static AHL_DEV float lo(uint32_t w) { return unpack_lo(w); }
+  static AHL_DEV float hi(uint32_t w) { return unpack_hi(w); }
+  // state counts of a quantiser with <= 8 significant bits give the same step whether it is
+  // computed as 2 B / n or as B * fl(2 / n) (see div)
+  static constexpr int kExactStepBits = 8;
 };
 
 // float16: like bfloat16, every elementwise result is rounded to the tensor dtype (round to
@@ -170,9 +177,13 @@ struct F16 {
     asm("v_cvt_f32_f16 %0, %1" : "=v"(r) : "v"(h));
     return r;
   }
-  static AHL_DEV elem to_elem(float x) { return __builtin_bit_cast(uint16_t, (_Float16)x); }
+  static AHL_DEV elem to_elem(float x) {
+    uint32_t h;
+    asm("v_cvt_f16_f32 %0, %1" : "=v"(h) : "v"(x));
+    return (elem)h;
+  }
   static AHL_DEV float load(const void* p, int64_t i) { return (float)((const _Float16*)p)[i]; }
-  static AHL_DEV void store(void* p, int64_t i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
+  static AHL_DEV void store(void* p, int64_t i, float v) { ((elem*)p)[i] = to_elem(v); }
   static AHL_DEV void unpack(const u32x4& v, float* f) {
     f[0] = f16_lo(v.x); f[1] = f16_hi(v.x); f[2] = f16_lo(v.y); f[3] = f16_hi(v.y);
     f[4] = f16_lo(v.z); f[5] = f16_hi(v.z); f[6] = f16_lo(v.w); f[7] = f16_hi(v.w);
@@ -185,6 +196,52 @@ struct F16 {
   // 11-bit significands: the product with an approximate reciprocal can land on the other side
   // of a rounding boundary, so the IEEE quotient is taken (the caller rounds it with rd()).
   static AHL_DEV float div(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
+  // the packing conversion as an instruction, for the reason given at rd()
+  static AHL_DEV uint32_t pack2(float lo, float hi) {
+    uint32_t w;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(w) : "v"(lo), "v"(hi));
+    return w;
+  }
+  static AHL_DEV float lo(uint32_t w) { return f16_lo(w); }
+  static AHL_DEV float hi(uint32_t w) { return f16_hi(w); }
+  static constexpr int kExactStepBits = 0;   // the quantiser's step always by division
+};
+
+// round two fp32 values to the 16-bit dtype D, keeping them in fp32 registers (3 instructions)
+template <class D>
+AHL_DEV void round2(float& a, float& b) {
+  const uint32_t p = D::pack2(a, b);
+  a = D::lo(p);
+  b = D::hi(p);
+}
+
+// ---- MFMA wrappers: one 32 x 32 x 16 product of 16-bit operands (8 per lane) ----
+typedef _Float16 f16x8m __attribute__((ext_vector_type(8)));
+template <class D>
+struct Mma16;
+template <>
+struct Mma16<BF16> {
+  static AHL_DEV void run(const u32x4& a, const u32x4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+  static AHL_DEV void run_zero(const u32x4& a, const u32x4& b, f32x16& c) {   // c = a x b
+    const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                __builtin_bit_cast(bf16x8, b), z, 0, 0, 0);
+  }
+};
+template <>
+struct Mma16<F16> {
+  static AHL_DEV void run(const u32x4& a, const u32x4& b, f32x16& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8m, a),
+                                               __builtin_bit_cast(f16x8m, b), c, 0, 0, 0);
+  }
+  static AHL_DEV void run_zero(const u32x4& a, const u32x4& b, f32x16& c) {
+    const f32x16 z = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8m, a),
+                                               __builtin_bit_cast(f16x8m, b), z, 0, 0, 0);
+  }
 };
 
 static constexpr float kTinyF32 = 1.17549435e-38f;  // finfo(float32).tiny == finfo(bfloat16).tiny

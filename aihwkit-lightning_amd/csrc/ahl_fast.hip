@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void k_dac_rows(const void* __restrict__ x, in
 // QM, what happens to a tile's outputs after the noise: 0 nothing, 1 clamp at the bound, 2 ADC
 // quantisation and clamp, 3 the same without the rounding step (skip_rounding). Compile-time, so
 // that the per-group epilogue has no branches apart from the rare "something left the range".
-template <int IRMODE, bool NOISE, int QM, int NBJ>
+template <class D, int IRMODE, bool NOISE, int QM, int NBJ>
 __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs a) {
   constexpr bool ADC = QM >= 2, CLAMP = QM >= 1, ROUND = QM != 3;
   constexpr int BN = 64 * NBJ;   // block columns
@@ -174,10 +174,10 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
       *(u32x4*)(ldsB + (row0 + 32 * j) * kLdsStrideF + cv * 16) = rawB[j];
     if (IRMODE == AHL_IR_DYNAMIC && first && tid < 128) {
       const int64_t m = m0 + tid;
-      const float irm = m < a.M ? BF16::load(a.ir, (int64_t)tt * a.M + m) : 0.0f;
+      const float irm = m < a.M ? D::load(a.ir, (int64_t)tt * a.M + m) : 0.0f;
       float* rc = rowc + (tt & 1) * 384;
-      rc[tid] = BF16::rd(a.noise_scale * irm);
-      rc[128 + tid] = BF16::rd(irm * a.out_bound);
+      rc[tid] = D::rd(a.noise_scale * irm);
+      rc[128 + tid] = D::rd(irm * a.out_bound);
     }
     __syncthreads();
   };
@@ -211,14 +211,14 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
         if (s == 0 && cin == 0) {  // first step of a K-tile starts from zero
 #pragma unroll
           for (int bj = 0; bj < NBJ; ++bj) {
-            mma_bf16_zero(a0, fb[s & 1][bj], acc[0][bj]);
-            mma_bf16_zero(a1, fb[s & 1][bj], acc[1][bj]);
+            Mma16<D>::run_zero(a0, fb[s & 1][bj], acc[0][bj]);
+            Mma16<D>::run_zero(a1, fb[s & 1][bj], acc[1][bj]);
           }
         } else {
 #pragma unroll
           for (int bj = 0; bj < NBJ; ++bj) {
-            mma_bf16(a0, fb[s & 1][bj], acc[0][bj]);
-            mma_bf16(a1, fb[s & 1][bj], acc[1][bj]);
+            Mma16<D>::run(a0, fb[s & 1][bj], acc[0][bj]);
+            Mma16<D>::run(a1, fb[s & 1][bj], acc[1][bj]);
           }
         }
       }
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
     // prefetch registers are dead while the epilogue runs.
     if (ch + 1 < nchunks) { stage(t + 1, true); prestaged = true; }
     // ---------------- per-K-tile epilogue ----------------
-    const float ir_t = IRMODE == AHL_IR_STATIC ? BF16::load(a.ir, t) : 0.0f;
+    const float ir_t = IRMODE == AHL_IR_STATIC ? D::load(a.ir, t) : 0.0f;
     const float tmax = (NOISE || bound_on) ? a.tile_max[t] : 0.0f;
     const float* rc_t = rowc + (t & 1) * 384;
 #pragma unroll
@@ -238,17 +238,17 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
       const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
       const bool nvalid = n < a.N;
       float wch = 0.0f;
-      if ((NOISE || bound_on) && nvalid) wch = BF16::load(a.wmax, (int64_t)t * a.N + n);
+      if ((NOISE || bound_on) && nvalid) wch = D::load(a.wmax, (int64_t)t * a.N + n);
       const float wr = a.noise_per_channel ? wch : tmax;
       const float wb = a.bound_per_channel ? wch : tmax;
       float nscale = 0.0f, B = 0.0f, r = 1.0f, rcp = 1.0f;
       if (IRMODE == AHL_IR_STATIC) {
-        if (NOISE) nscale = BF16::rd(wr * BF16::rd(a.noise_scale * ir_t));
+        if (NOISE) nscale = D::rd(wr * D::rd(a.noise_scale * ir_t));
         if (bound_on) {
-          B = BF16::rd(BF16::rd(ir_t * a.out_bound) * wb);
+          B = D::rd(D::rd(ir_t * a.out_bound) * wb);
           if (ADC) {
-            r = adc_step(B, a);
-            rcp = __fdiv_rn(1.0f, fmaxf(r, kTinyF32));
+            r = adc_step<D>(B, a);
+            rcp = __fdiv_rn(1.0f, fmaxf(r, D::tiny()));
           }
         }
       }
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
             float y[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) y[c] = acc[bi][bj][4 * g + c];
-            rd2(y[0], y[1]); rd2(y[2], y[3]);
+            round2<D>(y[0], y[1]); round2<D>(y[2], y[3]);
             float ns[4], Bv[4], rv[4], rcpv[4];
 #pragma unroll
             for (int c = 0; c < 4; ++c) { ns[c] = nscale; Bv[c] = B; rv[c] = r; rcpv[c] = rcp; }
@@ -294,20 +294,20 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
                 for (int c = 0; c < 4; ++c) Bv[c] = br[c] * wb;
               }
-              if (NOISE) { rd2(ns[0], ns[1]); rd2(ns[2], ns[3]); }
+              if (NOISE) { round2<D>(ns[0], ns[1]); round2<D>(ns[2], ns[3]); }
               if (bound_on) {
-                rd2(Bv[0], Bv[1]); rd2(Bv[2], Bv[3]);
+                round2<D>(Bv[0], Bv[1]); round2<D>(Bv[2], Bv[3]);
                 if (ADC) {
                   if (__builtin_expect(a.step_by_division != 0, 0)) {
 #pragma unroll
-                    for (int c = 0; c < 4; ++c) rv[c] = adc_step(Bv[c], a);
+                    for (int c = 0; c < 4; ++c) rv[c] = adc_step<D>(Bv[c], a);
                   } else {
 #pragma unroll
                     for (int c = 0; c < 4; ++c) rv[c] = Bv[c] * a.step_factor;
-                    rd2(rv[0], rv[1]); rd2(rv[2], rv[3]);
+                    round2<D>(rv[0], rv[1]); round2<D>(rv[2], rv[3]);
                   }
 #pragma unroll
-                  for (int c = 0; c < 4; ++c) rcpv[c] = __builtin_amdgcn_rcpf(fmaxf(rv[c], kTinyF32));
+                  for (int c = 0; c < 4; ++c) rcpv[c] = __builtin_amdgcn_rcpf(fmaxf(rv[c], D::tiny()));
                 }
               }
             }
@@ -316,19 +316,19 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
               // product of the reference to reproduce, and the sum is rounded once
 #pragma unroll
               for (int c = 0; c < 4; ++c) y[c] = __builtin_fmaf(ns[c], xi[4 * gg + c], y[c]);
-              rd2(y[0], y[1]); rd2(y[2], y[3]);
+              round2<D>(y[0], y[1]); round2<D>(y[2], y[3]);
             }
             if (ADC) {
 #pragma unroll
-              for (int c = 0; c < 4; ++c) y[c] *= rcpv[c];
-              rd2(y[0], y[1]); rd2(y[2], y[3]);
+              for (int c = 0; c < 4; ++c) y[c] = D::div(y[c], fmaxf(rv[c], D::tiny()), rcpv[c]);
+              round2<D>(y[0], y[1]); round2<D>(y[2], y[3]);
               if (ROUND) {
 #pragma unroll
                 for (int c = 0; c < 4; ++c) y[c] = rintf(y[c]);
               }
 #pragma unroll
               for (int c = 0; c < 4; ++c) y[c] *= rv[c];
-              rd2(y[0], y[1]); rd2(y[2], y[3]);
+              round2<D>(y[0], y[1]); round2<D>(y[2], y[3]);
             }
             if (CLAMP) {
 #pragma unroll
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
               const uint32_t tp = totp[bi][bj][2 * g + pr];
               tpo[2 * gg + pr] = tp;
               totp[bi][bj][2 * g + pr] =
-                  pack_bf16x2(unpack_lo(tp) + y[2 * pr], unpack_hi(tp) + y[2 * pr + 1]);
+                  D::pack2(D::lo(tp) + y[2 * pr], D::hi(tp) + y[2 * pr + 1]);
             }
           }
           if (CLAMP) {
@@ -365,7 +365,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
               for (int q = 0; q < 4; ++q)
                 totp[bi][bj][4 * gp + q] =
-                    pack_bf16x2(unpack_lo(tpo[q]) + y8[2 * q], unpack_hi(tpo[q]) + y8[2 * q + 1]);
+                    D::pack2(D::lo(tpo[q]) + y8[2 * q], D::hi(tpo[q]) + y8[2 * q + 1]);
               any_clamp |= over ? 1u : 0u;
             }
           }
@@ -405,13 +405,13 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
     for (int bj = 0; bj < NBJ; ++bj) {
       const int64_t n = n0 + wn * WN + bj * 32 + (lane & 31);
       const bool add_bias = a.bias != nullptr && !one_tile;
-      const float b = (add_bias && n < a.N) ? BF16::load(a.bias, n) : 0.0f;
+      const float b = (add_bias && n < a.N) ? D::load(a.bias, n) : 0.0f;
 #pragma unroll
       for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
         for (int pr = 0; pr < 8; ++pr) {
           uint32_t tp = totp[bi][bj][pr];
-          if (add_bias) tp = pack_bf16x2(unpack_lo(tp) + b, unpack_hi(tp) + b);
+          if (add_bias) tp = D::pack2(D::lo(tp) + b, D::hi(tp) + b);
           const int ro = bi * 32 + 8 * (pr >> 1) + 2 * (pr & 1);
           *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)tp;
           *(uint16_t*)(obase + (ro + 1) * kOutStride + bj * 64) = (uint16_t)(tp >> 16);
@@ -436,6 +436,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 
 // y[m, n] = rd(...rd(rd(0 + part[0]) + part[1])... ) (+ bias): the running total of k_fwd_fast over
 // the tiles, for results that were computed one tile per block. One 16-byte vector per thread.
+template <class D>
 __global__ __launch_bounds__(256) void k_tile_sum(const uint16_t* __restrict__ part, int32_t n_tiles,
                                                   int64_t M, int64_t N, const uint16_t* __restrict__ bias,
                                                   uint16_t* __restrict__ y, int64_t ldy) {
@@ -446,17 +447,17 @@ __global__ __launch_bounds__(256) void k_tile_sum(const uint16_t* __restrict__ p
   float tot[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int t = 0; t < n_tiles; ++t) {
     float e[8];
-    BF16::unpack(ld16(part + ((int64_t)t * M + m) * N + n), e);
+    D::unpack(ld16(part + ((int64_t)t * M + m) * N + n), e);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) tot[i] = BF16::rd(tot[i] + e[i]);
+    for (int i = 0; i < 8; ++i) tot[i] = D::rd(tot[i] + e[i]);
   }
   if (bias != nullptr) {
     float b[8];
-    BF16::unpack(ld16(bias + n), b);
+    D::unpack(ld16(bias + n), b);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) tot[i] = BF16::rd(tot[i] + b[i]);
+    for (int i = 0; i < 8; ++i) tot[i] = D::rd(tot[i] + b[i]);
   }
-  st16(y + m * ldy + n, BF16::pack(tot));
+  st16(y + m * ldy + n, D::pack(tot));
 }
 
 __global__ void k_zero_u32(uint32_t* p) { *p = 0u; }
@@ -475,11 +476,11 @@ static int significant_bits(float v) {
   return bits;
 }
 
-template <int IRMODE, int NBJ>
+template <class D, int IRMODE, int NBJ>
 static void launch_fast(const FastFwdArgs& a, bool noise, int qm, hipStream_t s) {
   constexpr int lds_bytes = (128 + 64 * NBJ) * kLdsStrideF + 2 * 384 * (int)sizeof(float);
   const dim3 block(256), grid((unsigned)(cdiv(a.M, 128) * cdiv(a.N, 64 * NBJ) * (a.part ? a.n_tiles : 1)));
-#define AHL_FWD(NZ, Q) hipLaunchKernelGGL((k_fwd_fast<IRMODE, NZ, Q, NBJ>), grid, block, lds_bytes, s, a)
+#define AHL_FWD(NZ, Q) hipLaunchKernelGGL((k_fwd_fast<D, IRMODE, NZ, Q, NBJ>), grid, block, lds_bytes, s, a)
   if (noise) {
     if (qm == 0) AHL_FWD(true, 0); else if (qm == 1) AHL_FWD(true, 1);
     else if (qm == 2) AHL_FWD(true, 2); else AHL_FWD(true, 3);
@@ -488,6 +489,13 @@ static void launch_fast(const FastFwdArgs& a, bool noise, int qm, hipStream_t s)
     else if (qm == 2) AHL_FWD(false, 2); else AHL_FWD(false, 3);
   }
 #undef AHL_FWD
+}
+
+template <class D>
+static void launch_fast_modes(const FastFwdArgs& a, int ir_mode, bool few, bool noise, int qm, hipStream_t s) {
+  if (ir_mode == AHL_IR_NONE) few ? launch_fast<D, 0, 1>(a, noise, qm, s) : launch_fast<D, 0, 2>(a, noise, qm, s);
+  else if (ir_mode == AHL_IR_STATIC) few ? launch_fast<D, 1, 1>(a, noise, qm, s) : launch_fast<D, 1, 2>(a, noise, qm, s);
+  else few ? launch_fast<D, 2, 1>(a, noise, qm, s) : launch_fast<D, 2, 2>(a, noise, qm, s);
 }
 
 namespace ahl {
@@ -510,7 +518,7 @@ int64_t fast_fwd_ws_bytes(int64_t M, int64_t N, int32_t n_tiles) {
 // Whether ahl_linear_fwd can take the bf16 fast path for these arguments.
 bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, const void* w,
                        int64_t ldw, int64_t K, const Tiling& tl) {
-  if (cfg->dtype != AHL_BF16 || xq == nullptr) return false;
+  if ((cfg->dtype != AHL_BF16 && cfg->dtype != AHL_F16) || xq == nullptr) return false;
   if (cfg->out_res > 0.0f && !(cfg->out_bound > 0.0f)) return false;  // an ADC needs its bound
   if (!aligned16(xq) || !aligned16(w) || ldxq % 8 != 0 || ldw % 8 != 0) return false;
   if (cfg->tile_stride > 0) {  // padded tile layout: any split
@@ -545,7 +553,8 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   a.noise_per_channel = cfg->out_noise_per_channel; a.bound_per_channel = cfg->bound_per_channel;
   a.skip_rounding = cfg->skip_rounding; a.clamp_on = cfg->out_bound > 0.0f ? 1 : 0;
   const bool states = cfg->out_res > 1.0f;
-  a.step_by_division = (adc && states && significant_bits(cfg->out_res) > 8) ? 1 : 0;
+  const int exact_bits = cfg->dtype == AHL_F16 ? F16::kExactStepBits : BF16::kExactStepBits;
+  a.step_by_division = (adc && states && significant_bits(cfg->out_res) > exact_bits) ? 1 : 0;
   a.step_factor = !adc ? 0.0f : states ? 2.0f / cfg->out_res : 2.0f * cfg->out_res;
   a.seed = cfg->seed; a.offset = cfg->offset; a.seed_state = cfg->seed_state;
   if (cdiv(M, 128) * cdiv(N, 64) > 0x7fffffff) return AHL_ERR_ARG;
@@ -565,15 +574,22 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   // Large grids go to the kernel that runs a tile's epilogue inside the next tile's product loop
   // (same results bit for bit); AHL_FORWARD_KERNEL=blocks in the environment keeps them here.
   const char* pick = getenv("AHL_FORWARD_KERNEL");
-  if (!(pick != nullptr && strcmp(pick, "blocks") == 0) && pipe_fwd_eligible(a, cfg->ir_mode) &&
+  if (cfg->dtype == AHL_BF16 && !(pick != nullptr && strcmp(pick, "blocks") == 0) &&
+      pipe_fwd_eligible(a, cfg->ir_mode) &&
       launch_pipe_fwd(a, cfg->ir_mode, noise, qm, s))
     return check_launch("ahl_linear_fwd(pipe)");
-  if (cfg->ir_mode == AHL_IR_NONE) few ? launch_fast<0, 1>(a, noise, qm, s) : launch_fast<0, 2>(a, noise, qm, s);
-  else if (cfg->ir_mode == AHL_IR_STATIC) few ? launch_fast<1, 1>(a, noise, qm, s) : launch_fast<1, 2>(a, noise, qm, s);
-  else few ? launch_fast<2, 1>(a, noise, qm, s) : launch_fast<2, 2>(a, noise, qm, s);
-  if (split)
-    hipLaunchKernelGGL(k_tile_sum, dim3((unsigned)cdiv(M * (N / 8), 256)), dim3(256), 0, s, a.part,
-                       tl.n_tiles, M, N, (const uint16_t*)bias, (uint16_t*)y, ldy);
+  const dim3 sum_grid((unsigned)cdiv(M * (N / 8), 256));
+  if (cfg->dtype == AHL_F16) {
+    launch_fast_modes<F16>(a, cfg->ir_mode, few, noise, qm, s);
+    if (split)
+      hipLaunchKernelGGL(k_tile_sum<F16>, sum_grid, dim3(256), 0, s, a.part, tl.n_tiles, M, N,
+                         (const uint16_t*)bias, (uint16_t*)y, ldy);
+  } else {
+    launch_fast_modes<BF16>(a, cfg->ir_mode, few, noise, qm, s);
+    if (split)
+      hipLaunchKernelGGL(k_tile_sum<BF16>, sum_grid, dim3(256), 0, s, a.part, tl.n_tiles, M, N,
+                         (const uint16_t*)bias, (uint16_t*)y, ldy);
+  }
   return check_launch("ahl_linear_fwd(fast)");
 }
 

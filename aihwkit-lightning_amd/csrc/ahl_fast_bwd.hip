@@ -60,10 +60,6 @@ struct BwdArgs {
   float* split;                        // slices > 1: fp32 partial results [slices][rows][K]
 };
 
-AHL_DEV void mma16(const u32x4& a, const u32x4& b, f32x16& c) {
-  c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                              __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-}
 
 // Everything after the product loop: the fp32 partial result of a slice, or the 256 x 256 result
 // written through LDS with the input-range epilogue of the input gradient.
@@ -72,7 +68,7 @@ struct BwdPos {
   int t, slice;
 };
 
-template <int MODE>
+template <class D, int MODE>
 AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2], char* lds,
                         float (*red)[3]) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -102,7 +98,7 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
   // the forward input needed by the input-range gradient is fetched the same way ----
   float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
   const bool do_ir = MODE == MODE_DX && a.ir_static != 0;
-  const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
+  const float ir_t = do_ir ? D::load(a.ir, t) : 0.0f;
   constexpr int kOutStride = 256 * 2 + 16;
   const int vcol = tid & 31, vrow = tid >> 5;  // 16-byte vector column, row within a pass of 16
   // column of this thread's vectors in x / dx: the operand column itself, or, with dense x / dx
@@ -124,7 +120,7 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
-          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)f32_to_bf16_bits(acc[bi][bj][v]);
+          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = D::to_elem(acc[bi][bj][v]);
         }
   }
   __syncthreads();
@@ -164,21 +160,21 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
         const int j = head + 8 * l32;
         float d[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) d[i] = bf16_bits_to_f32(*(const uint16_t*)(lrow + (j + i) * 2));
+        for (int i = 0; i < 8; ++i) d[i] = D::load(lrow, j + i);
         if (do_ir) {
           float xv[8];
-          BF16::unpack(ld16(a.x + e0 + j), xv);
+          D::unpack(ld16(a.x + e0 + j), xv);
 #pragma unroll
           for (int i = 0; i < 8; ++i) d[i] = element(d[i], xv[i]);
         }
-        st16(a.out + e0 + j, BF16::pack(d));
+        st16(a.out + e0 + j, D::pack(d));
       }
       // up to 7 elements before the first and after the last vector
       const int j1 = l32 < head ? l32 : tail0 + (l32 - head);
       if (l32 < head + (count - tail0)) {
-        float d = bf16_bits_to_f32(*(const uint16_t*)(lrow + j1 * 2));
-        if (do_ir) d = element(d, bf16_bits_to_f32(a.x[e0 + j1]));
-        a.out[e0 + j1] = (uint16_t)f32_to_bf16_bits(d);
+        float d = D::load(lrow, j1);
+        if (do_ir) d = element(d, D::load(a.x, e0 + j1));
+        a.out[e0 + j1] = D::to_elem(d);
       }
     }
   } else
@@ -201,8 +197,8 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
       if (r0 + row >= R || !ovalid) continue;
       if (do_ir) {
         float d[8], xv[8];
-        BF16::unpack(d4, d);
-        BF16::unpack(xr[j], xv);
+        D::unpack(d4, d);
+        D::unpack(xr[j], xv);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
@@ -216,7 +212,7 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
           }
           if (fabsf(xv[i]) > ir_t) d[i] = 0.0f;
         }
-        d4 = BF16::pack(d);
+        d4 = D::pack(d);
       }
       st16(op + (int64_t)(16 * (8 * half + j)) * a.ldo, d4);
     }
@@ -236,7 +232,7 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
 
 // TAIL: the contraction length is not a multiple of 64 (its last chunk is loaded with
 // predicates); the TAIL = false instantiation has no trace of that in its hot loop.
-template <int MODE, bool TAIL>
+template <class D, int MODE, bool TAIL>
 __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   __shared__ float red[8][3];
@@ -372,7 +368,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
     for (int j = 0; j < 4; ++j) {
       if (bias) {
         float e[8];
-        BF16::unpack(rawA[j], e);
+        D::unpack(rawA[j], e);
 #pragma unroll
         for (int i = 0; i < 8; ++i) bsum[i] += e[i];
       }
@@ -433,7 +429,7 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
 #pragma unroll
         for (int bi = 0; bi < 4; ++bi)
 #pragma unroll
-          for (int bj = 0; bj < 2; ++bj) mma16(fa[bi], fb[bj], acc[bi][bj]);
+          for (int bj = 0; bj < 2; ++bj) Mma16<D>::run(fa[bi], fb[bj], acc[bi][bj]);
       }
       if (ch + 1 < nchunks) {
         char* na = lds + ((ch + 1) & 1) * 2 * kOperandLds;
@@ -464,10 +460,11 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   }
 
   const BwdPos pos = {r0, c0, R, brow, bcol, nkb, t, slice};
-  bwd_finish<MODE>(a, pos, acc, lds, red);
+  bwd_finish<D, MODE>(a, pos, acc, lds, red);
 }
 
-// out[r, c] = bf16(sum over slices of split[s][r][c]), slices added in order
+// out[r, c] = the sum over slices of split[s][r][c], slices added in order, rounded to the dtype
+template <class D>
 __global__ __launch_bounds__(256) void k_split_reduce(const float* __restrict__ split, int slices,
                                                       int64_t R, int64_t K, uint16_t* __restrict__ out,
                                                       int64_t ldo) {
@@ -485,13 +482,14 @@ __global__ __launch_bounds__(256) void k_split_reduce(const float* __restrict__ 
     for (int u = 0; u < 4; ++u)
       if (s + u < slices) sum += part[u];
   }
-  u32x2 pk = {pack_bf16x2(sum.x, sum.y), pack_bf16x2(sum.z, sum.w)};
+  u32x2 pk = {D::pack2(sum.x, sum.y), D::pack2(sum.z, sum.w)};
   *(u32x2*)(out + r * ldo + c) = pk;
 }
 
 // Sliced input gradient: sums the slices' partial results in order, rounds once, and applies the
 // epilogue of the unsliced kernel (input-range mask and partial sums, column mapping onto a dense
 // dx). One block: 16 rows x 256 columns; partial sums go to partial[(row block, column block)].
+template <class D>
 __global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
   __shared__ float red[8][3];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -509,7 +507,7 @@ __global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
     ocol = ovalid ? (int64_t)t * a.dense_tile + in_tile : 0;
   }
   const bool do_ir = a.ir_static != 0;
-  const float ir_t = do_ir ? bf16_bits_to_f32(a.ir[t]) : 0.0f;
+  const float ir_t = do_ir ? D::load(a.ir, t) : 0.0f;
   float s_up = 0.0f, s_lo = 0.0f, cnt = 0.0f;
   if (row < a.M && ovalid) {
     f32x4 lo4 = {0.f, 0.f, 0.f, 0.f}, hi4 = {0.f, 0.f, 0.f, 0.f};
@@ -529,10 +527,10 @@ __global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
     }
     float d[8] = {lo4.x, lo4.y, lo4.z, lo4.w, hi4.x, hi4.y, hi4.z, hi4.w};
 #pragma unroll
-    for (int i = 0; i < 8; ++i) d[i] = bf16_bits_to_f32(f32_to_bf16_bits(d[i]));
+    for (int i = 0; i < 8; i += 2) round2<D>(d[i], d[i + 1]);
     if (do_ir) {
       float xv[8];
-      BF16::unpack(ld16(a.x + row * a.ldx + ocol), xv);
+      D::unpack(ld16(a.x + row * a.ldx + ocol), xv);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         if (a.ir_static == 1 + AHL_IR_GRAD_LEARNED) {
@@ -547,7 +545,7 @@ __global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
         if (fabsf(xv[i]) > ir_t) d[i] = 0.0f;
       }
     }
-    st16(a.out + row * a.ldo + ocol, BF16::pack(d));
+    st16(a.out + row * a.ldo + ocol, D::pack(d));
   }
   if (do_ir) {
     s_up = wave_sum(s_up); s_lo = wave_sum(s_lo); cnt = wave_sum(cnt);
@@ -562,9 +560,10 @@ __global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
   }
 }
 
-// dbias[n] = bf16(sum of the partial rows): 16 columns per block, 16 threads per column that
+// dbias[n] = the sum of the partial rows, rounded to the dtype: 16 columns per block, 16 threads per column that
 // each add every 16th row, combined in a fixed order (the partial rows can be hundreds when the
 // weight gradient is sliced)
+template <class D>
 __global__ __launch_bounds__(256) void k_bias_final(const float* partial, int rows, int64_t N,
                                                     uint16_t* dbias) {
   __shared__ float part[16][17];
@@ -579,15 +578,32 @@ __global__ __launch_bounds__(256) void k_bias_final(const float* partial, int ro
     float sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) sum += part[i][col];
-    dbias[n] = (uint16_t)f32_to_bf16_bits(sum);
+    dbias[n] = D::to_elem(sum);
   }
 }
 
-// Whether the fast backward kernels can be used: bf16, equal K-tiles of a multiple of 256
+template <class D, int MODE, bool TAIL>
+static void launch_bwd_one(dim3 grid, hipStream_t s, const BwdArgs& a) {
+  hipFuncSetAttribute((const void*)k_bwd_fast<D, MODE, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+  hipLaunchKernelGGL((k_bwd_fast<D, MODE, TAIL>), grid, dim3(512), kBwdLds, s, a);
+}
+
+template <int MODE>
+static void launch_bwd(int32_t dtype, bool tail, dim3 grid, hipStream_t s, const BwdArgs& a) {
+  if (dtype == AHL_F16) {
+    if (tail) launch_bwd_one<F16, MODE, true>(grid, s, a);
+    else launch_bwd_one<F16, MODE, false>(grid, s, a);
+  } else {
+    if (tail) launch_bwd_one<BF16, MODE, true>(grid, s, a);
+    else launch_bwd_one<BF16, MODE, false>(grid, s, a);
+  }
+}
+
+// Whether the fast backward kernels can be used: a 16-bit dtype, equal K-tiles of a multiple of 256
 // columns, output channels in whole 16-byte vectors. Any number of rows M: a contraction length
 // that is not a multiple of 64 ends in one predicated chunk.
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N) {
-  if (dtype != AHL_BF16) return false;
+  if (dtype != AHL_BF16 && dtype != AHL_F16) return false;
   if (tl.extra != 0 || tl.base % 256 != 0) return false;
   return K % 256 == 0 && N % 8 == 0 && N >= 8 && M >= 1;
 }
@@ -621,7 +637,7 @@ int64_t fast_dx_ws_bytes(int64_t M, int64_t K, int64_t N) {
   return fast_dx_partial_bytes(M, K, N) + (slices > 1 ? slices * M * K * 4 : 0);
 }
 
-int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dx(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, void* ws, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
@@ -641,15 +657,12 @@ int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint3
   a.split = slices > 1 ? (float*)((char*)ws + fast_dx_partial_bytes(M, K, N)) : nullptr;
   const int64_t nb = cdiv(M, 256) * (K / 256) * slices;
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
-  if (N % 64 == 0) {
-    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    hipLaunchKernelGGL((k_bwd_fast<MODE_DX, false>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
-  } else {
-    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DX, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    hipLaunchKernelGGL((k_bwd_fast<MODE_DX, true>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  const dim3 grid((unsigned)nb), reduce_grid((unsigned)(cdiv(M, 16) * (K / 256)));
+  launch_bwd<MODE_DX>(dtype, N % 64 != 0, grid, s, a);
+  if (slices > 1) {
+    if (dtype == AHL_F16) hipLaunchKernelGGL(k_dx_split_reduce<F16>, reduce_grid, dim3(512), 0, s, a);
+    else hipLaunchKernelGGL(k_dx_split_reduce<BF16>, reduce_grid, dim3(512), 0, s, a);
   }
-  if (slices > 1)
-    hipLaunchKernelGGL(k_dx_split_reduce, dim3((unsigned)(cdiv(M, 16) * (K / 256))), dim3(512), 0, s, a);
   return check_launch("ahl_linear_bwd_dx(fast)");
 }
 
@@ -675,7 +688,7 @@ int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N) {
   return bias + (slices > 1 ? slices * N * K * 4 : 0);
 }
 
-int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
                    hipStream_t s) {
@@ -693,19 +706,24 @@ int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint3
       ? (float*)((char*)ws + ((int64_t)slices * (K / 256) * N * 4 + 255) / 256 * 256) : nullptr;
   const int64_t nb = cdiv(N, 256) * (K / 256) * slices;
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
-  if (M % 64 == 0) {
-    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW, false>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    hipLaunchKernelGGL((k_bwd_fast<MODE_DW, false>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+  launch_bwd<MODE_DW>(dtype, M % 64 != 0, dim3((unsigned)nb), s, a);
+  const dim3 reduce_grid((unsigned)cdiv(N * K, 1024)), bias_grid((unsigned)cdiv(N, 16));
+  const int bias_rows = (int)(K / 256) * slices;
+  if (dtype == AHL_F16) {
+    if (slices > 1)
+      hipLaunchKernelGGL(k_split_reduce<F16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, slices, N, K,
+                         (uint16_t*)dw, lddw);
+    if (dbias)
+      hipLaunchKernelGGL(k_bias_final<F16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, N,
+                         (uint16_t*)dbias);
   } else {
-    hipFuncSetAttribute((const void*)k_bwd_fast<MODE_DW, true>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-    hipLaunchKernelGGL((k_bwd_fast<MODE_DW, true>), dim3((unsigned)nb), dim3(512), kBwdLds, s, a);
+    if (slices > 1)
+      hipLaunchKernelGGL(k_split_reduce<BF16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, slices, N, K,
+                         (uint16_t*)dw, lddw);
+    if (dbias)
+      hipLaunchKernelGGL(k_bias_final<BF16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, N,
+                         (uint16_t*)dbias);
   }
-  if (slices > 1)
-    hipLaunchKernelGGL(k_split_reduce, dim3((unsigned)cdiv(N * K, 1024)), dim3(256), 0, s,
-                       (const float*)a.split, slices, N, K, (uint16_t*)dw, lddw);
-  if (dbias)
-    hipLaunchKernelGGL(k_bias_final, dim3((unsigned)cdiv(N, 16)), dim3(256), 0, s,
-                       (const float*)bias_partial, (int)(K / 256) * slices, N, (uint16_t*)dbias);
   return check_launch("ahl_linear_bwd_dw(fast)");
 }
 

@@ -48,14 +48,15 @@ AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
                                               __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
-// step of an ADC with bound B (bf16 value held in fp32): rd(rd(2B) / n) for n states, rd(2B * res)
+// step of an ADC with bound B (a value of the 16-bit dtype held in fp32): rd(rd(2B) / n) for n states, rd(2B * res)
 // for a relative resolution. 2B is exact, so the second form is one product with the factor
 // 2 * res; for n with <= 8 significant bits the product with fl(2 / n) rounds to the same bf16 as
 // the quotient (see BF16::div). Only other n need the division; that case is a branch on a
 // launch constant, so the common one carries no division code.
+template <class D = BF16>
 AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
-  if (__builtin_expect(a.step_by_division != 0, 0)) return BF16::rd(__fdiv_rn(B + B, a.out_res));
-  return BF16::rd(B * a.step_factor);
+  if (__builtin_expect(a.step_by_division != 0, 0)) return D::rd(__fdiv_rn(B + B, a.out_res));
+  return D::rd(B * a.step_factor);
 }
 
 }  // namespace ahl

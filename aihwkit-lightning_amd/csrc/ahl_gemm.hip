@@ -709,14 +709,14 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
 int64_t fast_fwd_ws_bytes(int64_t M, int64_t N, int32_t n_tiles);
 __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N);
-int launch_fast_dx(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dx(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
                    void* dx, int64_t lddx, void* ws, int64_t M, int64_t K, int64_t N,
                    const Tiling& tl, int ir_static, int32_t dense_tile, const Tiling* dense,
                    hipStream_t s);
 int64_t fast_dx_ws_bytes(int64_t M, int64_t K, int64_t N);
 int64_t fast_dx_row_blocks(int64_t M, int64_t K, int64_t N, bool element_mode);
-int launch_fast_dw(const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
+int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
                    hipStream_t s);
@@ -766,7 +766,7 @@ extern "C" {
 
 int64_t ahl_linear_fwd_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_tiles, int32_t dtype) {
   (void)K;
-  if (dtype != AHL_BF16 || M <= 0 || N <= 0 || n_tiles <= 0) return 0;
+  if ((dtype != AHL_BF16 && dtype != AHL_F16) || M <= 0 || N <= 0 || n_tiles <= 0) return 0;
   return fast_fwd_ws_bytes(M, N, n_tiles);
 }
 
@@ -875,7 +875,7 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     // columns and maps its output columns back onto the dense x / dx in its epilogue
     const int64_t stride = cfg->tile_stride, padded = (int64_t)n_tiles * stride;
     if (stride < widest_tile(tl) || ldw < padded || padded > 0x3fffffff) return AHL_ERR_ARG;
-    if (cfg->dtype != AHL_BF16 || N % 8 != 0 || N < 8 || !aligned16(g) || !aligned16(w_eff) ||
+    if ((cfg->dtype != AHL_BF16 && cfg->dtype != AHL_F16) || N % 8 != 0 || N < 8 || !aligned16(g) || !aligned16(w_eff) ||
         ldg % 8 != 0 || ldw % 8 != 0 || (keep && !aligned16(keep)))
       return AHL_ERR_UNSUPPORTED;
     const Tiling ptl{n_tiles, (int32_t)stride, 0};
@@ -888,16 +888,19 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
     // the element-wise epilogue addresses x and dx with one offset and aligns its vectors on dx
     if (!vectors && (!aligned16(dx) || (is_static && (!aligned16(x) || ldx != lddx))))
       return AHL_ERR_UNSUPPORTED;
-    const int rc = launch_fast_dx(g, ldg, keep, clamp_flag, cfg->flag_token, w_eff, ldw, x, ldx, ir, dx, lddx, ws,
+    const int rc = launch_fast_dx(cfg->dtype, g, ldg, keep, clamp_flag, cfg->flag_token, w_eff, ldw, x, ldx, ir, dx, lddx, ws,
                                   M, padded, N, ptl, is_static ? 1 + cfg->ir_grad_rule : 0,
                                   vectors ? tl.base : 0, vectors ? nullptr : &tl, s);
     if (rc != AHL_OK) return rc;
-    if (is_static)
-      hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
-                         (const float*)partial, fast_dx_row_blocks(M, padded, N, !vectors),
-                         (int32_t)(padded / 256), per_tile,
-                         per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
-                         cfg->ir_grad_rule);
+    if (is_static) {
+      AHL_DISPATCH_DTYPE(cfg->dtype, {
+        hipLaunchKernelGGL((k_ir_grad_finalize<D>), dim3(n_tiles), dim3(64), 0, s,
+                           (const float*)partial, fast_dx_row_blocks(M, padded, N, !vectors),
+                           (int32_t)(padded / 256), per_tile,
+                           per_tile, tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
+                           cfg->ir_grad_rule);
+      });
+    }
     return check_launch("ahl_linear_bwd_dx(fast, padded weights)");
   }
   void* wt = (char*)ws + dx_partial_bytes(M, K, n_tiles);
@@ -906,16 +909,18 @@ int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* keep, const ui
                     (!keep || aligned16(keep)) &&
                     (!is_static || (ldx % 8 == 0 && aligned16(x)));
   if (fast) {
-    int rc = launch_fast_dx(g, ldg, keep, clamp_flag, cfg->flag_token, w_eff, ldw, x, ldx, ir, dx, lddx, ws, M, K,
+    int rc = launch_fast_dx(cfg->dtype, g, ldg, keep, clamp_flag, cfg->flag_token, w_eff, ldw, x, ldx, ir, dx, lddx, ws, M, K,
                             N, tl, is_static ? 1 + cfg->ir_grad_rule : 0, 0, nullptr, s);
     if (rc != AHL_OK) return rc;
     if (is_static) {
       const int32_t per_tile = tl.base / 256;
-      hipLaunchKernelGGL((k_ir_grad_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s,
-                         (const float*)partial, fast_dx_row_blocks(M, K, N, false),
-                         (int32_t)(K / 256), per_tile, per_tile,
-                         tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
-                         cfg->ir_grad_rule);
+      AHL_DISPATCH_DTYPE(cfg->dtype, {
+        hipLaunchKernelGGL((k_ir_grad_finalize<D>), dim3(n_tiles), dim3(64), 0, s,
+                           (const float*)partial, fast_dx_row_blocks(M, K, N, false),
+                           (int32_t)(K / 256), per_tile, per_tile,
+                           tl, M, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage,
+                           cfg->ir_grad_rule);
+      });
     }
     return check_launch("ahl_linear_bwd_dx(fast)");
   }
@@ -1032,19 +1037,19 @@ int ahl_linear_bwd_dw(const void* g, int64_t ldg, const uint32_t* keep, const ui
     // workspace, then the data columns are copied into the dense dw
     const int64_t stride = cfg->tile_stride, padded = (int64_t)n_tiles * stride;
     if (!xq || stride < widest_tile(tl) || ldxq < padded || padded > 0x3fffffff) return AHL_ERR_ARG;
-    if (cfg->dtype != AHL_BF16 || N % 8 != 0 || N < 8 || !aligned16(g) || !aligned16(xq) ||
+    if ((cfg->dtype != AHL_BF16 && cfg->dtype != AHL_F16) || N % 8 != 0 || N < 8 || !aligned16(g) || !aligned16(xq) ||
         ldg % 8 != 0 || ldxq % 8 != 0 || (keep && !aligned16(keep)))
       return AHL_ERR_UNSUPPORTED;
     void* dwp = (char*)ws + align256(fast_dw_ws_bytes(M, padded, N));
     const Tiling ptl{n_tiles, (int32_t)stride, 0};
-    const int rc = launch_fast_dw(g, ldg, keep, clamp_flag, cfg->flag_token, xq, ldxq, dwp, padded, dbias, ws, M,
+    const int rc = launch_fast_dw(cfg->dtype, g, ldg, keep, clamp_flag, cfg->flag_token, xq, ldxq, dwp, padded, dbias, ws, M,
                                   padded, N, ptl, s);
     if (rc != AHL_OK) return rc;
     return launch_unpad_tiles(dwp, padded, AHL_BF16, N, K, tl, stride, dw, lddw, s);
   }
   if (xq && fast_bwd_eligible(cfg->dtype, tl, M, K, N) && aligned16(g) && aligned16(xq) &&
       ldg % 8 == 0 && ldxq % 8 == 0 && lddw % 8 == 0 && aligned16(dw) && (!keep || aligned16(keep)))
-    return launch_fast_dw(g, ldg, keep, clamp_flag, cfg->flag_token, xq, ldxq, dw, lddw, dbias, ws, M, K, N, tl, s);
+    return launch_fast_dw(cfg->dtype, g, ldg, keep, clamp_flag, cfg->flag_token, xq, ldxq, dw, lddw, dbias, ws, M, K, N, tl, s);
   const int32_t dac_on = cfg->inp_res > 0.0f ? 1 : 0;
   DwArgs a;
   a.M = M; a.N = N; a.K = K; a.tl = tl; a.dw = dw; a.lddw = lddw;

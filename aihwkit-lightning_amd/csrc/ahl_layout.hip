@@ -117,7 +117,7 @@ int launch_unpad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t r
 using namespace ahl;
 
 extern "C" int64_t ahl_tile_stride(int64_t K, int32_t n_tiles, int32_t dtype) {
-  if (K <= 0 || n_tiles <= 0 || n_tiles > K || dtype != AHL_BF16) return 0;
+  if (K <= 0 || n_tiles <= 0 || n_tiles > K || (dtype != AHL_BF16 && dtype != AHL_F16)) return 0;
   if (K % n_tiles == 0 && (K / n_tiles) % 256 == 0) return 0;  // dense tiles are aligned already
   return padded_stride(K, n_tiles);
 }

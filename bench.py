@@ -116,6 +116,8 @@ OTHER_WORKLOADS = {
     "mlp_3072_8192": "LLaMA-style MLP block, hidden 3072, intermediate 8192, SiLU gating, three "
                      "AnalogLinear layers, bf16, 4096 tokens, tiles of 512, learned input range, 8-bit "
                      "DAC/ADC, out_noise 0.067, fwd+bwd",
+    "linear_4096_f16": "the headline layer and step in float16 (AnalogLinear 4096->4096, 8192 tokens, "
+                       "8 tiles x 512, learned range, 8-bit DAC/ADC, both noises, fwd+bwd)",
     "lstm_1024": "AnalogRNN, 2 LSTM layers 1024->1024 bf16, 64 steps x 64 sequences, tiles of 512, "
                  "fwd+bwd through time",
     "lstm_1024_eval": "AnalogRNN, 2 LSTM layers 1024->1024 bf16, 64 steps x 64 sequences, tiles of "
@@ -139,6 +141,13 @@ def build_other(name):
         x = torch.randn(128, 256, 28, 28, generator=gen).to(torch.bfloat16)
         g = torch.randn(128, 256, 28, 28, generator=gen).to(torch.bfloat16)
         flops = 3 * 2.0 * (128 * 28 * 28) * (256 * 9) * 256
+    elif name == "linear_4096_f16":
+        layer = AnalogLinear(4096, 4096, bias=True, dtype=torch.float16, rpu_config=_analog_cfg(512))
+        layer.set_weights_and_biases((0.02 * torch.randn(4096, 4096, generator=gen)).to(torch.float16),
+                                     torch.zeros(4096, dtype=torch.float16))
+        x = torch.randn(8192, 4096, generator=gen).to(torch.float16)
+        g = torch.randn(8192, 4096, generator=gen).to(torch.float16)
+        flops = 3 * 2.0 * 8192 * 4096 * 4096
     elif name == "fwd_dynamic_4096":
         cfg = _analog_cfg(512, noise=False)
         cfg.forward.out_noise = 0.04
@@ -543,7 +552,8 @@ def main():
         print(json.dumps({
             "metric": "TFLOP/s of the workload's matrix products", "value": res["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
             "steps": ns.steps, "warmup": ns.warmup, "ms_per_step": res["ms_per_step"],
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f16" if ns.workload.endswith("_f16") else "bf16",
             "data": "synthetic", "config": {k: v for k, v in res.items() if k not in ("ms_per_step", "tflops")},
         }))
         return
@@ -632,7 +642,7 @@ def main():
     del layer, x, g
     torch.cuda.empty_cache()
     others = {}
-    for name in ("fwd_dynamic_4096", "mlp_3072_8192", "lstm_1024"):
+    for name in ("fwd_dynamic_4096", "mlp_3072_8192", "linear_4096_f16", "lstm_1024"):
         res = time_other(name, 10, 3, graph=True) if name != "lstm_1024" else time_other(name, 4, 2, graph=True)
         res["frac_of_bf16_mfma_peak"] = round(res["tflops"] / PEAK_BF16_TFLOPS, 4)
         others[name] = res

@@ -10,9 +10,9 @@
  *   - dtype is AHL_F32, AHL_BF16 or AHL_F16 and applies to every pointer documented as "dtype".
  *     In AHL_BF16 / AHL_F16 every elementwise result is rounded to the 16-bit type
  *     (round-to-nearest-even) exactly where the reference's torch-mode rounds when it runs on
- *     tensors of that type. The MFMA kernels for large shapes exist for AHL_BF16 only; AHL_F16
- *     runs on the general kernels (the reference's accelerated slot takes float32 and float16,
- *     triton_utils/triton_linear.py:630).
+ *     tensors of that type. Both 16-bit types have the MFMA kernels for large shapes (the
+ *     reference's accelerated slot takes float32 and float16, triton_utils/triton_linear.py:630);
+ *     AHL_F32 runs on general kernels.
  *   - K-tiles ("analog tiles" along the input dimension) are described by `tile_ends_host`,
  *     the reference's `upper_end_of_slices` (nn/modules/linear.py:76-80) as a HOST int32 array
  *     of n_tiles cumulative end offsets. It must follow the reference's split rule

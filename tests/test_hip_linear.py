@@ -174,11 +174,20 @@ SHAPES = [
 ]
 
 
-# float16 runs on the general kernels: a selection of the shapes above once more in float16
+# float16 has the same kernel set as bfloat16 (the forward for large grids excepted): a selection
+# of the shapes above once more in float16, and two grids of a few hundred blocks
 SHAPES += [dict(c, name=c["name"].replace("bf16", "f16"), dtype="f16") for c in SHAPES if c["name"] in (
     "edge_bf16", "vec_bf16_static", "vec_bf16_dynamic", "vec_bf16_many_tiles", "fast_bf16_clamped",
     "fast_bf16_dynamic_clamped", "one_token_bf16", "pad_bf16_uneven_clamped", "tail_bf16_both_dynamic",
     "bf16_10bit_static", "bf16_odd_states_static", "pad_bf16_lsq", "sliced_dw_bf16_clamped")]
+SHAPES += [
+    case("grid_f16_static_clamped", dtype="f16", M=1536, K=1024, N=1024, max_input_size=512,
+         ir_mode="static", inp_res=254, out_res=254, out_bound=0.9, clip="channel", clip_sigma=2.5,
+         ir_decay=0.01, ir_init=3.0, w_scale=0.02, seed=61),
+    case("grid_f16_dynamic_clamped", dtype="f16", M=1024, K=1024, N=1280, max_input_size=256,
+         ir_mode="dynamic", inp_res=254, out_res=254, out_bound=0.9, clip="channel", clip_sigma=2.5,
+         w_scale=0.02, seed=62),
+]
 
 
 @pytest.mark.parametrize("c", SHAPES, ids=[c["name"] for c in SHAPES])
@@ -334,7 +343,7 @@ def test_cpu_tensor_is_rejected():
         layer(torch.randn(4, 16))
 
 
-@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("per_channel", [False, True])
 def test_output_noise_statistics(dtype, per_channel):
     """Per tile, the injected noise is N(0, out_noise/sqrt(T) * IR_t * wmax): mean and std of
@@ -355,7 +364,7 @@ def test_output_noise_statistics(dtype, per_channel):
     per_tile = (0.5 / 2 ** 0.5) * ir[:, None] * (wmax if per_channel else wmax.amax(1, keepdim=True))
     expected = per_tile.pow(2).sum(0).sqrt()  # [N] or [1]: tiles add independently
     z = (noisy - clean) / expected
-    tol = 0.01 if dtype == "f32" else 0.02  # bf16 rounding of the sum adds its own small variance
+    tol = 0.02 if dtype == "bf16" else 0.01  # bf16 rounding of the sum adds its own small variance
     assert abs(float(z.mean())) < 0.01
     assert abs(float(z.std()) - 1.0) < tol
     # successive calls draw fresh noise; the same torch seed replays it
