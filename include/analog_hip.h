@@ -125,7 +125,7 @@ typedef struct AhlModifierCfg {
 } AhlModifierCfg;
 
 /* ---- padded tile layout ------------------------------------------------------------------
- * The MFMA kernels of the bf16 path want every K-tile to start on a 256-column boundary. The
+ * The MFMA kernels of the 16-bit dtypes want every K-tile to start on a 256-column boundary. The
  * reference's split rule (nn/modules/linear.py:155-170) gives that only for some shapes
  * (4096 inputs in tiles of 512 do, 11008 in tiles of 512 or 2304 in tiles of 576 do not). For
  * the others the two operands the library produces itself -- the quantised input xq (ahl_dac)
@@ -223,7 +223,7 @@ int ahl_ir_moving_update(void* ir, int32_t* idx, const float* val, int32_t dtype
  * z = sigmoid(i_z + h_z); n = tanh(i_n + r h_n); h' = n + z (h - n)) and what autograd derives
  * from them, with the dtype rounding after every operation that the torch chain has.
  * All matrices dense row-major, 16-byte aligned; gates [rows, 4 hidden] / [rows, 3 hidden], states
- * [rows, hidden]; hidden a multiple of 8 (bf16) or 4 (fp32).
+ * [rows, hidden]; hidden a multiple of 8 (bf16, fp16) or 4 (fp32).
  * lstm fwd: hgates may be null (one product over [x, h], cells.py:244-267); act [rows, 4 hidden]
  *   receives the activated gates for the backward pass (null: not wanted).
  * lstm bwd: dcy may be null (c' unused downstream); dgates is the gradient of both products'
@@ -324,10 +324,10 @@ int ahl_dac(const void* x, int64_t ldx, void* xq, int64_t ldxq, const void* ir_i
  *   output noise, ADC quantise, clamp to the output bound; per-tile results summed in dtype;
  *   bias added last.
  *   x        dtype [M, K] raw input; the clamp + DAC then run fused in the A-tile staging.
- *   xq       dtype [M, K] from ahl_dac, or NULL. bf16 calls whose tiles are equal multiples of
+ *   xq       dtype [M, K] from ahl_dac, or NULL. 16-bit calls whose tiles are equal multiples of
  *            64 take a faster kernel when xq is given (x may then be NULL); with
  *            cfg->tile_stride > 0, xq and w_eff are in the padded tile layout and every split
- *            takes that kernel (bf16 only; AHL_ERR_UNSUPPORTED otherwise).
+ *            takes that kernel (16-bit dtypes only; AHL_ERR_UNSUPPORTED otherwise).
  *   ir       dtype [T] (AHL_IR_STATIC) or [T, M] (AHL_IR_DYNAMIC) or NULL (AHL_IR_NONE)
  *   wmax     dtype [T, N] from ahl_weight_prep, or NULL when neither noise nor bound is on
  *   tile_max float [T]    from ahl_weight_prep, or NULL likewise
@@ -361,7 +361,7 @@ int ahl_linear_fwd(const void* x, int64_t ldx, const void* xq, int64_t ldxq, con
  *   clamp_flag: NULL, or the flag written by ahl_linear_fwd (the mask is ignored when it reads 0).
  *   ws needs ahl_linear_bwd_dx_ws_bytes(M, K, N, n_tiles, dtype, cfg->tile_stride) bytes.
  *   With cfg->tile_stride > 0, w_eff is in the padded tile layout (x and dx stay dense: the
- *   kernel maps its columns back in the epilogue); needs bf16 and N a multiple of 8.
+ *   kernel maps its columns back in the epilogue); needs a 16-bit dtype and N a multiple of 8.
  * Slot of TritonLinear.backward, triton_utils/triton_linear.py:695-764.                  */
 int ahl_linear_bwd_dx(const void* g, int64_t ldg, const uint32_t* clamp_mask, const uint32_t* clamp_flag,
                       const void* w_eff, int64_t ldw, const void* x, int64_t ldx, const void* ir,
