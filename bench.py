@@ -33,8 +33,8 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 TRAFFIC_TABLE = os.path.join("profiles", "linear_fwd_bwd_4096x4096_8192tok_bf16_hbm_traffic.txt")
 TRAFFIC_ROWS = {
     "linear_fwd": "ahl::k_fwd_pipe<",
-    "linear_bwd_dx(+ir_grad)": "ahl::k_bwd_fast<0",
-    "linear_bwd_dw(+bias_grad)": "ahl::k_bwd_fast<1",
+    "linear_bwd_dx(+ir_grad)": "ahl::k_bwd_fast<ahl::BF16, 0",
+    "linear_bwd_dw(+bias_grad)": "ahl::k_bwd_fast<ahl::BF16, 1",
 }
 
 
