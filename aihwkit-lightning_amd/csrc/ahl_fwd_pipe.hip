@@ -264,10 +264,10 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
       if (t + 1 < a.n_tiles) write_rowc(t + 1);
     } else {
       // The "did an output leave the range" branch of unit u is taken in the middle of unit
-      // u + 1: a branch on a vector compare waits for the compare to leave the pipeline. What the
-      // rare path needs of the unit stays in registers until then.
+      // u + 1: a branch on a vector compare waits for the compare to leave the pipeline. The
+      // unit's outputs stay in registers until then and join the running totals after it, so
+      // that the (not so rare, with clipped weights) clamp path has no sums to redo.
       float yp[8], Bp[8];
-      uint32_t tpo[4];
       bool overp = false;
       auto resolve = [&](int pu) __attribute__((always_inline)) {
         if (!(EPI && CLAMP)) return;
@@ -282,11 +282,13 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
               clamp_record(cl && nbase + 32 * pbj < a.N, 32 * (pbi & 1) + 8 * g + (e & 3), cwords[pbi >> 1][pbj]);
             yp[e] = fminf(fmaxf(yp[e], -Bp[e]), Bp[e]);
           }
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            totp[pbi][pbj][4 * pgp + q] =
-                pack_bf16x2(unpack_lo(tpo[q]) + yp[2 * q], unpack_hi(tpo[q]) + yp[2 * q + 1]);
           any_clamp |= overp ? 1u : 0u;
+        }
+        // total = rd(total + y), bf16 pairs
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t tp = totp[pbi][pbj][4 * pgp + q];
+          totp[pbi][pbj][4 * pgp + q] = pack_bf16x2(unpack_lo(tp) + yp[2 * q], unpack_hi(tp) + yp[2 * q + 1]);
         }
       };
 #pragma unroll
@@ -314,7 +316,6 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
         float wr_ = 0.0f, wb_ = 0.0f;
         u32x4 pc = {0u, 0u, 0u, 0u};
         uint32_t k0 = (uint32_t)nk.seed, k1 = (uint32_t)(nk.seed >> 32);
-        uint32_t tp_old[4];
         // noise, ADC of elements e, e + 1
         auto element_pair = [&](int e) __attribute__((always_inline)) {
           if (NOISE) {
@@ -364,12 +365,11 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
           }
         };
         auto totals = [&](int gg) __attribute__((always_inline)) {
-          // total = rd(total + y), bf16 pairs
+          // without a clamp there is nothing to wait for: total = rd(total + y) right away
 #pragma unroll
           for (int pr = 0; pr < 2; ++pr) {
             const int idx = 2 * (2 * gp + gg) + pr;
             const uint32_t tp = totp[bi][bj][idx];
-            tp_old[2 * gg + pr] = tp;
             totp[bi][bj][idx] = pack_bf16x2(unpack_lo(tp) + y[4 * gg + 2 * pr], unpack_hi(tp) + y[4 * gg + 2 * pr + 1]);
           }
         };
@@ -409,8 +409,8 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
             if (piece == 10) element_pair(2);
             if (piece == 11) { row_consts(1); element_pair(4); }
             if (piece == 12) element_pair(6);
-            if (piece == 13) totals(0);
-            if (piece == 14) totals(1);
+            if (!CLAMP && piece == 13) totals(0);
+            if (!CLAMP && piece == 14) totals(1);
             if (CLAMP && piece == 15) {
               // a running maximum in a vector register and ONE compare: compares whose results
               // go to scalar registers, and the scalar ORs that collect them, stall the wave
@@ -431,8 +431,6 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
         if (EPI && CLAMP) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) { yp[e] = y[e]; Bp[e] = Bv[e]; }
-#pragma unroll
-          for (int q = 0; q < 4; ++q) tpo[q] = tp_old[q];
           overp = over;
         }
         if (!MMA) __builtin_amdgcn_sched_barrier(0);
