@@ -375,6 +375,58 @@ def time_other(name, steps, warmup, graph=False):
     return res
 
 
+def time_reference_speed_test():
+    """The workload of the reference's own speed script (its tests/test_speed.py:221-279): float16,
+    512 rows, square layers of 128 ... 2048 inputs as one tile, input range + DAC, ADC (bound 12),
+    output noise 0.02, additive weight noise, layer-wise clipping at 2 sigma; one step = forward,
+    `out.sum().backward()`, `AnalogOptimizer(AdamW, lr=0).step()` (which clips the weights).
+    Microseconds per step, eager and replayed from one HIP graph."""
+    from aihwkit_lightning.nn import AnalogLinear
+    from aihwkit_lightning.nn.graphs import CapturedStep
+    from aihwkit_lightning.optim import AnalogOptimizer
+    from aihwkit_lightning.simulator.configs import (
+        TorchInferenceRPUConfig, WeightClipType, WeightNoiseInjectionType,
+    )
+
+    out = {}
+    for size in (128, 256, 512, 1024, 2048):
+        cfg = TorchInferenceRPUConfig()
+        cfg.mapping.max_input_size = -1
+        cfg.forward.inp_res, cfg.forward.out_res, cfg.forward.out_bound = 254, 254, 12
+        cfg.forward.out_noise = 0.02
+        ir = cfg.pre_post.input_range
+        ir.enable, ir.learn_input_range, ir.init_from_data = True, True, 0
+        cfg.clip.type, cfg.clip.sigma = WeightClipType.LAYER_GAUSSIAN, 2.0
+        cfg.modifier.noise_type, cfg.modifier.std_dev = WeightNoiseInjectionType.ADD_NORMAL, 0.01
+        layer = AnalogLinear(size, size, bias=True, rpu_config=cfg).to(device="cuda", dtype=torch.float16)
+        optims = {"eager": AnalogOptimizer(torch.optim.AdamW, layer.analog_layers, layer.parameters(), lr=0.0),
+                  # torch's optimizers record into a graph only in their capturable form
+                  "graph": AnalogOptimizer(torch.optim.AdamW, layer.analog_layers, layer.parameters(), lr=0.0,
+                                           capturable=True)}
+        inp = torch.randn(512, size, device="cuda", dtype=torch.float16, requires_grad=True)
+        which = ["eager"]
+
+        def step():
+            layer(inp).sum().backward()
+            optims[which[0]].step()
+
+        def timed(fn, reps=300):
+            preheat(fn, 0.2)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / reps * 1e6
+
+        eager = timed(step)
+        which[0] = "graph"
+        replay = CapturedStep(step)
+        replay()
+        out[str(size)] = {"us_eager": round(eager, 1), "us_graph_replay": round(timed(replay), 1)}
+    return out
+
+
 def event_time_ms(fn, reps):
     """Average duration of fn() over `reps` back-to-back calls, HIP events on the current stream."""
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -532,7 +584,7 @@ def main():
                         help="headline workload only: skip the other configurations' short runs")
     parser.add_argument("--kernels-only", action="store_true",
                         help="only launch the individual kernels (for rocprofv3 runs)")
-    parser.add_argument("--workload", default="linear", choices=["linear", "post_training", *OTHER_WORKLOADS],
+    parser.add_argument("--workload", default="linear", choices=["linear", "post_training", "reference_speed_test", *OTHER_WORKLOADS],
                         help="'linear' is the headline workload; the others print their own line")
     ns = parser.parse_args()
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -543,6 +595,16 @@ def main():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
 
+    if ns.workload == "reference_speed_test":
+        res = time_reference_speed_test()
+        print(json.dumps({
+            "metric": "microseconds per forward + backward + optimizer step", "value": res["2048"]["us_eager"],
+            "unit": "us", "n_gpus": 1, "steps": 300, "warmup": 0, "ms_per_step": res["2048"]["us_eager"] / 1e3,
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "the reference's tests/test_speed.py fwd+bwd+step benchmark: float16, 512 rows, "
+                                   "square AnalogLinear of 128 ... 2048 (value: 2048), all non-idealities on",
+                       "us_per_step": res}}))
+        return
     if ns.workload == "post_training":
         print(json.dumps(time_post_training(not ns.no_cpu)))
         return
