@@ -2,10 +2,13 @@
 against the CPU oracle and the reference's golden vectors.
 
 Acceptance rule (the path's stated tolerance): noise disabled -> outputs and gradients within
-1e-5 (fp32) / 1e-2 (bf16) relative to the tensor scale; elements outside that must be at most one
-ADC LSB off and at most 0.1 % of the tensor. Noise enabled -> mean and std of the injected noise
+1e-5 (fp32) / 1e-2 (bf16) / 1e-3 (fp16) relative to the tensor scale; elements outside that must
+be at most one ADC LSB off (without an ADC: one step of the 16-bit type) and at most 0.1 % of the
+tensor. Noise enabled -> mean and std of the injected noise
 within 1 % of the configured values.
 """
+import math
+
 import pytest
 import torch
 
@@ -20,6 +23,8 @@ NOISELESS = [
     if c["kind"] == "fwd_bwd" and c["out_noise"] == 0 and c["weight_noise"] == "none"
 ]
 RTOL = {"f32": 1e-5, "bf16": 1e-2, "f16": 1e-3}
+# spacing of the 16-bit values in [0.5, 1)
+ROUNDING_STEP = {"bf16": 2.0 ** -8, "f16": 2.0 ** -11}
 
 
 def adc_lsb(c, wmax_scale=None):
@@ -39,6 +44,14 @@ def check_against(res, ref, c, tag):
 
     rtol = RTOL[c["dtype"]]
     lsb = adc_lsb(c)
+    if lsb is None and c["dtype"] in ROUNDING_STEP:
+        # Without an ADC the last rounding is the tile product's own, to the 16-bit type. A product
+        # whose fp32 sum lies within a few fp32 steps of the midpoint between two 16-bit values is
+        # rounded up or down by the order of the summation, which differs between the MFMA kernels
+        # and the CPU: such an element may be one 16-bit step (at the tensor's largest magnitude,
+        # the bound of a tile product) away, under the same 0.1 % cap as the ADC's steps.
+        top = float(ref["out"].abs().max())
+        lsb = ROUNDING_STEP[c["dtype"]] * 2.0 ** math.ceil(math.log2(max(top, 1e-30)))
     assert_close_lsb(res["out"], ref["out"].float().to(res["out"].dtype), rtol, lsb, what=f"{tag} out")
     # gradients: an output LSB flip never enters them (straight-through), only clamp-mask flips
     for key in ("dx", "dw", "db", "dir", "dlwc"):
