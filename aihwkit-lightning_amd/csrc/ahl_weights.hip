@@ -62,8 +62,9 @@ struct ModArgs {
 
 // One thread per group of 8 consecutive inputs of one channel (one Philox call gives the 8
 // normals of the group); consecutive threads walk along the row, so that with VEC every wave
-// reads and writes contiguous 16-byte vectors.
-template <class D, bool VEC>
+// reads and writes contiguous 16-byte vectors. A group lies in at most two tiles when tiles are
+// at least 7 inputs wide; NARROW (narrower tiles) looks the tile up element by element.
+template <class D, bool VEC, bool NARROW = false>
 __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t blocks_per_row) {
   const int64_t n = blockIdx.x / blocks_per_row;
   const int32_t kb = (int32_t)((blockIdx.x % blocks_per_row) * 256 + threadIdx.x) * 8;
@@ -108,11 +109,18 @@ __global__ __launch_bounds__(256) void k_weight_modify(ModArgs a, uint32_t block
     };
     const int t0 = a.tl.tile_of(kb), t1 = a.tl.tile_of(klast);
     TileConst c = tile_const(t0);
-    const int32_t t1_start = t1 != t0 ? a.tl.start(t1) : 0x7fffffff;  // a group spans at most 2 tiles
-    const TileConst c1 = t1 != t0 ? tile_const(t1) : c;
+    const int32_t t1_start = t1 != t0 ? a.tl.start(t1) : 0x7fffffff;
+    const TileConst c1 = !NARROW && t1 != t0 ? tile_const(t1) : c;
+    int tn = t0;                              // NARROW: the tile of element e, walked along
+    int32_t tn_end = a.tl.start(t0 + 1);
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const TileConst& ce = kb + e >= t1_start ? c1 : c;
+      if (NARROW && kb + e >= tn_end && kb + e <= klast) {
+        ++tn;
+        tn_end = a.tl.start(tn + 1);
+        c = tile_const(tn);
+      }
+      const TileConst& ce = !NARROW && kb + e >= t1_start ? c1 : c;
       float x = v[e];
       if (a.quant_type != AHL_QUANT_NONE)
         x = wquant_apply<D>(x, ce.q, a.maxq, a.quant_type != AHL_QUANT_CLIP_LEARNED);
@@ -427,7 +435,9 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       const int64_t bpr = cdiv(cdiv(K, 8), 256);
       if (bpr * N > 0x7fffffff) return AHL_ERR_ARG;
       const bool vec_mod = vec && K % 8 == 0 && aligned16(w_eff) && ld_eff % D::EPV == 0;
-      if (vec_mod)
+      if (tl.base < 7)
+        hipLaunchKernelGGL((k_weight_modify<D, false, true>), dim3((unsigned)(bpr * N)), dim3(256), 0, s, a, (uint32_t)bpr);
+      else if (vec_mod)
         hipLaunchKernelGGL((k_weight_modify<D, true>), dim3((unsigned)(bpr * N)), dim3(256), 0, s, a, (uint32_t)bpr);
       else
         hipLaunchKernelGGL((k_weight_modify<D, false>), dim3((unsigned)(bpr * N)), dim3(256), 0, s, a, (uint32_t)bpr);

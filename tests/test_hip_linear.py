@@ -193,6 +193,14 @@ SHAPES += [dict(c, name=c["name"].replace("bf16", "f16"), dtype="f16") for c in 
     "edge_bf16", "vec_bf16_static", "vec_bf16_dynamic", "vec_bf16_many_tiles", "fast_bf16_clamped",
     "fast_bf16_dynamic_clamped", "one_token_bf16", "pad_bf16_uneven_clamped", "tail_bf16_both_dynamic",
     "bf16_10bit_static", "bf16_odd_states_static", "pad_bf16_lsq", "sliced_dw_bf16_clamped")]
+# tiles narrower than the 8 inputs one thread of the weight kernels handles (several tiles per
+# thread), with the on-the-fly weight quantiser per tile and channel
+SHAPES += [
+    case(f"narrow_tiles_{dt}_{ms}", dtype=dt, M=17, K=100, N=24, max_input_size=ms, ir_mode="static",
+         inp_res=254, ir_init=2.0, ir_decay=0.01, weight_quant="discretize_per_channel", modifier_res=30,
+         w_scale=0.1, seed=63)
+    for dt in ("f32", "bf16", "f16") for ms in (1, 3, 6)
+]
 SHAPES += [
     case("grid_f16_static_clamped", dtype="f16", M=1536, K=1024, N=1024, max_input_size=512,
          ir_mode="static", inp_res=254, out_res=254, out_bound=0.9, clip="channel", clip_sigma=2.5,

@@ -134,6 +134,17 @@ def test_clip_weights_closed_form(dtype, per_channel):
         assert mism < 2e-3
 
 
+@pytest.mark.parametrize("per_channel", [False, True])
+def test_clip_weights_of_a_single_weight_is_left_alone(per_channel):
+    """The unbiased std of one value is NaN; the reference's clamp at +-NaN then turns the weight
+    into NaN. Here such a row (or one-weight matrix) stays as it is -- a stated difference."""
+    w = torch.tensor([[0.7], [-1.2], [0.0]]) if per_channel else torch.tensor([[0.7]])
+    dev = w.cuda().clone()
+    ops().clip_weights(dev, 2.0, 1 if per_channel else 0)
+    assert torch.equal(dev.cpu(), w)
+    assert torch.isnan(om.clip_weights(w, 2.0, per_channel)).all()
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("vectors", [1, 63, 256, 257, 768, 1024, 2048, 2049],
                          ids=lambda v: f"{v}_vectors")
@@ -192,16 +203,17 @@ def test_quantize_weights_matches_reference(name):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 @pytest.mark.parametrize("scales", ["small", "all_large", "mixed"])
-@pytest.mark.parametrize("cols,tile", [(512, 256), (2560, 1280), (300, 100)],
-                         ids=["held", "long_segments", "unaligned_tiles"])
+@pytest.mark.parametrize("cols,tile", [(512, 256), (2560, 1280), (300, 100), (100, 3), (26, 1)],
+                         ids=["held", "long_segments", "unaligned_tiles", "tiles_of_3", "tiles_of_1"])
 @pytest.mark.parametrize("rows", [24, 700])
 def test_quantize_weights_per_channel_scale_switch(rows, cols, tile, scales, dtype):
     """The per-channel quantiser against the oracle where the reference's resolution convention
     matters: it reads the scales as numbers of states only if EVERY scale of a tile exceeds one.
     `small`: none does (the one-pass kernel alone); `all_large`: all do; `mixed`: some channels do,
     so the switch stays off but their segments wait for the tile minimum. Segments held in
-    registers, segments longer than that, and a split the one-pass kernel does not take; a
-    handful of channels and more than one block's worth of them."""
+    registers, segments longer than that, a split the one-pass kernel does not take, and tiles
+    narrower than the 8 inputs a thread of the general kernel handles (several tiles per thread);
+    a handful of channels and more than one block's worth of them."""
     from aihwkit_lightning.nn.modules.hip_utils import library as L
 
     gen = torch.Generator().manual_seed(cols + len(scales))
