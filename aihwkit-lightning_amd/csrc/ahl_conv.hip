@@ -650,13 +650,14 @@ extern "C" int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geo
                   make_small_div((int32_t)oh_span), make_small_div(cpb),
                   {make_small_div(g.str[0]), make_small_div(g.str[1]), make_small_div(g.str[2])}};
       AHL_DISPATCH_DTYPE(dtype, {
+        // a refusal of the LDS size shows at the launch that follows (check_launch)
         if (pixels == 256) {
-          hipFuncSetAttribute((const void*)k_col2im_wide<D>,
+          (void)hipFuncSetAttribute((const void*)k_col2im_wide<D>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
           hipLaunchKernelGGL((k_col2im_wide<D>), dim3((unsigned)tblocks), dim3(256), (size_t)lds_bytes,
                              (hipStream_t)stream, dcols, ldc, g, fp, dx);
         } else {
-          hipFuncSetAttribute((const void*)k_col2im_tiled<D>,
+          (void)hipFuncSetAttribute((const void*)k_col2im_tiled<D>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
           hipLaunchKernelGGL((k_col2im_tiled<D>), dim3((unsigned)tblocks), dim3(512), (size_t)lds_bytes,
                              (hipStream_t)stream, dcols, ldc, g, fp, dx);

@@ -584,7 +584,8 @@ __global__ __launch_bounds__(256) void k_bias_final(const float* partial, int ro
 
 template <class D, int MODE, bool TAIL>
 static void launch_bwd_one(dim3 grid, hipStream_t s, const BwdArgs& a) {
-  hipFuncSetAttribute((const void*)k_bwd_fast<D, MODE, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+  // a refusal shows at the launch that follows (check_launch reads the last error)
+  (void)hipFuncSetAttribute((const void*)k_bwd_fast<D, MODE, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
   hipLaunchKernelGGL((k_bwd_fast<D, MODE, TAIL>), grid, dim3(512), kBwdLds, s, a);
 }
 

@@ -524,7 +524,8 @@ template <int IRMODE, bool NOISE, int QM, int CPT>
 static void launch_pipe_one(const FastFwdArgs& a, hipStream_t s) {
   constexpr int NBI = 2;
   const dim3 block(1024 / NBI), grid((unsigned)(cdiv(a.M, 256) * cdiv(a.N, 128)));
-  hipFuncSetAttribute((const void*)k_fwd_pipe<IRMODE, NOISE, QM, CPT, NBI>,
+  // a refusal shows at the launch that follows (check_launch reads the last error)
+  (void)hipFuncSetAttribute((const void*)k_fwd_pipe<IRMODE, NOISE, QM, CPT, NBI>,
                       hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
   hipLaunchKernelGGL((k_fwd_pipe<IRMODE, NOISE, QM, CPT, NBI>), grid, block, kPLdsBytes, s, a);
 }

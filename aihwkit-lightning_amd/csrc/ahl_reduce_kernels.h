@@ -58,7 +58,7 @@ __global__ __launch_bounds__(256) void k_tile_minmax(const void* __restrict__ v,
 }
 
 // p[0..n) = v (a fill kernel instead of a memset node, so callers may capture it in a graph)
-static __global__ void k_fill_u32(uint32_t* p, uint32_t v, int n) {
+__attribute__((unused)) static __global__ void k_fill_u32(uint32_t* p, uint32_t v, int n) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
 }
