@@ -110,6 +110,7 @@ struct F32 {
   }
   // x / d, where rcp_d is 1/d: fp32 tensors use the IEEE quotient like torch on the CPU.
   static AHL_DEV float div(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
+  static AHL_DEV float div_exact_rcp(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
 };
 
 struct BF16 {
@@ -140,6 +141,7 @@ struct BF16 {
   // x * fl32(1/d) to bf16 gives bit-identical results to rounding fl32(x / d). The caller
   // rounds the returned value with rd().
   static AHL_DEV float div(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
+  static AHL_DEV float div_exact_rcp(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
   // two values as one register of 16-bit halves (rounded to nearest even), and back
   static AHL_DEV uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
   static AHL_DEV float lo(uint32_t w) { return unpack_lo(w); }
@@ -193,9 +195,25 @@ struct F16 {
                pack_f16x2(f[6], f[7])};
     return v;
   }
-  // 11-bit significands: the product with an approximate reciprocal can land on the other side
-  // of a rounding boundary, so the IEEE quotient is taken (the caller rounds it with rd()).
-  static AHL_DEV float div(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
+  // 11-bit significands. With the CORRECTLY ROUNDED fp32 reciprocal, rounding x * rcp_d to
+  // float16 equals rounding x / d for every pair of float16 values (exhaustive over the
+  // significands), as for bfloat16; the caller rounds the returned value with rd().
+  static AHL_DEV float div_exact_rcp(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
+  // With a reciprocal that is one fp32 step off (v_rcp_f32) a few products land on the other
+  // side of a float16 rounding boundary, so the fp32 IEEE quotient is needed. For float16-valued
+  // x and d it takes one correction step instead of the full division
+  // sequence: q0 = x * rcp_d (rcp_d within one fp32 step of 1 / d), r = x - d * q0 (exact in an
+  // fma: x is a multiple of the product's last place and the difference has < 14 bits),
+  // q1 = q0 + r * rcp_d = (x / d) (1 + e), |e| < 2^-45. x / d cannot lie within 2^-36 (relative) of
+  // a midpoint between two fp32 values (d times a 25-bit odd number has more bits than x), so q1
+  // IS the correctly rounded fp32 quotient. Zero and non-finite x keep q0 (sign of zero, inf).
+  static AHL_DEV float div(float x, float d, float rcp_d) {
+    const float q0 = x * rcp_d;
+    const float r = __builtin_fmaf(-d, q0, x);
+    const float q1 = __builtin_fmaf(r, rcp_d, q0);
+    // class bits 3, 4, 7, 8: normal or subnormal of either sign (not zero, infinite or NaN)
+    return __builtin_amdgcn_classf(q0, 0x198) ? q1 : q0;
+  }
   // the packing conversion as an instruction, for the reason given at rd()
   static AHL_DEV uint32_t pack2(float lo, float hi) {
     uint32_t w;
@@ -400,7 +418,7 @@ AHL_DEV float dac_apply(float x, const Dac& d, bool skip_rounding) {
   float v = x;
   if (CLAMP) v = fminf(fmaxf(v, -d.ir), d.ir);
   if (QUANT) {
-    float q = D::rd(D::div(v, d.rc, d.rcp));
+    float q = D::rd(D::div_exact_rcp(v, d.rc, d.rcp));
     if (!skip_rounding) q = rintf(q);  // v_rndne_f32: round half to even like torch.round
     v = D::rd(q * d.r);
   }

@@ -320,7 +320,9 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
             }
             if (ADC) {
 #pragma unroll
-              for (int c = 0; c < 4; ++c) y[c] = D::div(y[c], fmaxf(rv[c], D::tiny()), rcpv[c]);
+              for (int c = 0; c < 4; ++c)
+                y[c] = IRMODE == AHL_IR_STATIC ? D::div_exact_rcp(y[c], fmaxf(rv[c], D::tiny()), rcpv[c])
+                                               : D::div(y[c], fmaxf(rv[c], D::tiny()), rcpv[c]);
               round2<D>(y[0], y[1]); round2<D>(y[2], y[3]);
               if (ROUND) {
 #pragma unroll
@@ -502,7 +504,7 @@ namespace ahl {
 
 // ahl_fwd_pipe.hip: the kernel for large grids
 bool pipe_fwd_eligible(const FastFwdArgs& a, int ir_mode);
-bool launch_pipe_fwd(const FastFwdArgs& a, int ir_mode, bool noise, int qm, hipStream_t s);
+bool launch_pipe_fwd(int32_t dtype, const FastFwdArgs& a, int ir_mode, bool noise, int qm, hipStream_t s);
 
 // Few rows (a recurrent step, a decoding step): the 128 x 64 output blocks alone leave most CUs
 // idle and every block walks the whole contraction with one chunk in flight. With a workspace
@@ -574,9 +576,8 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   // Large grids go to the kernel that runs a tile's epilogue inside the next tile's product loop
   // (same results bit for bit); AHL_FORWARD_KERNEL=blocks in the environment keeps them here.
   const char* pick = getenv("AHL_FORWARD_KERNEL");
-  if (cfg->dtype == AHL_BF16 && !(pick != nullptr && strcmp(pick, "blocks") == 0) &&
-      pipe_fwd_eligible(a, cfg->ir_mode) &&
-      launch_pipe_fwd(a, cfg->ir_mode, noise, qm, s))
+  if (!(pick != nullptr && strcmp(pick, "blocks") == 0) && pipe_fwd_eligible(a, cfg->ir_mode) &&
+      launch_pipe_fwd(cfg->dtype, a, cfg->ir_mode, noise, qm, s))
     return check_launch("ahl_linear_fwd(pipe)");
   const dim3 sum_grid((unsigned)cdiv(M * (N / 8), 256));
   if (cfg->dtype == AHL_F16) {

@@ -1,4 +1,5 @@
-// bf16 analog forward for large grids with a learned (static) input range: the per-K-tile
+// Analog forward in a 16-bit type (bf16, float16) for large grids with a learned (static) input
+// range ("bf16" below stands for either: same registers, same packing). The per-K-tile
 // epilogue of tile t - 1 runs inside the product loop of tile t, and the operands go from global
 // memory straight into LDS two chunks ahead.
 //
@@ -58,7 +59,7 @@ template <bool V> using flag = std::integral_constant<bool, V>;
 // reads per flop but was 25 % slower: a SIMD issues at most one instruction of ONE wave per 4-5
 // cycles whatever its kind, and vector throughput for the epilogue's instruction mix is up to
 // 1.9 x higher with two waves.
-template <int IRMODE, bool NOISE, int QM, int CPT, int NBI>
+template <class D, int IRMODE, bool NOISE, int QM, int CPT, int NBI>
 __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastFwdArgs a) {
   constexpr bool ADC = QM >= 2, CLAMP = QM >= 1, ROUND = QM != 3;
   constexpr bool bound_on = CLAMP;
@@ -147,10 +148,10 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
   auto write_rowc = [&](int tt) __attribute__((always_inline)) {
     if (IRMODE == AHL_IR_DYNAMIC && (NOISE || bound_on) && tid < 256) {
       const int64_t m = m0 + tid;
-      const float irm = m < a.M ? BF16::load(a.ir, (int64_t)tt * a.M + m) : 0.0f;
+      const float irm = m < a.M ? D::load(a.ir, (int64_t)tt * a.M + m) : 0.0f;
       float* rc = rowc + (tt & 1) * 512;
-      rc[tid] = BF16::rd(a.noise_scale * irm);
-      rc[256 + tid] = BF16::rd(irm * a.out_bound);
+      rc[tid] = D::rd(a.noise_scale * irm);
+      rc[256 + tid] = D::rd(irm * a.out_bound);
     }
   };
 
@@ -213,7 +214,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
     constexpr bool MMA = decltype(mma_c)::value, EPI = decltype(epi_c)::value;
     const int te = t - 1;
     if (EPI && (NOISE || bound_on)) {
-      const float ir_t = IRMODE == AHL_IR_STATIC ? BF16::load(a.ir, te) : 0.0f;
+      const float ir_t = IRMODE == AHL_IR_STATIC ? D::load(a.ir, te) : 0.0f;
       const float tmax = a.tile_max[te];
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj) {
@@ -221,12 +222,12 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
         const float wb_ = a.bound_per_channel ? wch[bj] : tmax;
         float nscale = 0.0f, Bc = 0.0f, rc = 1.0f, rcpc = 1.0f;
         if (IRMODE == AHL_IR_STATIC) {
-          if (NOISE) nscale = BF16::rd(wr_ * BF16::rd(a.noise_scale * ir_t));
+          if (NOISE) nscale = D::rd(wr_ * D::rd(a.noise_scale * ir_t));
           if (bound_on) {
-            Bc = BF16::rd(BF16::rd(ir_t * a.out_bound) * wb_);
+            Bc = D::rd(D::rd(ir_t * a.out_bound) * wb_);
             if (ADC) {
-              rc = adc_step(Bc, a);
-              rcpc = __fdiv_rn(1.0f, fmaxf(rc, kTinyF32));
+              rc = adc_step<D>(Bc, a);
+              rcpc = __fdiv_rn(1.0f, fmaxf(rc, D::tiny()));
             }
           }
         }
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
     if (MMA && (NOISE || bound_on)) {
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj)
-        wch[bj] = nbase + 32 * bj < a.N ? BF16::load(a.wmax, (int64_t)t * a.N + nbase + 32 * bj) : 0.0f;
+        wch[bj] = nbase + 32 * bj < a.N ? D::load(a.wmax, (int64_t)t * a.N + nbase + 32 * bj) : 0.0f;
     }
     const float* rc_t = rowc + (te & 1) * 512;
 
@@ -256,8 +257,8 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
         for (int i = 0; i < NBI; ++i)
 #pragma unroll
           for (int j = 0; j < 2; ++j) {
-            if (sg == 0) mma_bf16_zero(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
-            else mma_bf16(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
+            if (sg == 0) Mma16<D>::run_zero(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
+            else Mma16<D>::run(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
           }
         if (s == 3) end_chunk();
       }
@@ -288,7 +289,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const uint32_t tp = totp[pbi][pbj][4 * pgp + q];
-          totp[pbi][pbj][4 * pgp + q] = pack_bf16x2(unpack_lo(tp) + yp[2 * q], unpack_hi(tp) + yp[2 * q + 1]);
+          totp[pbi][pbj][4 * pgp + q] = D::pack2(D::lo(tp) + yp[2 * q], D::hi(tp) + yp[2 * q + 1]);
         }
       };
 #pragma unroll
@@ -308,8 +309,8 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
             const int sg = u * KPU + m / MPS, s = sg & 3;
             if (m % MPS == 0 && s < 3) read_frags(s + 1, (s + 1) & 1);
             const int i = (m >> 1) % NBI, j = m & 1;
-            if (sg == 0) mma_bf16_zero(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
-            else mma_bf16(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
+            if (sg == 0) Mma16<D>::run_zero(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
+            else Mma16<D>::run(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
           }
         };
         float y[8], xi[8], ns[8], Bv[8], rv[8], rcpv[8];
@@ -323,14 +324,20 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
             // of the reference to reproduce, and the sum is rounded once
             y[e] = __builtin_fmaf(ns[e], xi[e], y[e]);
             y[e + 1] = __builtin_fmaf(ns[e + 1], xi[e + 1], y[e + 1]);
-            rd2(y[e], y[e + 1]);
+            round2<D>(y[e], y[e + 1]);
           }
           if (ADC) {
-            y[e] *= rcpv[e]; y[e + 1] *= rcpv[e + 1];
-            rd2(y[e], y[e + 1]);
+            if (IRMODE == AHL_IR_STATIC) {   // the per-column reciprocal is correctly rounded
+              y[e] = D::div_exact_rcp(y[e], fmaxf(rv[e], D::tiny()), rcpv[e]);
+              y[e + 1] = D::div_exact_rcp(y[e + 1], fmaxf(rv[e + 1], D::tiny()), rcpv[e + 1]);
+            } else {
+              y[e] = D::div(y[e], fmaxf(rv[e], D::tiny()), rcpv[e]);
+              y[e + 1] = D::div(y[e + 1], fmaxf(rv[e + 1], D::tiny()), rcpv[e + 1]);
+            }
+            round2<D>(y[e], y[e + 1]);
             if (ROUND) { y[e] = rintf(y[e]); y[e + 1] = rintf(y[e + 1]); }
             y[e] *= rv[e]; y[e + 1] *= rv[e + 1];
-            rd2(y[e], y[e + 1]);
+            round2<D>(y[e], y[e + 1]);
           }
         };
         // dynamic range: the constants of the four consecutive rows of group gg
@@ -342,24 +349,24 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
               const f32x4 nr = *(const f32x4*)(rc_t + rl0);
 #pragma unroll
               for (int c = 0; c < 4; ++c) nsg[c] = wr_ * nr[c];
-              rd2(nsg[0], nsg[1]); rd2(nsg[2], nsg[3]);
+              round2<D>(nsg[0], nsg[1]); round2<D>(nsg[2], nsg[3]);
             }
             if (bound_on) {
               const f32x4 br = *(const f32x4*)(rc_t + 256 + rl0);
 #pragma unroll
               for (int c = 0; c < 4; ++c) Bg[c] = br[c] * wb_;
-              rd2(Bg[0], Bg[1]); rd2(Bg[2], Bg[3]);
+              round2<D>(Bg[0], Bg[1]); round2<D>(Bg[2], Bg[3]);
               if (ADC) {
                 if (__builtin_expect(a.step_by_division != 0, 0)) {
 #pragma unroll
-                  for (int c = 0; c < 4; ++c) rg[c] = adc_step(Bg[c], a);
+                  for (int c = 0; c < 4; ++c) rg[c] = adc_step<D>(Bg[c], a);
                 } else {
 #pragma unroll
                   for (int c = 0; c < 4; ++c) rg[c] = Bg[c] * a.step_factor;
-                  rd2(rg[0], rg[1]); rd2(rg[2], rg[3]);
+                  round2<D>(rg[0], rg[1]); round2<D>(rg[2], rg[3]);
                 }
 #pragma unroll
-                for (int c = 0; c < 4; ++c) rcg[c] = __builtin_amdgcn_rcpf(fmaxf(rg[c], kTinyF32));
+                for (int c = 0; c < 4; ++c) rcg[c] = __builtin_amdgcn_rcpf(fmaxf(rg[c], D::tiny()));
               }
             }
           }
@@ -370,7 +377,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
           for (int pr = 0; pr < 2; ++pr) {
             const int idx = 2 * (2 * gp + gg) + pr;
             const uint32_t tp = totp[bi][bj][idx];
-            totp[bi][bj][idx] = pack_bf16x2(unpack_lo(tp) + y[4 * gg + 2 * pr], unpack_hi(tp) + y[4 * gg + 2 * pr + 1]);
+            totp[bi][bj][idx] = D::pack2(D::lo(tp) + y[4 * gg + 2 * pr], D::hi(tp) + y[4 * gg + 2 * pr + 1]);
           }
         };
         bool over = false;
@@ -389,8 +396,8 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
 #pragma unroll
               for (int q = 0; q < 4; ++q) {
                 const uint32_t pv = pend[bi][bj][4 * gp + q];
-                y[2 * q] = unpack_lo(pv);
-                y[2 * q + 1] = unpack_hi(pv);
+                y[2 * q] = D::lo(pv);
+                y[2 * q + 1] = D::hi(pv);
               }
               if (NOISE) {
                 const uint32_t mrow = (uint32_t)(m0 + rbase + 16 * gp);
@@ -463,7 +470,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-          for (int v = 0; v < 8; ++v) pend[i][j][v] = pack_bf16x2(acc[i][j][2 * v], acc[i][j][2 * v + 1]);
+          for (int v = 0; v < 8; ++v) pend[i][j][v] = D::pack2(acc[i][j][2 * v], acc[i][j][2 * v + 1]);
     }
   };
 
@@ -484,13 +491,13 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
 #pragma unroll
     for (int bj = 0; bj < 2; ++bj) {
       const bool add_bias = a.bias != nullptr;
-      const float b = (add_bias && nbase + 32 * bj < a.N) ? BF16::load(a.bias, nbase + 32 * bj) : 0.0f;
+      const float b = (add_bias && nbase + 32 * bj < a.N) ? D::load(a.bias, nbase + 32 * bj) : 0.0f;
 #pragma unroll
       for (int bi = 0; bi < NBI; ++bi)
 #pragma unroll
         for (int pr = 0; pr < 8; ++pr) {
           uint32_t tp = totp[bi][bj][pr];
-          if (add_bias) tp = pack_bf16x2(unpack_lo(tp) + b, unpack_hi(tp) + b);
+          if (add_bias) tp = D::pack2(D::lo(tp) + b, D::hi(tp) + b);
           const int ro = bi * 32 + 8 * (pr >> 1) + 2 * (pr & 1);
           *(uint16_t*)(obase + ro * kOutStride + bj * 64) = (uint16_t)tp;
           *(uint16_t*)(obase + (ro + 1) * kOutStride + bj * 64) = (uint16_t)(tp >> 16);
@@ -520,22 +527,23 @@ bool pipe_fwd_eligible(const FastFwdArgs& a, int ir_mode) {
   return a.ldx <= (1 << 21) && a.ldw <= (1 << 21);
 }
 
-template <int IRMODE, bool NOISE, int QM, int CPT>
+template <class D, int IRMODE, bool NOISE, int QM, int CPT>
 static void launch_pipe_one(const FastFwdArgs& a, hipStream_t s) {
   constexpr int NBI = 2;
   const dim3 block(1024 / NBI), grid((unsigned)(cdiv(a.M, 256) * cdiv(a.N, 128)));
   // a refusal shows at the launch that follows (check_launch reads the last error)
-  (void)hipFuncSetAttribute((const void*)k_fwd_pipe<IRMODE, NOISE, QM, CPT, NBI>,
+  (void)hipFuncSetAttribute((const void*)k_fwd_pipe<D, IRMODE, NOISE, QM, CPT, NBI>,
                       hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
-  hipLaunchKernelGGL((k_fwd_pipe<IRMODE, NOISE, QM, CPT, NBI>), grid, block, kPLdsBytes, s, a);
+  hipLaunchKernelGGL((k_fwd_pipe<D, IRMODE, NOISE, QM, CPT, NBI>), grid, block, kPLdsBytes, s, a);
 }
 
 // Launches the kernel if this combination is built; false otherwise (the caller falls back).
-bool launch_pipe_fwd(const FastFwdArgs& a, int ir_mode, bool noise, int qm, hipStream_t s) {
+bool launch_pipe_fwd(int32_t dtype, const FastFwdArgs& a, int ir_mode, bool noise, int qm, hipStream_t s) {
   const int cpt = a.tile / 64;
 #define AHL_PIPE(I, NZ, Q, C)                                                          \
   if (ir_mode == I && noise == NZ && qm == Q && cpt == C) {                            \
-    launch_pipe_one<I, NZ, Q, C>(a, s);                                                \
+    if (dtype == AHL_F16) launch_pipe_one<F16, I, NZ, Q, C>(a, s);                     \
+    else launch_pipe_one<BF16, I, NZ, Q, C>(a, s);                                     \
     return true;                                                                       \
   }
   AHL_PIPE(1, true, 2, 8)

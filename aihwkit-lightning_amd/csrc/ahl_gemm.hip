@@ -306,7 +306,7 @@ __global__ __launch_bounds__(256) void k_linear_fwd(FwdArgs a) {
                 if (a.noise_on) y = D::rd(__builtin_fmaf(nscale, xi[4 * gg + c], y));
                 if (a.bound_on) {
                   if (a.adc_on) {
-                    float q = D::rd(D::div(y, rc, rcp));
+                    float q = D::rd(D::div_exact_rcp(y, rc, rcp));
                     if (!a.skip_rounding) q = rintf(q);
                     y = D::rd(q * r);
                   }

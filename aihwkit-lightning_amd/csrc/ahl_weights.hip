@@ -27,7 +27,7 @@ AHL_DEV WQuant make_wquant(float wm, float n_states, bool all_gt1) {
 
 template <class D>
 AHL_DEV float wquant_apply(float w, const WQuant& q, float maxq, bool round = true) {
-  float v = D::rd(D::div(w, q.rc, q.rcp));
+  float v = D::rd(D::div_exact_rcp(w, q.rc, q.rcp));
   v = fminf(fmaxf(v, -maxq), maxq);
   if (round) v = rintf(v);
   return D::rd(v * q.step);
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(256) void k_learned_clip_bwd(ClipBwdArgs a) {
   for (int32_t k = a.tl.start(t) + lane; k < a.tl.start(t + 1); k += 64) {
     const float w = D::load(a.w, n * a.ldw + k);
     const float g = D::load(a.dw, n * a.lddw + k);
-    const float qw = D::rd(D::div(w, q.rc, q.rcp));
+    const float qw = D::rd(D::div_exact_rcp(w, q.rc, q.rcp));
     const bool small = qw < -a.maxq, big = qw > a.maxq;
     // (indicator terms) * grad * grad_scale, evaluated in fp32 as torch promotes them
     float term;

@@ -227,6 +227,36 @@ def test_bf16_division_by_reciprocal_is_exact():
         assert torch.equal((x * bumped).to(torch.bfloat16), exact)
 
 
+def test_float16_division_through_the_reciprocal():
+    """How the kernels divide float16 values x / d (both exact in fp32), exhaustive over all pairs
+    of 11-bit significands (the significands decide; a few exponent pairs on top):
+    * with the correctly rounded fp32 reciprocal, float16(x * rcp) == float16(x / d) -- what the
+      paths whose reciprocal comes from an IEEE division use;
+    * with a reciprocal one fp32 step off (the hardware's approximate reciprocal) that fails for a
+      few pairs, and one correction step, q0 = x * rcp, r = fma(-d, q0, x), q1 = fma(r, rcp, q0),
+      gives the IEEE fp32 quotient bit for bit."""
+    def fma32(a, b, c):  # the products below are exact in float64 (at most 11 + 24 bits)
+        return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(np.float32)
+
+    sig = (1024 + np.arange(1024)).astype(np.float32)
+    x0, d0 = np.repeat(sig, 1024), np.tile(sig, 1024)
+    off_by_one_fails = 0
+    for ex, ed in ((0, 0), (-14, 15), (15, -14), (3, -2)):
+        x = np.ldexp(x0, ex - 10).astype(np.float32)
+        d = np.ldexp(d0, ed - 10).astype(np.float32)
+        want = (x / d).astype(np.float32)
+        exact_rcp = (np.float32(1.0) / d).astype(np.float32)
+        assert np.array_equal((x * exact_rcp).astype(np.float16), want.astype(np.float16)), (ex, ed)
+        for towards in (None, np.inf, -np.inf):
+            rcp = exact_rcp if towards is None else np.nextafter(exact_rcp, np.float32(towards))
+            q0 = (x * rcp).astype(np.float32)
+            if towards is not None:
+                off_by_one_fails += int((q0.astype(np.float16) != want.astype(np.float16)).sum())
+            q1 = fma32(fma32(-d, q0, x), rcp, q0)
+            assert np.array_equal(q1, want), (ex, ed, towards)
+    assert off_by_one_fails > 0
+
+
 def test_box_muller16_statistics():
     """The device transform (two 16-bit uniforms per pair) has mean 0 and variance 1 to 1e-3
     when enumerated over a full grid of its inputs."""
