@@ -25,7 +25,8 @@ from helpers import assert_close_lsb
 
 pytestmark = pytest.mark.gpu
 
-T_DTYPE = {"f32": torch.float32, "bf16": torch.bfloat16}
+T_DTYPE = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+SIXTEEN_BIT = ("bf16", "f16")
 
 
 def _layer(c, w, ir=None):
@@ -48,10 +49,10 @@ def _rd(t, dtype):
     return t.to(T_DTYPE[dtype]).float()
 
 
-def _bf16_ulp(v):
-    """Spacing of bf16 numbers at the magnitude of v (fp32 tensor)."""
-    _, e = torch.frexp(v.abs().clamp_min(1e-30))
-    return torch.ldexp(torch.ones_like(v), e - 8)
+def _ulp16(v, dtype):
+    """Spacing of the 16-bit type's numbers at the magnitude of v (fp32 tensor; normal range)."""
+    _, e = torch.frexp(v.abs().clamp_min(2.0 ** -14))
+    return torch.ldexp(torch.ones_like(v), e - (8 if dtype == "bf16" else 11))
 
 
 def _rounded_noise_var(sigma, ulp):
@@ -100,7 +101,7 @@ MLP_UP = dict(M=4096, K=3072, N=8192, max_input_size=512)
 
 # ---------------------------------------------------------------------------------------------
 # (i) / (ii) output noise per tile, ADC off
-@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
 @pytest.mark.parametrize("per_channel", [False, True], ids=["per_tile_max", "per_channel"])
 @pytest.mark.parametrize("ir_mode", ["static", "dynamic"])
 def test_output_noise_per_tile_statistics(dtype, per_channel, ir_mode):
@@ -115,7 +116,7 @@ def test_output_noise_per_tile_statistics(dtype, per_channel, ir_mode):
     xd = x.cuda()
     ranges = [3.0, 2.0, 2.5, 3.5, 1.5, 3.0, 2.75, 2.25]
     # fp32 runs on the general kernels (~12 ms per forward): three tiles are enough there
-    tiles = range(n_tiles) if dtype == "bf16" else (0, 3, 7)
+    tiles = range(n_tiles) if dtype in SIXTEEN_BIT else (0, 3, 7)
     for t in tiles:
         if ir_mode == "static":
             ir = torch.zeros(n_tiles)
@@ -134,8 +135,8 @@ def test_output_noise_per_tile_statistics(dtype, per_channel, ir_mode):
         clean = layer(xin).float()
         sigma = _noise_scale(c, ir_rows, wmax[t], n_tiles)
         var = sigma ** 2
-        if dtype == "bf16":
-            var = _rounded_noise_var(sigma, _bf16_ulp(clean))
+        if dtype in SIXTEEN_BIT:
+            var = _rounded_noise_var(sigma, _ulp16(clean, dtype))
         z = (noisy - clean).detach() / var.sqrt()
         mean, std = _moments(z)
         assert abs(mean) < 0.01, f"tile {t}: mean {mean}"
@@ -164,7 +165,7 @@ def _emulate_levels(c, acc, sigma, bound, step, gen):
     (FULL, "static", 0.04), (FULL, "static", 0.4), (FULL, "dynamic", 0.04), (FULL, "dynamic", 0.4),
     (MLP_UP, "static", 0.067), (MLP_UP, "static", 0.67),
 ], ids=["c3", "c3_x10", "c2", "c2_x10", "c4", "c4_x10"])
-@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("dtype", ["bf16", "f32", "f16"])
 def test_output_noise_with_adc_and_clamp(shape, ir_mode, out_noise, dtype):
     """Noise, ADC and clamp together at the benchmark shapes (learned range: the forward of
     configuration 3 and of the MLP block; dynamic range: configuration 2), one tile at a time:
@@ -209,7 +210,7 @@ def test_output_noise_with_adc_and_clamp(shape, ir_mode, out_noise, dtype):
         bound, step = _adc(c, ir_rows, wmax[t])
         levels = torch.round(noisy / step)
         on_grid = _rd(levels * step, dtype)
-        if dtype == "bf16":   # exactly a level, or clamped to the bound itself
+        if dtype in SIXTEEN_BIT:   # exactly a level, or clamped to the bound itself
             assert bool(((on_grid == noisy) | (noisy.abs() == bound)).all())
         else:
             assert float((on_grid - noisy).abs().max()) <= 1e-6 * float(bound.max())
@@ -264,7 +265,7 @@ def test_weight_noise_statistics_at_full_size(dtype, kind):
         sigma = _rd(0.02 * ref, dtype)
         var = (sigma ** 2).expand(n, 512)
         if dtype == "bf16":
-            var = _rounded_noise_var(sigma.expand(n, 512), _bf16_ulp(wd[:, sl]))
+            var = _rounded_noise_var(sigma.expand(n, 512), _ulp16(wd[:, sl], dtype))
         mean, std = _moments((w_eff[:, sl] - wd[:, sl]) / var.sqrt())
         assert abs(mean) < 0.01, f"tile {t}: mean {mean}"
         assert abs(std - 1.0) < 0.01, f"tile {t}: std {std}"
