@@ -149,6 +149,7 @@ struct BF16 {
   // state counts of a quantiser with <= 8 significant bits give the same step whether it is
   // computed as 2 B / n or as B * fl(2 / n) (see div)
   static constexpr int kExactStepBits = 8;
+  static constexpr bool kDoubleCanOverflow = false;   // 2 x a finite value overflows only near 3e38
 };
 
 // float16: like bfloat16, every elementwise result is rounded to the tensor dtype (round to
@@ -222,7 +223,9 @@ struct F16 {
   }
   static AHL_DEV float lo(uint32_t w) { return f16_lo(w); }
   static AHL_DEV float hi(uint32_t w) { return f16_hi(w); }
-  static constexpr int kExactStepBits = 0;   // the quantiser's step always by division
+  // state counts with <= 11 significant bits: rd(2B / n) == rd(rd(2B) * fl(1 / n)), as for div
+  static constexpr int kExactStepBits = 11;
+  static constexpr bool kDoubleCanOverflow = true;    // 2B is inf for B > 32752
 };
 
 // round two fp32 values to the 16-bit dtype D, keeping them in fp32 registers (3 instructions)

@@ -302,9 +302,7 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
                     for (int c = 0; c < 4; ++c) rv[c] = adc_step<D>(Bv[c], a);
                   } else {
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) rv[c] = Bv[c] * a.step_factor;
-                    round2<D>(rv[0], rv[1]); round2<D>(rv[2], rv[3]);
+                    adc_step4<D>(Bv, rv, a);
                   }
 #pragma unroll
                   for (int c = 0; c < 4; ++c) rcpv[c] = __builtin_amdgcn_rcpf(fmaxf(rv[c], D::tiny()));

@@ -53,10 +53,31 @@ AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
 // 2 * res; for n with <= 8 significant bits the product with fl(2 / n) rounds to the same bf16 as
 // the quotient (see BF16::div). Only other n need the division; that case is a branch on a
 // launch constant, so the common one carries no division code.
+// float16: the same holds for n with <= 11 significant bits (BOTH facts are checked exhaustively
+// on the CPU), but 2B itself can leave the type's range (B > 32752): it is rounded first, so that
+// such a bound gives the infinite step the reference gets.
 template <class D = BF16>
 AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
-  if (__builtin_expect(a.step_by_division != 0, 0)) return D::rd(__fdiv_rn(B + B, a.out_res));
+  if (__builtin_expect(a.step_by_division != 0, 0)) return D::rd(__fdiv_rn(D::rd(B + B), a.out_res));
+  if (D::kDoubleCanOverflow) return D::rd(D::rd(B + B) * (0.5f * a.step_factor));
   return D::rd(B * a.step_factor);
+}
+
+// the same for four bounds at once, rounded in pairs (the product form only)
+template <class D>
+AHL_DEV void adc_step4(const float* B, float* r, const FastFwdArgs& a) {
+  if (D::kDoubleCanOverflow) {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) r[c] = B[c] + B[c];
+    round2<D>(r[0], r[1]); round2<D>(r[2], r[3]);
+    const float hf = 0.5f * a.step_factor;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) r[c] *= hf;
+  } else {
+#pragma unroll
+    for (int c = 0; c < 4; ++c) r[c] = B[c] * a.step_factor;
+  }
+  round2<D>(r[0], r[1]); round2<D>(r[2], r[3]);
 }
 
 }  // namespace ahl

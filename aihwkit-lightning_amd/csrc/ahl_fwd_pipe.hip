@@ -361,9 +361,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
 #pragma unroll
                   for (int c = 0; c < 4; ++c) rg[c] = adc_step<D>(Bg[c], a);
                 } else {
-#pragma unroll
-                  for (int c = 0; c < 4; ++c) rg[c] = Bg[c] * a.step_factor;
-                  round2<D>(rg[0], rg[1]); round2<D>(rg[2], rg[3]);
+                  adc_step4<D>(Bg, rg, a);
                 }
 #pragma unroll
                 for (int c = 0; c < 4; ++c) rcg[c] = __builtin_amdgcn_rcpf(fmaxf(rg[c], D::tiny()));

@@ -192,7 +192,15 @@ SHAPES = [
 SHAPES += [dict(c, name=c["name"].replace("bf16", "f16"), dtype="f16") for c in SHAPES if c["name"] in (
     "edge_bf16", "vec_bf16_static", "vec_bf16_dynamic", "vec_bf16_many_tiles", "fast_bf16_clamped",
     "fast_bf16_dynamic_clamped", "one_token_bf16", "pad_bf16_uneven_clamped", "tail_bf16_both_dynamic",
-    "bf16_10bit_static", "bf16_odd_states_static", "pad_bf16_lsq", "sliced_dw_bf16_clamped")]
+    "bf16_10bit_static", "bf16_16bit_dynamic", "bf16_odd_states_static", "pad_bf16_lsq",
+    "sliced_dw_bf16_clamped")]
+# float16 takes the ADC step by a product for state counts of up to 11 significant bits (the
+# twins above) and by a division beyond: 4095 states, learned and dynamic range
+SHAPES += [
+    case(f"f16_12bit_{mode}", dtype="f16", M=200, K=512, N=136, max_input_size=256, ir_mode=mode,
+         inp_res=4095, out_res=4095, out_bound=0.6, ir_decay=0.01, ir_init=2.0, w_scale=0.1, seed=64)
+    for mode in ("static", "dynamic")
+]
 # tiles narrower than the 8 inputs one thread of the weight kernels handles (several tiles per
 # thread), with the on-the-fly weight quantiser per tile and channel
 SHAPES += [

@@ -231,7 +231,8 @@ def test_float16_division_through_the_reciprocal():
     """How the kernels divide float16 values x / d (both exact in fp32), exhaustive over all pairs
     of 11-bit significands (the significands decide; a few exponent pairs on top):
     * with the correctly rounded fp32 reciprocal, float16(x * rcp) == float16(x / d) -- what the
-      paths whose reciprocal comes from an IEEE division use;
+      paths whose reciprocal comes from an IEEE division use, and the ADC step rd(2B) / n for
+      state counts n of up to 11 significant bits (n is then a float16 value like d);
     * with a reciprocal one fp32 step off (the hardware's approximate reciprocal) that fails for a
       few pairs, and one correction step, q0 = x * rcp, r = fma(-d, q0, x), q1 = fma(r, rcp, q0),
       gives the IEEE fp32 quotient bit for bit."""
