@@ -9,6 +9,7 @@ exactly between two ADC levels for several per cent of the outputs, where the la
 fp32 sum decides and a CPU and a GPU sum legitimately differ), and fast_mode (its range gradient
 is the difference of two large bf16-rounded sums; the golden cases cover it).
 """
+import math
 import random
 
 import pytest
@@ -18,7 +19,7 @@ from conv_cases import conv_case, make_conv_inputs, out_size
 from golden_cases import DTYPES, case
 from helpers import assert_close_lsb, case_input_range, oracle_cfg, oracle_fwd_bwd
 from oracle import conv_mode as oc
-from test_hip_linear import check_against
+from test_hip_linear import ROUNDING_STEP, check_against
 
 pytestmark = pytest.mark.gpu
 
@@ -116,6 +117,8 @@ def conv_cases(seed, count):
 
 
 CONV = conv_cases(0, 48)
+# a third of them once more in float16
+CONV += [dict(c, dtype="f16", name=c["name"] + "_f16") for c in conv_cases(0, 48)[::3]]
 
 
 @pytest.mark.parametrize("c", CONV, ids=[c["name"] for c in CONV])
@@ -152,13 +155,25 @@ def test_random_convolutions(c):
         ref_out, dx = ref_out[0], dx[0]
     rtol = {"f32": 1e-5, "bf16": 1e-2, "f16": 1e-3}[c["dtype"]]
     lsb = None
-    if c["ir_mode"] != "none":  # an upper bound of the ADC step: 2 * range * out_bound * max|w| / 254
+    if c["ir_mode"] == "static":  # an upper bound of the ADC step: 2 * range * out_bound * max|w| / 254
         lsb = 2 * 2.0 * c["out_bound"] * float(w.abs().max()) / 254 * 1.05
+    elif c["ir_mode"] == "dynamic":  # the range is the patch's own abs-max
+        lsb = 2 * float(x.abs().max()) * c["out_bound"] * float(w.abs().max()) / 254 * 1.05
+    elif c["dtype"] in ROUNDING_STEP:
+        # no ADC: a tile product on a rounding midpoint of the 16-bit type (see check_against)
+        top = float(ref_out.abs().max())
+        lsb = ROUNDING_STEP[c["dtype"]] * 2.0 ** math.ceil(math.log2(max(top, 1e-30)))
+    def step16(ref):
+        # float16 gradients: a per-tile partial on a rounding midpoint, as for the outputs
+        if c["dtype"] != "f16":
+            return None
+        return ROUNDING_STEP["f16"] * 2.0 ** math.ceil(math.log2(max(float(ref.abs().max()), 1e-30)))
+
     assert_close_lsb(out.detach().cpu().float(), ref_out.float(), rtol, lsb, what="out")
-    assert_close_lsb(xin.grad.cpu().float(), dx.float(), rtol, None, what="dx")
+    assert_close_lsb(xin.grad.cpu().float(), dx.float(), rtol, step16(dx), what="dx")
     wgrad = layer.weight.grad.cpu()
-    assert_close_lsb((wgrad.squeeze(-2) if one else wgrad).float(), dw.float(), rtol, None, what="dw")
+    assert_close_lsb((wgrad.squeeze(-2) if one else wgrad).float(), dw.float(), rtol, step16(dw), what="dw")
     if b is not None:
-        assert_close_lsb(layer.bias.grad.cpu().float(), db.float(), rtol, None, what="db")
+        assert_close_lsb(layer.bias.grad.cpu().float(), db.float(), rtol, step16(db), what="db")
     if dir_ is not None and layer.input_range.grad is not None:
         assert_close_lsb(layer.input_range.grad.cpu().float(), dir_.float(), rtol, None, what="dir")
