@@ -704,7 +704,8 @@ def main():
     del layer, x, g
     torch.cuda.empty_cache()
     others = {}
-    for name in ("fwd_dynamic_4096", "mlp_3072_8192", "linear_4096_f16", "lstm_1024"):
+    for name in ("fwd_dynamic_4096", "mlp_3072_8192", "linear_4096_f16", "linear_11008", "conv2d_256",
+                 "lstm_1024"):
         res = time_other(name, 10, 3, graph=True) if name != "lstm_1024" else time_other(name, 4, 2, graph=True)
         res["frac_of_bf16_mfma_peak"] = round(res["tflops"] / PEAK_BF16_TFLOPS, 4)
         others[name] = res
@@ -714,6 +715,12 @@ def main():
         "workload": post["config"]["workload"], "ms": post["ms_per_step"], "parts_ms": post["config"]["ms"],
         "GB/s": post["value"], "frac_hbm": post["roofline"]["frac"],
         "cpu_baseline": post.get("cpu_baseline"),
+    }
+    # the workload of the reference's own speed script (float16, small layers, optimizer step)
+    others["reference_speed_test"] = {
+        "workload": "the reference's tests/test_speed.py fwd+bwd+step benchmark: float16, 512 rows, square "
+                    "AnalogLinear of 128 ... 2048, all non-idealities on",
+        "us_per_step": time_reference_speed_test(),
     }
     result["other_configs"] = others
     print(json.dumps(result))
