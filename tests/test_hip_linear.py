@@ -254,6 +254,51 @@ def test_leading_dims_and_1d_input():
             assert param.grad is not None and not bool(param.grad.any())
 
 
+def _as_view(t, layout):
+    """A device tensor equal to ``t`` [M, K] whose memory is laid out as ``layout`` says."""
+    rows, cols = t.shape
+    if layout == "offset_by_one_element":      # data pointer not on a 16-byte boundary
+        buf = torch.empty(rows * cols + 3, dtype=t.dtype, device="cuda")
+        view = buf[1:1 + rows * cols].view(rows, cols)
+    elif layout == "columns_3_on_of_wider_rows":  # odd offset and a row stride larger than K
+        view = torch.empty(rows, cols + 5, dtype=t.dtype, device="cuda")[:, 3:3 + cols]
+    elif layout == "wider_rows":
+        view = torch.empty(rows, cols + 8, dtype=t.dtype, device="cuda")[:, :cols]
+    elif layout == "transposed":
+        view = torch.empty(cols, rows, dtype=t.dtype, device="cuda").t()
+    else:
+        return t.cuda()
+    view.copy_(t)
+    return view
+
+
+@pytest.mark.parametrize("layout", ["offset_by_one_element", "columns_3_on_of_wider_rows", "wider_rows",
+                                    "transposed"])
+@pytest.mark.parametrize("name", ["fast_bf16_clamped", "fast_f16_dynamic_clamped", "edge_f32",
+                                  "pad_bf16_uneven_clamped"])
+def test_inputs_and_gradients_that_are_views(name, layout):
+    """The input and the incoming gradient as views of other storage (misaligned pointers, row
+    strides that are not K, a transposed buffer): the same results, bit for bit, as with
+    contiguous tensors."""
+    from hip_helpers import hip_fwd_bwd, make_layer
+
+    c = next(s for s in SHAPES if s["name"] == name)
+    x, w, b, g = make_inputs(c)
+    want = hip_fwd_bwd(c, inputs=(x, w, b, g))
+    layer = make_layer(c, inputs=(x, w, b, g))
+    xin = _as_view(x, layout).requires_grad_(True)
+    torch.manual_seed(c["noise_seed"])
+    out = layer(xin)
+    out.backward(_as_view(g, layout))
+    assert torch.equal(out.detach().cpu(), want["out"])
+    assert torch.equal(xin.grad.cpu(), want["dx"])
+    assert torch.equal(layer.weight.grad.cpu(), want["dw"])
+    if want["db"] is not None:
+        assert torch.equal(layer.bias.grad.cpu(), want["db"])
+    if want["dir"] is not None:
+        assert torch.equal(layer.input_range.grad.cpu(), want["dir"])
+
+
 @pytest.mark.parametrize("name", ["sliced_dx_bf16_clamped", "pad_bf16_384_static_clamped",
                                   "pad_bf16_uneven_clamped"])
 def test_no_grad_forward_equals_the_differentiable_forward(name):
