@@ -87,6 +87,29 @@ def test_full_size_analog_matches_oracle(ir_mode, dtype):
                          what=f"{c['name']} {key}")
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("out_bound", [10.0, 0.9], ids=["rare_clamps", "frequent_clamps"])
+def test_the_two_forward_kernels_agree_bit_for_bit(dtype, out_bound, monkeypatch):
+    """Large grids with a learned range run the kernel that works a tile's epilogue off inside the
+    next tile's product loop; AHL_FORWARD_KERNEL=blocks in the environment keeps them on the kernel
+    for small grids. Same seed, output noise, ADC and clamp on: outputs (noise draws included),
+    clamp-dependent gradients and all, bit for bit."""
+    from hip_helpers import hip_fwd_bwd
+
+    c = case(f"two_kernels_{dtype}", ir_mode="static", inp_res=254, out_res=254, out_bound=out_bound,
+             out_noise=0.04, clip="channel", clip_sigma=2.5, ir_decay=0.01, ir_init=3.0, w_scale=0.02,
+             seed=43, **dict(FULL, dtype=dtype))
+    inputs = make_inputs(c)
+    monkeypatch.delenv("AHL_FORWARD_KERNEL", raising=False)
+    piped = hip_fwd_bwd(c, inputs=inputs)
+    monkeypatch.setenv("AHL_FORWARD_KERNEL", "blocks")
+    blocks = hip_fwd_bwd(c, inputs=inputs)
+    for key in ("out", "dx", "dw", "db", "dir"):
+        if piped.get(key) is not None:
+            assert torch.equal(piped[key], blocks[key]), key
+    assert bool(piped["out"].float().std() > 0)
+
+
 def test_llama_mlp_block_matches_oracle():
     """Configuration 4 of the baseline: a LLaMA-style MLP block (hidden 3072, intermediate 8192,
     SiLU gating: down(silu(gate(x)) * up(x))), bf16, 4096 tokens, tiles of 512, 8-bit DAC/ADC,
