@@ -44,14 +44,16 @@ def check_against(res, ref, c, tag):
 
     rtol = RTOL[c["dtype"]]
     lsb = adc_lsb(c)
-    if lsb is None and c["dtype"] in ROUNDING_STEP:
-        # Without an ADC the last rounding is the tile product's own, to the 16-bit type. A product
-        # whose fp32 sum lies within a few fp32 steps of the midpoint between two 16-bit values is
-        # rounded up or down by the order of the summation, which differs between the MFMA kernels
-        # and the CPU: such an element may be one 16-bit step (at the tensor's largest magnitude,
-        # the bound of a tile product) away, under the same 0.1 % cap as the ADC's steps.
+    if c["dtype"] in ROUNDING_STEP:
+        # Without an ADC (or with one finer than the type itself: 65534 states) the last rounding
+        # is the tile product's own, to the 16-bit type. A product whose fp32 sum lies within a few
+        # fp32 steps of the midpoint between two 16-bit values is rounded up or down by the order of
+        # the summation, which differs between the MFMA kernels and the CPU: such an element may be
+        # one 16-bit step (at the tensor's largest magnitude, the bound of a tile product) away,
+        # under the same 0.1 % cap as the ADC's steps.
         top = float(ref["out"].abs().max())
-        lsb = ROUNDING_STEP[c["dtype"]] * 2.0 ** math.ceil(math.log2(max(top, 1e-30)))
+        step16 = ROUNDING_STEP[c["dtype"]] * 2.0 ** math.ceil(math.log2(max(top, 1e-30)))
+        lsb = step16 if lsb is None else torch.clamp_min(torch.as_tensor(lsb, dtype=torch.float64), step16)
     assert_close_lsb(res["out"], ref["out"].float().to(res["out"].dtype), rtol, lsb, what=f"{tag} out")
     # gradients: an output LSB flip never enters them (straight-through), only clamp-mask flips
     for key in ("dx", "dw", "db", "dir", "dlwc"):
