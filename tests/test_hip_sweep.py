@@ -66,6 +66,31 @@ LINEAR += [dict(c, dtype="f16", name=c["name"] + "_f16") for c in linear_cases(2
 LINEAR += [dict(c, dtype="f16", name=c["name"] + "_f16") for c in linear_cases(3, 48)]
 
 
+def resolution_cases(seed, count):
+    """DAC / ADC / weight-quantiser resolutions of every kind (numbers of states with few and with
+    many significant bits, odd ones, relative resolutions) for the two 16-bit types: the quotient
+    and step arithmetic of the kernels (products with reciprocals, a correction step, divisions)."""
+    res = [2, 3, 5, 14, 30, 254, 255, 1000, 1022, 2046, 2047, 2048, 4094, 4095, 65534, 1 / 254, 1 / 30,
+           0.37, 1 / 1022]
+    rng = random.Random(seed)
+    cases = []
+    for i in range(count):
+        kw = dict(M=rng.choice([17, 130, 256, 300]), K=rng.choice([64, 256, 512, 1024]),
+                  N=rng.choice([8, 72, 128, 256]), max_input_size=rng.choice([-1, 64, 128, 256]),
+                  ir_mode=rng.choice(["static", "dynamic"]), inp_res=rng.choice(res), out_res=rng.choice(res),
+                  out_bound=rng.choice([0.3, 0.6, 2.0, 10.0]), ir_init=rng.choice([1.0, 2.0, 3.0]),
+                  ir_decay=0.01, w_scale=0.1, seed=4000 + 100 * seed + i, clip=rng.choice(["none", "channel"]),
+                  clip_sigma=2.5, bias=rng.random() < 0.5)
+        if rng.random() < 0.3:
+            kw.update(weight_quant=rng.choice(["discretize", "discretize_per_channel"]),
+                      modifier_res=rng.choice(res))
+        cases += [case(f"res_{seed}_{i}_{dt}", dtype=dt, **kw) for dt in ("f16", "bf16")]
+    return cases
+
+
+LINEAR += resolution_cases(1, 40)
+
+
 @pytest.fixture(autouse=True)
 def _pad_channels_at_test_sizes(monkeypatch):
     """The host pads odd output widths only for large products; lower the threshold so that the
