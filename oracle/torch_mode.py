@@ -229,6 +229,35 @@ def ir_fast_update(x_t: Tensor, ir: Tensor, idx: Tensor, x_min: Tensor, x_max: T
     ir[t] = max(x_min[t].abs(), x_max[t].abs())
 
 
+# Test instrumentation: when set, ``PRODUCT_HOOK(xq, w_eff, y, post)`` sees every tile product of
+# :func:`linear_forward` before noise / ADC / clamp and returns the product to go on with. The tie
+# analysis of the GPU parity tests uses it to find (and to resolve the other way) products whose
+# exact value lies within the fp32 accumulation error of a rounding decision; nothing else sets it.
+PRODUCT_HOOK = None
+# The same for the DAC: ``DAC_HOOK(xc, step, xq, skip_rounding)`` sees the clamped input of a tile,
+# its quantisation step and the quantised input, and returns the quantised input to go on with.
+# Networks of several layers use it: the input of a later layer comes out of exp / tanh, whose
+# last place differs between a CPU and a GPU, so a DAC level can hang on that last place.
+DAC_HOOK = None
+
+
+def tile_output(y: Tensor, post: Dict) -> Tuple[Tensor, Optional[Tensor]]:
+    """What follows the product of one tile (torch_utils/torch_linear.py:255-309): output noise
+    (``post["noise"]``: the scaled normal draw), ADC with step ``post["step"]``, clamp to
+    ``post["bound"]``. Returns the tile output and the mask of unclamped elements (or None)."""
+    if post["noise"] is not None:
+        y = y + post["noise"]
+    keep = None
+    if post["bound"] is not None:
+        bound = post["bound"]
+        if post["step"] is not None:
+            y = quantize(y, post["step"], post["skip_rounding"])
+        if post["clamp"]:
+            keep = (y >= -bound) & (y <= bound)
+            y = torch.clamp(y, min=-bound, max=bound)
+    return y, keep
+
+
 def linear_forward(
     x: Tensor,
     weights: Tensor,
@@ -278,7 +307,10 @@ def linear_forward(
             xc = x_t
         rec["ir"] = ir_t
         if cfg.inp_res > 0:
-            xq = quantize(xc, quant_step(ir_t, cfg.inp_res), cfg.skip_rounding)
+            dac_step = quant_step(ir_t, cfg.inp_res)
+            xq = quantize(xc, dac_step, cfg.skip_rounding)
+            if DAC_HOOK is not None:
+                xq = DAC_HOOK(xc, dac_step, xq, cfg.skip_rounding)
         else:
             xq = xc
         w_t = weights[:, lo:hi]
@@ -296,19 +328,20 @@ def linear_forward(
                                       None if w_xi is None else w_xi[t])
         # one fp32-accumulated product, rounded once to the tensor dtype
         y = matmul_rounded(xq, w_eff.T)
+        post: Dict = {"noise": None, "bound": None, "step": None, "clamp": cfg.out_bound > 0,
+                      "skip_rounding": cfg.skip_rounding}
         if noise_on:
             wr = wmax_t.view(1, -1) if cfg.out_noise_per_channel else wmax_t.max()
             xi = torch.randn_like(y) if out_xi is None else out_xi[t]
-            y = y + wr * (cfg.out_noise / sqrt(n_tiles) * ir_t) * xi
-        keep = None
+            post["noise"] = wr * (cfg.out_noise / sqrt(n_tiles) * ir_t) * xi
         if bound_on:
             wb = wmax_t.view(1, -1) if cfg.bound_per_channel else wmax_t.max()
-            bound = (ir_t * cfg.out_bound) * wb
+            post["bound"] = (ir_t * cfg.out_bound) * wb
             if adc_on:
-                y = quantize(y, quant_step(bound, cfg.out_res), cfg.skip_rounding)
-            if cfg.out_bound > 0:
-                keep = (y >= -bound) & (y <= bound)
-                y = torch.clamp(y, min=-bound, max=bound)
+                post["step"] = quant_step(post["bound"], cfg.out_res)
+        if PRODUCT_HOOK is not None:
+            y = PRODUCT_HOOK(xq, w_eff, y, post)
+        y, keep = tile_output(y, post)
         out = out + y
         rec.update(xq=xq, w_eff=w_eff, keep=keep)
         saved["tiles"].append(rec)

@@ -59,7 +59,7 @@ def test_full_size_analog_matches_oracle(ir_mode, dtype):
     inputs = make_inputs(c)
     res = hip_fwd_bwd(c, inputs=inputs)
     torch.set_num_threads(16)
-    ref = oracle_fwd_bwd(c)
+    ref = oracle_fwd_bwd(c, ties=False)   # the float64 tie analysis is for small cases; the rule is stated below
     # An ADC level that flips in one tile (rounding-boundary tie, from the different fp32
     # accumulation order of the two GEMMs) moves that tile's output by one ADC step; the bf16
     # running sum over the 8 tiles can then land on the neighbouring bf16 value of a partial sum

@@ -13,7 +13,8 @@ import pytest
 import torch
 
 from golden_cases import CASES, DTYPES, case, make_inputs
-from helpers import assert_close_lsb, golden, golden_tensor, oracle_fwd_bwd
+from helpers import (assert_close_lsb, assert_close_ties, golden, golden_tensor, oracle_fwd_bwd,
+                     rel_scale_mismatch)
 from oracle import torch_mode as om
 
 pytestmark = pytest.mark.gpu
@@ -39,10 +40,13 @@ def adc_lsb(c, wmax_scale=None):
     return 2.0 * ir_max * c["out_bound"] * w_max / n
 
 
-def check_against(res, ref, c, tag):
+def check_against(res, ref, c, tag, ties=None):
+    """``ties``: the oracle's record of the decisions that hang on the accumulation order
+    (``helpers.tie_allowances``; taken from ``ref["_ties"]`` when the oracle produced ``ref``)."""
     from hip_helpers import hip_fwd_bwd  # noqa: F401  (import checks the package loads)
 
     rtol = RTOL[c["dtype"]]
+    ties = ref.get("_ties") if ties is None else ties
     lsb = adc_lsb(c)
     if c["dtype"] in ROUNDING_STEP:
         # Without an ADC (or with one finer than the type itself: 65534 states) the last rounding
@@ -54,13 +58,22 @@ def check_against(res, ref, c, tag):
         top = float(ref["out"].abs().max())
         step16 = ROUNDING_STEP[c["dtype"]] * 2.0 ** math.ceil(math.log2(max(top, 1e-30)))
         lsb = step16 if lsb is None else torch.clamp_min(torch.as_tensor(lsb, dtype=torch.float64), step16)
-    assert_close_lsb(res["out"], ref["out"].float().to(res["out"].dtype), rtol, lsb, what=f"{tag} out")
-    # gradients: an output LSB flip never enters them (straight-through), only clamp-mask flips
+    want = ref["out"].float().to(res["out"].dtype)
+    assert_close_lsb(res["out"], want, rtol, lsb, what=f"{tag} out")
+    if ties is not None:
+        # an output may be a step off only where the oracle itself finds a tile product within the
+        # accumulation error of a change of ADC level or clamp decision
+        stray = rel_scale_mismatch(res["out"], want, rtol) & ~ties["near_out"]
+        assert not bool(stray.any()), f"{tag} out: {int(stray.sum())} elements differ where no tile has a tie"
+    # Gradients: a flipped ADC level never enters them (straight-through); a flipped clamp decision
+    # of one (row, channel, tile) does, over the whole tile span of that row of dx and of that
+    # channel of dw (and from there the input-range and learnable-clip gradients). The bias
+    # gradient does not see the mask.
     for key in ("dx", "dw", "db", "dir", "dlwc"):
         if ref.get(key) is None:
             continue
         assert res.get(key) is not None, f"{tag}: no {key} from the HIP path"
-        assert_close_lsb(res[key].float(), ref[key].float(), rtol, None, what=f"{tag} {key}")
+        assert_close_ties(res[key].float(), ref[key].float(), rtol, ties, key, what=f"{tag} {key}")
 
 
 @pytest.mark.parametrize("c", NOISELESS, ids=[c["name"] for c in NOISELESS])
@@ -72,7 +85,7 @@ def test_golden_cases_match_oracle_and_reference(c):
     check_against(res, ref, c, c["name"] + " vs oracle")
     gold = {k: golden_tensor(f"{c['name']}/{k}") if f"{c['name']}/{k}" in golden() else None
             for k in ("out", "dx", "dw", "db", "dir", "dlwc")}
-    check_against(res, gold, c, c["name"] + " vs reference")
+    check_against(res, gold, c, c["name"] + " vs reference", ties=ref["_ties"])
 
 
 SHAPES = [
