@@ -263,8 +263,11 @@ class HipLinear(Function):
             stride,
             state_ptr,
             # what "something was clamped" looks like in this call's one-word flag: a value of
-            # its own per call, so that the forward need not clear the word first
-            next_flag_token(),
+            # its own per call, so that the forward need not clear the word first. A call that is
+            # being recorded into a graph passes 0 instead (the library's own clearing launch is
+            # recorded): a token baked into the recording would be the same on every replay, and
+            # after the first replay that clamps every later one would find a stale match
+            0 if torch.cuda.is_current_stream_capturing() else next_flag_token(),
         ]
         fcfg = [
             float(fwd.inp_res), float(fwd.out_res), float(fwd.out_bound),

@@ -4,6 +4,7 @@ Each op allocates its outputs and scratch with torch (device memory plumbing onl
 device pointers, sizes and the current HIP stream to one C entry point, and returns. The ops are
 registered for the CUDA (= ROCm/HIP) dispatch key only: calling them on CPU tensors raises.
 """
+import threading
 from ctypes import byref, c_void_p
 from functools import lru_cache
 from typing import List, Optional, Tuple
@@ -30,8 +31,14 @@ def dtype_id(dtype: torch.dtype) -> int:
 # Shape inference ("fake" / meta kernels, what torch.compile and torch.library.opcheck ask an
 # op for) runs the op's own Python with the launches left out: inside `_shapes_only()` pointers
 # and the stream are null, every entry point returns 0 (the OK status; as a workspace size: no
-# workspace) without being called, and sizes may be symbolic.
-_SHAPES_ONLY = [0]
+# workspace) without being called, and sizes may be symbolic. The switch is per thread: while one
+# thread traces, the autograd engine's device thread (which runs the backward ops) must go on
+# launching.
+class _ShapesOnly(threading.local):
+    depth = 0
+
+
+_SHAPES_ONLY = _ShapesOnly()
 
 
 class _NoLaunch:
@@ -42,22 +49,22 @@ class _NoLaunch:
 
 
 def _lib():
-    return _NoLaunch() if _SHAPES_ONLY[0] else L.load()
+    return _NoLaunch() if _SHAPES_ONLY.depth else L.load()
 
 
 def _shapes_only(fn):
     """``fn`` as a fake kernel: same outputs (shapes, dtypes, devices), nothing launched."""
     def fake(*args, **kwargs):
-        _SHAPES_ONLY[0] += 1
+        _SHAPES_ONLY.depth += 1
         try:
             return fn(*args, **kwargs)
         finally:
-            _SHAPES_ONLY[0] -= 1
+            _SHAPES_ONLY.depth -= 1
     return fake
 
 
 def _ptr(tensor: Optional[Tensor]):
-    if tensor is None or _SHAPES_ONLY[0]:
+    if tensor is None or _SHAPES_ONLY.depth:
         return None
     return c_void_p(tensor.data_ptr())
 
@@ -67,11 +74,11 @@ def _ref(struct):
 
 
 def _aligned16(tensor: Tensor) -> bool:
-    return bool(_SHAPES_ONLY[0]) or tensor.data_ptr() % 16 == 0
+    return bool(_SHAPES_ONLY.depth) or tensor.data_ptr() % 16 == 0
 
 
 def _stream():
-    if _SHAPES_ONLY[0]:
+    if _SHAPES_ONLY.depth:
         return None
     # the raw handle of torch's current stream, without building a Stream object per launch
     return c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))  # pylint: disable=protected-access
@@ -237,7 +244,7 @@ def conv_geom(geom: List[int]) -> L.AhlConvGeom:
     geometry struct."""
     if len(geom) != 17:
         raise HipBackendError(f"a convolution geometry has 17 integers, got {len(geom)}")
-    if _SHAPES_ONLY[0]:
+    if _SHAPES_ONLY.depth:
         return None
     out = L.AhlConvGeom()
     out.batch, out.channels = int(geom[0]), int(geom[1])
@@ -252,7 +259,7 @@ def conv_geom(geom: List[int]) -> L.AhlConvGeom:
 
 def conv_out_size(geom: List[int]) -> List[int]:
     """Output extents (3) of a convolution geometry; host arithmetic in the library."""
-    if _SHAPES_ONLY[0]:   # the same formula on what may be symbolic sizes
+    if _SHAPES_ONLY.depth:   # the same formula on what may be symbolic sizes
         return [(geom[2 + i] + 2 * geom[11 + i] - geom[14 + i] * (geom[5 + i] - 1) - 1) // geom[8 + i] + 1
                 for i in range(3)]
     out = (L.c_int32 * 3)()
@@ -656,7 +663,7 @@ def linear_fwd(
         keep[:, :, m_rows:].zero_()   # the padding rows: defined contents for whoever compares masks
     flag = torch.empty((1,) if want_keep else (0,), dtype=torch.int32, device=ref.device)
     ws_bytes = 0
-    if xq is not None and SPLIT_FEW_ROW_FORWARD and not _SHAPES_ONLY[0]:
+    if xq is not None and SPLIT_FEW_ROW_FORWARD and not _SHAPES_ONLY.depth:
         ws_bytes = _fwd_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype)
     ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=ref.device) if ws_bytes else None
     L.check(

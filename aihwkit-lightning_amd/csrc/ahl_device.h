@@ -111,6 +111,7 @@ struct F32 {
   // x / d, where rcp_d is 1/d: fp32 tensors use the IEEE quotient like torch on the CPU.
   static AHL_DEV float div(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
   static AHL_DEV float div_exact_rcp(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
+  static AHL_DEV float div_to_round(float x, float d, float /*rcp_d*/) { return __fdiv_rn(x, d); }
 };
 
 struct BF16 {
@@ -142,6 +143,7 @@ struct BF16 {
   // rounds the returned value with rd().
   static AHL_DEV float div(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
   static AHL_DEV float div_exact_rcp(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
+  static AHL_DEV float div_to_round(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
   // two values as one register of 16-bit halves (rounded to nearest even), and back
   static AHL_DEV uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
   static AHL_DEV float lo(uint32_t w) { return unpack_lo(w); }
@@ -197,9 +199,18 @@ struct F16 {
     return v;
   }
   // 11-bit significands. With the CORRECTLY ROUNDED fp32 reciprocal, rounding x * rcp_d to
-  // float16 equals rounding x / d for every pair of float16 values (exhaustive over the
-  // significands), as for bfloat16; the caller rounds the returned value with rd().
-  static AHL_DEV float div_exact_rcp(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
+  // float16 equals rounding x / d for every pair of float16 values whose quotient is a NORMAL
+  // float16 (exhaustive over the significands), as for bfloat16. A quotient below 2^-14 is rounded
+  // on the subnormal grid, where the exact quotient can be a tie that fl32(1 / d) tips (x = 5.424e-6,
+  // d = 14 is one of them): there the corrected quotient of div() is taken, which is the IEEE fp32
+  // quotient for subnormal x as well. The caller rounds the returned value with rd().
+  static AHL_DEV float div_exact_rcp(float x, float d, float rcp_d) {
+    const float q0 = x * rcp_d;
+    return fabsf(q0) < 6.2e-5f ? div(x, d, rcp_d) : q0;
+  }
+  // The same for a quotient that is rounded to an integer next: below 2^-14 that is zero (with the
+  // quotient's sign) whichever neighbour on the subnormal grid the float16 rounding picked.
+  static AHL_DEV float div_to_round(float x, float /*d*/, float rcp_d) { return x * rcp_d; }
   // With a reciprocal that is one fp32 step off (v_rcp_f32) a few products land on the other
   // side of a float16 rounding boundary, so the fp32 IEEE quotient is needed. For float16-valued
   // x and d it takes one correction step instead of the full division

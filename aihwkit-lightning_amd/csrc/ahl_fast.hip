@@ -319,8 +319,9 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
             if (ADC) {
 #pragma unroll
               for (int c = 0; c < 4; ++c)
-                y[c] = IRMODE == AHL_IR_STATIC ? D::div_exact_rcp(y[c], fmaxf(rv[c], D::tiny()), rcpv[c])
-                                               : D::div(y[c], fmaxf(rv[c], D::tiny()), rcpv[c]);
+                y[c] = IRMODE != AHL_IR_STATIC ? D::div(y[c], fmaxf(rv[c], D::tiny()), rcpv[c])
+                       : ROUND ? D::div_to_round(y[c], fmaxf(rv[c], D::tiny()), rcpv[c])
+                               : D::div_exact_rcp(y[c], fmaxf(rv[c], D::tiny()), rcpv[c]);
               round2<D>(y[0], y[1]); round2<D>(y[2], y[3]);
               if (ROUND) {
 #pragma unroll

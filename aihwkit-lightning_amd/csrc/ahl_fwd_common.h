@@ -53,13 +53,19 @@ AHL_DEV void mma_bf16(const u32x4& a, const u32x4& b, f32x16& c) {
 // 2 * res; for n with <= 8 significant bits the product with fl(2 / n) rounds to the same bf16 as
 // the quotient (see BF16::div). Only other n need the division; that case is a branch on a
 // launch constant, so the common one carries no division code.
-// float16: the same holds for n with <= 11 significant bits (BOTH facts are checked exhaustively
-// on the CPU), but 2B itself can leave the type's range (B > 32752): it is rounded first, so that
+// float16: the same holds for n with <= 11 significant bits and steps that are normal float16 values
+// (BOTH facts are checked exhaustively on the CPU; smaller steps are divided), but 2B itself can leave the type's range (B > 32752): it is rounded first, so that
 // such a bound gives the infinite step the reference gets.
 template <class D = BF16>
 AHL_DEV float adc_step(float B, const FastFwdArgs& a) {
   if (__builtin_expect(a.step_by_division != 0, 0)) return D::rd(__fdiv_rn(D::rd(B + B), a.out_res));
-  if (D::kDoubleCanOverflow) return D::rd(D::rd(B + B) * (0.5f * a.step_factor));
+  if (D::kDoubleCanOverflow) {
+    const float s = D::rd(D::rd(B + B) * (0.5f * a.step_factor));
+    // a step below the smallest normal float16 is rounded on the subnormal grid, where the product
+    // with fl(1 / n) can fall on the other side of a tie than the quotient: divide there
+    if (__builtin_expect(s < 6.2e-5f && a.out_res > 1.0f, 0)) return D::rd(__fdiv_rn(D::rd(B + B), a.out_res));
+    return s;
+  }
   return D::rd(B * a.step_factor);
 }
 
@@ -71,8 +77,16 @@ AHL_DEV void adc_step4(const float* B, float* r, const FastFwdArgs& a) {
     for (int c = 0; c < 4; ++c) r[c] = B[c] + B[c];
     round2<D>(r[0], r[1]); round2<D>(r[2], r[3]);
     const float hf = 0.5f * a.step_factor;
+    float twoB[4];
 #pragma unroll
-    for (int c = 0; c < 4; ++c) r[c] *= hf;
+    for (int c = 0; c < 4; ++c) { twoB[c] = r[c]; r[c] *= hf; }
+    round2<D>(r[0], r[1]); round2<D>(r[2], r[3]);
+    // subnormal steps: by division (see adc_step)
+    if (__builtin_expect(fminf(fminf(r[0], r[1]), fminf(r[2], r[3])) < 6.2e-5f && a.out_res > 1.0f, 0)) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) r[c] = D::rd(__fdiv_rn(twoB[c], a.out_res));
+    }
+    return;
   } else {
 #pragma unroll
     for (int c = 0; c < 4; ++c) r[c] = B[c] * a.step_factor;

@@ -328,8 +328,10 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
           }
           if (ADC) {
             if (IRMODE == AHL_IR_STATIC) {   // the per-column reciprocal is correctly rounded
-              y[e] = D::div_exact_rcp(y[e], fmaxf(rv[e], D::tiny()), rcpv[e]);
-              y[e + 1] = D::div_exact_rcp(y[e + 1], fmaxf(rv[e + 1], D::tiny()), rcpv[e + 1]);
+              y[e] = ROUND ? D::div_to_round(y[e], fmaxf(rv[e], D::tiny()), rcpv[e])
+                           : D::div_exact_rcp(y[e], fmaxf(rv[e], D::tiny()), rcpv[e]);
+              y[e + 1] = ROUND ? D::div_to_round(y[e + 1], fmaxf(rv[e + 1], D::tiny()), rcpv[e + 1])
+                               : D::div_exact_rcp(y[e + 1], fmaxf(rv[e + 1], D::tiny()), rcpv[e + 1]);
             } else {
               y[e] = D::div(y[e], fmaxf(rv[e], D::tiny()), rcpv[e]);
               y[e + 1] = D::div(y[e + 1], fmaxf(rv[e + 1], D::tiny()), rcpv[e + 1]);

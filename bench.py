@@ -328,12 +328,16 @@ PREHEAT_S = 0.5
 
 
 def preheat(fn, seconds=PREHEAT_S):
-    """Run fn() back to back for `seconds` of wall clock, untimed (see PREHEAT_S)."""
+    """Run fn() back to back for `seconds` of wall clock, untimed (see PREHEAT_S); returns the
+    number of calls made."""
     t0 = time.perf_counter()
+    calls = 0
     while time.perf_counter() - t0 < seconds:
         for _ in range(10):
             fn()
+        calls += 10
         torch.cuda.synchronize()
+    return calls
 
 
 def time_other(name, steps, warmup, graph=False):
@@ -439,41 +443,93 @@ def event_time_ms(fn, reps):
     return start.elapsed_time(stop) / reps
 
 
-def kernel_rooflines(layer, x, g, reps):
-    """Per-kernel timings of the three MFMA kernels through the same custom ops the layer uses."""
+def mfma_kernel_times(x, g, weight, bias, ir, in_sizes, dynamic, out_noise, weight_noise, reps):
+    """ms per launch of the three MFMA kernels of one layer call (and of the two passes in front of
+    them), through the same custom ops the layer uses, plus torch.matmul (the vendor library) on the
+    same three products with the same operands -- what a plain product of each shape takes on this
+    box, with none of the analog work. ``g`` None: forward only."""
     from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
     from aihwkit_lightning.nn.modules.hip_utils import library as L
 
-    in_sizes = layer.in_sizes
-    wmax, tile_max, _, w_eff = OPS.weight_prep(
-        layer.weight.data, in_sizes, L.AHL_QUANT_NONE, L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02,
-        11, 1, True)
-    ir = layer.input_range.detach()
-    icfg = [L.AHL_IR_STATIC, 0, 1, 1, 0, 12345, 0]
-    fcfg = [254.0, 254.0, 10.0, 0.04, 0.01, 0.95]
-    xq, _ = OPS.dac(x, ir, in_sizes, icfg, fcfg)
-    y, keep, flag = OPS.linear_fwd(None, xq, w_eff, layer.bias.data, ir, wmax, tile_max, in_sizes, icfg,
-                                   fcfg, True)
-    flops = 2.0 * M_TOKENS * K_IN * N_OUT
-    out = {}
-    t = event_time_ms(lambda: OPS.linear_fwd(None, xq, w_eff, layer.bias.data, ir, wmax, tile_max,
-                                             in_sizes, icfg, fcfg, True), reps)
-    out["linear_fwd"] = t
-    t = event_time_ms(lambda: OPS.linear_bwd_dx(g, keep, flag, w_eff, x, ir, in_sizes, icfg, fcfg), reps)
-    out["linear_bwd_dx(+ir_grad)"] = t
-    t = event_time_ms(lambda: OPS.linear_bwd_dw(g, keep, flag, None, xq, ir, in_sizes, icfg, fcfg, True), reps)
-    out["linear_bwd_dw(+bias_grad)"] = t
+    noise_type = L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL if weight_noise else L.AHL_NOISE_NONE
+    prep = lambda: OPS.weight_prep(weight, in_sizes, L.AHL_QUANT_NONE, noise_type, 1.0, weight_noise,   # noqa: E731
+                                   11, 1, True)
+    wmax, tile_max, _, w_eff = prep()
+    w_eff = weight if w_eff is None else w_eff
+    icfg = [L.AHL_IR_DYNAMIC if dynamic else L.AHL_IR_STATIC, 0, 1, 1, 0, 12345, 0]
+    fcfg = [254.0, 254.0, 10.0, out_noise, 0.01, 0.95]
+    xq, ir_rows = OPS.dac(x, ir, in_sizes, icfg, fcfg)
+    ir_used = ir_rows if dynamic else ir
+    fwd = lambda: OPS.linear_fwd(None, xq, w_eff, bias, ir_used, wmax, tile_max, in_sizes, icfg, fcfg,   # noqa: E731
+                                 g is not None)
+    _, keep, flag = fwd()
+    out = {"linear_fwd": event_time_ms(fwd, reps)}
+    if g is not None:
+        out["linear_bwd_dx(+ir_grad)"] = event_time_ms(
+            lambda: OPS.linear_bwd_dx(g, keep, flag, w_eff, x, ir_used, in_sizes, icfg, fcfg), reps)
+        out["linear_bwd_dw(+bias_grad)"] = event_time_ms(
+            lambda: OPS.linear_bwd_dw(g, keep, flag, None, xq, ir_used, in_sizes, icfg, fcfg, bias is not None), reps)
     out["dac"] = event_time_ms(lambda: OPS.dac(x, ir, in_sizes, icfg, fcfg), reps)
-    t = event_time_ms(lambda: OPS.weight_prep(layer.weight.data, in_sizes, L.AHL_QUANT_NONE,
-                                              L.AHL_NOISE_ADD_NORMAL_PER_CHANNEL, 1.0, 0.02, 11, 1,
-                                              True), reps)
-    out["weight_prep"] = t
+    out["weight_prep"] = event_time_ms(prep, reps)
+    vendor = {"fwd": event_time_ms(lambda: torch.matmul(xq, w_eff.t()), reps)}
+    if g is not None:
+        vendor["dx"] = event_time_ms(lambda: torch.matmul(g, w_eff), reps)
+        vendor["dw"] = event_time_ms(lambda: torch.matmul(g.t(), xq), reps)
+    return out, vendor
+
+
+MFMA_KERNELS = ("linear_fwd", "linear_bwd_dx(+ir_grad)", "linear_bwd_dw(+bias_grad)")
+
+
+def mfma_roofline(times, flops):
+    """The roofline object of the slowest MFMA kernel among ``times`` ({name: ms per launch})."""
+    dom = max((k for k in times if k.split(":")[-1] in MFMA_KERNELS), key=lambda k: times[k])
+    achieved = flops[dom] / (times[dom] * 1e-3) / 1e12
+    return {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+            "ms_per_launch": {k: round(v, 4) for k, v in times.items()}}
+
+
+def kernel_rooflines(layer, x, g, reps):
+    """Per-kernel timings of the headline layer, the vendor library's plain products beside them."""
+    times, vendor = mfma_kernel_times(x, g, layer.weight.data, layer.bias.data, layer.input_range.detach(),
+                                      layer.in_sizes, False, 0.04, 0.02, reps)
     # a plain device copy of known size (256 MiB read + 256 MiB written): the yardstick that
     # HBM byte counters of a profiler run of this command are scaled by
     src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=x.device)
     dst = torch.empty_like(src)
-    out["copy_256MiB"] = event_time_ms(lambda: dst.copy_(src), reps)
-    return out, flops
+    times["copy_256MiB"] = event_time_ms(lambda: dst.copy_(src), reps)
+    return times, vendor, 2.0 * M_TOKENS * K_IN * N_OUT
+
+
+def other_config_roofline(name, reps=10):
+    """The roofline of the slowest MFMA kernel of the dynamic-range forward / the MLP block."""
+    gen = torch.Generator().manual_seed(3)
+    bf = torch.bfloat16
+    if name == "fwd_dynamic_4096":
+        x = torch.randn(8192, 4096, generator=gen).to(bf).cuda()
+        w = (0.02 * torch.randn(4096, 4096, generator=gen)).to(bf).cuda()
+        times, vendor = mfma_kernel_times(x, None, w, torch.zeros(4096, dtype=bf, device="cuda"), None,
+                                          [512] * 8, True, 0.04, 0.0, reps)
+        roof = mfma_roofline(times, {"linear_fwd": 2.0 * 8192 * 4096 * 4096})
+        roof["vendor_plain_ms"] = {k: round(v, 4) for k, v in vendor.items()}
+        return roof
+    assert name == "mlp_3072_8192"
+    times, flops, vendors = {}, {}, {}
+    for proj, k, n in (("gate/up", 3072, 8192), ("down", 8192, 3072)):
+        x = torch.randn(4096, k, generator=gen).to(bf).cuda()
+        g = torch.randn(4096, n, generator=gen).to(bf).cuda()
+        w = (0.02 * torch.randn(n, k, generator=gen)).to(bf).cuda()
+        ir = torch.full((k // 512,), 3.0, dtype=bf, device="cuda")
+        t, vendor = mfma_kernel_times(x, g, w, None, ir, [512] * (k // 512), False, 0.067, 0.0, reps)
+        for key, val in t.items():
+            times[f"{proj}:{key}"] = val
+            flops[f"{proj}:{key}"] = 2.0 * 4096 * k * n
+        vendors[proj] = {key: round(val, 4) for key, val in vendor.items()}
+        del x, g, w
+    roof = mfma_roofline(times, flops)
+    roof["vendor_plain_ms"] = vendors
+    return roof
 
 
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
@@ -633,8 +689,8 @@ def main():
         out.backward(g)
 
     if ns.kernels_only:
-        kernels, _ = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 1))
-        print(json.dumps({"ms_per_launch": kernels}))
+        kernels, vendor, _ = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 1))
+        print(json.dumps({"ms_per_launch": kernels, "vendor_plain_ms": vendor}))
         return
 
     def timed(fn):
@@ -653,7 +709,7 @@ def main():
     # two agree.
     from aihwkit_lightning.nn.graphs import CapturedStep
     ms_cold = timed(step)            # W + K steps on a GPU that was idle until now
-    preheat(step)
+    preheat_steps = preheat(step)
     ms_eager = timed(step)           # the same W + K steps at sustained clocks: the headline
     replay = CapturedStep(step)
     replay()                         # the recording itself (the GPU idles meanwhile)
@@ -663,9 +719,8 @@ def main():
     step_flops = 3 * 2.0 * M_TOKENS * K_IN * N_OUT
     value = step_flops / (ms_per_step * 1e-3) / 1e12
 
-    kernels, gemm_flops = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 5))
-    dom = max(("linear_fwd", "linear_bwd_dx(+ir_grad)", "linear_bwd_dw(+bias_grad)"),
-              key=lambda k: kernels[k])
+    kernels, vendor, gemm_flops = kernel_rooflines(layer, x.detach(), g, max(ns.steps, 5))
+    dom = max(MFMA_KERNELS, key=lambda k: kernels[k])
     achieved = gemm_flops / (kernels[dom] * 1e-3) / 1e12
     result = {
         "metric": "AnalogLinear fwd+bwd TFLOP/s (4096^2, 8192 tok, bf16) + % MFMA peak",
@@ -681,7 +736,11 @@ def main():
             "ms_per_step_eager": round(ms_eager, 4), "ms_per_step_graph_replay": round(ms_graph, 4),
             # timed regions follow PREHEAT_S seconds of the same work, untimed, so that they run at
             # sustained clocks; the same W + K steps on the GPU as the process found it (idle):
-            "preheat_s": PREHEAT_S, "ms_per_step_cold_start": round(ms_cold, 4),
+            "preheat_s": PREHEAT_S, "preheat_steps": preheat_steps,
+            "ms_per_step_cold_start": round(ms_cold, 4),
+            # torch.matmul (the vendor library) on the three products of this step, same operands:
+            # what the plain products alone take on this box, no analog work (bench-only yardstick)
+            "vendor_plain_ms": {k: round(v, 4) for k, v in vendor.items()},
         },
         "roofline": {
             "bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
@@ -708,6 +767,9 @@ def main():
                  "lstm_1024"):
         res = time_other(name, 10, 3, graph=True) if name != "lstm_1024" else time_other(name, 4, 2, graph=True)
         res["frac_of_bf16_mfma_peak"] = round(res["tflops"] / PEAK_BF16_TFLOPS, 4)
+        if name in ("fwd_dynamic_4096", "mlp_3072_8192"):
+            torch.cuda.empty_cache()
+            res["roofline"] = other_config_roofline(name)
         others[name] = res
         torch.cuda.empty_cache()
     post = time_post_training(not ns.no_cpu)

@@ -94,7 +94,9 @@ typedef struct AhlLinearCfg {
                                     nothing, the backward reads "equal to this value" -- pass the
                                     same cfg to both, and a value that differs from call to call:
                                     a stale or accidental match only makes the backward apply a
-                                    mask that clamps nothing                                     */
+                                    mask that clamps nothing. Launches recorded into a HIP graph
+                                    repeat their by-value arguments on every replay: record them
+                                    with 0 (the clearing launch is a kernel and is recorded too)  */
   uint64_t seed;                 /* Philox key for this call                                    */
   uint64_t offset;               /* Philox counter offset for this call                         */
   const uint64_t* seed_state;    /* NULL, or a DEVICE uint64[2] = {key, call counter}: the kernels
@@ -379,7 +381,10 @@ int64_t ahl_linear_bwd_dx_ws_bytes(int64_t M, int64_t K, int64_t N, int32_t n_ti
  * size return AHL_ERR_WORKSPACE (nothing is launched). The call itself allocates and frees
  * nothing. All calls on one GPU share that GPU's array: calls that overlap on one GPU (different
  * streams or threads) race; calls on one stream, or ordered by events, are safe. Nothing in the
- * array has to be cleared between calls (every slot is written before it is read).            */
+ * array has to be cleared between calls (every slot is written before it is read).
+ * The first call on each device looks up the array's device address (hipGetSymbolAddress, which
+ * may load the library's code object on that device): make one call per device OUTSIDE any
+ * stream capture before the calls that are recorded into a graph.                             */
 #define AHL_STATIC_DX_SCRATCH_BYTES (16 * 1024 * 1024)
 int ahl_linear_bwd_dx_static(const void* g, int64_t ldg, const uint32_t* clamp_mask,
                              const uint32_t* clamp_flag, const void* w_eff, int64_t ldw,

@@ -111,6 +111,14 @@ CLAMP_TIES = [
          clip="channel", clip_sigma=2.5, bias=True),
 ]
 LINEAR += CLAMP_TIES
+# float16 with ADC steps below the smallest normal float16 value (bounds of a few 1e-3: small
+# weights): steps and quotients on the subnormal grid, where the kernels divide instead of
+# multiplying with a reciprocal
+LINEAR += [case(f"subnormal_step_{n}_f16", dtype="f16", M=130, K=256, N=72, max_input_size=128, ir_mode=mode,
+                inp_res=254, out_res=n, out_bound=0.3, ir_init=1.0, ir_decay=0.01, w_scale=0.001, seed=4700 + i,
+                clip="channel", clip_sigma=2.5, bias=False)
+           for i, (n, mode) in enumerate([(14, "static"), (30, "dynamic"), (126, "static"), (254, "dynamic"),
+                                          (510, "static"), (1000, "static"), (1022, "dynamic")])]
 
 
 @pytest.fixture(autouse=True)

@@ -423,3 +423,25 @@ def test_fake_kernels_give_shapes_without_a_gpu():
         geom = [2, 8, 1, 12, 12, 1, 3, 3, 1, 1, 1, 0, 1, 1, 1, 1, 1]
         cols = OPS.im2col(torch.empty(2, 8, 1, 12, 12, device="cuda"), geom)
         assert cols.shape == (2, 144, 72) and OPS.col2im(cols, geom).shape == (2, 8, 1, 12, 12)
+
+
+def test_shape_inference_switch_is_per_thread():
+    """While one thread evaluates a fake kernel (torch.compile / opcheck tracing) the library stays
+    live for every other thread: the autograd engine's device thread runs the backward ops and must
+    launch them, not return unwritten buffers."""
+    import threading
+
+    from aihwkit_lightning.nn.modules.hip_utils import ops
+
+    seen = {}
+
+    def body():
+        seen["tracing thread"] = ops._SHAPES_ONLY.depth   # pylint: disable=protected-access
+        other = threading.Thread(target=lambda: seen.__setitem__("other thread", ops._SHAPES_ONLY.depth))
+        other.start()
+        other.join()
+        return 0
+
+    assert ops._shapes_only(body)() == 0   # pylint: disable=protected-access
+    assert seen == {"tracing thread": 1, "other thread": 0}
+    assert ops._SHAPES_ONLY.depth == 0   # pylint: disable=protected-access

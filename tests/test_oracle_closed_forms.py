@@ -258,6 +258,45 @@ def test_float16_division_through_the_reciprocal():
     assert off_by_one_fails > 0
 
 
+def test_float16_quotients_below_the_smallest_normal_value():
+    """A quotient below 2^-14 is rounded on float16's subnormal grid, where the exact quotient can be
+    a tie that the rounded reciprocal tips: float16(x * fl32(1 / d)) differs from float16(x / d) for
+    some pairs (x = 5.424e-6, d = 14 among them). The kernels therefore take the corrected quotient
+    q1 = fma(fma(-d, q0, x), rcp, q0) whenever |q0| < 6.2e-5 (F16::div_exact_rcp), and divide for an
+    ADC step that small (adc_step). Exhaustive over every finite float16 x, for the state counts the
+    resolution sweeps use and a few float16 steps as divisors: the guarded quotient equals the IEEE
+    fp32 quotient wherever the guard applies, and float16-rounds like it everywhere."""
+    def fma32(a, b, c):
+        return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(np.float32)
+
+    bits = np.arange(65536, dtype=np.uint16)
+    x = bits.view(np.float16).astype(np.float32)
+    x = x[np.isfinite(x)]
+    divisors = [14.0, 30.0, 126.0, 254.0, 510.0, 1000.0, 1022.0, 2046.0, 3.0, 5.0,
+                float(np.float16(0.0189)), float(np.float16(3.3e-3)), float(np.float16(1.7)), float(np.float16(6.5e-5))]
+    plain_fails = 0
+    for dv in divisors:
+        d = np.full_like(x, np.float32(dv))
+        want32 = (x / d).astype(np.float32)
+        rcp = (np.float32(1.0) / d).astype(np.float32)
+        q0 = (x * rcp).astype(np.float32)
+        q1 = fma32(fma32(-d, q0, x), rcp, q0)
+        q1 = np.where((x == 0) | ~np.isfinite(q0), q0, q1)   # zero keeps its sign (the device's class test)
+        small = np.abs(q0) < np.float32(6.2e-5)
+        with np.errstate(over="ignore"):
+            plain_fails += int((q0.astype(np.float16) != want32.astype(np.float16)).sum())
+            guarded = np.where(small, q1, q0)
+            assert np.array_equal(q1[small], want32[small]), dv
+            assert np.array_equal(guarded.astype(np.float16), want32.astype(np.float16)), dv
+            # the plain product is wrong only where the guard applies ...
+            wrong = q0.astype(np.float16) != want32.astype(np.float16)
+            assert not bool((wrong & ~small).any()), dv
+            # ... and rounding to an integer hides it (F16::div_to_round)
+            assert np.array_equal(np.rint(q0.astype(np.float16).astype(np.float32)),
+                                  np.rint(want32.astype(np.float16).astype(np.float32))), dv
+    assert plain_fails > 0
+
+
 def test_box_muller16_statistics():
     """The device transform (two 16-bit uniforms per pair) has mean 0 and variance 1 to 1e-3
     when enumerated over a full grid of its inputs."""

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 def _cfg(L, dtype, ir_mode, tile_stride=0):
     cfg = L.AhlLinearCfg()
-    cfg.dtype = L.AHL_BF16 if dtype == torch.bfloat16 else L.AHL_F32
+    cfg.dtype = {torch.bfloat16: L.AHL_BF16, torch.float16: L.AHL_F16, torch.float32: L.AHL_F32}[dtype]
     cfg.ir_mode = ir_mode
     cfg.inp_res, cfg.out_res, cfg.out_bound, cfg.out_noise = 254.0, 254.0, 10.0, 0.0
     cfg.bound_per_channel, cfg.training = 1, 1
@@ -36,21 +36,31 @@ def _both(L, lib, dtype, m_rows, k_in, n_out, tile, seed, with_mask):
     n_tiles = k_in // tile
     ir = torch.linspace(1.0, 3.0, n_tiles).to(dtype).cuda()
     ends = L.tile_ends_array([tile] * n_tiles)
+    # tiles that do not start on 256-column boundaries: the weights come in the padded tile layout
+    # (tile t at column t * stride, zeros up to the next tile), x and dx stay dense
+    cfg = _cfg(L, dtype, L.AHL_IR_STATIC)
+    stride = int(lib.ahl_tile_stride(k_in, n_tiles, cfg.dtype))
+    ldw = k_in
+    if stride > 0:
+        padded = torch.zeros(n_out, n_tiles * stride, dtype=dtype, device="cuda")
+        for t in range(n_tiles):
+            padded[:, t * stride:t * stride + tile] = w[:, t * tile:(t + 1) * tile]
+        w, ldw = padded, n_tiles * stride
     keep = flag = None
     if with_mask:
         rows = (m_rows + 63) // 64 * 64
         keep = (torch.rand(n_tiles, (n_out + 31) // 32, rows, generator=gen) < 0.1).to(torch.int32)
         keep = (keep * torch.randint(1, 2 ** 31 - 1, keep.shape, generator=gen, dtype=torch.int32)).cuda()
         flag = torch.ones(1, dtype=torch.int32, device="cuda")
-    cfg = _cfg(L, dtype, L.AHL_IR_STATIC)
+    cfg = _cfg(L, dtype, L.AHL_IR_STATIC, stride)
     stream = c_void_p(torch.cuda.current_stream().cuda_stream)
-    need = lib.ahl_linear_bwd_dx_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype, 0)
+    need = lib.ahl_linear_bwd_dx_ws_bytes(m_rows, k_in, n_out, n_tiles, cfg.dtype, stride)
     assert 0 < need <= L.STATIC_DX_SCRATCH_BYTES
     out = []
     for static in (False, True):
         dx = torch.full((m_rows, k_in), float("nan"), dtype=dtype, device="cuda")
         ir_grad = torch.full((n_tiles,), float("nan"), dtype=dtype, device="cuda")
-        head = [_ptr(g), n_out, _ptr(keep), _ptr(flag), _ptr(w), k_in, _ptr(x), k_in, _ptr(ir), _ptr(dx),
+        head = [_ptr(g), n_out, _ptr(keep), _ptr(flag), _ptr(w), ldw, _ptr(x), k_in, _ptr(ir), _ptr(dx),
                 k_in, _ptr(ir_grad), m_rows, k_in, n_out, ends, n_tiles, byref(cfg)]
         if static:
             rc = lib.ahl_linear_bwd_dx_static(*head, stream)
@@ -71,7 +81,13 @@ def _both(L, lib, dtype, m_rows, k_in, n_out, tile, seed, with_mask):
     (torch.bfloat16, (1024, 2048, 448, 512), (300, 512, 264, 256)),
     # fp32 general kernels: transposed weights + partial sums in the workspace
     (torch.float32, (96, 768, 640, 256), (17, 60, 24, 20)),
-], ids=["bf16_sliced", "bf16_one_slice", "f32_general"])
+    # the float16 instantiations of the MFMA kernel, sliced and not
+    (torch.float16, (64, 4096, 1024, 512), (300, 512, 264, 256)),
+    # padded tile layout (2304 inputs in tiles of 576, stride 768; then 1152 in tiles of 384,
+    # stride 512): the workspace size follows the padded width
+    (torch.bfloat16, (64, 2304, 1024, 576), (200, 1152, 128, 384)),
+    (torch.float16, (1024, 2304, 256, 576), (64, 1152, 512, 384)),
+], ids=["bf16_sliced", "bf16_one_slice", "f32_general", "f16", "bf16_padded", "f16_padded"])
 @pytest.mark.parametrize("with_mask", [False, True], ids=["no_mask", "mask"])
 def test_static_scratch_dx_equals_workspace_dx(dtype, first, second, with_mask):
     from aihwkit_lightning.nn.modules.hip_utils import library as L
