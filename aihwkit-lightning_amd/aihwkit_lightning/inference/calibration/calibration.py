@@ -16,7 +16,7 @@ from torch.utils.hooks import RemovableHandle
 from ...exceptions import ConfigError
 from ...nn import AnalogLinear
 from ...nn.modules.conv import _AnalogConvNd
-from ...nn.modules.hip_utils.ops import OPS
+from ...nn.modules.hip_utils.ops import OPS, direct
 from ...simulator.configs import TorchInferenceRPUConfig, WeightNoiseInjectionType
 
 
@@ -49,6 +49,7 @@ def _calibration_pre_forward(mod, args: Tuple, kwargs: Dict, calibration_type, c
     x_input = _tile_rows(mod, args, kwargs)
     if x_input.size(0) == 0:
         return
+    OPS = direct(x_input)   # a hook is never traced: the operators without the dispatcher hop  # noqa: N806
     ir_params = mod.rpu_config.pre_post.input_range
     if calibration_type == InputRangeCalibrationType.MAX:
         if key not in cache:

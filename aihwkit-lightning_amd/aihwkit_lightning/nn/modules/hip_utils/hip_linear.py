@@ -54,14 +54,9 @@ def check_supported(rpu_config: TorchInferenceRPUConfig) -> None:
 PAD_CHANNELS_MIN_WORK = 1 << 22
 
 
-def _ops_for(tensor: Tensor):
-    """Where HipLinear takes its operator calls from. It is an autograd node of its own, so
-    inside it the dispatcher adds nothing but time (about 10 us per call, three to six calls per
-    layer call): for a tensor on the current device the implementations are called directly. For
-    a tensor elsewhere the registered ops are used, whose dispatch switches the device."""
-    if tensor.device.index == torch.cuda.current_device():
-        return _impl
-    return _impl.OPS
+# Where HipLinear takes its operator calls from: it is an autograd node of its own, so inside it
+# the dispatcher adds nothing but time (three to six calls per layer call)
+_ops_for = _impl.direct
 
 
 # dtypes with MFMA kernels of their own (two-byte elements); float32 runs on the general kernels

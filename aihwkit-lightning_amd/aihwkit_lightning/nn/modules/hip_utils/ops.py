@@ -4,6 +4,7 @@ Each op allocates its outputs and scratch with torch (device memory plumbing onl
 device pointers, sizes and the current HIP stream to one C entry point, and returns. The ops are
 registered for the CUDA (= ROCm/HIP) dispatch key only: calling them on CPU tensors raises.
 """
+import sys
 import threading
 from ctypes import byref, c_void_p
 from functools import lru_cache
@@ -855,3 +856,13 @@ for _name, _fn in [
     torch.library.register_fake(f"aihwkit_hip::{_name}", _shapes_only(_fn), lib=LIB)
 
 OPS = torch.ops.aihwkit_hip
+
+
+def direct(tensor: Tensor):
+    """Where code that is never traced (an autograd node's own body, a calibration hook) takes its
+    operator calls from: this module's functions themselves for a tensor on the current device --
+    the dispatcher adds nothing there but time, about 10 us per call -- and the registered ops,
+    whose dispatch switches the device, for a tensor elsewhere."""
+    if tensor.device.index == torch.cuda.current_device():
+        return sys.modules[__name__]
+    return OPS

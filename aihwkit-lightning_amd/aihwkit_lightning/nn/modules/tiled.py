@@ -14,7 +14,7 @@ from torch import Tensor, no_grad
 from .base import AnalogLayerBase
 from .hip_utils import library as L
 from .hip_utils.hip_linear import HipLinear, QUANT_IDS, check_supported
-from .hip_utils.ops import OPS
+from .hip_utils.ops import OPS, direct
 from ...exceptions import HipBackendError
 from ...simulator.configs import WeightClipType, WeightQuantizationType
 
@@ -214,7 +214,9 @@ class TiledAnalogLayer(AnalogLayerBase):
         else:
             raise ValueError(f"Unknown clip type {clip_type}")
         self._require_device("clip_weights")
-        OPS.clip_weights(self.weight_matrix().data, float(sigma), kind)
+        # called after every optimizer step of every layer and never traced: no dispatcher hop
+        weights = self.weight_matrix().data
+        direct(weights).clip_weights(weights, float(sigma), kind)
 
     @no_grad()
     def quantize_weights(self) -> None:
@@ -237,10 +239,9 @@ class TiledAnalogLayer(AnalogLayerBase):
             self.weight_matrix().data.copy_(w_new)
         elif quant_type != WeightQuantizationType.NONE:
             self._require_device("quantize_weights")
-            OPS.quantize_weights(
-                self.weight_matrix().data, self.in_sizes, QUANT_IDS[quant_type],
-                float(self.rpu_config.modifier.res),
-            )
+            weights = self.weight_matrix().data
+            direct(weights).quantize_weights(weights, self.in_sizes, QUANT_IDS[quant_type],
+                                             float(self.rpu_config.modifier.res))
         super().quantize_weights()
 
     def _require_device(self, what: str) -> None:

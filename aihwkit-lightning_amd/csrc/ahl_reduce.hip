@@ -22,9 +22,11 @@ int record_hip_error(hipError_t e, const char* where) {
 // reproducible run to run.
 static constexpr int kStdRows = 16;  // rows per block of the whole-matrix clip kernels below
 
-// rows per wave: aim at >= 4096 waves, at most 16 rows each
+// rows per wave: aim at >= 1024 groups of rows (times the number of tiles: waves), at most 16 rows
+// each. Few fat waves with several rows' loads in flight finish a pass over a few tens of MB sooner
+// than many thin ones (k_running_absmax_rows).
 static int rows_per_wave(int64_t rows) {
-  const int64_t r = rows / 4096;
+  const int64_t r = rows / 1024;
   return (int)(r < 1 ? 1 : (r > 16 ? 16 : r));
 }
 
@@ -56,6 +58,62 @@ __global__ __launch_bounds__(256) void k_sliced_sums(const void* __restrict__ x,
     p[0] = s;
     p[1] = s2;
   }
+}
+
+// The same partial sums for 16-byte aligned rows whose tiles are NV x 64 vectors wide, with all of a
+// wave's RPW x NV loads issued before the first value is used (see k_running_absmax_rows). A lane
+// adds its values in the same order as k_sliced_sums does (row by row, ascending columns), so the
+// partial sums are the same to the bit.
+template <class D, int RPW, int NV>
+__global__ __launch_bounds__(256) void k_sliced_sums_rows(const void* __restrict__ x, int64_t rows,
+                                                          int64_t ld, Tiling tl,
+                                                          double* __restrict__ partial) {
+  constexpr int E = D::EPV;
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t grp = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
+  const int64_t r0 = grp * RPW;
+  if (r0 >= rows) return;
+  const typename D::elem* base = (const typename D::elem*)x + (int64_t)tl.base * t + lane * E;
+  u32x4 v[RPW][NV];
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) {
+    const int64_t r = r0 + i < rows ? r0 + i : rows - 1;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[i][j] = ld16(base + r * ld + j * 64 * E);
+  }
+  double s = 0.0, s2 = 0.0;
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) {
+    if (r0 + i >= rows) break;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      float e[E];
+      D::unpack(v[i][j], e);
+#pragma unroll
+      for (int q = 0; q < E; ++q) {
+        s += (double)e[q];
+        s2 += (double)e[q] * (double)e[q];
+      }
+    }
+  }
+  s = wave_sum(s);
+  s2 = wave_sum(s2);
+  if (lane == 0) {
+    double* p = partial + wave * 2;
+    p[0] = s;
+    p[1] = s2;
+  }
+}
+
+template <class D>
+static void launch_sums_rows(int nv, int rpw, dim3 grid, hipStream_t s, const void* x, int64_t rows, int64_t ld,
+                             const Tiling& tl, double* partial) {
+#define AHL_SUMS(R, V) hipLaunchKernelGGL((k_sliced_sums_rows<D, R, V>), grid, dim3(256), 0, s, x, rows, ld, tl, partial)
+  if (nv == 1) { if (rpw == 1) AHL_SUMS(1, 1); else if (rpw == 2) AHL_SUMS(2, 1); else AHL_SUMS(4, 1); }
+  else { if (rpw == 1) AHL_SUMS(1, 2); else if (rpw == 2) AHL_SUMS(2, 2); else AHL_SUMS(4, 2); }
+#undef AHL_SUMS
 }
 
 // out[t] = sqrt((S2 - S^2/n) / (n - 1)); one wave per tile, fixed summation order.
@@ -139,6 +197,45 @@ __global__ __launch_bounds__(256) void k_running_absmax(const void* __restrict__
   }
   m = wave_max(m);
   // most waves find the cached maximum already above theirs and skip the atomic
+  if (lane == 0 && __float_as_int(m) > __hip_atomic_load((int*)cache + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
+    atomicMax((int*)cache + t, __float_as_int(m));
+}
+
+// The same for 16-byte aligned rows whose tiles are NV x 64 vectors wide: a wave takes RPW rows of
+// one tile and issues all its RPW x NV 16-byte loads before it uses the first value (a wave that
+// walks its rows one after the other has one row's loads in flight, and a pass over a few tens of
+// MB is over before such waves have covered the latency). Rows beyond the matrix re-read the last
+// row: the maximum does not change. Measured at 2048 x 3072 fp32 (25 MB, launches replayed from a
+// graph): 7.2 us with one row per wave, 5.7 / 5.9 / 6.1 us with RPW = 2 / 4 / 8.
+template <class D, int RPW, int NV>
+__global__ __launch_bounds__(256) void k_running_absmax_rows(const void* __restrict__ x, int64_t rows,
+                                                             int64_t ld, Tiling tl, float* cache) {
+  constexpr int E = D::EPV;
+  const int lane = threadIdx.x & 63;
+  const int64_t wave = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t grp = wave / tl.n_tiles;
+  const int32_t t = (int32_t)(wave % tl.n_tiles);
+  const int64_t r0 = grp * RPW;
+  if (r0 >= rows) return;
+  const typename D::elem* base = (const typename D::elem*)x + (int64_t)tl.base * t + lane * E;
+  u32x4 v[RPW][NV];
+#pragma unroll
+  for (int i = 0; i < RPW; ++i) {
+    const int64_t r = r0 + i < rows ? r0 + i : rows - 1;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) v[i][j] = ld16(base + r * ld + j * 64 * E);
+  }
+  float m = 0.0f;
+#pragma unroll
+  for (int i = 0; i < RPW; ++i)
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      float e[E];
+      D::unpack(v[i][j], e);
+#pragma unroll
+      for (int q = 0; q < E; ++q) m = fmaxf(m, fabsf(e[q]));
+    }
+  m = wave_max(m);
   if (lane == 0 && __float_as_int(m) > __hip_atomic_load((int*)cache + t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))
     atomicMax((int*)cache + t, __float_as_int(m));
 }
@@ -473,8 +570,16 @@ int ahl_sliced_std(const void* x, int32_t dtype, int64_t rows, int64_t cols, int
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(x) && (ld % D::EPV == 0);
-    if (vec) hipLaunchKernelGGL((k_sliced_sums<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
-    else hipLaunchKernelGGL((k_sliced_sums<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
+    // equal tiles of 64 or 128 vectors: the kernel with all of a wave's loads in flight (same
+    // grouping of rows into waves, same sums)
+    const int nv = (vec && tl.extra == 0 && tl.base % (64 * D::EPV) == 0) ? tl.base / (64 * D::EPV) : 0;
+    if ((nv == 1 || nv == 2) && (rpw == 1 || rpw == 2 || rpw == 4)) {
+      launch_sums_rows<D>(nv, rpw, dim3((unsigned)nb), s, x, rows, ld, tl, (double*)ws_partials);
+    } else if (vec) {
+      hipLaunchKernelGGL((k_sliced_sums<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
+    } else {
+      hipLaunchKernelGGL((k_sliced_sums<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, (double*)ws_partials);
+    }
   });
   hipLaunchKernelGGL(k_std_finalize, dim3(n_tiles), dim3(256), 0, s, (const double*)ws_partials, nw, rows, tl, out,
                      (const uint32_t*)nullptr);
@@ -536,8 +641,17 @@ int ahl_running_absmax(const void* x, int32_t dtype, int64_t rows, int64_t cols,
   if (nb > 0x7fffffff) return AHL_ERR_ARG;
   AHL_DISPATCH_DTYPE(dtype, {
     const bool vec = aligned16(x) && (ld % D::EPV == 0);
-    if (vec) hipLaunchKernelGGL((k_running_absmax<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, cache);
-    else hipLaunchKernelGGL((k_running_absmax<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, cache);
+    // equal tiles of 64 or 128 vectors (256 / 512 fp32, 512 / 1024 16-bit columns), many rows
+    const int nv = (vec && tl.extra == 0 && tl.base % (64 * D::EPV) == 0) ? tl.base / (64 * D::EPV) : 0;
+    if ((nv == 1 || nv == 2) && rows >= 512) {
+      const int64_t nbr = cdiv(cdiv(rows, 2) * n_tiles, 4);
+      if (nv == 1) hipLaunchKernelGGL((k_running_absmax_rows<D, 2, 1>), dim3((unsigned)nbr), dim3(256), 0, s, x, rows, ld, tl, cache);
+      else hipLaunchKernelGGL((k_running_absmax_rows<D, 2, 2>), dim3((unsigned)nbr), dim3(256), 0, s, x, rows, ld, tl, cache);
+    } else if (vec) {
+      hipLaunchKernelGGL((k_running_absmax<D, true>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, cache);
+    } else {
+      hipLaunchKernelGGL((k_running_absmax<D, false>), dim3((unsigned)nb), dim3(256), 0, s, x, rows, ld, tl, rpw, cache);
+    }
   });
   return check_launch("ahl_running_absmax");
 }

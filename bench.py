@@ -237,8 +237,9 @@ def time_post_training(with_cpu):
     batches (the kernel the calibration hook calls; 16 distinct batches, 403 MB, visited in turn).
     One timed pass over fresh matrices, wall clock around it."""
     from aihwkit_lightning.nn import AnalogLinear
-    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+    from aihwkit_lightning.nn.modules.hip_utils import ops
 
+    OPS = ops.direct(torch.empty(0, device="cuda"))   # what the calibration hook calls  # noqa: N806
     n, k, m, n_mat, n_batch = 8192, 3072, 2048, 64, 256
     gen = torch.Generator(device="cuda").manual_seed(4)
 
@@ -427,7 +428,17 @@ def time_reference_speed_test():
         which[0] = "graph"
         replay = CapturedStep(step)
         replay()
-        out[str(size)] = {"us_eager": round(eager, 1), "us_graph_replay": round(timed(replay), 1)}
+        # the same eager step with torch's own Linear and optimizer: what the host side of any
+        # eager step costs on this box (autograd, AdamW's launches), with no analog work at all
+        plain = torch.nn.Linear(size, size).to(device="cuda", dtype=torch.float16)
+        plain_opt = torch.optim.AdamW(plain.parameters(), lr=0.0)
+
+        def plain_step():
+            plain(inp).sum().backward()
+            plain_opt.step()
+
+        out[str(size)] = {"us_eager": round(eager, 1), "us_graph_replay": round(timed(replay), 1),
+                          "us_eager_torch_linear": round(timed(plain_step), 1)}
     return out
 
 
