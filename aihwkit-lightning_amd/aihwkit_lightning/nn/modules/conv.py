@@ -9,12 +9,14 @@ HIP kernels behind the same C ABI as the operator; this module only strings them
 from functools import reduce
 from typing import List, Optional, Tuple, Union
 
+import torch
 from torch import Tensor
 from torch.autograd import Function
 from torch.nn import Conv1d, Conv2d, Conv3d
 from torch.nn.modules.conv import _ConvNd
 from torch.nn.modules.utils import _pair, _single, _triple
 
+from .hip_utils.hip_conv import HipConv, direct_conv_applies
 from .hip_utils.ops import OPS, conv_out_size
 from .linear import is_at_least_volta_gpu  # noqa: F401  (re-exported)
 from .tiled import TiledAnalogLayer
@@ -172,11 +174,24 @@ class _AnalogConvNd(TiledAnalogLayer, _ConvNd):
         n_spatial = len(self.kernel_size)
         geom = self.geometry(tuple(inp.shape))
         out_size = conv_out_size(geom)[3 - n_spatial:]
+        if direct_conv_applies(self, inp, geom, self.training and self._init_phase_active()):
+            # the three products read the (padded, channels-last) image itself: no patch matrix
+            out = self._conv_on_the_image(inp, geom).view(geom[0], self.out_channels, *out_size)
+            return out.squeeze(0) if unbatched else out
         rows = PatchRows.apply(inp, geom)  # [B, L, K]
         out = self.analog_mvm(rows)  # [B, L, N]
         out = SwapLastTwo.apply(out)  # [B, N, L]
         out = out.view(geom[0], self.out_channels, *out_size)
         return out.squeeze(0) if unbatched else out
+
+    @torch.compiler.disable
+    def _conv_on_the_image(self, inp: Tensor, geom: List[int]) -> Tensor:
+        weight, bias, input_range = self.weight_matrix(), self.bias, self.input_range
+        if not torch.is_grad_enabled():   # see TiledAnalogLayer.analog_mvm
+            inp, weight, bias, input_range = (None if t is None else t.detach()
+                                              for t in (inp, weight, bias, input_range))
+        return HipConv.apply(inp, weight, bias, input_range, self.in_sizes, self.rpu_config,
+                             self.training, geom)
 
     @classmethod
     def _from_digital(cls, module: _ConvNd, rpu_config: TorchInferenceRPUConfig, weight: Tensor):

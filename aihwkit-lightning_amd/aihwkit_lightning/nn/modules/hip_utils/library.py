@@ -14,7 +14,7 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 13
+ABI_VERSION = 14
 STATIC_DX_SCRATCH_BYTES = 16 * 1024 * 1024
 
 AHL_F32, AHL_BF16, AHL_F16 = 0, 1, 2
@@ -181,6 +181,25 @@ SIGNATURES = {
     "ahl_linear_bwd_dw_ws_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int32, c_int32, c_int32,
                                              c_int64]),
     "ahl_tile_stride": (c_int64, [c_int64, c_int32, c_int32]),
+    "ahl_conv_direct_rows": (c_int32, [POINTER(AhlConvGeom), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64)]),
+    "ahl_conv_direct_supported": (c_int32, [POINTER(AhlConvGeom), c_int32, c_int64, _I32P, c_int32]),
+    "ahl_conv_image_rows": (c_int32, [c_void_p, POINTER(AhlConvGeom), c_int32, c_void_p, _I32P, c_int32,
+                                      POINTER(AhlLinearCfg), c_void_p, c_void_p, c_void_p]),
+    "ahl_conv_weight_layout": (c_int32, [c_void_p, c_int64, c_int32, c_int64, POINTER(AhlConvGeom), _I32P,
+                                         c_int32, c_int32, c_int64, c_void_p, c_int64, c_void_p]),
+    "ahl_conv_fwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, POINTER(AhlConvGeom), c_int64, _I32P, c_int32,
+                               POINTER(AhlLinearCfg), c_void_p]),
+    "ahl_conv_output": (c_int32, [c_void_p, POINTER(AhlConvGeom), c_int32, c_int64, c_void_p, c_void_p]),
+    "ahl_conv_grad_rows": (c_int32, [c_void_p, POINTER(AhlConvGeom), c_int32, c_int64, c_void_p, c_void_p]),
+    "ahl_conv_bwd_dw_ws_bytes": (c_int64, [POINTER(AhlConvGeom), c_int64, _I32P, c_int32, POINTER(c_int64)]),
+    "ahl_conv_bwd_dw": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  POINTER(AhlConvGeom), c_int64, _I32P, c_int32, POINTER(AhlLinearCfg),
+                                  c_void_p, c_void_p]),
+    "ahl_conv_bwd_dx_ws_bytes": (c_int64, [POINTER(AhlConvGeom), c_int32]),
+    "ahl_conv_bwd_dx": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_void_p, POINTER(AhlConvGeom), c_int64, _I32P, c_int32,
+                                  POINTER(AhlLinearCfg), c_void_p, c_void_p]),
     "ahl_row_nonzero": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                   c_void_p]),
     "ahl_sliced_std_kept": (c_int32, [c_void_p, c_int32, c_int64, c_int64, c_int64, _I32P, c_int32,

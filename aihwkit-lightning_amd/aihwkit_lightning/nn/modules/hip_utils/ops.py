@@ -4,6 +4,7 @@ Each op allocates its outputs and scratch with torch (device memory plumbing onl
 device pointers, sizes and the current HIP stream to one C entry point, and returns. The ops are
 registered for the CUDA (= ROCm/HIP) dispatch key only: calling them on CPU tensors raises.
 """
+import os
 import sys
 import threading
 from ctypes import byref, c_void_p
@@ -856,6 +857,14 @@ for _name, _fn in [
     torch.library.register_fake(f"aihwkit_hip::{_name}", _shapes_only(_fn), lib=LIB)
 
 OPS = torch.ops.aihwkit_hip
+
+# what the autograd functions that call the library themselves (hip_conv.py) share with the ops here
+ptr, linear_cfg, current_stream = _ptr, _linear_cfg, _stream
+
+
+def os_environ_no_rounding() -> bool:
+    """The reference's test switch ``_AIHWKIT_NO_ROUNDING``."""
+    return bool(os.environ.get("_AIHWKIT_NO_ROUNDING", False))
 
 
 def direct(tensor: Tensor):

@@ -19,7 +19,7 @@ OBJ_DIR = os.path.join(CSRC, "build")
 LIB_DIR = os.path.join(HERE, "aihwkit_lightning", "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "libanalog_hip.so")
 SOURCES = ["ahl_reduce.hip", "ahl_weights.hip", "ahl_gemm.hip", "ahl_fast.hip", "ahl_fwd_pipe.hip", "ahl_fast_bwd.hip",
-           "ahl_conv.hip", "ahl_layout.hip", "ahl_calib.hip", "ahl_rnn.hip"]
+           "ahl_conv.hip", "ahl_conv_direct.hip", "ahl_layout.hip", "ahl_calib.hip", "ahl_rnn.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",

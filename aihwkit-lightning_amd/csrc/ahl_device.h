@@ -56,6 +56,39 @@ AHL_DEV void block_to_tile(int64_t bid, int64_t nb, int64_t nbm, int64_t nbn, in
 }
 
 // ---------------------------------------------------------------------------------------------
+// A convolution read straight off the image (stride 1, dilation 1), instead of off a patch matrix.
+// The image is kept zero-padded and channels-last as a flat [pixels, C] matrix; the outputs are
+// numbered on the same PADDED pixel grid (row p is the output whose receptive field has its
+// first corner at padded pixel p; rows whose field would leave the image are computed and
+// dropped). A kernel offset ("tap") is then ONE constant row offset for every output:
+//   tap = (id * kh + ih) * kw + iw   ->   rows (id * hp + ih) * wp + iw.
+// The contraction of a K-tile runs over (tap, channel) instead of the reference's (channel, tap)
+// -- the same terms, so the tile's sum is the same up to the order of the fp32 additions -- and a
+// 64-wide chunk of it is 64 consecutive channels of one tap: the same 128-byte row segment a
+// matrix operand has, at a row offset that depends on the chunk only.
+struct ConvMap {
+  int32_t on;          // 0: a plain matrix operand
+  int32_t sign;        // +1: output row m reads rows m + offset(tap); -1: rows m + lead - offset(tap)
+  int32_t lead;        // sign -1: rows of zeros in front of the operand (= the largest offset)
+  int32_t cg;          // 64-wide chunks per tap
+  int32_t tile_base;   // columns between the starts of two tiles inside an operand row
+  int32_t kh, kw;      // kernel extents of the two inner dimensions
+  int32_t hp, wp;      // padded image extents of the two inner dimensions
+  int64_t alloc_rows;  // rows the operand's allocation holds (all readable, zero beyond the data)
+};
+AHL_DEV int32_t conv_tap_rows(const ConvMap& c, int32_t tap) {
+  const int32_t iw = tap % c.kw, r = tap / c.kw;
+  const int32_t ih = r % c.kh, id = r / c.kh;
+  return (id * c.hp + ih) * c.wp + iw;
+}
+// element offset inside the operand of chunk i of tile t, relative to the output row's own row
+AHL_DEV int32_t conv_chunk_offset(const ConvMap& c, int32_t t, int32_t i, int32_t ld) {
+  const int32_t tap = i / c.cg;
+  const int32_t rows = c.sign > 0 ? conv_tap_rows(c, tap) : c.lead - conv_tap_rows(c, tap);
+  return rows * ld + t * c.tile_base + (i - tap * c.cg) * 64;
+}
+
+// ---------------------------------------------------------------------------------------------
 // Clamp-mask layout: one bit per (tile, row, column). Word [(t * ceil(N/32) + n / 32) * M + m]
 // has bit (n % 32) set where the tile-t output of element (m, n) left the ADC range (and so
 // passes no gradient). One 64-lane ballot over a 32x32 MFMA result register yields two such

@@ -132,7 +132,8 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
   // row panel is computed once, the k position advances as the scalar offset, and rows beyond
   // the matrix read as zero (out-of-range check of the descriptor) -- no per-chunk address
   // arithmetic and no predicates.
-  const int64_t rowsA = a.M - m0, rowsB = a.N - n0;
+  // (an image operand reads rows beyond its block's: the descriptor spans the allocation)
+  const int64_t rowsA = (a.conv.on ? a.conv.alloc_rows : a.M) - m0, rowsB = a.N - n0;
   const uint64_t bytesA = (uint64_t)rowsA * (uint64_t)a.ldx * 2u, bytesB = (uint64_t)rowsB * (uint64_t)a.ldw * 2u;
   const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc(
       (void*)((const uint16_t*)a.xq + m0 * a.ldx), 0,
@@ -146,21 +147,23 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
 #pragma unroll
   for (int j = 0; j < NB; ++j) voB[j] = (int)(((int64_t)(row0 + 32 * j) * a.ldw + cv * 8) * 2);
   u32x4 rawA[4], rawB[NB];
-  auto load = [&](int32_t kc) {
+  // chunk li of tile lt: the weights at column lt * tile_stride + 64 li, the input at the same
+  // column or, read off an image, at the chunk's (tap, channels) position
+  auto load = [&](int lt, int li) {
+    const int32_t kcB = lt * a.tile_stride + li * 64;
+    const int32_t kcA = a.conv.on ? conv_chunk_offset(a.conv, lt, li, (int32_t)a.ldx) : kcB;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      rawA[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsA, voA[j], kc * 2, 0));
+      rawA[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsA, voA[j], kcA * 2, 0));
 #pragma unroll
     for (int j = 0; j < NB; ++j)
-      rawB[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsB, voB[j], kc * 2, 0));
+      rawB[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsB, voB[j], kcB * 2, 0));
   };
-  const int32_t k_first = t_first * a.tile_stride;
-  load(k_first);
+  load(t_first, 0);
   const int cpt = a.tile / 64, nchunks = (one_tile ? 1 : a.n_tiles) * cpt;
-  // k offset of the chunk after the one being loaded: next 64 columns, or the next tile's start
-  int32_t knext = k_first + 64;
-  int lcin = 1;  // position inside its tile of the chunk at knext
-  if (lcin == cpt) { lcin = 0; knext = k_first + a.tile_stride; }
+  // tile and position inside it of the chunk after the one being loaded
+  int lt = t_first, lcin = 1;
+  if (lcin == cpt) { lcin = 0; ++lt; }
   int t = t_first, cin = 0;
   // registers -> LDS for the chunk held in rawA/rawB; `tt` is its K-tile, `first` whether it
   // opens that tile (then the dynamic-mode per-row constants of the tile are written too)
@@ -186,9 +189,8 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
     if (!prestaged) stage(t, cin == 0);
     prestaged = false;
     if (ch + 1 < nchunks) {
-      load(knext);
-      knext += 64;
-      if (++lcin == cpt) { lcin = 0; knext += a.tile_stride - a.tile; }
+      load(lt, lcin);
+      if (++lcin == cpt) { lcin = 0; ++lt; }
     }
 
     {
@@ -534,11 +536,14 @@ bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, co
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
                     void* y, int64_t ldy, uint32_t* keep, uint32_t* clamp_flag, const void* ir,
                     const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
-                    const Tiling& tl, const AhlLinearCfg* cfg, void* ws, hipStream_t s) {
+                    const Tiling& tl, const AhlLinearCfg* cfg, void* ws, hipStream_t s,
+                    const ConvMap* conv) {
   FastFwdArgs a;
   a.xq = xq; a.ldx = ldxq; a.w = w_eff; a.ldw = ldw; a.bias = bias; a.y = y; a.ldy = ldy;
   a.keep = keep; a.clamp_flag = clamp_flag; a.ir = ir; a.wmax = wmax; a.tile_max = tile_max;
   a.M = M; a.N = N; a.n_tiles = tl.n_tiles;
+  memset(&a.conv, 0, sizeof(a.conv));
+  if (conv != nullptr) a.conv = *conv;
   if (cfg->tile_stride > 0) {  // padded tile layout: only the chunks that hold data are visited
     a.tile = (int32_t)cdiv(widest_tile(tl), 64) * 64;
     a.tile_stride = cfg->tile_stride;
@@ -568,14 +573,14 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   // When those are too few to give every CU a block (few rows: a recurrent step, a small batch),
   // the 128 x 64 blocks double the count.
   const bool few = cdiv(M, 128) * cdiv(N, 128) < 200;
-  const bool split = ws != nullptr && aligned16(ws) && (!bias || aligned16(bias)) &&
+  const bool split = ws != nullptr && aligned16(ws) && (!bias || aligned16(bias)) && !a.conv.on &&
                      fast_fwd_split(M, N, tl.n_tiles);
   a.part = split ? (uint16_t*)ws : nullptr;
   const int qm = adc ? (cfg->skip_rounding ? 3 : 2) : (a.clamp_on ? 1 : 0);
   // Large grids go to the kernel that runs a tile's epilogue inside the next tile's product loop
   // (same results bit for bit); AHL_FORWARD_KERNEL=blocks in the environment keeps them here.
   const char* pick = getenv("AHL_FORWARD_KERNEL");
-  if (!(pick != nullptr && strcmp(pick, "blocks") == 0) && pipe_fwd_eligible(a, cfg->ir_mode) &&
+  if (!(pick != nullptr && strcmp(pick, "blocks") == 0) && !a.conv.on && pipe_fwd_eligible(a, cfg->ir_mode) &&
       launch_pipe_fwd(cfg->dtype, a, cfg->ir_mode, noise, qm, s))
     return check_launch("ahl_linear_fwd(pipe)");
   const dim3 sum_grid((unsigned)cdiv(M * (N / 8), 256));

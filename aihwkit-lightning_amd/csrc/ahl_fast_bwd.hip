@@ -58,6 +58,10 @@ struct BwdArgs {
                                        // into this many slices, one block each; > 1 when the
                                        // output tiles alone are too few to fill the chip
   float* split;                        // slices > 1: fp32 partial results [slices][rows][K]
+  ConvMap conv;                        // DW, conv.on: b is a padded channels-last image [pixels, C] and
+                                       // output column c of tile t (at t * tile + c, c < conv_cols) is
+                                       // (tap c / tile_base, channel t * tile_base + c % tile_base)
+  int32_t conv_cols;                   // columns of a tile that hold data (taps x channels per tile)
 };
 
 
@@ -300,6 +304,19 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   }
 #pragma unroll
   for (int j = 0; j < 4; ++j) pb[j] = a.b + (int64_t)(km_row + 16 * j) * a.ldb + c0 + km_cv * 8;  // + l0 * ldb
+  // weight gradient of a convolution read off the image: this thread's 8 columns are 8 channels of
+  // one tap, i.e. of the image rows `tap offset` further on; columns in the padding between two
+  // tiles contribute zeros
+  bool b_valid = true;
+  if (MODE == MODE_DW && a.conv.on) {
+    const int32_t in_tile = (int32_t)(c0 - (int64_t)t * a.tile) + km_cv * 8;
+    b_valid = in_tile < a.conv_cols;
+    const int32_t tap = b_valid ? in_tile / a.conv.tile_base : 0;
+    const int32_t ch = b_valid ? in_tile - tap * a.conv.tile_base : 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      pb[j] = a.b + (int64_t)(km_row + 16 * j + conv_tap_rows(a.conv, tap)) * a.ldb + t * a.conv.tile_base + ch;
+  }
   const int64_t a_step = MODE == MODE_DX ? 64 : 64 * a.ldg;
   const int64_t k_step = MODE == MODE_DX ? 2 * clamp_rows(a.M) : 64;   // 64 columns = 2 words; or 64 rows
   const int64_t b_step = 64 * a.ldb;
@@ -347,6 +364,10 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
         if (a_ok) rawA[j] = ld16(pa[j]);
         if (b_ok) rawB[j] = ld16(pb[j]);
       }
+    }
+    if (MODE == MODE_DW && !b_valid) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) rawB[j] = zero4;
     }
     if (masked) pk += k_step;
 #pragma unroll
@@ -650,6 +671,7 @@ int launch_fast_dx(int32_t dtype, const void* g, int64_t ldg, const uint32_t* ke
   a.dense_tile = dense_tile;
   a.dense_base = dense ? dense->base : 0;
   a.dense_extra = dense ? dense->extra : 0;
+  memset(&a.conv, 0, sizeof(a.conv)); a.conv_cols = 0;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = flag_token;
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
@@ -692,9 +714,11 @@ int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N) {
 int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
-                   hipStream_t s) {
+                   hipStream_t s, const ConvMap* conv, int32_t conv_cols) {
   BwdArgs a;
   const int slices = fast_dw_slices(M, K, N);
+  memset(&a.conv, 0, sizeof(a.conv)); a.conv_cols = 0;
+  if (conv != nullptr) { a.conv = *conv; a.conv_cols = conv_cols; }
   float* bias_partial = (float*)ws;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = flag_token;
   a.b = (const uint16_t*)xq; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;

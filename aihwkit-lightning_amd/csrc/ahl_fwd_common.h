@@ -35,6 +35,7 @@ struct FastFwdArgs {
   const uint64_t* seed_state;    // null, or device {key, call counter} that replaces seed / offset
   uint16_t* part;                // null, or [T, M, N]: every block takes ONE K-tile and leaves its
                                  // result there; k_tile_sum adds the tiles in order (few rows)
+  ConvMap conv;                  // conv.on: xq is a padded channels-last image (see ConvMap)
 };
 
 AHL_DEV void mma_bf16_zero(const u32x4& a, const u32x4& b, f32x16& c) {

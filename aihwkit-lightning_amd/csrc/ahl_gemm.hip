@@ -705,7 +705,8 @@ bool fast_fwd_eligible(const AhlLinearCfg* cfg, const void* xq, int64_t ldxq, co
 int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw, const void* bias,
                     void* y, int64_t ldy, uint32_t* keep, uint32_t* clamp_flag, const void* ir,
                     const void* wmax, const float* tile_max, int64_t M, int64_t K, int64_t N,
-                    const Tiling& tl, const AhlLinearCfg* cfg, void* ws, hipStream_t s);
+                    const Tiling& tl, const AhlLinearCfg* cfg, void* ws, hipStream_t s,
+                    const ConvMap* conv = nullptr);
 int64_t fast_fwd_ws_bytes(int64_t M, int64_t N, int32_t n_tiles);
 __global__ void k_set_u32(uint32_t* p, uint32_t v) { *p = v; }
 bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, int64_t N);
@@ -719,7 +720,7 @@ int64_t fast_dx_row_blocks(int64_t M, int64_t K, int64_t N, bool element_mode);
 int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
-                   hipStream_t s);
+                   hipStream_t s, const ConvMap* conv = nullptr, int32_t conv_cols = 0);
 int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N);
 int launch_pad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows, const Tiling& tl,
                      int64_t stride, void* dst, int64_t ld_dst, hipStream_t s);

@@ -461,6 +461,74 @@ int ahl_col2im(const void* dcols, int64_t ldc, const AhlConvGeom* geom, int32_t 
 int ahl_transpose_batched(const void* src, int64_t ld_src, int32_t dtype, int64_t batch,
                           int64_t rows, int64_t cols, void* dst, int64_t ld_dst, void* stream);
 
+/* ---- convolution read off the image, without the patch matrix --------------------------------
+ * For 16-bit dtypes, stride 1, dilation 1, a static (or no) input range, out_channels a multiple
+ * of 64 and K-tiles that hold whole channels in multiples of 64 (ahl_conv_direct_supported), the
+ * three products of _AnalogConvNd.forward / its autograd (nn/modules/conv.py:310-360) read a
+ * zero-padded, channels-last copy of the image instead of the [B * L, C * kvol] patch matrix that
+ * unfold writes: outputs are numbered on the PADDED pixel grid (P = B * prod(in + 2 pad) rows; a
+ * row whose receptive field would leave the padded image is computed and dropped), and a kernel
+ * offset is one constant row offset. A K-tile's contraction runs over (tap, channel) instead of
+ * (channel, tap): the same terms in another order. Results equal the patch path's up to the order
+ * of the fp32 additions inside a tile.
+ * Pixel-row buffers ("rows" below) are dtype [rows, width] matrices, rows from
+ * ahl_conv_direct_rows: `lead` rows of zeros, the P pixels, zeros to the end.
+ * ahl_conv_image_rows and ahl_conv_grad_rows write EVERY row of their buffers (the zeros of the
+ * lead, of the padding pixels and of the tail included): the caller need not clear them.      */
+int ahl_conv_direct_rows(const AhlConvGeom* geom, int64_t* pixels, int64_t* lead, int64_t* rows);
+int ahl_conv_direct_supported(const AhlConvGeom* geom, int32_t dtype, int64_t N, const int32_t* tile_ends_host,
+                              int32_t n_tiles);
+
+/* xq_rows[lead + p, c] = DAC(x[b, c, d, h, w]) at the padded pixel p of (b, d, h, w): clamp to the
+ * range of channel c's K-tile and quantise (cfg->ir_mode AHL_IR_STATIC; AHL_IR_NONE copies). x_rows,
+ * if not NULL, receives the unmodified values in the same layout (the input-range gradient needs
+ * them). Replaces unfold + the per-tile clamp/DAC of torch_utils/torch_linear.py:134-192.    */
+int ahl_conv_image_rows(const void* x, const AhlConvGeom* geom, int32_t dtype, const void* ir,
+                        const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg, void* xq_rows,
+                        void* x_rows, void* stream);
+
+/* Weight layouts for the three products, from / to the layer's [N, C * kvol] matrix
+ * (weight.view(out_channels, -1)): mode 0 reorders every tile's columns to (tap, channel) -- the
+ * forward's operand; mode 1 is its inverse from a matrix whose tiles start every `stride` columns
+ * (what ahl_conv_bwd_dw leaves) ; mode 2 writes [C, kvol * N] for the input gradient.          */
+int ahl_conv_weight_layout(const void* src, int64_t ld_src, int32_t dtype, int64_t N, const AhlConvGeom* geom,
+                           const int32_t* tile_ends_host, int32_t n_tiles, int32_t mode, int64_t stride, void* dst,
+                           int64_t ld_dst, void* stream);
+
+/* The analog forward on the padded pixel grid: y_rows [P, N] (no lead rows), clamp mask
+ * [T, ceil(N/32), rows64(P)] and flag as ahl_linear_fwd writes them; w_taps from
+ * ahl_conv_weight_layout mode 0; ir, wmax, tile_max, bias, cfg as for ahl_linear_fwd.
+ * Slot of TorchLinear.linear as called from nn/modules/conv.py:325-352.                       */
+int ahl_conv_fwd(const void* xq_rows, const void* w_taps, const void* bias, void* y_rows, uint32_t* clamp_mask,
+                 uint32_t* clamp_flag, const void* ir, const void* wmax, const float* tile_max,
+                 const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
+                 const AhlLinearCfg* cfg, void* stream);
+
+/* y[b, n, *out] = y_rows[row of that output, n] (replaces out.transpose(-1, -2).contiguous() and
+ * the view of nn/modules/conv.py:356-366), and its adjoint g_rows[lead + row, n] = g[b, n, *out].   */
+int ahl_conv_output(const void* y_rows, const AhlConvGeom* geom, int32_t dtype, int64_t N, void* y, void* stream);
+int ahl_conv_grad_rows(const void* g_out, const AhlConvGeom* geom, int32_t dtype, int64_t N, void* g_rows,
+                       void* stream);
+
+/* Weight gradient (and bias gradient if dbias != NULL) from the gradient rows and the quantised
+ * image rows; dw_tiled is [N, padded_cols] with tile t at column t * (padded_cols / n_tiles), its
+ * columns in (tap, channel) order (ahl_conv_weight_layout mode 1 turns it into the layer's order). */
+int64_t ahl_conv_bwd_dw_ws_bytes(const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
+                                 int64_t* padded_cols);
+int ahl_conv_bwd_dw(const void* g_rows, const uint32_t* clamp_mask, const uint32_t* clamp_flag, const void* xq_rows,
+                    void* dw_tiled, void* dbias, const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host,
+                    int32_t n_tiles, const AhlLinearCfg* cfg, void* ws, void* stream);
+
+/* Input gradient dx [B, C, *in] and, with a static range, ir_grad [T] (the autograd of unfold,
+ * the product and the range clamp: torch_utils/torch_linear.py:29-108): w_dx from
+ * ahl_conv_weight_layout mode 2; x_rows the unquantised image rows, x the input itself (both only
+ * with a static range); dimg_rows [P, C] is scratch the caller provides.                       */
+int64_t ahl_conv_bwd_dx_ws_bytes(const AhlConvGeom* geom, int32_t n_tiles);
+int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* clamp_mask, const uint32_t* clamp_flag, const void* w_dx,
+                    const void* x_rows, const void* x, const void* ir, void* dimg_rows, void* dx, void* ir_grad,
+                    const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
+                    const AhlLinearCfg* cfg, void* ws, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -22,7 +22,7 @@ pytestmark = pytest.mark.gpu
 
 CONV_GOLDEN = dict(np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
                                         "conv_cases.npz")))
-RTOL = {"f32": 1e-5, "bf16": 1e-2}
+RTOL = {"f32": 1e-5, "bf16": 1e-2, "f16": 1e-3}
 
 GEOMS = [
     # batch, C, size(3), kernel(3), stride(3), padding(3), dilation(3)
@@ -205,6 +205,79 @@ SHAPES = [
 def test_seeded_convolutions_match_oracle(c):
     inputs = make_conv_inputs(c)
     check(hip_conv_fwd_bwd(c, inputs), oracle_conv_fwd_bwd(c, inputs), c, c["name"])
+
+
+# Convolutions the layer runs WITHOUT the patch matrix (16-bit, stride 1, dilation 1, a learned
+# static range or none, K-tiles of whole channels in multiples of 64, out_channels a multiple of
+# 64): against the oracle (the reference's unfold + linear model) and against the patch path.
+_IMG = dict(inp_res=254, out_res=254, clip="channel", clip_sigma=2.5, ir_decay=0.01, ir_mode="static")
+DIRECT = [
+    # three tiles of 64 channels x 9 taps, ranges that clip some inputs, no output clamps
+    conv_case("direct_bf16_three_tiles", 2, 2, 192, (9, 11), (3, 3), (1, 1), (1, 1), N=64, dtype="bf16",
+              max_input_size=576, ir_values=[1.5, 3.0, 2.0], out_bound=12.0, seed=60, **_IMG),
+    # one tile of 128 channels (the 128-wide input-gradient blocks), 5 x 3 kernel, uneven padding,
+    # a bound that clamps, 300 output channels would not do: 128
+    conv_case("direct_bf16_clamped", 2, 3, 128, (8, 7), (5, 3), (1, 1), (2, 0), N=128, dtype="bf16",
+              max_input_size=-1, ir_values=[2.0], out_bound=3.0, w_scale=0.05, seed=61, **_IMG),
+    conv_case("direct_f16_two_tiles", 2, 2, 128, (10, 10), (3, 3), (1, 1), (1, 1), N=64, dtype="f16",
+              max_input_size=600, ir_values=[2.5, 1.5], out_bound=12.0, seed=62, **_IMG),
+    # no padding, 1 x 1 kernel: the image rows ARE the patch rows
+    conv_case("direct_bf16_pointwise", 2, 2, 64, (6, 5), (1, 1), (1, 1), (0, 0), N=64, dtype="bf16",
+              ir_values=[2.0], out_bound=12.0, seed=63, **_IMG),
+    # volumes and sequences
+    conv_case("direct_bf16_volume", 3, 2, 64, (4, 6, 5), (2, 3, 3), (1, 1, 1), (1, 1, 0), N=64, dtype="bf16",
+              ir_values=[2.0], out_bound=12.0, seed=64, **_IMG),
+    conv_case("direct_bf16_sequence", 1, 3, 128, (70,), (5,), (1,), (2,), N=64, dtype="bf16",
+              max_input_size=320, ir_values=[2.0, 1.0], out_bound=12.0, seed=65, **_IMG),
+    # no converters at all: the plain convolution in 16-bit arithmetic
+    conv_case("direct_bf16_plain", 2, 2, 64, (9, 9), (3, 3), (1, 1), (1, 1), N=64, dtype="bf16", seed=66),
+    # evaluation mode (no input-range gradient, nothing kept for a backward pass of the range)
+    conv_case("direct_bf16_eval", 2, 2, 64, (9, 9), (3, 3), (1, 1), (1, 1), N=64, dtype="bf16",
+              ir_values=[2.0], out_bound=12.0, seed=67, training=False, **_IMG),
+    # an unbatched image
+    conv_case("direct_bf16_unbatched", 2, 0, 64, (12, 9), (3, 3), (1, 1), (1, 1), N=64, dtype="bf16",
+              ir_values=[2.0], out_bound=12.0, seed=68, **_IMG),
+]
+
+
+@pytest.mark.parametrize("c", DIRECT, ids=[c["name"] for c in DIRECT])
+def test_convolutions_read_off_the_image(c, monkeypatch):
+    from aihwkit_lightning.nn.modules.hip_utils import hip_conv
+
+    inputs = make_conv_inputs(c)
+    calls = []
+    real = hip_conv.HipConv.forward
+    monkeypatch.setattr(hip_conv.HipConv, "forward",
+                        staticmethod(lambda *a: calls.append(1) or real(*a)))
+    res = hip_conv_fwd_bwd(c, inputs)
+    assert calls, "the layer did not call the image path"
+    check(res, oracle_conv_fwd_bwd(c, inputs), c, c["name"] + " vs oracle")
+    monkeypatch.setattr(hip_conv, "ENABLED", False)
+    del calls[:]
+    patches = hip_conv_fwd_bwd(c, inputs)
+    assert not calls
+    check(res, patches, c, c["name"] + " vs the patch path")
+
+
+def test_image_path_declines_what_it_does_not_cover():
+    from aihwkit_lightning.nn.modules.hip_utils import hip_conv
+
+    base = dict(N=64, dtype="bf16", ir_values=[2.0], out_bound=12.0, **_IMG)
+    declined = [
+        conv_case("strided", 2, 2, 64, (9, 9), (3, 3), (2, 1), (1, 1), **base),
+        conv_case("dilated", 2, 2, 64, (9, 9), (3, 3), (1, 1), (1, 1), (1, 2), **base),
+        conv_case("odd_channels", 2, 2, 48, (9, 9), (3, 3), (1, 1), (1, 1), **base),
+        conv_case("odd_outputs", 2, 2, 64, (9, 9), (3, 3), (1, 1), (1, 1), **{**base, "N": 40}),
+        conv_case("split_taps", 2, 2, 64, (9, 9), (3, 3), (1, 1), (1, 1),
+                  **{**base, "max_input_size": 300, "ir_values": [2.0, 2.0]}),
+        conv_case("dynamic", 2, 2, 64, (9, 9), (3, 3), (1, 1), (1, 1),
+                  **{**base, "ir_mode": "dynamic", "ir_values": None}),
+        conv_case("fp32", 2, 2, 64, (9, 9), (3, 3), (1, 1), (1, 1), **{**base, "dtype": "f32"}),
+    ]
+    for c in declined:
+        x, w, b, _ = make_conv_inputs(c)
+        layer = make_conv_layer(c, w, b)
+        assert not hip_conv.direct_conv_applies(layer, x.cuda(), layer.geometry(tuple(x.shape)), False), c["name"]
 
 
 def test_conv1d_state_dict_round_trip_with_torch():

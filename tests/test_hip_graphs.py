@@ -197,3 +197,72 @@ def test_recurrent_training_step_in_one_graph_equals_eager_step():
         outs.append(noisy().detach().float().clone())
         torch.cuda.synchronize()
     assert not torch.equal(outs[0], outs[1]) and not torch.equal(outs[1], outs[2])
+
+
+def test_convolution_step_on_the_image_in_one_graph_equals_eager_step():
+    """A convolution that runs without the patch matrix, forward + backward in one graph, with a
+    bound that clamps (the clamp flag under replay) and replays with a different input in between:
+    every replay equals the eager step on the same input bit for bit. With output noise on, every
+    replay draws new noise."""
+    from conv_cases import conv_case, make_conv_inputs
+    from test_hip_conv import make_conv_layer
+    from aihwkit_lightning.nn.graphs import CapturedStep
+    from aihwkit_lightning.nn.modules.hip_utils import hip_conv
+
+    c = conv_case("graph_conv", 2, 4, 128, (12, 10), (3, 3), (1, 1), (1, 1), N=128, dtype="bf16",
+                  max_input_size=576, ir_mode="static", ir_values=[2.0, 1.5], inp_res=254, out_res=254,
+                  out_bound=2.0, clip="channel", clip_sigma=2.5, ir_decay=0.01, w_scale=0.05, seed=90)
+    x, w, b, g = make_conv_inputs(c)
+    inputs = [x.cuda(), (0.05 * x).cuda()]   # the second one clamps nothing
+    eager_results = []
+    for xin in inputs:
+        eager = make_conv_layer(c, w, b)
+        xe = xin.clone().requires_grad_(True)
+        out = eager(xe)
+        out.backward(g.cuda())
+        eager_results.append((out.detach(), xe.grad, eager.weight.grad, eager.bias.grad, eager.input_range.grad))
+    layer = make_conv_layer(c, w, b)
+    xs, gs = inputs[0].clone().requires_grad_(True), g.cuda()
+    calls = []
+    real = hip_conv.HipConv.forward
+    hip_conv.HipConv.forward = staticmethod(lambda *a: calls.append(1) or real(*a))
+    try:
+        def step():
+            xs.grad = None
+            layer.zero_grad(set_to_none=True)
+            out = layer(xs)
+            out.backward(gs)
+            return out
+
+        replay = CapturedStep(step)
+    finally:
+        hip_conv.HipConv.forward = real
+    assert calls, "the recorded step did not take the image path"
+    for i, which in enumerate([0, 1, 0, 0, 1]):
+        with torch.no_grad():
+            xs.copy_(inputs[which])
+        out = replay()
+        torch.cuda.synchronize()
+        want = eager_results[which]
+        got = (out, xs.grad, layer.weight.grad, layer.bias.grad, layer.input_range.grad)
+        for name, a, e in zip(("out", "dx", "dw", "db", "dir"), got, want):
+            assert torch.equal(a, e), f"{name}, replay {i} (input {which})"
+        _ = (out.float().flatten(1) @ out.float().flatten(1).t()).sum().item()
+
+    noisy = dict(c, out_noise=0.3, name="graph_conv_noise")
+    layer = make_conv_layer(noisy, w, b)
+    xn = inputs[0].clone().requires_grad_(True)
+
+    def noisy_step():
+        xn.grad = None
+        layer.zero_grad(set_to_none=True)
+        out = layer(xn)
+        out.backward(gs)
+        return out
+
+    replay = CapturedStep(noisy_step)
+    outs = []
+    for _ in range(3):
+        outs.append(replay().detach().clone())
+        torch.cuda.synchronize()
+    assert not torch.equal(outs[0], outs[1]) and not torch.equal(outs[1], outs[2])
