@@ -752,30 +752,37 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
 // ir_grad[t] from the blocks' partial sums and the clipped-entry counts (reference
 // torch_utils/torch_linear.py:92-106; the roundings of k_ir_grad_finalize).
 template <class D>
-__global__ __launch_bounds__(64) void k_conv_ir_finalize(const float* __restrict__ partial, int64_t row_blocks,
-                                                         int32_t col_blocks, int32_t per_tile,
-                                                         const uint32_t* __restrict__ count,
-                                                         int64_t count_rows, int32_t count_cols,
-                                                         int32_t count_per_tile,
-                                                         double numel, const void* ir, void* ir_grad,
-                                                         float decay, float min_pct) {
-  const int t = blockIdx.x, lane = threadIdx.x;
+__global__ __launch_bounds__(256) void k_conv_ir_finalize(const float* __restrict__ partial, int64_t row_blocks,
+                                                          int32_t col_blocks, int32_t per_tile,
+                                                          const uint32_t* __restrict__ count,
+                                                          int64_t count_rows, int32_t count_cols,
+                                                          int32_t count_per_tile,
+                                                          double numel, const void* ir, void* ir_grad,
+                                                          float decay, float min_pct) {
+  __shared__ double part[4][2];
+  __shared__ unsigned long long part_count[4];
+  const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   double s_up = 0.0, s_lo = 0.0;
   // clipped patch entries of the tile: the gather blocks' counts [count_rows][count_cols], this
   // tile's columns
   unsigned long long clipped = 0;
-  for (int64_t i = lane; i < count_rows * count_per_tile; i += 64)
+  for (int64_t i = tid; i < count_rows * count_per_tile; i += 256)
     clipped += count[(i / count_per_tile) * count_cols + (int64_t)t * count_per_tile + i % count_per_tile];
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) clipped += __shfl_xor(clipped, o, 64);
   const int64_t total = row_blocks * per_tile;
-  for (int64_t i = lane; i < total; i += 64) {
+  for (int64_t i = tid; i < total; i += 256) {
     const int64_t rb = i / per_tile, cb = (int64_t)t * per_tile + i % per_tile;
     const float* p = partial + (rb * col_blocks + cb) * 2;
     s_up += (double)p[0]; s_lo += (double)p[1];
   }
   s_up = wave_sum(s_up); s_lo = wave_sum(s_lo);
-  if (lane == 0) {
+  if (lane == 0) { part[wave][0] = s_up; part[wave][1] = s_lo; part_count[wave] = clipped; }
+  __syncthreads();
+  if (tid == 0) {
+    s_up = (part[0][0] + part[1][0]) + (part[2][0] + part[3][0]);
+    s_lo = (part[0][1] + part[1][1]) + (part[2][1] + part[3][1]);
+    clipped = (part_count[0] + part_count[1]) + (part_count[2] + part_count[3]);
     const float irv = D::load(ir, t);
     float gr = D::rd(0.0f + D::rd((float)s_up));
     gr = D::rd(gr - D::rd((float)s_lo));
@@ -1023,11 +1030,11 @@ int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* keep, const uint32_t* cl
   if (is_static) {
     const double numel = (double)g.B * g.out[0] * g.out[1] * g.out[2] * (double)tl.base;
     if (cfg->dtype == AHL_F16)
-      hipLaunchKernelGGL((k_conv_ir_finalize<F16>), dim3(n_tiles), dim3(64), 0, s, (const float*)partial, row_blocks,
+      hipLaunchKernelGGL((k_conv_ir_finalize<F16>), dim3(n_tiles), dim3(256), 0, s, (const float*)partial, row_blocks,
                          partial_cols, partial_per_tile, (const uint32_t*)count, (int64_t)g.B * cdiv(S, 64), g.C / 64, ct / 64,
                          numel, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
     else
-      hipLaunchKernelGGL((k_conv_ir_finalize<BF16>), dim3(n_tiles), dim3(64), 0, s, (const float*)partial, row_blocks,
+      hipLaunchKernelGGL((k_conv_ir_finalize<BF16>), dim3(n_tiles), dim3(256), 0, s, (const float*)partial, row_blocks,
                          partial_cols, partial_per_tile, (const uint32_t*)count, (int64_t)g.B * cdiv(S, 64), g.C / 64, ct / 64,
                          numel, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
   }
