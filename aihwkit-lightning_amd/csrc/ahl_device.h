@@ -434,6 +434,10 @@ AHL_DEV int64_t cdiv_dev(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // 16-byte global load / store of one `vec`
 AHL_DEV u32x4 ld16(const void* p) { return *(const u32x4*)p; }
 AHL_DEV void st16(void* p, const u32x4& v) { *(u32x4*)p = v; }
+// The same for data that is touched once (streaming passes over a whole matrix): non-temporal, so
+// that the lines do not displace what other kernels keep in the caches.
+AHL_DEV u32x4 ld16_stream(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
+AHL_DEV void st16_stream(void* p, const u32x4& v) { __builtin_nontemporal_store(v, (u32x4*)p); }
 
 }  // namespace ahl
 

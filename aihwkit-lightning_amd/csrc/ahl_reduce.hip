@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void k_sliced_sums_rows(const void* __restrict
   for (int i = 0; i < RPW; ++i) {
     const int64_t r = r0 + i < rows ? r0 + i : rows - 1;
 #pragma unroll
-    for (int j = 0; j < NV; ++j) v[i][j] = ld16(base + r * ld + j * 64 * E);
+    for (int j = 0; j < NV; ++j) v[i][j] = ld16_stream(base + r * ld + j * 64 * E);
   }
   double s = 0.0, s2 = 0.0;
 #pragma unroll
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void k_running_absmax_rows(const void* __restr
   for (int i = 0; i < RPW; ++i) {
     const int64_t r = r0 + i < rows ? r0 + i : rows - 1;
 #pragma unroll
-    for (int j = 0; j < NV; ++j) v[i][j] = ld16(base + r * ld + j * 64 * E);
+    for (int j = 0; j < NV; ++j) v[i][j] = ld16_stream(base + r * ld + j * 64 * E);
   }
   float m = 0.0f;
 #pragma unroll
@@ -390,7 +390,7 @@ __global__ __launch_bounds__(256) void k_clip_rows_held(void* w, int64_t rows, i
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int32_t v = lane + 64 * i;
-    held[i] = ld16(row + (int64_t)(v < nv ? v : 0) * E);
+    held[i] = ld16_stream(row + (int64_t)(v < nv ? v : 0) * E);
   }
   double s = 0.0, s2 = 0.0;
 #pragma unroll

@@ -230,7 +230,7 @@ AHL_DEV void quantize_segment(const ModArgs& a, int64_t n, int32_t t, float mx, 
 #pragma unroll
     for (int e = 0; e < 8; ++e) v[e] = wquant_apply<D>(v[e], q, a.maxq);
 #pragma unroll
-    for (int qv = 0; qv < VPG; ++qv) st16(dst + (int64_t)g * 8 + qv * E, D::pack(v + qv * E));
+    for (int qv = 0; qv < VPG; ++qv) st16_stream(dst + (int64_t)g * 8 + qv * E, D::pack(v + qv * E));
   }
 }
 
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(256) void k_quantize_rows(ModArgs a, void* __restri
   for (int32_t g = g0 + lane; g < g1; g += 64, ++it) {
     float v[8];
 #pragma unroll
-    for (int q = 0; q < VPG; ++q) D::unpack(ld16(row + (int64_t)g * 8 + q * E), v + q * E);
+    for (int q = 0; q < VPG; ++q) D::unpack(ld16_stream(row + (int64_t)g * 8 + q * E), v + q * E);
 #pragma unroll
     for (int e = 0; e < 8; ++e) mx = fmaxf(mx, fabsf(v[e]));
     if (it < 2) {
