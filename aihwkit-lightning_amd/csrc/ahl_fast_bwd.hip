@@ -636,7 +636,7 @@ bool fast_bwd_eligible(int32_t dtype, const Tiling& tl, int64_t M, int64_t K, in
 int fast_dx_slices(int64_t M, int64_t K, int64_t N) {
   const int64_t tiles = cdiv(M, 256) * (K / 256);
   if (tiles >= 128) return 1;
-  int64_t s = cdiv(256, tiles);
+  int64_t s = 256 / tiles;   // one block per CU: tiles * s blocks must fit one round of 256
   const int64_t chunks = cdiv(N, 64), most = chunks / 4;
   if (s > most) s = most;
   if (s <= 1) return 1;
@@ -695,7 +695,7 @@ int launch_fast_dx(int32_t dtype, const void* g, int64_t ldg, const uint32_t* ke
 int fast_dw_slices(int64_t M, int64_t K, int64_t N) {
   const int64_t tiles = cdiv(N, 256) * (K / 256);
   if (tiles >= 128) return 1;
-  int64_t s = cdiv(256, tiles);
+  int64_t s = 256 / tiles;   // one block per CU: 257 blocks take as long as 512
   const int64_t chunks = cdiv(M, 64), most = chunks / 8;
   if (s > most) s = most;
   if (s <= 1) return 1;
