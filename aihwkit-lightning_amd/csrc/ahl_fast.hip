@@ -580,7 +580,7 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
   // Large grids go to the kernel that runs a tile's epilogue inside the next tile's product loop
   // (same results bit for bit); AHL_FORWARD_KERNEL=blocks in the environment keeps them here.
   const char* pick = getenv("AHL_FORWARD_KERNEL");
-  if (!(pick != nullptr && strcmp(pick, "blocks") == 0) && !a.conv.on && pipe_fwd_eligible(a, cfg->ir_mode) &&
+  if (!(pick != nullptr && strcmp(pick, "blocks") == 0) && pipe_fwd_eligible(a, cfg->ir_mode) &&
       launch_pipe_fwd(cfg->dtype, a, cfg->ir_mode, noise, qm, s))
     return check_launch("ahl_linear_fwd(pipe)");
   const dim3 sum_grid((unsigned)cdiv(M * (N / 8), 256));

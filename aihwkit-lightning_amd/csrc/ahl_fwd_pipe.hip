@@ -59,7 +59,10 @@ template <bool V> using flag = std::integral_constant<bool, V>;
 // reads per flop but was 25 % slower: a SIMD issues at most one instruction of ONE wave per 4-5
 // cycles whatever its kind, and vector throughput for the epilogue's instruction mix is up to
 // 1.9 x higher with two waves.
-template <class D, int IRMODE, bool NOISE, int QM, int CPT, int NBI>
+// EXTRA: K-tiles of more than CPT chunks (any multiple of 64 columns from 576 up; the K-tiles of a
+// convolution read off the image, whose A operand takes its chunk offsets from the ConvMap): the
+// first CPT chunks of a tile carry the epilogue of the tile before, the others are product only.
+template <class D, int IRMODE, bool NOISE, int QM, int CPT, int NBI, bool EXTRA = false>
 __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastFwdArgs a) {
   constexpr bool ADC = QM >= 2, CLAMP = QM >= 1, ROUND = QM != 3;
   constexpr bool bound_on = CLAMP;
@@ -97,7 +100,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
   uint32_t any_clamp = 0u;
 
   // operand loads through buffer descriptors (see k_fwd_fast)
-  const int64_t rowsA = a.M - m0, rowsB = a.N - n0;
+  const int64_t rowsA = (EXTRA && a.conv.on ? a.conv.alloc_rows : a.M) - m0, rowsB = a.N - n0;
   const uint64_t bytesA = (uint64_t)rowsA * (uint64_t)a.ldx * 2u, bytesB = (uint64_t)rowsB * (uint64_t)a.ldw * 2u;
   const __amdgpu_buffer_rsrc_t rsA = __builtin_amdgcn_make_buffer_rsrc(
       (void*)((const uint16_t*)a.xq + m0 * a.ldx), 0,
@@ -124,12 +127,19 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
     voB[j] = (int)(((int64_t)row * a.ldw + (((lane & 7) ^ ((row >> 1) & 7)) * 8)) * 2);
   }
   int st_load = 0;   // stage the next chunk is loaded into
+  const int cpt = EXTRA ? a.tile / 64 : CPT;   // chunks per K-tile
+  const int nchunks = a.n_tiles * cpt;
+  int32_t knext = 0;   // k offset of the next chunk to load
+  int lcin = 0;        // its position inside its tile
+  int lt = 0;          // its tile (EXTRA)
   auto load = [&](int32_t kc) __attribute__((always_inline)) {
     char* sa = lds + st_load * kPStage + wave * (8 * NLA * kPRow);
     char* sb = lds + st_load * kPStage + kPLdsA + wave * (8 * NLB * kPRow);
+    // an image operand: the chunk's (tap, channels) position instead of the weights' column
+    const int32_t kcA = (EXTRA && a.conv.on) ? conv_chunk_offset(a.conv, lt, lcin, (int32_t)a.ldx) : kc;
 #pragma unroll
     for (int j = 0; j < NLA; ++j)
-      load_to_lds16(rsA, sa + j * 8 * kPRow, voA[j], kc * 2);
+      load_to_lds16(rsA, sa + j * 8 * kPRow, voA[j], kcA * 2);
 #pragma unroll
     for (int j = 0; j < NLB; ++j)
       load_to_lds16(rsB, sb + j * 8 * kPRow, voB[j], kc * 2);
@@ -137,12 +147,9 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
   };
   constexpr int kLoads = NLA + NLB;   // vector memory operations of one chunk, per wave
 
-  const int nchunks = a.n_tiles * CPT;
-  int32_t knext = 0;   // k offset of the next chunk to load
-  int lcin = 0;        // its position inside its tile
   auto advance = [&]() __attribute__((always_inline)) {
     knext += 64;
-    if (++lcin == CPT) { lcin = 0; knext += a.tile_stride - a.tile; }
+    if (++lcin == cpt) { lcin = 0; ++lt; knext += a.tile_stride - a.tile; }
   };
   // dynamic range: the per-row constants of tile tt, one row per thread
   auto write_rowc = [&](int tt) __attribute__((always_inline)) {
@@ -199,6 +206,23 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
     rdB += wrap ? -(kPStages - 1) * kPStage : kPStage;
     asm volatile("" : "+v"(rdA), "+v"(rdB));
     ++ch;
+  };
+
+  // EXTRA: the chunks of a tile beyond the first CPT, product only
+  auto plain_chunks = [&]() __attribute__((always_inline)) {
+    if (!EXTRA) return;
+    for (int x = CPT; x < cpt; ++x) {
+      read_frags(0, 0);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        if (s < 3) read_frags(s + 1, (s + 1) & 1);
+#pragma unroll
+        for (int i = 0; i < NBI; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) Mma16<D>::run(fa[s & 1][i], fb[s & 1][j], acc[i][j]);
+      }
+      end_chunk();
+    }
   };
 
   // One K-tile phase: the product of tile t (MMA) and the epilogue of tile t - 1 (EPI).
@@ -262,6 +286,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
           }
         if (s == 3) end_chunk();
       }
+      plain_chunks();
       if (t + 1 < a.n_tiles) write_rowc(t + 1);
     } else {
       // The "did an output leave the range" branch of unit u is taken in the middle of unit
@@ -448,6 +473,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
         }
       }
       resolve(NU - 1);
+      if (MMA) plain_chunks();
     }
     if (EPI && CLAMP && a.keep != nullptr) {
       // the clamp-mask words of tile te: per 32-column block, 64 rows are 256 contiguous bytes
@@ -519,7 +545,11 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
 // Grids of at least one block per CU, tiles of 256 / 512 columns, no split over K-tiles.
 bool pipe_fwd_eligible(const FastFwdArgs& a, int ir_mode) {
   if (a.part != nullptr || ir_mode == AHL_IR_NONE) return false;
-  if (a.tile != 256 && a.tile != 512) return false;
+  // tiles of 256 or 512 columns, or any multiple of 64 from 576 up (the chunks beyond the eighth
+  // are product only); an image operand only in the latter form
+  const bool longer = a.tile > 512 && a.tile % 64 == 0;
+  if (a.tile != 256 && a.tile != 512 && !longer) return false;
+  if (a.conv.on && !longer) return false;
   // at least one block per CU, and no round of blocks that leaves more than a fifth of the CUs idle
   const int64_t nb = cdiv(a.M, 256) * cdiv(a.N, 128);
   if (nb < 256 || nb * 5 < cdiv(nb, 256) * 256 * 4) return false;
@@ -527,14 +557,14 @@ bool pipe_fwd_eligible(const FastFwdArgs& a, int ir_mode) {
   return a.ldx <= (1 << 21) && a.ldw <= (1 << 21);
 }
 
-template <class D, int IRMODE, bool NOISE, int QM, int CPT>
+template <class D, int IRMODE, bool NOISE, int QM, int CPT, bool EXTRA = false>
 static void launch_pipe_one(const FastFwdArgs& a, hipStream_t s) {
   constexpr int NBI = 2;
   const dim3 block(1024 / NBI), grid((unsigned)(cdiv(a.M, 256) * cdiv(a.N, 128)));
   // a refusal shows at the launch that follows (check_launch reads the last error)
-  (void)hipFuncSetAttribute((const void*)k_fwd_pipe<D, IRMODE, NOISE, QM, CPT, NBI>,
+  (void)hipFuncSetAttribute((const void*)k_fwd_pipe<D, IRMODE, NOISE, QM, CPT, NBI, EXTRA>,
                       hipFuncAttributeMaxDynamicSharedMemorySize, kPLdsBytes);
-  hipLaunchKernelGGL((k_fwd_pipe<D, IRMODE, NOISE, QM, CPT, NBI>), grid, block, kPLdsBytes, s, a);
+  hipLaunchKernelGGL((k_fwd_pipe<D, IRMODE, NOISE, QM, CPT, NBI, EXTRA>), grid, block, kPLdsBytes, s, a);
 }
 
 // Launches the kernel if this combination is built; false otherwise (the caller falls back).
@@ -555,6 +585,16 @@ bool launch_pipe_fwd(int32_t dtype, const FastFwdArgs& a, int ir_mode, bool nois
   AHL_PIPE(1, true, 0, 4)
   AHL_PIPE(1, false, 0, 4)
 #undef AHL_PIPE
+  // longer tiles: with the ADC (the configurations that are measured); others stay on k_fwd_fast
+#define AHL_PIPE_LONG(NZ)                                                              \
+  if (ir_mode == 1 && noise == NZ && qm == 2 && cpt > 8) {                             \
+    if (dtype == AHL_F16) launch_pipe_one<F16, 1, NZ, 2, 8, true>(a, s);               \
+    else launch_pipe_one<BF16, 1, NZ, 2, 8, true>(a, s);                               \
+    return true;                                                                       \
+  }
+  AHL_PIPE_LONG(true)
+  AHL_PIPE_LONG(false)
+#undef AHL_PIPE_LONG
   return false;
 }
 

@@ -110,6 +110,50 @@ def test_the_two_forward_kernels_agree_bit_for_bit(dtype, out_bound, monkeypatch
     assert bool(piped["out"].float().std() > 0)
 
 
+@pytest.mark.parametrize("dtype,tile,noise", [("bf16", 576, 0.04), ("f16", 640, 0.04), ("bf16", 1088, 0.0)])
+def test_the_two_forward_kernels_agree_on_longer_tiles(dtype, tile, noise, monkeypatch):
+    """K-tiles of more than 512 columns (any multiple of 64): the first eight chunks of a tile carry
+    the epilogue of the tile before, the others are product only. Same results as the kernel for
+    small grids, bit for bit, with noise, ADC and clamps."""
+    from hip_helpers import hip_fwd_bwd
+
+    c = case(f"long_tiles_{dtype}_{tile}", dtype=dtype, M=4096, K=2 * tile, N=2048, max_input_size=tile,
+             ir_mode="static", inp_res=254, out_res=254, out_bound=0.9, out_noise=noise, clip="channel",
+             clip_sigma=2.5, ir_decay=0.01, ir_init=3.0, w_scale=0.02, seed=47)
+    inputs = make_inputs(c)
+    monkeypatch.delenv("AHL_FORWARD_KERNEL", raising=False)
+    piped = hip_fwd_bwd(c, inputs=inputs)
+    monkeypatch.setenv("AHL_FORWARD_KERNEL", "blocks")
+    blocks = hip_fwd_bwd(c, inputs=inputs)
+    for key in ("out", "dx", "dw", "db", "dir"):
+        if piped.get(key) is not None:
+            assert torch.equal(piped[key], blocks[key]), key
+    assert bool(piped["out"].float().std() > 0)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_the_two_forward_kernels_agree_on_an_image(dtype, monkeypatch):
+    """A convolution read off the image with enough pixels for the large-grid forward kernel (its A
+    operand's chunk offsets come from the tap map): same outputs and gradients as with the kernel
+    for small grids, bit for bit, noise included."""
+    from conv_cases import conv_case, make_conv_inputs
+    from test_hip_conv import hip_conv_fwd_bwd
+
+    c = conv_case(f"image_two_kernels_{dtype}", 2, 64, 128, (28, 28), (3, 3), (1, 1), (1, 1), N=256, dtype=dtype,
+                  max_input_size=576, ir_mode="static", ir_values=[2.0, 1.5], inp_res=254, out_res=254,
+                  out_bound=1.5, out_noise=0.04, clip="channel", clip_sigma=2.5, ir_decay=0.01,
+                  w_scale=0.02, seed=48)
+    inputs = make_conv_inputs(c)
+    monkeypatch.delenv("AHL_FORWARD_KERNEL", raising=False)
+    piped = hip_conv_fwd_bwd(c, inputs)
+    monkeypatch.setenv("AHL_FORWARD_KERNEL", "blocks")
+    blocks = hip_conv_fwd_bwd(c, inputs)
+    for key in ("out", "dx", "dw", "db", "dir"):
+        if piped.get(key) is not None:
+            assert torch.equal(piped[key], blocks[key]), key
+    assert bool(piped["out"].float().std() > 0)
+
+
 def test_llama_mlp_block_matches_oracle():
     """Configuration 4 of the baseline: a LLaMA-style MLP block (hidden 3072, intermediate 8192,
     SiLU gating: down(silu(gate(x)) * up(x))), bf16, 4096 tokens, tiles of 512, 8-bit DAC/ADC,
