@@ -390,10 +390,14 @@ AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, u
 // row `row` for l < 32 and of row `row + 4` for l >= 32, rows counted within the wave's tile)
 // in `words`, where lane L keeps the mask word of row L. Must be called by the whole wave.
 AHL_DEV void clamp_record(bool clamped, int row, uint32_t& words) {
+  // the ballot is wave-uniform: its halves go into lanes `row` and `row + 4` directly
+  // (v_writelane_b32; a select per lane would cost two compares that write scalar registers)
   const uint64_t b = __builtin_amdgcn_ballot_w64(clamped);
-  const int lane = (int)(threadIdx.x & 63u);
-  words = lane == row ? (uint32_t)b : words;
-  words = lane == row + 4 ? (uint32_t)(b >> 32) : words;
+  const uint32_t lo = (uint32_t)b, hi = (uint32_t)(b >> 32);
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0"
+               : "+v"(words) : "s"(lo), "s"(row) : "m0");
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0"
+               : "+v"(words) : "s"(hi), "s"(row + 4) : "m0");
 }
 
 // Zeroes the elements of a vector of 8 bf16 whose bit in the low byte of `bits` is set.
