@@ -97,13 +97,15 @@ AHL_DEV int64_t row_of(const RowMap& m, int32_t b, int32_t s) {
 }
 // The inverse: pixel p of the padded grid -> index into a [B, nch, S] tensor's (b, s), or -1 when
 // p lies outside the box (padding, outputs that do not exist).
-AHL_DEV bool box_of(const RowMap& m, int64_t p, int32_t& b, int32_t& s) {
-  const int32_t w = (int32_t)(p % m.p2) - m.o2;
-  const int64_t q1 = p / m.p2;
-  const int32_t h = (int32_t)(q1 % m.p1) - m.o1;
-  const int64_t q0 = q1 / m.p1;
-  const int32_t d = (int32_t)(q0 % m.p0) - m.o0;
-  b = (int32_t)(q0 / m.p0);
+AHL_DEV bool box_of(const RowMap& m, int64_t p64, int32_t& b, int32_t& s) {
+  const uint32_t p = (uint32_t)p64;   // pixels are fewer than 2^30: 32-bit divisions
+  const uint32_t q1 = p / (uint32_t)m.p2;
+  const int32_t w = (int32_t)(p - q1 * (uint32_t)m.p2) - m.o2;
+  const uint32_t q0 = q1 / (uint32_t)m.p1;
+  const int32_t h = (int32_t)(q1 - q0 * (uint32_t)m.p1) - m.o1;
+  const uint32_t qb = q0 / (uint32_t)m.p0;
+  const int32_t d = (int32_t)(q0 - qb * (uint32_t)m.p0) - m.o0;
+  b = (int32_t)qb;
   s = (d * m.d1 + h) * m.d2 + w;
   return w >= 0 && w < m.d2 && h >= 0 && h < m.d1 && d >= 0 && d < m.d0;
 }
@@ -133,10 +135,17 @@ __global__ __launch_bounds__(256) void k_conv_scatter(const uint16_t* __restrict
   const bool inside = pix >= 0 && pix < P && box_of(map, pix, b, sp);
   Dac dac = {0.0f, 1.0f, 1.0f, 1.0f};
   if (IRMODE == AHL_IR_STATIC) dac = make_dac<D>(D::load(ir, c0 / ct), inp_res);
+  // every load is issued (lanes with nothing to read load the tensor's first element) and the
+  // values are selected afterwards: a load behind a branch would be waited for before the next
   const uint16_t* col = src + ((int64_t)b * nch + c0 + wave * 16) * S + sp;
   float v[16];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) v[i] = (inside && c0 + wave * 16 + i < nch) ? D::load(col, (int64_t)i * S) : 0.0f;
+  for (int i = 0; i < 16; ++i) {
+    const bool ok = inside && c0 + wave * 16 + i < nch;
+    v[i] = D::load(ok ? col + (int64_t)i * S : src, 0);
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) v[i] = (inside && c0 + wave * 16 + i < nch) ? v[i] : 0.0f;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int32_t cl = wave * 16 + i;
@@ -212,18 +221,26 @@ __global__ __launch_bounds__(256) void k_conv_gather(const uint16_t* __restrict_
   __syncthreads();
   const int32_t s = s0 + lane;
   uint32_t cnt = 0;   // at most 16 channels x kvol per lane
+  const bool live = s < S;
+  const int64_t at0 = ((int64_t)b * nch + c0 + wave * 16) * S + (live ? s : 0);
+  float xv[16];
+  float irv = 0.0f;
+  if (MASK) {
+    irv = D::load(ir, c0 / ct);   // the block's 64 channels lie in one K-tile
+#pragma unroll
+    for (int i = 0; i < 16; ++i)   // all loads issued, none behind a branch
+      xv[i] = D::load((live && c0 + wave * 16 + i < nch) ? x + at0 + (int64_t)i * S : x, 0);
+  }
+#pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int32_t cl = wave * 16 + i, c = c0 + cl;
-    if (s >= S || c >= nch) continue;
+    if (!live || c >= nch) continue;
     float v = D::load(tile, lane * (2 * kTileWords) + cl);
-    const int64_t at = ((int64_t)b * nch + c) * S + s;
     if (MASK) {
-      const float irv = D::load(ir, c / ct);
-      const float xv = D::load(x, at);
-      if (xv >= irv || xv <= -irv) cnt += (uint32_t)taps[lane];
-      if (fabsf(xv) > irv) v = 0.0f;
+      if (xv[i] >= irv || xv[i] <= -irv) cnt += (uint32_t)taps[lane];
+      if (fabsf(xv[i]) > irv) v = 0.0f;
     }
-    D::store(dst, at, v);
+    D::store(dst, at0 + (int64_t)i * S, v);
   }
   if (MASK) {
     // one count per block (its 64 channels lie in one tile: ct is a multiple of 64), summed per
