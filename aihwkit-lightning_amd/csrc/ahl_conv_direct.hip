@@ -536,7 +536,14 @@ template <class D>
 __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   __shared__ float red[8][2];
+  // four mask bits -> the two dwords that keep the elements whose bit is clear (entry n: element
+  // pairs (0, 1) and (2, 3) of the nibble); 16 entries of 8 bytes lie in 32 different banks
+  __shared__ uint2 keep_lut[16];
   const int tid = threadIdx.x, lane = tid & 63;
+  if (tid < 16) {
+    auto pair = [](uint32_t two) { return ((two & 1u) ? 0u : 0xffffu) | ((two & 2u) ? 0u : 0xffff0000u); };
+    keep_lut[tid] = make_uint2(pair((uint32_t)tid & 3u), pair((uint32_t)tid >> 2));
+  }
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int h = lane >> 5, r = lane & 31;
@@ -628,8 +635,9 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
   constexpr int kLoads = 4 + 2 + 2;   // vector memory operations of one chunk, per wave
   const int cg = a.N / 64, nchunks = a.kvol * cg;
   int st_load = 0, ltap = 0, lcin = 0;   // stage, tap and position in the tap of the next chunk to load
+  int tap_w = 0, tap_h = 0, tap_d = 0;   // the tap's kernel coordinates (no divisions per chunk)
   auto load = [&]() __attribute__((always_inline)) {
-    const int32_t shift = conv_tap_rows(a.conv, ltap);
+    const int32_t shift = (tap_d * a.conv.hp + tap_h) * a.conv.wp + tap_w;
     const int32_t kcA = (a.conv.lead - shift) * (int32_t)a.ldg + lcin * 64;
     const int32_t kcB = (ltap * cg + lcin) * 64;
     char* sa = lds + st_load * kDxStage + wave * (32 * kDxRow);
@@ -648,7 +656,10 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
       load_to_lds4(rsK, sk + j * 256, ok ? (int)(word * 4) : -1);
     }
     st_load = st_load == kDxStages - 1 ? 0 : st_load + 1;
-    if (++lcin == cg) { lcin = 0; ++ltap; }
+    if (++lcin == cg) {
+      lcin = 0; ++ltap;
+      if (++tap_w == a.conv.kw) { tap_w = 0; if (++tap_h == a.conv.kh) { tap_h = 0; ++tap_d; } }
+    }
   };
 
   load();
@@ -682,8 +693,13 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
       if (s < 3) read_frags(s + 1, (s + 1) & 1);
       if (masked) {   // values s * 16 + h * 8 ... + 7 of the chunk: byte (2 s + h) of the row's 8
         const int sh = 8 * ((2 * s + h) & 3);
-        fa[s & 1][0] = zero_where_set8(fa[s & 1][0], (s < 2 ? k00 : k01) >> sh);
-        fa[s & 1][1] = zero_where_set8(fa[s & 1][1], (s < 2 ? k10 : k11) >> sh);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const uint32_t byte = (i == 0 ? (s < 2 ? k00 : k01) : (s < 2 ? k10 : k11)) >> sh;
+          const uint2 lo2 = keep_lut[byte & 15u], hi2 = keep_lut[(byte >> 4) & 15u];
+          fa[s & 1][i].x &= lo2.x; fa[s & 1][i].y &= lo2.y;
+          fa[s & 1][i].z &= hi2.x; fa[s & 1][i].w &= hi2.y;
+        }
       }
 #pragma unroll
       for (int i = 0; i < 2; ++i)
