@@ -259,6 +259,46 @@ def test_convolutions_read_off_the_image(c, monkeypatch):
     check(res, patches, c, c["name"] + " vs the patch path")
 
 
+_SWEEP = [
+    # ndim, batch, C, size, kernel, padding, N, channels per tile (0: one tile), dtype
+    (2, 1, 64, (5, 40), (3, 5), (1, 2), 64, 0, "bf16"),          # one image, wide kernel
+    (2, 3, 128, (13, 6), (7, 3), (3, 1), 192, 64, "bf16"),       # 7-tall kernel, N = 3 x 64
+    (2, 2, 256, (6, 6), (1, 1), (1, 1), 128, 128, "f16"),        # 1 x 1 kernel WITH padding
+    (2, 2, 64, (4, 4), (4, 4), (0, 0), 64, 0, "bf16"),           # kernel == image: one output per image
+    (2, 5, 64, (17, 3), (3, 3), (0, 1), 64, 0, "f16"),           # padding in one dimension only
+    (3, 1, 64, (5, 5, 5), (3, 3, 3), (1, 1, 1), 64, 0, "bf16"),  # 27 taps
+    (3, 2, 128, (3, 8, 4), (1, 3, 2), (0, 1, 1), 64, 64, "bf16"),  # even kernel extent, two tiles
+    (1, 2, 64, (300,), (9,), (4,), 128, 0, "bf16"),              # long sequence, 9 taps
+    (1, 4, 192, (33,), (3,), (0,), 64, 64, "f16"),               # three tiles, no padding
+    (2, 0, 128, (9, 10), (3, 3), (2, 2), 64, 64, "bf16"),        # unbatched, padding wider than the kernel needs
+]
+
+
+@pytest.mark.parametrize("spec", _SWEEP, ids=[f"geom{i}" for i in range(len(_SWEEP))])
+def test_image_path_equals_patch_path_over_geometries(spec, monkeypatch):
+    """Index arithmetic of the image path (padded grid, tap offsets, lead rows, layouts) over kernel
+    shapes, paddings and tilings: outputs and every gradient against the patch path on the same
+    layer and inputs (the patch path is the one compared with the reference's goldens)."""
+    from aihwkit_lightning.nn.modules.hip_utils import hip_conv
+
+    ndim, batch, chan, size, kernel, padding, n_out, ct, dtype = spec
+    kvol = 1
+    for k in kernel:
+        kvol *= k
+    tiles = 1 if ct == 0 else chan // ct
+    c = conv_case("sweep", ndim, batch, chan, size, kernel, (1,) * ndim, padding, N=n_out, dtype=dtype,
+                  max_input_size=-1 if ct == 0 else ct * kvol, ir_values=[1.5 + 0.5 * t for t in range(tiles)],
+                  out_bound=2.0, w_scale=0.05, seed=70 + len(size) + chan, **_IMG)
+    inputs = make_conv_inputs(c)
+    calls = []
+    real = hip_conv.HipConv.forward
+    monkeypatch.setattr(hip_conv.HipConv, "forward", staticmethod(lambda *a: calls.append(1) or real(*a)))
+    res = hip_conv_fwd_bwd(c, inputs)
+    assert calls, "the layer did not call the image path"
+    monkeypatch.setattr(hip_conv, "ENABLED", False)
+    check(res, hip_conv_fwd_bwd(c, inputs), c, f"{spec} vs the patch path")
+
+
 def test_image_path_declines_what_it_does_not_cover():
     from aihwkit_lightning.nn.modules.hip_utils import hip_conv
 
