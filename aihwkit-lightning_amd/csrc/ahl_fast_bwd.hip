@@ -385,6 +385,9 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   float bsum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int kb_idx = (int)bcol;
   auto stage = [&](char* sa, char* sb, bool masked, bool bias) {
+    // clamps are rare in most layers: a chunk whose mask words are all zero for the wave skips the
+    // table reads and the ANDs
+    if (masked) masked = __any((rawK[0] | rawK[1] | rawK[2] | rawK[3]) != 0u);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       if (bias) {
