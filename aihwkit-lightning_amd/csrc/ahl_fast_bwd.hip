@@ -62,6 +62,10 @@ struct BwdArgs {
                                        // output column c of tile t (at t * tile + c, c < conv_cols) is
                                        // (tap c / tile_base, channel t * tile_base + c % tile_base)
   int32_t conv_cols;                   // columns of a tile that hold data (taps x channels per tile)
+  int64_t col_base;                    // DW on a column range of the weights: the range's first column
+                                       // (the K-tile of a block is (col_base + its first column) / tile)
+  int64_t mask_N;                      // output channels the clamp-mask planes were laid out for (N, also
+                                       // when this launch covers a range of them)
 };
 
 
@@ -252,11 +256,11 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   block_to_tile(blockIdx.x % nb, nb, nb / nkb, nkb, 4, brow, bcol);
   const int64_t r0 = brow * 256;                     // DX: m0; DW: n0
   const int64_t c0 = bcol * 256;                     // k0
-  const int t = (int)(c0 / a.tile);
+  const int t = (int)((c0 + (MODE == MODE_DW ? a.col_base : 0)) / a.tile);
   const int64_t R = MODE == MODE_DX ? a.M : a.N;      // output rows
   const int64_t L = MODE == MODE_DX ? a.N : a.M;      // contraction length
   const bool use_keep = a.keep != nullptr && clamp_flag_says_clamped(a.clamp_flag, a.flag_token);
-  const uint32_t* plane = use_keep ? a.keep + (int64_t)t * clamp_plane_words(a.M, a.N) : nullptr;
+  const uint32_t* plane = use_keep ? a.keep + (int64_t)t * clamp_plane_words(a.M, a.mask_N) : nullptr;
 
   f32x16 acc[4][2];
 #pragma unroll
@@ -674,7 +678,7 @@ int launch_fast_dx(int32_t dtype, const void* g, int64_t ldg, const uint32_t* ke
   a.dense_tile = dense_tile;
   a.dense_base = dense ? dense->base : 0;
   a.dense_extra = dense ? dense->extra : 0;
-  memset(&a.conv, 0, sizeof(a.conv)); a.conv_cols = 0;
+  memset(&a.conv, 0, sizeof(a.conv)); a.conv_cols = 0; a.col_base = 0; a.mask_N = N;
   a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = flag_token;
   a.b = (const uint16_t*)w_eff; a.ldb = ldw; a.x = (const uint16_t*)x; a.ldx = ldx;
   a.ir = (const uint16_t*)ir; a.out = (uint16_t*)dx; a.ldo = lddx; a.partial = partial; a.bias_partial = nullptr;
@@ -695,9 +699,16 @@ int launch_fast_dx(int32_t dtype, const void* g, int64_t ldg, const uint32_t* ke
 // Slices of the contraction for the weight gradient: N x K / 65536 output tiles are too few to
 // fill 256 CUs when the layer is narrow (a convolution with many patches and few channels), so
 // the rows m are cut until there are about 256 blocks, each with at least 8 chunks of 64 rows.
-int fast_dw_slices(int64_t M, int64_t K, int64_t N) {
-  const int64_t tiles = cdiv(N, 256) * (K / 256);
-  if (tiles >= 128) return 1;
+//
+// A weight gradient whose 256 x 256 output tiles fill whole rounds of the 256 CUs plus a rest of at
+// most half a round is cut in two launches: the tiles of the full rounds, and the rest with its
+// contraction sliced so that it fills one round of shorter blocks (1.5 rounds paid as 2 become
+// 1 + 0.5). The cut runs along the columns (a range of weight columns: xq and dw shifted, K-tiles
+// counted from col_base) or along the rows (a range of output channels: g, dw, the bias gradient
+// and the mask words shifted), whichever leaves whole rounds in front.
+struct DwPart { int64_t n0, n, k0, k; int slices; };
+
+static int dw_slices_for(int64_t tiles, int64_t M) {
   int64_t s = 256 / tiles;   // one block per CU: 257 blocks take as long as 512
   const int64_t chunks = cdiv(M, 64), most = chunks / 8;
   if (s > most) s = most;
@@ -706,51 +717,101 @@ int fast_dw_slices(int64_t M, int64_t K, int64_t N) {
   return (int)cdiv(chunks, cdiv(chunks, s));
 }
 
-// Workspace of launch_fast_dw: [partial bias sums: slices x K/256 x N floats | slices > 1:
-// partial results slices x N x K floats]
+int fast_dw_slices(int64_t M, int64_t K, int64_t N) {
+  const int64_t tiles = cdiv(N, 256) * (K / 256);
+  return tiles >= 128 ? 1 : dw_slices_for(tiles, M);
+}
+
+static int dw_parts(int64_t M, int64_t K, int64_t N, bool whole_only, DwPart parts[2]) {
+  const int64_t nrows = cdiv(N, 256), nkb = K / 256, tiles = nrows * nkb;
+  parts[0] = {0, N, 0, K, fast_dw_slices(M, K, N)};
+  if (whole_only || tiles <= 256 || tiles % 256 == 0) return 1;
+  for (int64_t kb1 = nkb - 1; kb1 >= 1; --kb1) {
+    const int64_t rest = nrows * (nkb - kb1);
+    if ((nrows * kb1) % 256 != 0 || rest > 128) continue;
+    const int sl = dw_slices_for(rest, M);
+    if (sl < 2) break;
+    parts[0] = {0, N, 0, kb1 * 256, 1};
+    parts[1] = {0, N, kb1 * 256, K - kb1 * 256, sl};
+    return 2;
+  }
+  if (N % 256 != 0) return 1;
+  for (int64_t r1 = nrows - 1; r1 >= 1; --r1) {
+    const int64_t rest = (nrows - r1) * nkb;
+    if ((r1 * nkb) % 256 != 0 || rest > 128) continue;
+    const int sl = dw_slices_for(rest, M);
+    if (sl < 2) break;
+    parts[0] = {0, r1 * 256, 0, K, 1};
+    parts[1] = {r1 * 256, N - r1 * 256, 0, K, sl};
+    return 2;
+  }
+  return 1;
+}
+
+static int64_t dw_part_bias_bytes(const DwPart& p) { return ((int64_t)p.slices * (p.k / 256) * p.n * 4 + 255) / 256 * 256; }
+static int64_t dw_part_bytes(const DwPart& p) {
+  return dw_part_bias_bytes(p) + (p.slices > 1 ? ((int64_t)p.slices * p.n * p.k * 4 + 255) / 256 * 256 : 0);
+}
+
+// Workspace of launch_fast_dw, per launch: [partial bias sums: slices x k/256 x n floats |
+// slices > 1: partial results slices x n x k floats]
 int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N) {
-  const int64_t slices = fast_dw_slices(M, K, N);
-  const int64_t bias = (slices * (K / 256) * N * 4 + 255) / 256 * 256;
-  return bias + (slices > 1 ? slices * N * K * 4 : 0);
+  DwPart parts[2];
+  const int np = dw_parts(M, K, N, false, parts);
+  int64_t bytes = 0;
+  for (int i = 0; i < np; ++i) bytes += dw_part_bytes(parts[i]);
+  return bytes;
 }
 
 int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
                    hipStream_t s, const ConvMap* conv, int32_t conv_cols) {
-  BwdArgs a;
-  const int slices = fast_dw_slices(M, K, N);
-  memset(&a.conv, 0, sizeof(a.conv)); a.conv_cols = 0;
-  if (conv != nullptr) { a.conv = *conv; a.conv_cols = conv_cols; }
-  float* bias_partial = (float*)ws;
-  a.g = (const uint16_t*)g; a.ldg = ldg; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = flag_token;
-  a.b = (const uint16_t*)xq; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;
-  a.out = (uint16_t*)dw; a.ldo = lddw; a.partial = nullptr;
-  a.bias_partial = dbias ? bias_partial : nullptr;
-  a.M = M; a.N = N; a.K = K; a.tile = tl.base; a.ir_static = 0; a.dense_tile = 0;
-  a.dense_base = 0; a.dense_extra = 0;
-  a.slices = slices;
-  a.split = slices > 1
-      ? (float*)((char*)ws + ((int64_t)slices * (K / 256) * N * 4 + 255) / 256 * 256) : nullptr;
-  const int64_t nb = cdiv(N, 256) * (K / 256) * slices;
-  if (nb > 0x7fffffff) return AHL_ERR_ARG;
-  launch_bwd<MODE_DW>(dtype, M % 64 != 0, dim3((unsigned)nb), s, a);
-  const dim3 reduce_grid((unsigned)cdiv(N * K, 1024)), bias_grid((unsigned)cdiv(N, 16));
-  const int bias_rows = (int)(K / 256) * slices;
-  if (dtype == AHL_F16) {
-    if (slices > 1)
-      hipLaunchKernelGGL(k_split_reduce<F16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, slices, N, K,
-                         (uint16_t*)dw, lddw);
-    if (dbias)
-      hipLaunchKernelGGL(k_bias_final<F16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, N,
-                         (uint16_t*)dbias);
-  } else {
-    if (slices > 1)
-      hipLaunchKernelGGL(k_split_reduce<BF16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, slices, N, K,
-                         (uint16_t*)dw, lddw);
-    if (dbias)
-      hipLaunchKernelGGL(k_bias_final<BF16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, N,
-                         (uint16_t*)dbias);
+  DwPart parts[2];
+  // an image operand maps its columns itself: one launch
+  const int np = dw_parts(M, K, N, conv != nullptr, parts);
+  char* wsp = (char*)ws;
+  for (int i = 0; i < np; ++i) {
+    const DwPart& p = parts[i];
+    // the bias gradient comes from the launch(es) that cover column 0 of the weights
+    void* dbias_p = (dbias && p.k0 == 0) ? (char*)dbias + p.n0 * 2 : nullptr;
+    BwdArgs a;
+    memset(&a.conv, 0, sizeof(a.conv)); a.conv_cols = 0;
+    if (conv != nullptr) { a.conv = *conv; a.conv_cols = conv_cols; }
+    float* bias_partial = (float*)wsp;
+    a.g = (const uint16_t*)g + p.n0; a.ldg = ldg;
+    // mask words of channel n lie at word column n / 32 of a plane laid out for all N channels
+    a.keep = keep ? keep + (p.n0 >> 5) * ((M + 63) & ~(int64_t)63) : nullptr;
+    a.clamp_flag = clamp_flag; a.flag_token = flag_token;
+    a.b = (const uint16_t*)xq + p.k0; a.ldb = ldxq; a.x = nullptr; a.ldx = 0; a.ir = nullptr;
+    a.out = (uint16_t*)dw + p.n0 * lddw + p.k0; a.ldo = lddw; a.partial = nullptr;
+    a.bias_partial = dbias_p ? bias_partial : nullptr;
+    a.M = M; a.N = p.n; a.K = p.k; a.tile = tl.base; a.ir_static = 0; a.dense_tile = 0;
+    a.dense_base = 0; a.dense_extra = 0;
+    a.col_base = p.k0; a.mask_N = N;
+    a.slices = p.slices;
+    a.split = p.slices > 1 ? (float*)(wsp + dw_part_bias_bytes(p)) : nullptr;
+    const int64_t nb = cdiv(p.n, 256) * (p.k / 256) * p.slices;
+    if (nb > 0x7fffffff) return AHL_ERR_ARG;
+    launch_bwd<MODE_DW>(dtype, M % 64 != 0, dim3((unsigned)nb), s, a);
+    const dim3 reduce_grid((unsigned)cdiv(p.n * p.k, 1024)), bias_grid((unsigned)cdiv(p.n, 16));
+    const int bias_rows = (int)(p.k / 256) * p.slices;
+    if (dtype == AHL_F16) {
+      if (p.slices > 1)
+        hipLaunchKernelGGL(k_split_reduce<F16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, p.slices, p.n, p.k,
+                           a.out, lddw);
+      if (dbias_p)
+        hipLaunchKernelGGL(k_bias_final<F16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, p.n,
+                           (uint16_t*)dbias_p);
+    } else {
+      if (p.slices > 1)
+        hipLaunchKernelGGL(k_split_reduce<BF16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, p.slices, p.n, p.k,
+                           a.out, lddw);
+      if (dbias_p)
+        hipLaunchKernelGGL(k_bias_final<BF16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, p.n,
+                           (uint16_t*)dbias_p);
+    }
+    wsp += dw_part_bytes(p);
   }
   return check_launch("ahl_linear_bwd_dw(fast)");
 }

@@ -154,6 +154,50 @@ def test_the_two_forward_kernels_agree_on_an_image(dtype, monkeypatch):
     assert bool(piped["out"].float().std() > 0)
 
 
+@pytest.mark.parametrize("n_out,k_in", [(8192, 3072), (3072, 8192), (2048, 4096)],
+                         ids=["cut_along_columns", "cut_along_rows", "one_launch"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_weight_gradient_whose_tiles_do_not_fill_whole_rounds(n_out, k_in, dtype):
+    """384 output tiles of 256 x 256 are 1.5 rounds of the 256 CUs: the weight gradient then runs as
+    two launches (the tiles of the full round; the rest with its contraction sliced). Through the
+    operators, with a bound that clamps 5 % of the outputs: dW against (g without the clamped
+    outputs of the column's K-tile)^T xq computed with torch from the kernel's own clamp mask, the
+    bias gradient against the column sums of g."""
+    from aihwkit_lightning.nn.modules.hip_utils.ops import OPS
+    from aihwkit_lightning.nn.modules.hip_utils import library as L
+
+    m_rows, tile = 1024, 512
+    gen = torch.Generator().manual_seed(52)
+    x = torch.randn(m_rows, k_in, generator=gen).to(dtype).cuda()
+    g = torch.randn(m_rows, n_out, generator=gen).to(dtype).cuda()
+    w = (0.02 * torch.randn(n_out, k_in, generator=gen)).to(dtype).cuda()
+    bias = torch.zeros(n_out, dtype=dtype, device="cuda")
+    in_sizes = [tile] * (k_in // tile)
+    ir = torch.full((len(in_sizes),), 3.0, dtype=dtype, device="cuda")
+    wmax, tile_max, _, _ = OPS.weight_prep(w, in_sizes, L.AHL_QUANT_NONE, L.AHL_NOISE_NONE, 1.0, 0.0, 0, 1, False)
+    icfg = [L.AHL_IR_STATIC, 0, 1, 1, 0, 0, 0]
+    fcfg = [254.0, 254.0, 3.6, 0.0, 0.01, 0.95]
+    xq, _ = OPS.dac(x, ir, in_sizes, icfg, fcfg)
+    _, keep, flag = OPS.linear_fwd(None, xq, w, bias, ir, wmax, tile_max, in_sizes, icfg, fcfg, True)
+    dw, db = OPS.linear_bwd_dw(g, keep, flag, None, xq, ir, in_sizes, icfg, fcfg, True)
+    torch.cuda.synchronize()
+    # keep: [T, ceil(N / 32), rows64(M)] words, bit n % 32 of word (n / 32, m) set where clamped
+    words = keep.view(torch.int32)[:, :, :m_rows].to(torch.int64) & 0xFFFFFFFF
+    shifts = torch.arange(32, device="cuda", dtype=torch.int64).view(1, 1, 32, 1)
+    clamped = ((words.unsqueeze(2) >> shifts) & 1).reshape(len(in_sizes), -1, m_rows)[:, :n_out]   # [T, N, M]
+    frac = float(clamped.float().mean())
+    assert 0.01 < frac < 0.2, frac
+    want = torch.empty(n_out, k_in, dtype=torch.float32, device="cuda")
+    for t in range(len(in_sizes)):
+        gm = g.float() * (1.0 - clamped[t].t().float())
+        want[:, t * tile:(t + 1) * tile] = gm.t() @ xq[:, t * tile:(t + 1) * tile].float()
+    scale = float(want.abs().max())
+    tol = 4e-3 if dtype == torch.bfloat16 else 1e-3    # one rounding of the fp32 sum to the dtype
+    assert float((dw.float() - want).abs().max()) <= tol * scale
+    want_db = g.float().sum(0)
+    assert float((db.float() - want_db).abs().max()) <= tol * float(want_db.abs().max())
+
+
 def test_llama_mlp_block_matches_oracle():
     """Configuration 4 of the baseline: a LLaMA-style MLP block (hidden 3072, intermediate 8192,
     SiLU gating: down(silu(gate(x)) * up(x))), bf16, 4096 tokens, tiles of 512, 8-bit DAC/ADC,
