@@ -151,12 +151,17 @@ class HipConv(Function):
         if ir_mode == L.AHL_IR_STATIC:
             ir_dev = input_range.detach().contiguous()
         # the image as zero-padded channels-last pixel rows, quantised per K-tile on the way (the
-        # entry point writes every row of the buffers, the zeros included)
+        # entry point writes every row of the buffers, the zeros included); with a static range
+        # and a backward pass to come also what that pass needs to know about x: the range flags
+        # of every element and the clipped-entry counts
         xq_rows = torch.empty((rows, channels), dtype=dtype, device=dev)
-        keep_raw = ir_mode == L.AHL_IR_STATIC and need_dx
-        x_rows = torch.empty((rows, channels), dtype=dtype, device=dev) if keep_raw else None
+        keep_flags = ir_mode == L.AHL_IR_STATIC and need_dx
+        flag_rows = counts = None
+        if keep_flags:
+            flag_rows = torch.empty((rows, channels), dtype=torch.uint8, device=dev)
+            counts = torch.empty((lib.ahl_conv_count_words(byref(cgeom)),), dtype=torch.int32, device=dev)
         _check(lib.ahl_conv_image_rows(ops.ptr(inp), byref(cgeom), dt, ops.ptr(ir_dev), ends, n_tiles,
-                                       byref(cfg), ops.ptr(xq_rows), ops.ptr(x_rows), stream),
+                                       byref(cfg), ops.ptr(xq_rows), ops.ptr(flag_rows), ops.ptr(counts), stream),
                "ahl_conv_image_rows")
         w_taps = torch.empty_like(w_eff)
         _check(lib.ahl_conv_weight_layout(ops.ptr(w_eff), k_in, dt, n_out, byref(cgeom), ends, n_tiles, 0, 0,
@@ -181,14 +186,14 @@ class HipConv(Function):
         ctx.need_dx, ctx.need_dw, ctx.ir_needs_grad = need_dx, need_dw, ir_needs_grad
         ctx.ir_mode, ctx.has_bias = ir_mode, bias is not None
         ctx.save_for_backward(
-            xq_rows if need_dw else None, x_rows, inp if keep_raw else None,
+            xq_rows if need_dw else None, flag_rows, counts,
             w_eff if need_dx else None, keep, flag, ir_dev,
         )
         return y
 
     @staticmethod
     def backward(ctx, grad_out: Tensor):
-        xq_rows, x_rows, inp, w_eff, keep, flag, ir_dev = ctx.saved_tensors
+        xq_rows, flag_rows, counts, w_eff, keep, flag, ir_dev = ctx.saved_tensors
         lib = L.load()
         geom, in_sizes = ctx.geom, ctx.in_sizes
         cgeom = ops.conv_geom(geom)
@@ -238,7 +243,7 @@ class HipConv(Function):
             dx = torch.empty((geom[0], channels, geom[2], geom[3], geom[4]), dtype=dtype, device=dev)
             ir_grad = torch.empty((n_tiles,), dtype=dtype, device=dev) if static else None
             _check(lib.ahl_conv_bwd_dx(ops.ptr(g_rows), ops.ptr(keep), ops.ptr(flag), ops.ptr(w_dx),
-                                       ops.ptr(x_rows), ops.ptr(inp), ops.ptr(ir_dev), ops.ptr(dimg), ops.ptr(dx),
+                                       ops.ptr(flag_rows), ops.ptr(counts), ops.ptr(ir_dev), ops.ptr(dimg), ops.ptr(dx),
                                        ops.ptr(ir_grad), byref(cgeom), n_out, ends, n_tiles, byref(cfg),
                                        ops.ptr(ws), stream), "ahl_conv_bwd_dx")
             if ctx.needs_input_grad[0]:

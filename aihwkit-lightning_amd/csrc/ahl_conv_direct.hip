@@ -97,7 +97,7 @@ AHL_DEV int64_t row_of(const RowMap& m, int32_t b, int32_t s) {
 }
 // The inverse: pixel p of the padded grid -> index into a [B, nch, S] tensor's (b, s), or -1 when
 // p lies outside the box (padding, outputs that do not exist).
-AHL_DEV bool box_of(const RowMap& m, int64_t p64, int32_t& b, int32_t& s) {
+AHL_DEV bool box_of(const RowMap& m, int64_t p64, int32_t& b, int32_t& s, int32_t (&pc)[3]) {
   const uint32_t p = (uint32_t)p64;   // pixels are fewer than 2^30: 32-bit divisions
   const uint32_t q1 = p / (uint32_t)m.p2;
   const int32_t w = (int32_t)(p - q1 * (uint32_t)m.p2) - m.o2;
@@ -107,6 +107,7 @@ AHL_DEV bool box_of(const RowMap& m, int64_t p64, int32_t& b, int32_t& s) {
   const int32_t d = (int32_t)(q0 - qb * (uint32_t)m.p0) - m.o0;
   b = (int32_t)qb;
   s = (d * m.d1 + h) * m.d2 + w;
+  pc[0] = d + m.o0; pc[1] = h + m.o1; pc[2] = w + m.o2;   // coordinates on the padded grid
   return w >= 0 && w < m.d2 && h >= 0 && h < m.d1 && d >= 0 && d < m.d0;
 }
 
@@ -116,25 +117,41 @@ static constexpr int kTileWords = 33;   // LDS row stride of the 64 x 64 transpo
 // [B, nch, S] -> pixel rows: dst[lead + row(b, s), c] = f(src[b, c, s]), f = the DAC of channel
 // c's K-tile (clamp to the tile's range, quantise) or the identity; every other row of dst (the
 // lead rows, the padding pixels, the rows behind the last pixel) is written as zeros, so dst
-// need not be cleared beforehand. With `raw` set the unmodified values go to a second buffer of
-// the same shape. One block: 64 consecutive rows of dst x 64 channels, turned in LDS; global
-// memory is read along s (consecutive rows of dst are consecutive s up to the padding) and
-// written along c, 16 bytes at a time. ct is a multiple of 64: a block's channels share a K-tile.
+// need not be cleared beforehand. One block: 64 consecutive rows of dst x 64 channels, turned in
+// LDS; global memory is read along s (consecutive rows of dst are consecutive s up to the padding)
+// and written along c, 16 bytes at a time. ct is a multiple of 64: a block's channels share a K-tile.
+// With `flags` set (static range, a backward pass will follow) the kernel also leaves what the
+// input gradient needs to know about x, one byte per element in the layout of dst:
+//   bit 0: x >= ir, bit 1: x <= -ir (the entries whose gradient goes to the range, reference
+//   torch_utils/torch_linear.py:92-106), bit 2: |x| > ir (the straight-through mask, :44-54),
+// and per block the number of PATCH ENTRIES with bit 0 or 1 (for the decay switch, :98-103): a
+// pixel is seen by one patch for every tap under which some valid output lies, so it counts that
+// many times.
+struct TapSpan { int32_t k0, k1, k2, out0, out1, out2; };
+
 template <class D, int IRMODE>
 __global__ __launch_bounds__(256) void k_conv_scatter(const uint16_t* __restrict__ src, int32_t nch, int32_t S,
                                                       RowMap map, int32_t lead, int64_t P, int64_t rows,
                                                       uint16_t* __restrict__ dst,
-                                                      uint16_t* __restrict__ raw, const void* __restrict__ ir,
+                                                      uint8_t* __restrict__ flags, uint32_t* __restrict__ count,
+                                                      TapSpan taps, const void* __restrict__ ir,
                                                       int32_t ct, float inp_res, int32_t skip_rounding) {
-  __shared__ uint32_t tile[2][64 * kTileWords];
+  __shared__ uint32_t tile[64 * kTileWords];
+  __shared__ uint32_t ftile[64 * 17];   // flags, one byte per element, 68 bytes per row
+  __shared__ uint32_t wave_count[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t r0 = (int64_t)blockIdx.x * 64;
   const int32_t c0 = blockIdx.y * 64;
   int32_t b = 0, sp = 0;
+  int32_t pc[3] = {0, 0, 0};
   const int64_t pix = r0 + lane - lead;
-  const bool inside = pix >= 0 && pix < P && box_of(map, pix, b, sp);
+  const bool inside = pix >= 0 && pix < P && box_of(map, pix, b, sp, pc);
   Dac dac = {0.0f, 1.0f, 1.0f, 1.0f};
-  if (IRMODE == AHL_IR_STATIC) dac = make_dac<D>(D::load(ir, c0 / ct), inp_res);
+  float irv = 0.0f;
+  if (IRMODE == AHL_IR_STATIC) {
+    irv = D::load(ir, c0 / ct);
+    dac = make_dac<D>(irv, inp_res);
+  }
   // every load is issued (lanes with nothing to read load the tensor's first element) and the
   // values are selected afterwards: a load behind a branch would be waited for before the next
   const uint16_t* col = src + ((int64_t)b * nch + c0 + wave * 16) * S + sp;
@@ -146,6 +163,7 @@ __global__ __launch_bounds__(256) void k_conv_scatter(const uint16_t* __restrict
   }
 #pragma unroll
   for (int i = 0; i < 16; ++i) v[i] = (inside && c0 + wave * 16 + i < nch) ? v[i] : 0.0f;
+  uint32_t clipped = 0;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int32_t cl = wave * 16 + i;
@@ -153,10 +171,29 @@ __global__ __launch_bounds__(256) void k_conv_scatter(const uint16_t* __restrict
     if (IRMODE == AHL_IR_STATIC)
       q = inp_res > 0.0f ? dac_apply<D, true, true>(v[i], dac, skip_rounding != 0)
                          : dac_apply<D, true, false>(v[i], dac, false);
-    ((uint16_t*)tile[0])[lane * (2 * kTileWords) + cl] = D::to_elem(q);
-    if (raw != nullptr) ((uint16_t*)tile[1])[lane * (2 * kTileWords) + cl] = D::to_elem(v[i]);
+    ((uint16_t*)tile)[lane * (2 * kTileWords) + cl] = D::to_elem(q);
+    if (IRMODE == AHL_IR_STATIC && flags != nullptr) {
+      const bool edge = v[i] >= irv || v[i] <= -irv;
+      const uint32_t f = (v[i] >= irv ? 1u : 0u) | (v[i] <= -irv ? 2u : 0u) | (fabsf(v[i]) > irv ? 4u : 0u);
+      ((uint8_t*)ftile)[lane * 68 + cl] = (uint8_t)f;
+      clipped += edge ? 1u : 0u;
+    }
+  }
+  if (IRMODE == AHL_IR_STATIC && flags != nullptr) {
+    // patches that see this lane's pixel: per dimension, the taps k with 0 <= coordinate - k < outputs
+    auto span = [](int32_t c, int32_t k, int32_t out) {
+      const int32_t lo = c - (out - 1) > 0 ? c - (out - 1) : 0, hi = c < k - 1 ? c : k - 1;
+      return hi >= lo ? hi - lo + 1 : 0;
+    };
+    uint32_t cnt = inside ? clipped * (uint32_t)(span(pc[0], taps.k0, taps.out0) * span(pc[1], taps.k1, taps.out1) *
+                                                 span(pc[2], taps.k2, taps.out2)) : 0u;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) cnt += __shfl_xor(cnt, o, 64);
+    if (lane == 0) wave_count[wave] = cnt;
   }
   __syncthreads();
+  if (IRMODE == AHL_IR_STATIC && flags != nullptr && tid == 0)
+    count[(int64_t)blockIdx.x * gridDim.y + blockIdx.y] = (wave_count[0] + wave_count[1]) + (wave_count[2] + wave_count[3]);
   const int vec = tid & 7;
   if (c0 + vec * 8 >= nch) return;
 #pragma unroll
@@ -164,33 +201,23 @@ __global__ __launch_bounds__(256) void k_conv_scatter(const uint16_t* __restrict
     const int r = (tid >> 3) + 32 * half;
     const int64_t row = r0 + r;
     if (row >= rows) continue;
-    const uint32_t* t0 = tile[0] + r * kTileWords + vec * 4;
+    const uint32_t* t0 = tile + r * kTileWords + vec * 4;
     const u32x4 v0 = {t0[0], t0[1], t0[2], t0[3]};
     st16(dst + row * nch + c0 + vec * 8, v0);
-    if (raw != nullptr) {
-      const uint32_t* t1 = tile[1] + r * kTileWords + vec * 4;
-      const u32x4 v1 = {t1[0], t1[1], t1[2], t1[3]};
-      st16(raw + row * nch + c0 + vec * 8, v1);
+    if (IRMODE == AHL_IR_STATIC && flags != nullptr) {
+      const uint32_t* f0 = ftile + r * 17 + vec * 2;
+      const u32x2 fv = {f0[0], f0[1]};
+      *(u32x2*)(flags + row * nch + c0 + vec * 8) = fv;
     }
   }
 }
 
 // ---------------------------------------------------------------------------------------------
-// pixel rows -> [B, nch, S]: dst[b, c, s] = src[lead + row(b, s), c]. MASK: the straight-through
-// rule of the learned input range on the way (dst zeroed where |x[b, c, s]| > ir of channel c's
-// tile; reference torch_utils/torch_linear.py:44-54), and the number of PATCH ENTRIES whose
-// input lies on or beyond the range, per tile (for the decay switch, :98-103): a pixel is seen by
-// one patch for every tap under which some valid output lies, so it counts that many times.
-template <class D, bool MASK>
+// pixel rows -> [B, nch, S]: dst[b, c, s] = src[lead + row(b, s), c].
+template <class D>
 __global__ __launch_bounds__(256) void k_conv_gather(const uint16_t* __restrict__ src, int32_t nch, int32_t S,
-                                                     RowMap map, int32_t lead, uint16_t* __restrict__ dst,
-                                                     const uint16_t* __restrict__ x, const void* __restrict__ ir,
-                                                     int32_t ct, int32_t k0, int32_t k1, int32_t k2,
-                                                     int32_t out0, int32_t out1, int32_t out2,
-                                                     uint32_t* __restrict__ count) {
+                                                     RowMap map, int32_t lead, uint16_t* __restrict__ dst) {
   __shared__ uint32_t tile[64 * kTileWords];
-  __shared__ int32_t taps[64];
-  __shared__ uint32_t wave_count[4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int32_t s0 = blockIdx.x * 64, c0 = blockIdx.y * 64, b = blockIdx.z;
   const int vec = tid & 7;
@@ -203,55 +230,15 @@ __global__ __launch_bounds__(256) void k_conv_gather(const uint16_t* __restrict_
     uint32_t* t0 = tile + r * kTileWords + vec * 4;
     t0[0] = v.x; t0[1] = v.y; t0[2] = v.z; t0[3] = v.w;
   }
-  if (MASK && tid < 64) {
-    // patches that see pixel s0 + tid: per dimension, the taps k with 0 <= coordinate - k < outputs
-    int32_t n = 0;
-    if (s0 + tid < S) {
-      const int32_t s = s0 + tid;
-      const int32_t w = s % map.d2 + map.o2, r = s / map.d2;
-      const int32_t h = r % map.d1 + map.o1, d = r / map.d1 + map.o0;
-      auto span = [](int32_t c, int32_t k, int32_t out) {
-        const int32_t lo = c - (out - 1) > 0 ? c - (out - 1) : 0, hi = c < k - 1 ? c : k - 1;
-        return hi >= lo ? hi - lo + 1 : 0;
-      };
-      n = span(d, k0, out0) * span(h, k1, out1) * span(w, k2, out2);
-    }
-    taps[tid] = n;
-  }
   __syncthreads();
   const int32_t s = s0 + lane;
-  uint32_t cnt = 0;   // at most 16 channels x kvol per lane
-  const bool live = s < S;
-  const int64_t at0 = ((int64_t)b * nch + c0 + wave * 16) * S + (live ? s : 0);
-  float xv[16];
-  float irv = 0.0f;
-  if (MASK) {
-    irv = D::load(ir, c0 / ct);   // the block's 64 channels lie in one K-tile
-#pragma unroll
-    for (int i = 0; i < 16; ++i)   // all loads issued, none behind a branch
-      xv[i] = D::load((live && c0 + wave * 16 + i < nch) ? x + at0 + (int64_t)i * S : x, 0);
-  }
+  if (s >= S) return;
+  const int64_t at0 = ((int64_t)b * nch + c0 + wave * 16) * S + s;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    const int32_t cl = wave * 16 + i, c = c0 + cl;
-    if (!live || c >= nch) continue;
-    float v = D::load(tile, lane * (2 * kTileWords) + cl);
-    if (MASK) {
-      if (xv[i] >= irv || xv[i] <= -irv) cnt += (uint32_t)taps[lane];
-      if (fabsf(xv[i]) > irv) v = 0.0f;
-    }
-    D::store(dst, at0 + (int64_t)i * S, v);
-  }
-  if (MASK) {
-    // one count per block (its 64 channels lie in one tile: ct is a multiple of 64), summed per
-    // tile by k_conv_ir_finalize: no atomics, nothing to clear beforehand
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) cnt += __shfl_xor(cnt, o, 64);
-    if (lane == 0) wave_count[wave] = cnt;
-    __syncthreads();
-    if (tid == 0)
-      count[((int64_t)b * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y] =
-          (wave_count[0] + wave_count[1]) + (wave_count[2] + wave_count[3]);
+    const int32_t cl = wave * 16 + i;
+    if (c0 + cl >= nch) continue;
+    D::store(dst, at0 + (int64_t)i * S, D::load(tile, lane * (2 * kTileWords) + cl));
   }
 }
 
@@ -296,10 +283,10 @@ struct ConvDxArgs {
   const uint32_t* keep;                // clamp mask [T, ceil(N/32), rows64(P)] or null
   const uint32_t* clamp_flag; uint32_t flag_token;
   const uint16_t* w; int64_t ldw;      // [C, kvol * N] (k_conv_weights mode 2)
-  const uint16_t* x;                   // the unquantised padded image rows [rows, C], or null
-  const void* ir;                      // [T] (with x)
+  const uint8_t* flags;                // per element of the padded image rows [rows, C]: bit 0 x >= ir,
+                                       // bit 1 x <= -ir, bit 2 |x| > ir (k_conv_scatter); or null
   uint16_t* out; int64_t ldo;          // dimg [P, C]
-  float* partial;                      // [row blocks][column blocks][2] (with x)
+  float* partial;                      // [row blocks][column blocks][2] (with flags)
   int64_t P, rows;
   int32_t N, C, ct, kvol;
   ConvMap conv;                        // sign -1
@@ -349,27 +336,28 @@ __global__ __launch_bounds__(256, 2) void k_conv_dx(ConvDxArgs a) {
       for (int v = 0; v < 16; ++v) { acc[i][j][v] = 0.0f; tot[i][j][v] = 0.0f; }
 
   // which of this lane's 64 outputs have their input on or beyond the range (per tap the same pixel)
-  uint64_t up = 0, lo = 0;
-  const bool do_ir = a.x != nullptr;
+  // and which are zeroed by the straight-through rule (|x| > range)
+  uint64_t up = 0, lo = 0, zr = 0;
+  const bool do_ir = a.flags != nullptr;
   if (do_ir) {
-    const float irv = D::load(a.ir, t_out);
-    // all loads first (rows beyond the last pixel are rows of zeros of the buffer), then the tests
+    // all loads first (rows beyond the last pixel carry zero flags), then the tests
 #pragma unroll
     for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
       for (int bj = 0; bj < 2; ++bj) {
-        float xv[16];
+        uint32_t fv[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int64_t m = m0 + wm * 64 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
           const int32_t c = n0 + wn * 64 + bj * 32 + (lane & 31);
-          xv[v] = D::load(a.x, (m + a.conv.lead) * a.C + c);
+          fv[v] = a.flags[(m + a.conv.lead) * a.C + c];
         }
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const uint64_t bit = 1ull << ((bi * 2 + bj) * 16 + v);
-          if (xv[v] >= irv) up |= bit;
-          if (xv[v] <= -irv) lo |= bit;
+          const int e = (bi * 2 + bj) * 16 + v;
+          up |= (uint64_t)(fv[v] & 1u) << e;
+          lo |= (uint64_t)((fv[v] >> 1) & 1u) << e;
+          zr |= (uint64_t)((fv[v] >> 2) & 1u) << e;
         }
       }
   }
@@ -490,7 +478,8 @@ __global__ __launch_bounds__(256, 2) void k_conv_dx(ConvDxArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
-          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = D::to_elem(tot[bi][bj][v]);
+          const bool zero = (zr >> ((bi * 2 + bj) * 16 + v)) & 1ull;
+          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = D::to_elem(zero ? 0.0f : tot[bi][bj][v]);
         }
     __syncthreads();
     constexpr int VPR = BN / 8, RPP = 256 / VPR;
@@ -567,11 +556,11 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
   // which of this lane's 64 outputs have their input on or beyond the range (per tap the same pixel)
   // bit e of up / lo: this lane's output e (MFMA block e >> 4, register e & 15) has its input on or
   // beyond the upper / lower end of the range (per tap the same pixel)
-  uint32_t up[2] = {0u, 0u}, lo[2] = {0u, 0u};
-  const bool do_ir = a.x != nullptr;
+  // zr: the outputs that the straight-through rule zeroes (|x| > range)
+  uint32_t up[2] = {0u, 0u}, lo[2] = {0u, 0u}, zr[2] = {0u, 0u};
+  const bool do_ir = a.flags != nullptr;
   if (do_ir) {
-    const float irv = D::load(a.ir, t_wave);
-    float xv[2][2][16];   // all 64 loads in flight at once (rows beyond the pixels are zeros)
+    uint32_t fv[2][2][16];   // all 64 loads in flight at once (rows beyond the pixels carry zero flags)
 #pragma unroll
     for (int bi = 0; bi < 2; ++bi)
 #pragma unroll
@@ -580,7 +569,7 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
         for (int v = 0; v < 16; ++v) {
           const int64_t m = m0 + wm * 64 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
           const int32_t c = n0 + wn * 64 + bj * 32 + r;
-          xv[bi][bj][v] = D::load(a.x, (m + a.conv.lead) * a.C + c);
+          fv[bi][bj][v] = a.flags[(m + a.conv.lead) * a.C + c];
         }
 #pragma unroll
     for (int bi = 0; bi < 2; ++bi)
@@ -588,9 +577,10 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
       for (int bj = 0; bj < 2; ++bj)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const uint32_t bit = 1u << (bj * 16 + v);
-          if (xv[bi][bj][v] >= irv) up[bi] |= bit;
-          if (xv[bi][bj][v] <= -irv) lo[bi] |= bit;
+          const int e = bj * 16 + v;
+          up[bi] |= (fv[bi][bj][v] & 1u) << e;
+          lo[bi] |= ((fv[bi][bj][v] >> 1) & 1u) << e;
+          zr[bi] |= ((fv[bi][bj][v] >> 2) & 1u) << e;
         }
   }
   // the same for the wave: most of the 64 registers have no clipped input in any lane
@@ -759,7 +749,8 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int ro = bi * 32 + 8 * (v >> 2) + (v & 3);
-          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = D::to_elem(tot[bi][bj][v]);
+          const bool zero = (zr[bi] >> (bj * 16 + v)) & 1u;
+          *(uint16_t*)(obase + ro * kOutStride + bj * 64) = D::to_elem(zero ? 0.0f : tot[bi][bj][v]);
         }
     __syncthreads();
     const int vcol = tid & 15, vrow = tid >> 4;
@@ -861,24 +852,32 @@ int ahl_conv_direct_supported(const AhlConvGeom* geom, int32_t dtype, int64_t N,
   return channels_per_tile(g, tl) > 0 ? 1 : 0;
 }
 
+int64_t ahl_conv_count_words(const AhlConvGeom* geom) {
+  DirectGeom g;
+  if (!make_direct(geom, &g)) return -1;
+  return cdiv(g.rows, 64) * cdiv(g.C, 64);
+}
+
 int ahl_conv_image_rows(const void* x, const AhlConvGeom* geom, int32_t dtype, const void* ir,
                         const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg, void* xq_rows,
-                        void* x_rows, void* stream) {
+                        uint8_t* flag_rows, uint32_t* counts, void* stream) {
   DirectGeom g;
   Tiling tl;
   if (!x || !xq_rows || !cfg || !direct_dtype(dtype) || !make_direct(geom, &g)) return AHL_ERR_ARG;
+  if ((flag_rows == nullptr) != (counts == nullptr)) return AHL_ERR_ARG;
   if (!make_tiling(tile_ends_host, n_tiles, (int64_t)g.C * g.kvol, &tl)) return AHL_ERR_TILING;
   const int32_t ct = channels_per_tile(g, tl);
   if (ct == 0 || cfg->ir_mode == AHL_IR_DYNAMIC || (cfg->ir_mode == AHL_IR_STATIC && !ir)) return AHL_ERR_UNSUPPORTED;
-  if (cfg->ir_mode == AHL_IR_NONE && cfg->inp_res > 0.0f) return AHL_ERR_ARG;
+  if (cfg->ir_mode == AHL_IR_NONE && (cfg->inp_res > 0.0f || flag_rows)) return AHL_ERR_ARG;
   const int32_t S = g.in[0] * g.in[1] * g.in[2];
   const RowMap map = {g.in[0], g.in[1], g.in[2], g.pad[0], g.pad[1], g.pad[2], g.pin[0], g.pin[1], g.pin[2]};
+  const TapSpan taps = {g.ker[0], g.ker[1], g.ker[2], g.out[0], g.out[1], g.out[2]};
   const dim3 grid((unsigned)cdiv(g.rows, 64), (unsigned)cdiv(g.C, 64));
   hipStream_t s = (hipStream_t)stream;
 #define AHL_SCATTER(DT, MODE)                                                                          \
   hipLaunchKernelGGL((k_conv_scatter<DT, MODE>), grid, dim3(256), 0, s, (const uint16_t*)x, g.C, S, map, \
-                     g.lead, g.P, g.rows, (uint16_t*)xq_rows, (uint16_t*)x_rows, ir, ct, cfg->inp_res,   \
-                     cfg->skip_rounding)
+                     g.lead, g.P, g.rows, (uint16_t*)xq_rows, flag_rows, counts, taps, ir, ct,           \
+                     cfg->inp_res, cfg->skip_rounding)
   if (dtype == AHL_F16) { if (cfg->ir_mode == AHL_IR_STATIC) AHL_SCATTER(F16, 1); else AHL_SCATTER(F16, 0); }
   else { if (cfg->ir_mode == AHL_IR_STATIC) AHL_SCATTER(BF16, 1); else AHL_SCATTER(BF16, 0); }
 #undef AHL_SCATTER
@@ -895,10 +894,12 @@ int ahl_conv_grad_rows(const void* g_out, const AhlConvGeom* geom, int32_t dtype
   hipStream_t s = (hipStream_t)stream;
   if (dtype == AHL_F16)
     hipLaunchKernelGGL((k_conv_scatter<F16, 0>), grid, dim3(256), 0, s, (const uint16_t*)g_out, (int32_t)N, S, map,
-                       g.lead, g.P, g.rows, (uint16_t*)g_rows, (uint16_t*)nullptr, (const void*)nullptr, 64, 0.0f, 0);
+                       g.lead, g.P, g.rows, (uint16_t*)g_rows, (uint8_t*)nullptr, (uint32_t*)nullptr, TapSpan{1, 1, 1, 1, 1, 1},
+                       (const void*)nullptr, 64, 0.0f, 0);
   else
     hipLaunchKernelGGL((k_conv_scatter<BF16, 0>), grid, dim3(256), 0, s, (const uint16_t*)g_out, (int32_t)N, S, map,
-                       g.lead, g.P, g.rows, (uint16_t*)g_rows, (uint16_t*)nullptr, (const void*)nullptr, 64, 0.0f, 0);
+                       g.lead, g.P, g.rows, (uint16_t*)g_rows, (uint8_t*)nullptr, (uint32_t*)nullptr, TapSpan{1, 1, 1, 1, 1, 1},
+                       (const void*)nullptr, 64, 0.0f, 0);
   return check_launch("ahl_conv_grad_rows");
 }
 
@@ -911,13 +912,11 @@ int ahl_conv_output(const void* y_rows, const AhlConvGeom* geom, int32_t dtype, 
   hipStream_t s = (hipStream_t)stream;
   // the output rows carry no lead: row p of y_rows is output p
   if (dtype == AHL_F16)
-    hipLaunchKernelGGL((k_conv_gather<F16, false>), grid, dim3(256), 0, s, (const uint16_t*)y_rows, (int32_t)N, S, map, 0,
-                       (uint16_t*)y, (const uint16_t*)nullptr, (const void*)nullptr, 1, 1, 1, 1, 1, 1, 1,
-                       (uint32_t*)nullptr);
+    hipLaunchKernelGGL((k_conv_gather<F16>), grid, dim3(256), 0, s, (const uint16_t*)y_rows, (int32_t)N, S, map, 0,
+                       (uint16_t*)y);
   else
-    hipLaunchKernelGGL((k_conv_gather<BF16, false>), grid, dim3(256), 0, s, (const uint16_t*)y_rows, (int32_t)N, S, map, 0,
-                       (uint16_t*)y, (const uint16_t*)nullptr, (const void*)nullptr, 1, 1, 1, 1, 1, 1, 1,
-                       (uint32_t*)nullptr);
+    hipLaunchKernelGGL((k_conv_gather<BF16>), grid, dim3(256), 0, s, (const uint16_t*)y_rows, (int32_t)N, S, map, 0,
+                       (uint16_t*)y);
   return check_launch("ahl_conv_output");
 }
 
@@ -994,14 +993,13 @@ int ahl_conv_bwd_dw(const void* g_rows, const uint32_t* keep, const uint32_t* cl
 int64_t ahl_conv_bwd_dx_ws_bytes(const AhlConvGeom* geom, int32_t n_tiles) {
   DirectGeom g;
   if (!make_direct(geom, &g) || n_tiles <= 0) return -1;
-  // [row blocks][C / 64][2] floats, then one 32-bit count per block of the gather kernel
-  const int64_t S = (int64_t)g.in[0] * g.in[1] * g.in[2];
-  return (cdiv(g.P, 128) * (g.C / 64) * 2 * 4 + 255) / 256 * 256 + (int64_t)g.B * cdiv(S, 64) * (g.C / 64) * 4;
+  // the blocks' partial sums of the range gradient: [row blocks][C / 64][2] floats
+  return (cdiv(g.P, 128) * (g.C / 64) * 2 * 4 + 255) / 256 * 256;
 }
 
 int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* keep, const uint32_t* clamp_flag, const void* w_dx,
-                    const void* x_rows, const void* x, const void* ir, void* dimg_rows, void* dx, void* ir_grad,
-                    const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
+                    const uint8_t* flag_rows, const uint32_t* counts, const void* ir, void* dimg_rows, void* dx,
+                    void* ir_grad, const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
                     const AhlLinearCfg* cfg, void* ws, void* stream) {
   DirectGeom g;
   Tiling tl;
@@ -1010,7 +1008,8 @@ int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* keep, const uint32_t* cl
   const int32_t ct = channels_per_tile(g, tl);
   if (ct == 0 || N <= 0 || N % 64 != 0) return AHL_ERR_UNSUPPORTED;
   const bool is_static = cfg->ir_mode == AHL_IR_STATIC;
-  if (is_static && (!x_rows || !x || !ir || !ir_grad || !ws || cfg->ir_grad_rule != AHL_IR_GRAD_LEARNED)) return AHL_ERR_ARG;
+  if (is_static && (!flag_rows || !counts || !ir || !ir_grad || !ws || cfg->ir_grad_rule != AHL_IR_GRAD_LEARNED))
+    return AHL_ERR_ARG;
   hipStream_t s = (hipStream_t)stream;
   // blocks: 256 x 128 (channel counts that are multiples of 128), else 128 x 128 or 256 x 64
   const bool pipe = g.C % 128 == 0;
@@ -1021,11 +1020,10 @@ int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* keep, const uint32_t* cl
   // partial sums per (row block, column block); the 256 x 128 blocks leave one pair per 64 columns
   const int32_t partial_cols = pipe ? g.C / 64 : col_blocks, partial_per_tile = pipe ? ct / 64 : ct / bn_cols;
   float* partial = (float*)ws;
-  uint32_t* count = ws ? (uint32_t*)((char*)ws + (cdiv(g.P, 128) * (g.C / 64) * 2 * 4 + 255) / 256 * 256) : nullptr;
   ConvDxArgs a;
   a.g = (const uint16_t*)g_rows; a.ldg = N; a.keep = keep; a.clamp_flag = clamp_flag; a.flag_token = cfg->flag_token;
   a.w = (const uint16_t*)w_dx; a.ldw = (int64_t)g.kvol * N;
-  a.x = is_static ? (const uint16_t*)x_rows : nullptr; a.ir = ir;
+  a.flags = is_static ? flag_rows : nullptr;
   a.out = (uint16_t*)dimg_rows; a.ldo = g.C; a.partial = partial;
   a.P = g.P; a.rows = g.rows; a.N = (int32_t)N; a.C = g.C; a.ct = ct; a.kvol = g.kvol;
   a.conv = make_map(g, -1, (int32_t)(N / 64), 0, g.rows);
@@ -1049,26 +1047,24 @@ int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* keep, const uint32_t* cl
       else hipLaunchKernelGGL((k_conv_dx<BF16, 4, 1>), grid, dim3(256), lds_bytes, s, a);
     }
   }
-  // pixel rows -> [B, C, *spatial], with the range mask and the clipped-entry counts
+  // pixel rows -> [B, C, *spatial] (the range mask is applied already)
   const int32_t S = g.in[0] * g.in[1] * g.in[2];
   const RowMap map = {g.in[0], g.in[1], g.in[2], g.pad[0], g.pad[1], g.pad[2], g.pin[0], g.pin[1], g.pin[2]};
   const dim3 ggrid((unsigned)cdiv(S, 64), (unsigned)cdiv(g.C, 64), (unsigned)g.B);
-#define AHL_GATHER(DT, MASK)                                                                                   \
-  hipLaunchKernelGGL((k_conv_gather<DT, MASK>), ggrid, dim3(256), 0, s, (const uint16_t*)dimg_rows, g.C, S, map, 0, \
-                     (uint16_t*)dx, (const uint16_t*)x, ir, ct, g.ker[0], g.ker[1], g.ker[2], g.out[0], g.out[1],  \
-                     g.out[2], count)
-  if (cfg->dtype == AHL_F16) { if (is_static) AHL_GATHER(F16, true); else AHL_GATHER(F16, false); }
-  else { if (is_static) AHL_GATHER(BF16, true); else AHL_GATHER(BF16, false); }
-#undef AHL_GATHER
+  if (cfg->dtype == AHL_F16)
+    hipLaunchKernelGGL((k_conv_gather<F16>), ggrid, dim3(256), 0, s, (const uint16_t*)dimg_rows, g.C, S, map, 0, (uint16_t*)dx);
+  else
+    hipLaunchKernelGGL((k_conv_gather<BF16>), ggrid, dim3(256), 0, s, (const uint16_t*)dimg_rows, g.C, S, map, 0, (uint16_t*)dx);
   if (is_static) {
     const double numel = (double)g.B * g.out[0] * g.out[1] * g.out[2] * (double)tl.base;
+    // the clipped-entry counts of k_conv_scatter: [blocks of 64 rows][C / 64]
     if (cfg->dtype == AHL_F16)
       hipLaunchKernelGGL((k_conv_ir_finalize<F16>), dim3(n_tiles), dim3(256), 0, s, (const float*)partial, row_blocks,
-                         partial_cols, partial_per_tile, (const uint32_t*)count, (int64_t)g.B * cdiv(S, 64), g.C / 64, ct / 64,
+                         partial_cols, partial_per_tile, counts, cdiv(g.rows, 64), g.C / 64, ct / 64,
                          numel, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
     else
       hipLaunchKernelGGL((k_conv_ir_finalize<BF16>), dim3(n_tiles), dim3(256), 0, s, (const float*)partial, row_blocks,
-                         partial_cols, partial_per_tile, (const uint32_t*)count, (int64_t)g.B * cdiv(S, 64), g.C / 64, ct / 64,
+                         partial_cols, partial_per_tile, counts, cdiv(g.rows, 64), g.C / 64, ct / 64,
                          numel, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
   }
   return check_launch("ahl_conv_bwd_dx");

@@ -480,12 +480,18 @@ int ahl_conv_direct_supported(const AhlConvGeom* geom, int32_t dtype, int64_t N,
                               int32_t n_tiles);
 
 /* xq_rows[lead + p, c] = DAC(x[b, c, d, h, w]) at the padded pixel p of (b, d, h, w): clamp to the
- * range of channel c's K-tile and quantise (cfg->ir_mode AHL_IR_STATIC; AHL_IR_NONE copies). x_rows,
- * if not NULL, receives the unmodified values in the same layout (the input-range gradient needs
- * them). Replaces unfold + the per-tile clamp/DAC of torch_utils/torch_linear.py:134-192.    */
+ * range of channel c's K-tile and quantise (cfg->ir_mode AHL_IR_STATIC; AHL_IR_NONE copies).
+ * flag_rows / counts (both or neither; static range, when a backward pass will follow): what
+ * the input gradient needs to know about x -- flag_rows uint8 [rows, C] in the layout of xq_rows,
+ * bit 0: x >= range, bit 1: x <= -range (entries whose gradient goes to the range), bit 2:
+ * |x| > range (zeroed by the straight-through rule); counts uint32 [ahl_conv_count_words(geom)]:
+ * per block of the kernel, the number of patch entries with bit 0 or 1 (the decay switch).
+ * Replaces unfold + the per-tile clamp/DAC of torch_utils/torch_linear.py:134-192 and the
+ * bookkeeping of :44-54, :92-106.                                                           */
+int64_t ahl_conv_count_words(const AhlConvGeom* geom);
 int ahl_conv_image_rows(const void* x, const AhlConvGeom* geom, int32_t dtype, const void* ir,
                         const int32_t* tile_ends_host, int32_t n_tiles, const AhlLinearCfg* cfg, void* xq_rows,
-                        void* x_rows, void* stream);
+                        uint8_t* flag_rows, uint32_t* counts, void* stream);
 
 /* Weight layouts for the three products, from / to the layer's [N, C * kvol] matrix
  * (weight.view(out_channels, -1)): mode 0 reorders every tile's columns to (tap, channel) -- the
@@ -521,12 +527,12 @@ int ahl_conv_bwd_dw(const void* g_rows, const uint32_t* clamp_mask, const uint32
 
 /* Input gradient dx [B, C, *in] and, with a static range, ir_grad [T] (the autograd of unfold,
  * the product and the range clamp: torch_utils/torch_linear.py:29-108): w_dx from
- * ahl_conv_weight_layout mode 2; x_rows the unquantised image rows, x the input itself (both only
+ * ahl_conv_weight_layout mode 2; flag_rows and counts as ahl_conv_image_rows left them (only
  * with a static range); dimg_rows [P, C] is scratch the caller provides.                       */
 int64_t ahl_conv_bwd_dx_ws_bytes(const AhlConvGeom* geom, int32_t n_tiles);
 int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* clamp_mask, const uint32_t* clamp_flag, const void* w_dx,
-                    const void* x_rows, const void* x, const void* ir, void* dimg_rows, void* dx, void* ir_grad,
-                    const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
+                    const uint8_t* flag_rows, const uint32_t* counts, const void* ir, void* dimg_rows, void* dx,
+                    void* ir_grad, const AhlConvGeom* geom, int64_t N, const int32_t* tile_ends_host, int32_t n_tiles,
                     const AhlLinearCfg* cfg, void* ws, void* stream);
 
 #ifdef __cplusplus
