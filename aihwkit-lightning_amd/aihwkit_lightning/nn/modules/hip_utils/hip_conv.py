@@ -163,9 +163,17 @@ class HipConv(Function):
         _check(lib.ahl_conv_image_rows(ops.ptr(inp), byref(cgeom), dt, ops.ptr(ir_dev), ends, n_tiles,
                                        byref(cfg), ops.ptr(xq_rows), ops.ptr(flag_rows), ops.ptr(counts), stream),
                "ahl_conv_image_rows")
+        # the forward's operand and, for a step that wants dx, the input gradient's in the same launch
         w_taps = torch.empty_like(w_eff)
-        _check(lib.ahl_conv_weight_layout(ops.ptr(w_eff), k_in, dt, n_out, byref(cgeom), ends, n_tiles, 0, 0,
-                                          ops.ptr(w_taps), k_in, stream), "ahl_conv_weight_layout")
+        w_dx = None
+        if need_dx:
+            w_dx = torch.empty((channels, k_in // channels * n_out), dtype=dtype, device=dev)
+            _check(lib.ahl_conv_weight_layouts(ops.ptr(w_eff), k_in, dt, n_out, byref(cgeom), ends, n_tiles,
+                                               ops.ptr(w_taps), k_in, ops.ptr(w_dx), w_dx.size(1), stream),
+                   "ahl_conv_weight_layouts")
+        else:
+            _check(lib.ahl_conv_weight_layout(ops.ptr(w_eff), k_in, dt, n_out, byref(cgeom), ends, n_tiles, 0, 0,
+                                              ops.ptr(w_taps), k_in, stream), "ahl_conv_weight_layout")
         want_keep = fwd.out_bound > 0 and (need_dx or need_dw)
         y_rows = torch.empty((pixels, n_out), dtype=dtype, device=dev)
         keep = flag = None
@@ -187,13 +195,13 @@ class HipConv(Function):
         ctx.ir_mode, ctx.has_bias = ir_mode, bias is not None
         ctx.save_for_backward(
             xq_rows if need_dw else None, flag_rows, counts,
-            w_eff if need_dx else None, keep, flag, ir_dev,
+            w_dx, keep, flag, ir_dev,
         )
         return y
 
     @staticmethod
     def backward(ctx, grad_out: Tensor):
-        xq_rows, flag_rows, counts, w_eff, keep, flag, ir_dev = ctx.saved_tensors
+        xq_rows, flag_rows, counts, w_dx, keep, flag, ir_dev = ctx.saved_tensors
         lib = L.load()
         geom, in_sizes = ctx.geom, ctx.in_sizes
         cgeom = ops.conv_geom(geom)
@@ -233,9 +241,6 @@ class HipConv(Function):
         elif want_bias:
             grad_b = g.flatten(2).sum(dim=(0, 2)).to(dtype)
         if ctx.need_dx:
-            w_dx = torch.empty((channels, k_in // channels * n_out), dtype=dtype, device=dev)
-            _check(lib.ahl_conv_weight_layout(ops.ptr(w_eff), k_in, dt, n_out, byref(cgeom), ends, n_tiles, 2, 0,
-                                              ops.ptr(w_dx), w_dx.size(1), stream), "ahl_conv_weight_layout")
             static = ctx.ir_mode == L.AHL_IR_STATIC
             ws_bytes = lib.ahl_conv_bwd_dx_ws_bytes(byref(cgeom), n_tiles)
             ws = torch.empty((max(ws_bytes, 16),), dtype=torch.uint8, device=dev)

@@ -14,7 +14,7 @@ from ....exceptions import HipBackendError
 
 LIB_NAME = "libanalog_hip.so"
 LIB_DIR = os.path.normpath(os.path.join(os.path.dirname(__file__), "..", "..", "..", "_lib"))
-ABI_VERSION = 15
+ABI_VERSION = 16
 STATIC_DX_SCRATCH_BYTES = 16 * 1024 * 1024
 
 AHL_F32, AHL_BF16, AHL_F16 = 0, 1, 2
@@ -188,6 +188,8 @@ SIGNATURES = {
                                       POINTER(AhlLinearCfg), c_void_p, c_void_p, c_void_p, c_void_p]),
     "ahl_conv_weight_layout": (c_int32, [c_void_p, c_int64, c_int32, c_int64, POINTER(AhlConvGeom), _I32P,
                                          c_int32, c_int32, c_int64, c_void_p, c_int64, c_void_p]),
+    "ahl_conv_weight_layouts": (c_int32, [c_void_p, c_int64, c_int32, c_int64, POINTER(AhlConvGeom), _I32P,
+                                          c_int32, c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "ahl_conv_fwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                c_void_p, c_void_p, POINTER(AhlConvGeom), c_int64, _I32P, c_int32,
                                POINTER(AhlLinearCfg), c_void_p]),

@@ -38,8 +38,9 @@ int launch_fast_fwd(const void* xq, int64_t ldxq, const void* w_eff, int64_t ldw
 int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
-                   hipStream_t s, const ConvMap* conv, int32_t conv_cols);
-int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N);
+                   hipStream_t s, const ConvMap* conv, int32_t conv_cols, int block_cols);
+int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int block_cols);
+int fast_dw_image_block(int64_t M, int64_t tile_cols, int32_t n_tiles, int64_t N);
 
 struct DirectGeom {
   int32_t B, C;
@@ -252,16 +253,17 @@ __global__ __launch_bounds__(256) void k_conv_gather(const uint16_t* __restrict_
 template <class E>
 __global__ __launch_bounds__(256) void k_conv_weights(const E* __restrict__ src, int64_t ld_src, int32_t N,
                                                       int32_t C, int32_t kvol, int32_t ct, int32_t stride,
-                                                      int mode, E* __restrict__ dst, int64_t ld_dst) {
+                                                      int mode, E* __restrict__ dst, int64_t ld_dst,
+                                                      E* __restrict__ dst_dx, int64_t ld_dx) {
   const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const int64_t K = (int64_t)C * kvol;
   if (idx >= (int64_t)N * K) return;
-  if (mode == 2) {
+  if (dst_dx != nullptr) {   // mode 2, alone or (mode 0) beside the forward's layout
     const int32_t c = (int32_t)(idx / ((int64_t)kvol * N));
     const int32_t rem = (int32_t)(idx - (int64_t)c * kvol * N);
     const int32_t tap = rem / N, n = rem - tap * N;
-    dst[(int64_t)c * ld_dst + rem] = src[(int64_t)n * ld_src + (int64_t)c * kvol + tap];
-    return;
+    dst_dx[(int64_t)c * ld_dx + rem] = src[(int64_t)n * ld_src + (int64_t)c * kvol + tap];
+    if (mode == 2) return;
   }
   const int32_t n = (int32_t)(idx / K);
   const int32_t k = (int32_t)(idx - (int64_t)n * K);   // position in the layer's order
@@ -776,37 +778,37 @@ __global__ __launch_bounds__(512, 1) void k_conv_dx_pipe(ConvDxArgs a) {
 // ir_grad[t] from the blocks' partial sums and the clipped-entry counts (reference
 // torch_utils/torch_linear.py:92-106; the roundings of k_ir_grad_finalize).
 template <class D>
-__global__ __launch_bounds__(256) void k_conv_ir_finalize(const float* __restrict__ partial, int64_t row_blocks,
+__global__ __launch_bounds__(1024) void k_conv_ir_finalize(const float* __restrict__ partial, int64_t row_blocks,
                                                           int32_t col_blocks, int32_t per_tile,
                                                           const uint32_t* __restrict__ count,
                                                           int64_t count_rows, int32_t count_cols,
                                                           int32_t count_per_tile,
                                                           double numel, const void* ir, void* ir_grad,
                                                           float decay, float min_pct) {
-  __shared__ double part[4][2];
-  __shared__ unsigned long long part_count[4];
+  __shared__ double part[16][2];
+  __shared__ unsigned long long part_count[16];
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   double s_up = 0.0, s_lo = 0.0;
-  // clipped patch entries of the tile: the gather blocks' counts [count_rows][count_cols], this
-  // tile's columns
+  // clipped patch entries of the tile: the layout kernel's counts [count_rows][count_cols], this
+  // tile's columns. A thread walks rows (every 1024th), so that the loop holds no division and the
+  // loads of a pass are independent.
   unsigned long long clipped = 0;
-  for (int64_t i = tid; i < count_rows * count_per_tile; i += 256)
-    clipped += count[(i / count_per_tile) * count_cols + (int64_t)t * count_per_tile + i % count_per_tile];
+  for (int64_t r = tid; r < count_rows; r += 1024) {
+    const uint32_t* c = count + r * count_cols + (int64_t)t * count_per_tile;
+    for (int32_t j = 0; j < count_per_tile; ++j) clipped += c[j];
+  }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) clipped += __shfl_xor(clipped, o, 64);
-  const int64_t total = row_blocks * per_tile;
-  for (int64_t i = tid; i < total; i += 256) {
-    const int64_t rb = i / per_tile, cb = (int64_t)t * per_tile + i % per_tile;
-    const float* p = partial + (rb * col_blocks + cb) * 2;
-    s_up += (double)p[0]; s_lo += (double)p[1];
+  for (int64_t rb = tid; rb < row_blocks; rb += 1024) {
+    const float* p = partial + (rb * col_blocks + (int64_t)t * per_tile) * 2;
+    for (int32_t j = 0; j < per_tile; ++j) { s_up += (double)p[2 * j]; s_lo += (double)p[2 * j + 1]; }
   }
   s_up = wave_sum(s_up); s_lo = wave_sum(s_lo);
   if (lane == 0) { part[wave][0] = s_up; part[wave][1] = s_lo; part_count[wave] = clipped; }
   __syncthreads();
   if (tid == 0) {
-    s_up = (part[0][0] + part[1][0]) + (part[2][0] + part[3][0]);
-    s_lo = (part[0][1] + part[1][1]) + (part[2][1] + part[3][1]);
-    clipped = (part_count[0] + part_count[1]) + (part_count[2] + part_count[3]);
+    s_up = 0.0; s_lo = 0.0; clipped = 0;
+    for (int w = 0; w < 16; ++w) { s_up += part[w][0]; s_lo += part[w][1]; clipped += part_count[w]; }
     const float irv = D::load(ir, t);
     float gr = D::rd(0.0f + D::rd((float)s_up));
     gr = D::rd(gr - D::rd((float)s_lo));
@@ -930,10 +932,27 @@ int ahl_conv_weight_layout(const void* src, int64_t ld_src, int32_t dtype, int64
   const int32_t ct = channels_per_tile(g, tl);
   if (ct == 0) return AHL_ERR_UNSUPPORTED;
   const int64_t total = N * g.C * g.kvol;
+  const bool dx = mode == 2;
   hipLaunchKernelGGL((k_conv_weights<uint16_t>), dim3((unsigned)cdiv(total, 256)), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t*)src, ld_src, (int32_t)N, g.C, g.kvol, ct, (int32_t)stride, (int)mode, (uint16_t*)dst,
-                     ld_dst);
+                     (const uint16_t*)src, ld_src, (int32_t)N, g.C, g.kvol, ct, (int32_t)stride, (int)mode,
+                     dx ? nullptr : (uint16_t*)dst, dx ? 0 : ld_dst, dx ? (uint16_t*)dst : nullptr, dx ? ld_dst : 0);
   return check_launch("ahl_conv_weight_layout");
+}
+
+int ahl_conv_weight_layouts(const void* src, int64_t ld_src, int32_t dtype, int64_t N, const AhlConvGeom* geom,
+                            const int32_t* tile_ends_host, int32_t n_tiles, void* w_taps, int64_t ld_taps, void* w_dx,
+                            int64_t ld_dx, void* stream) {
+  DirectGeom g;
+  Tiling tl;
+  if (!src || !w_taps || !w_dx || N <= 0 || !direct_dtype(dtype) || !make_direct(geom, &g)) return AHL_ERR_ARG;
+  if (!make_tiling(tile_ends_host, n_tiles, (int64_t)g.C * g.kvol, &tl)) return AHL_ERR_TILING;
+  const int32_t ct = channels_per_tile(g, tl);
+  if (ct == 0) return AHL_ERR_UNSUPPORTED;
+  const int64_t total = N * g.C * g.kvol;
+  hipLaunchKernelGGL((k_conv_weights<uint16_t>), dim3((unsigned)cdiv(total, 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)src, ld_src, (int32_t)N, g.C, g.kvol, ct, 0, 0, (uint16_t*)w_taps, ld_taps,
+                     (uint16_t*)w_dx, ld_dx);
+  return check_launch("ahl_conv_weight_layouts");
 }
 
 int ahl_conv_fwd(const void* xq_rows, const void* w_taps, const void* bias, void* y_rows, uint32_t* keep,
@@ -965,9 +984,10 @@ int64_t ahl_conv_bwd_dw_ws_bytes(const AhlConvGeom* geom, int64_t N, const int32
   DirectGeom g;
   Tiling tl;
   if (!make_direct(geom, &g) || !make_tiling(tile_ends_host, n_tiles, (int64_t)g.C * g.kvol, &tl)) return -1;
-  const int64_t stride = cdiv(tl.base, 256) * 256, kp = stride * n_tiles;
+  const int bw = fast_dw_image_block(g.P, tl.base, n_tiles, N);
+  const int64_t stride = cdiv(tl.base, bw) * bw, kp = stride * n_tiles;
   if (padded_cols) *padded_cols = kp;
-  return fast_dw_ws_bytes(g.P, kp, N);
+  return fast_dw_ws_bytes(g.P, kp, N, bw);
 }
 
 int ahl_conv_bwd_dw(const void* g_rows, const uint32_t* keep, const uint32_t* clamp_flag, const void* xq_rows,
@@ -979,7 +999,10 @@ int ahl_conv_bwd_dw(const void* g_rows, const uint32_t* keep, const uint32_t* cl
   if (!make_tiling(tile_ends_host, n_tiles, (int64_t)g.C * g.kvol, &tl)) return AHL_ERR_TILING;
   const int32_t ct = channels_per_tile(g, tl);
   if (ct == 0 || N <= 0 || N % 8 != 0) return AHL_ERR_UNSUPPORTED;
-  const int32_t stride = (int32_t)(cdiv(tl.base, 256) * 256);
+  // columns per block and per K-tile of dw_tiled: the tile itself when blocks of 192 or 256 columns
+  // divide it, else the tile padded to whole blocks of 256
+  const int bw = fast_dw_image_block(g.P, tl.base, n_tiles, N);
+  const int32_t stride = (int32_t)(cdiv(tl.base, bw) * bw);
   const int64_t kp = (int64_t)stride * n_tiles;
   Tiling padded;
   padded.n_tiles = n_tiles; padded.base = stride; padded.extra = 0;
@@ -987,7 +1010,7 @@ int ahl_conv_bwd_dw(const void* g_rows, const uint32_t* keep, const uint32_t* cl
   const uint16_t* gb = (const uint16_t*)g_rows + (int64_t)g.lead * N;
   const uint16_t* xb = (const uint16_t*)xq_rows + (int64_t)g.lead * g.C;
   return launch_fast_dw(cfg->dtype, gb, N, keep, clamp_flag, cfg->flag_token, xb, g.C, dw_tiled, kp, dbias, ws, g.P, kp, N,
-                        padded, (hipStream_t)stream, &map, g.kvol * ct);
+                        padded, (hipStream_t)stream, &map, g.kvol * ct, bw);
 }
 
 int64_t ahl_conv_bwd_dx_ws_bytes(const AhlConvGeom* geom, int32_t n_tiles) {
@@ -1059,11 +1082,11 @@ int ahl_conv_bwd_dx(const void* g_rows, const uint32_t* keep, const uint32_t* cl
     const double numel = (double)g.B * g.out[0] * g.out[1] * g.out[2] * (double)tl.base;
     // the clipped-entry counts of k_conv_scatter: [blocks of 64 rows][C / 64]
     if (cfg->dtype == AHL_F16)
-      hipLaunchKernelGGL((k_conv_ir_finalize<F16>), dim3(n_tiles), dim3(256), 0, s, (const float*)partial, row_blocks,
+      hipLaunchKernelGGL((k_conv_ir_finalize<F16>), dim3(n_tiles), dim3(1024), 0, s, (const float*)partial, row_blocks,
                          partial_cols, partial_per_tile, counts, cdiv(g.rows, 64), g.C / 64, ct / 64,
                          numel, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
     else
-      hipLaunchKernelGGL((k_conv_ir_finalize<BF16>), dim3(n_tiles), dim3(256), 0, s, (const float*)partial, row_blocks,
+      hipLaunchKernelGGL((k_conv_ir_finalize<BF16>), dim3(n_tiles), dim3(1024), 0, s, (const float*)partial, row_blocks,
                          partial_cols, partial_per_tile, counts, cdiv(g.rows, 64), g.C / 64, ct / 64,
                          numel, ir, ir_grad, cfg->ir_decay, cfg->ir_input_min_percentage);
   }

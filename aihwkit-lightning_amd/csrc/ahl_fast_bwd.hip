@@ -76,11 +76,12 @@ struct BwdPos {
   int t, slice;
 };
 
-template <class D, int MODE>
-AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2], char* lds,
+template <class D, int MODE, int BN, int TI, int TJ>
+AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[TI][TJ], char* lds,
                         float (*red)[3]) {
+  constexpr int WN = BN / (32 * TJ);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave / WN, wn = wave % WN;
   const int h = lane >> 5;
   const int64_t r0 = pos.r0, c0 = pos.c0, R = pos.R, brow = pos.brow, bcol = pos.bcol, nkb = pos.nkb;
   const int t = pos.t, slice = pos.slice;
@@ -89,17 +90,19 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
     // the 32 lanes of a half wave write 128 contiguous bytes of one row
     float* sp = a.split + ((int64_t)slice * R) * a.K;
 #pragma unroll
-    for (int bi = 0; bi < 4; ++bi)
+    for (int bi = 0; bi < TI; ++bi)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int64_t row = r0 + wm * 128 + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
+        const int64_t row = r0 + wm * (TI * 32) + bi * 32 + 8 * (v >> 2) + 4 * h + (v & 3);
         if (row >= R) continue;
 #pragma unroll
-        for (int bj = 0; bj < 2; ++bj)
-          sp[row * a.K + c0 + wn * 64 + bj * 32 + (lane & 31)] = acc[bi][bj][v];
+        for (int bj = 0; bj < TJ; ++bj)
+          sp[row * a.K + c0 + wn * (TJ * 32) + bj * 32 + (lane & 31)] = acc[bi][bj][v];
       }
     return;
   }
+  // the narrower block only exists with a sliced contraction (the launcher sees to it)
+  if constexpr (BN == 256) {
 
   // ---- epilogue: the 256 x 256 result goes through LDS (the operand buffers are free after
   // the loop's last barrier) so that global memory is touched in row-contiguous 16-byte vectors;
@@ -236,37 +239,45 @@ AHL_DEV void bwd_finish(const BwdArgs& a, const BwdPos& pos, f32x16 (&acc)[4][2]
       p[0] = u; p[1] = l; p[2] = c; p[3] = 0.0f;
     }
   }
+  }
 }
 
 // TAIL: the contraction length is not a multiple of 64 (its last chunk is loaded with
 // predicates); the TAIL = false instantiation has no trace of that in its hot loop.
-template <class D, int MODE, bool TAIL>
+//
+// BN: output columns per block. 256: 2 x 4 waves of 128 x 64. 192 (weight gradient with a sliced
+// contraction only): 4 x 2 waves of 64 x 96, for K-tiles of 3 x 64 columns and their multiples that
+// blocks of 256 would cover with a quarter of their columns empty.
+template <class D, int MODE, bool TAIL, int BN>
 __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
+  static_assert(BN == 256 || (BN == 192 && MODE == MODE_DW), "block widths: 256, or 192 for the weight gradient");
+  constexpr int WN = BN == 256 ? 4 : 2, WM = 8 / WN;  // waves along the columns / the rows
+  constexpr int TI = 256 / (32 * WM), TJ = BN / (32 * WN);  // 32 x 32 tiles of a wave
   extern __shared__ __attribute__((aligned(16))) char lds[];
   __shared__ float red[8][3];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 2, wn = wave & 3;  // 2 x 4 waves
+  const int wm = wave / WN, wn = wave % WN;
   const int h = lane >> 5;
 
-  // ---- block -> output tile. columns of the output are k (both modes), 256 per block ----
-  const int64_t nkb = a.K / 256;
+  // ---- block -> output tile. columns of the output are k (both modes), BN per block ----
+  const int64_t nkb = a.K / BN;
   const int64_t nb = gridDim.x / a.slices;            // output tiles
   const int slice = (int)(blockIdx.x / nb);
   int64_t brow, bcol;
   block_to_tile(blockIdx.x % nb, nb, nb / nkb, nkb, 4, brow, bcol);
   const int64_t r0 = brow * 256;                     // DX: m0; DW: n0
-  const int64_t c0 = bcol * 256;                     // k0
+  const int64_t c0 = bcol * BN;                      // k0
   const int t = (int)((c0 + (MODE == MODE_DW ? a.col_base : 0)) / a.tile);
   const int64_t R = MODE == MODE_DX ? a.M : a.N;      // output rows
   const int64_t L = MODE == MODE_DX ? a.N : a.M;      // contraction length
   const bool use_keep = a.keep != nullptr && clamp_flag_says_clamped(a.clamp_flag, a.flag_token);
   const uint32_t* plane = use_keep ? a.keep + (int64_t)t * clamp_plane_words(a.M, a.mask_N) : nullptr;
 
-  f32x16 acc[4][2];
+  f32x16 acc[TI][TJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TI; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TJ; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
@@ -311,10 +322,11 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   // weight gradient of a convolution read off the image: this thread's 8 columns are 8 channels of
   // one tap, i.e. of the image rows `tap offset` further on; columns in the padding between two
   // tiles contribute zeros
-  bool b_valid = true;
+  // (a block narrower than the 256 columns the threads span leaves the last vectors of a row unused)
+  bool b_valid = BN == 256 || km_cv * 8 < BN;
   if (MODE == MODE_DW && a.conv.on) {
     const int32_t in_tile = (int32_t)(c0 - (int64_t)t * a.tile) + km_cv * 8;
-    b_valid = in_tile < a.conv_cols;
+    b_valid = b_valid && in_tile < a.conv_cols;
     const int32_t tap = b_valid ? in_tile / a.conv.tile_base : 0;
     const int32_t ch = b_valid ? in_tile - tap * a.conv.tile_base : 0;
 #pragma unroll
@@ -444,20 +456,20 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
       if (ch + 1 < nchunks) load(kMasked);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        u32x4 fa[4], fb[2];
+        u32x4 fa[TI], fb[TJ];
 #pragma unroll
-        for (int bi = 0; bi < 4; ++bi) {
+        for (int bi = 0; bi < TI; ++bi) {
           if (MODE == MODE_DX)
-            fa[bi] = *(const u32x4*)(sa + (wm * 128 + bi * 32 + (lane & 31)) * kRowkStride + s * 32 + h * 16);
+            fa[bi] = *(const u32x4*)(sa + (wm * (TI * 32) + bi * 32 + (lane & 31)) * kRowkStride + s * 32 + h * 16);
           else
-            fa[bi] = read_kmaj(sa, wm * 128 + bi * 32, s);
+            fa[bi] = read_kmaj(sa, wm * (TI * 32) + bi * 32, s);
         }
 #pragma unroll
-        for (int bj = 0; bj < 2; ++bj) fb[bj] = read_kmaj(sb, wn * 64 + bj * 32, s);
+        for (int bj = 0; bj < TJ; ++bj) fb[bj] = read_kmaj(sb, wn * (TJ * 32) + bj * 32, s);
 #pragma unroll
-        for (int bi = 0; bi < 4; ++bi)
+        for (int bi = 0; bi < TI; ++bi)
 #pragma unroll
-          for (int bj = 0; bj < 2; ++bj) Mma16<D>::run(fa[bi], fb[bj], acc[bi][bj]);
+          for (int bj = 0; bj < TJ; ++bj) Mma16<D>::run(fa[bi], fb[bj], acc[bi][bj]);
       }
       if (ch + 1 < nchunks) {
         char* na = lds + ((ch + 1) & 1) * 2 * kOperandLds;
@@ -488,15 +500,43 @@ __global__ __launch_bounds__(512, 2) void k_bwd_fast(BwdArgs a) {
   }
 
   const BwdPos pos = {r0, c0, R, brow, bcol, nkb, t, slice};
-  bwd_finish<D, MODE>(a, pos, acc, lds, red);
+  bwd_finish<D, MODE, BN, TI, TJ>(a, pos, acc, lds, red);
 }
 
-// out[r, c] = the sum over slices of split[s][r][c], slices added in order, rounded to the dtype
+// dbias[n] = the sum of the partial rows, rounded to the dtype: 16 columns per block, 16 threads per column that
+// each add every 16th row, combined in a fixed order (the partial rows can be hundreds when the
+// weight gradient is sliced)
+template <class D>
+AHL_DEV void bias_final_block(int64_t block, const float* partial, int rows, int64_t N, uint16_t* dbias) {
+  __shared__ float part[16][17];
+  const int col = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  const int64_t n = block * 16 + col;
+  float s = 0.0f;
+  if (n < N)
+    for (int i = grp; i < rows; i += 16) s += partial[(int64_t)i * N + n];
+  part[grp][col] = s;
+  __syncthreads();
+  if (grp == 0 && n < N) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sum += part[i][col];
+    dbias[n] = D::to_elem(sum);
+  }
+}
+
+// out[r, c] = the sum over slices of split[s][r][c], slices added in order, rounded to the dtype.
+// The first bias_blocks blocks (or none) finish the bias gradient in the same launch: a few long
+// chains of additions that start first and run beside the sums.
 template <class D>
 __global__ __launch_bounds__(256) void k_split_reduce(const float* __restrict__ split, int slices,
                                                       int64_t R, int64_t K, uint16_t* __restrict__ out,
-                                                      int64_t ldo) {
-  const int64_t idx = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+                                                      int64_t ldo, int64_t bias_blocks, const float* bias_partial,
+                                                      int bias_rows, uint16_t* dbias) {
+  if ((int64_t)blockIdx.x < bias_blocks) {   // uniform over the block
+    bias_final_block<D>((int64_t)blockIdx.x, bias_partial, bias_rows, R, dbias);
+    return;
+  }
+  const int64_t idx = (((int64_t)blockIdx.x - bias_blocks) * 256 + threadIdx.x) * 4;
   if (idx >= R * K) return;
   const int64_t r = idx / K, c = idx - r * K;  // K is a multiple of 256: the 4 share a row
   f32x4 sum = {0.f, 0.f, 0.f, 0.f};
@@ -588,43 +628,27 @@ __global__ __launch_bounds__(512) void k_dx_split_reduce(BwdArgs a) {
   }
 }
 
-// dbias[n] = the sum of the partial rows, rounded to the dtype: 16 columns per block, 16 threads per column that
-// each add every 16th row, combined in a fixed order (the partial rows can be hundreds when the
-// weight gradient is sliced)
 template <class D>
 __global__ __launch_bounds__(256) void k_bias_final(const float* partial, int rows, int64_t N,
                                                     uint16_t* dbias) {
-  __shared__ float part[16][17];
-  const int col = threadIdx.x & 15, grp = threadIdx.x >> 4;
-  const int64_t n = (int64_t)blockIdx.x * 16 + col;
-  float s = 0.0f;
-  if (n < N)
-    for (int i = grp; i < rows; i += 16) s += partial[(int64_t)i * N + n];
-  part[grp][col] = s;
-  __syncthreads();
-  if (grp == 0 && n < N) {
-    float sum = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sum += part[i][col];
-    dbias[n] = D::to_elem(sum);
-  }
+  bias_final_block<D>((int64_t)blockIdx.x, partial, rows, N, dbias);
 }
 
-template <class D, int MODE, bool TAIL>
+template <class D, int MODE, bool TAIL, int BN>
 static void launch_bwd_one(dim3 grid, hipStream_t s, const BwdArgs& a) {
   // a refusal shows at the launch that follows (check_launch reads the last error)
-  (void)hipFuncSetAttribute((const void*)k_bwd_fast<D, MODE, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
-  hipLaunchKernelGGL((k_bwd_fast<D, MODE, TAIL>), grid, dim3(512), kBwdLds, s, a);
+  (void)hipFuncSetAttribute((const void*)k_bwd_fast<D, MODE, TAIL, BN>, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLds);
+  hipLaunchKernelGGL((k_bwd_fast<D, MODE, TAIL, BN>), grid, dim3(512), kBwdLds, s, a);
 }
 
-template <int MODE>
+template <int MODE, int BN = 256>
 static void launch_bwd(int32_t dtype, bool tail, dim3 grid, hipStream_t s, const BwdArgs& a) {
   if (dtype == AHL_F16) {
-    if (tail) launch_bwd_one<F16, MODE, true>(grid, s, a);
-    else launch_bwd_one<F16, MODE, false>(grid, s, a);
+    if (tail) launch_bwd_one<F16, MODE, true, BN>(grid, s, a);
+    else launch_bwd_one<F16, MODE, false, BN>(grid, s, a);
   } else {
-    if (tail) launch_bwd_one<BF16, MODE, true>(grid, s, a);
-    else launch_bwd_one<BF16, MODE, false>(grid, s, a);
+    if (tail) launch_bwd_one<BF16, MODE, true, BN>(grid, s, a);
+    else launch_bwd_one<BF16, MODE, false, BN>(grid, s, a);
   }
 }
 
@@ -722,8 +746,22 @@ int fast_dw_slices(int64_t M, int64_t K, int64_t N) {
   return tiles >= 128 ? 1 : dw_slices_for(tiles, M);
 }
 
-static int dw_parts(int64_t M, int64_t K, int64_t N, bool whole_only, DwPart parts[2]) {
+// Columns per block for the weight gradient of an image operand whose K-tiles hold `tile_cols`
+// columns: 192 when that divides the tile, 256 does not, and the 192-wide blocks are few enough
+// for a sliced contraction (the narrower block has no unsliced epilogue); else 256, with the tile
+// padded to a multiple of it.
+int fast_dw_image_block(int64_t M, int64_t tile_cols, int32_t n_tiles, int64_t N) {
+  if (tile_cols % 256 == 0 || tile_cols % 192 != 0) return 256;
+  const int64_t tiles = cdiv(N, 256) * (tile_cols / 192) * n_tiles;
+  return tiles < 128 && dw_slices_for(tiles, M) > 1 ? 192 : 256;
+}
+
+static int dw_parts(int64_t M, int64_t K, int64_t N, bool whole_only, int bw, DwPart parts[2]) {
   const int64_t nrows = cdiv(N, 256), nkb = K / 256, tiles = nrows * nkb;
+  if (bw != 256) {  // the narrower blocks of an image operand: one launch, sliced
+    parts[0] = {0, N, 0, K, dw_slices_for(nrows * (K / bw), M)};
+    return 1;
+  }
   parts[0] = {0, N, 0, K, fast_dw_slices(M, K, N)};
   if (whole_only || tiles <= 256 || tiles % 256 == 0) return 1;
   for (int64_t kb1 = nkb - 1; kb1 >= 1; --kb1) {
@@ -748,28 +786,31 @@ static int dw_parts(int64_t M, int64_t K, int64_t N, bool whole_only, DwPart par
   return 1;
 }
 
-static int64_t dw_part_bias_bytes(const DwPart& p) { return ((int64_t)p.slices * (p.k / 256) * p.n * 4 + 255) / 256 * 256; }
-static int64_t dw_part_bytes(const DwPart& p) {
-  return dw_part_bias_bytes(p) + (p.slices > 1 ? ((int64_t)p.slices * p.n * p.k * 4 + 255) / 256 * 256 : 0);
+static int64_t dw_part_bias_bytes(const DwPart& p, int bw) { return ((int64_t)p.slices * (p.k / bw) * p.n * 4 + 255) / 256 * 256; }
+static int64_t dw_part_bytes(const DwPart& p, int bw) {
+  return dw_part_bias_bytes(p, bw) + (p.slices > 1 ? ((int64_t)p.slices * p.n * p.k * 4 + 255) / 256 * 256 : 0);
 }
 
 // Workspace of launch_fast_dw, per launch: [partial bias sums: slices x k/256 x n floats |
 // slices > 1: partial results slices x n x k floats]
-int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N) {
+int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int block_cols) {
   DwPart parts[2];
-  const int np = dw_parts(M, K, N, false, parts);
+  const int np = dw_parts(M, K, N, false, block_cols, parts);
   int64_t bytes = 0;
-  for (int i = 0; i < np; ++i) bytes += dw_part_bytes(parts[i]);
+  for (int i = 0; i < np; ++i) bytes += dw_part_bytes(parts[i], block_cols);
   return bytes;
 }
 
 int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
-                   hipStream_t s, const ConvMap* conv, int32_t conv_cols) {
+                   hipStream_t s, const ConvMap* conv, int32_t conv_cols, int block_cols) {
   DwPart parts[2];
+  const int bw = conv != nullptr ? block_cols : 256;
+  if (bw != 256 && (bw != 192 || K % 192 != 0 || tl.base % 192 != 0)) return AHL_ERR_ARG;
   // an image operand maps its columns itself: one launch
-  const int np = dw_parts(M, K, N, conv != nullptr, parts);
+  const int np = dw_parts(M, K, N, conv != nullptr, bw, parts);
+  if (bw != 256 && parts[0].slices < 2) return AHL_ERR_ARG;
   char* wsp = (char*)ws;
   for (int i = 0; i < np; ++i) {
     const DwPart& p = parts[i];
@@ -790,28 +831,31 @@ int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* ke
     a.dense_base = 0; a.dense_extra = 0;
     a.col_base = p.k0; a.mask_N = N;
     a.slices = p.slices;
-    a.split = p.slices > 1 ? (float*)(wsp + dw_part_bias_bytes(p)) : nullptr;
-    const int64_t nb = cdiv(p.n, 256) * (p.k / 256) * p.slices;
+    a.split = p.slices > 1 ? (float*)(wsp + dw_part_bias_bytes(p, bw)) : nullptr;
+    const int64_t nb = cdiv(p.n, 256) * (p.k / bw) * p.slices;
     if (nb > 0x7fffffff) return AHL_ERR_ARG;
-    launch_bwd<MODE_DW>(dtype, M % 64 != 0, dim3((unsigned)nb), s, a);
-    const dim3 reduce_grid((unsigned)cdiv(p.n * p.k, 1024)), bias_grid((unsigned)cdiv(p.n, 16));
-    const int bias_rows = (int)(p.k / 256) * p.slices;
+    if (bw == 192) launch_bwd<MODE_DW, 192>(dtype, M % 64 != 0, dim3((unsigned)nb), s, a);
+    else launch_bwd<MODE_DW>(dtype, M % 64 != 0, dim3((unsigned)nb), s, a);
+    // a sliced launch sums its slices and finishes the bias gradient in one more launch
+    const int64_t sum_blocks = cdiv(p.n * p.k, 1024), bias_blocks = dbias_p ? cdiv(p.n, 16) : 0;
+    const dim3 reduce_grid((unsigned)(sum_blocks + bias_blocks)), bias_grid((unsigned)cdiv(p.n, 16));
+    const int bias_rows = (int)(p.k / bw) * p.slices;
     if (dtype == AHL_F16) {
       if (p.slices > 1)
         hipLaunchKernelGGL(k_split_reduce<F16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, p.slices, p.n, p.k,
-                           a.out, lddw);
-      if (dbias_p)
+                           a.out, lddw, bias_blocks, (const float*)bias_partial, bias_rows, (uint16_t*)dbias_p);
+      else if (dbias_p)
         hipLaunchKernelGGL(k_bias_final<F16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, p.n,
                            (uint16_t*)dbias_p);
     } else {
       if (p.slices > 1)
         hipLaunchKernelGGL(k_split_reduce<BF16>, reduce_grid, dim3(256), 0, s, (const float*)a.split, p.slices, p.n, p.k,
-                           a.out, lddw);
-      if (dbias_p)
+                           a.out, lddw, bias_blocks, (const float*)bias_partial, bias_rows, (uint16_t*)dbias_p);
+      else if (dbias_p)
         hipLaunchKernelGGL(k_bias_final<BF16>, bias_grid, dim3(256), 0, s, (const float*)bias_partial, bias_rows, p.n,
                            (uint16_t*)dbias_p);
     }
-    wsp += dw_part_bytes(p);
+    wsp += dw_part_bytes(p, bw);
   }
   return check_launch("ahl_linear_bwd_dw(fast)");
 }

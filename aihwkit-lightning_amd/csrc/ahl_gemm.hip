@@ -720,8 +720,8 @@ int64_t fast_dx_row_blocks(int64_t M, int64_t K, int64_t N, bool element_mode);
 int launch_fast_dw(int32_t dtype, const void* g, int64_t ldg, const uint32_t* keep, const uint32_t* clamp_flag,
                    uint32_t flag_token, const void* xq, int64_t ldxq, void* dw, int64_t lddw, void* dbias,
                    void* ws, int64_t M, int64_t K, int64_t N, const Tiling& tl,
-                   hipStream_t s, const ConvMap* conv = nullptr, int32_t conv_cols = 0);
-int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N);
+                   hipStream_t s, const ConvMap* conv = nullptr, int32_t conv_cols = 0, int block_cols = 256);
+int64_t fast_dw_ws_bytes(int64_t M, int64_t K, int64_t N, int block_cols = 256);
 int launch_pad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows, const Tiling& tl,
                      int64_t stride, void* dst, int64_t ld_dst, hipStream_t s);
 int launch_unpad_tiles(const void* src, int64_t ld_src, int32_t dtype, int64_t rows, int64_t K,

@@ -524,7 +524,7 @@ using namespace ahl;
 // ============================================================================================
 extern "C" {
 
-int ahl_abi_version(void) { return 15; }
+int ahl_abi_version(void) { return 16; }
 
 int ahl_seed_advance(uint64_t* state, uint64_t delta, void* stream) {
   if (!state) return AHL_ERR_ARG;

@@ -500,6 +500,11 @@ int ahl_conv_image_rows(const void* x, const AhlConvGeom* geom, int32_t dtype, c
 int ahl_conv_weight_layout(const void* src, int64_t ld_src, int32_t dtype, int64_t N, const AhlConvGeom* geom,
                            const int32_t* tile_ends_host, int32_t n_tiles, int32_t mode, int64_t stride, void* dst,
                            int64_t ld_dst, void* stream);
+/* Modes 0 and 2 of ahl_conv_weight_layout in one launch: a training step's forward leaves the
+ * input gradient's operand beside its own.                                                      */
+int ahl_conv_weight_layouts(const void* src, int64_t ld_src, int32_t dtype, int64_t N, const AhlConvGeom* geom,
+                            const int32_t* tile_ends_host, int32_t n_tiles, void* w_taps, int64_t ld_taps, void* w_dx,
+                            int64_t ld_dx, void* stream);
 
 /* The analog forward on the padded pixel grid: y_rows [P, N] (no lead rows), clamp mask
  * [T, ceil(N/32), rows64(P)] and flag as ahl_linear_fwd writes them; w_taps from

@@ -271,6 +271,14 @@ _SWEEP = [
     (1, 2, 64, (300,), (9,), (4,), 128, 0, "bf16"),              # long sequence, 9 taps
     (1, 4, 192, (33,), (3,), (0,), 64, 64, "f16"),               # three tiles, no padding
     (2, 0, 128, (9, 10), (3, 3), (2, 2), 64, 64, "bf16"),        # unbatched, padding wider than the kernel needs
+    # enough pixels for a sliced weight gradient, K-tiles of 3 x 192 columns (the 192-wide blocks):
+    # 4 x 16 x 16 = 1024 padded pixels (whole chunks of 64), 4 x 18 x 18 (a partial last chunk),
+    # 6 x 192 columns in f16, 9 x 192 columns from 27 taps, and N beyond one row of blocks
+    (2, 4, 128, (14, 14), (3, 3), (1, 1), 64, 64, "bf16"),
+    (2, 4, 192, (16, 16), (3, 3), (1, 1), 128, 64, "bf16"),
+    (2, 4, 128, (16, 15), (3, 3), (1, 1), 64, 0, "f16"),
+    (3, 2, 64, (8, 9, 8), (3, 3, 3), (1, 1, 1), 64, 0, "bf16"),
+    (2, 4, 64, (16, 16), (3, 3), (1, 1), 320, 0, "bf16"),
 ]
 
 
