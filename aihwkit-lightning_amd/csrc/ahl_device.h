@@ -389,15 +389,19 @@ AHL_DEV void normal8(uint64_t seed, uint64_t offset, uint32_t stream_and_tile, u
 // Records the clamp bits of one register of a 32x32 MFMA result (lane l holds column l % 32 of
 // row `row` for l < 32 and of row `row + 4` for l >= 32, rows counted within the wave's tile)
 // in `words`, where lane L keeps the mask word of row L. Must be called by the whole wave.
+// v_writelane_b32 through the compiler (this clang declares no builtin for it): it then places the
+// wait states after the compare that produced the value itself, and a lane number that is a
+// constant after unrolling becomes an immediate operand.
+extern "C" __device__ int ahl_writelane(int value, int lane, int old) __asm("llvm.amdgcn.writelane.i32");
+
+AHL_DEV void clamp_record_bits(uint64_t b, int row, uint32_t& words) {
+  // the ballot is wave-uniform: its halves go into lanes `row` and `row + 4` directly (a select
+  // per lane would cost two compares that write scalar registers)
+  words = (uint32_t)ahl_writelane((int)(uint32_t)b, row, (int)words);
+  words = (uint32_t)ahl_writelane((int)(uint32_t)(b >> 32), row + 4, (int)words);
+}
 AHL_DEV void clamp_record(bool clamped, int row, uint32_t& words) {
-  // the ballot is wave-uniform: its halves go into lanes `row` and `row + 4` directly
-  // (v_writelane_b32; a select per lane would cost two compares that write scalar registers)
-  const uint64_t b = __builtin_amdgcn_ballot_w64(clamped);
-  const uint32_t lo = (uint32_t)b, hi = (uint32_t)(b >> 32);
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0"
-               : "+v"(words) : "s"(lo), "s"(row) : "m0");
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tv_writelane_b32 %0, %1, m0"
-               : "+v"(words) : "s"(hi), "s"(row + 4) : "m0");
+  clamp_record_bits(__builtin_amdgcn_ballot_w64(clamped), row, words);
 }
 
 // Zeroes the elements of a vector of 8 bf16 whose bit in the low byte of `bits` is set.

@@ -358,18 +358,21 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
           if (CLAMP) {
             const bool over = excess > 0.0f;
             if (__builtin_expect(__any(over), 0)) {
+              if (a.keep != nullptr) {
+                // the compare's scalar result is the wave's mask bits of two rows
+                const uint64_t cols = __builtin_amdgcn_ballot_w64(nvalid);
 #pragma unroll
-              for (int e = 0; e < 8; ++e) {
-                const bool cl = fabsf(y8[e]) > B8[e];
-                if (a.keep != nullptr)
-                  clamp_record(cl && nvalid, 32 * bi + 8 * (2 * gp + (e >> 2)) + (e & 3), cwords[bj]);
-                y8[e] = fminf(fmaxf(y8[e], -B8[e]), B8[e]);
+                for (int e = 0; e < 8; ++e)
+                  clamp_record_bits(__builtin_amdgcn_ballot_w64(fabsf(y8[e]) > B8[e]) & cols,
+                                    32 * bi + 8 * (2 * gp + (e >> 2)) + (e & 3), cwords[bj]);
               }
+#pragma unroll
+              for (int e = 0; e < 8; ++e) y8[e] = __builtin_amdgcn_fmed3f(y8[e], -B8[e], B8[e]);
 #pragma unroll
               for (int q = 0; q < 4; ++q)
                 totp[bi][bj][4 * gp + q] =
                     D::pack2(D::lo(tpo[q]) + y8[2 * q], D::hi(tpo[q]) + y8[2 * q + 1]);
-              any_clamp |= over ? 1u : 0u;
+              any_clamp = 1u;   // wave-uniform here; only "any lane" is read at the end
             }
           }
           // keep the scheduler from interleaving the 8 Philox/Box-Muller chains of a block:

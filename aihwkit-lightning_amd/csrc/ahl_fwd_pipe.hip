@@ -180,6 +180,7 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
   int st_read = 0;
   asm volatile("" : "+v"(rdA), "+v"(rdB));
   const int64_t nbase = n0 + wn * 64 + r;   // this lane's column in MFMA block bj: nbase + 32 bj
+  const bool ncheck = (a.N & 63) != 0;      // some block of 64 columns is not whole
   float wch[2] = {0.0f, 0.0f};              // per-channel abs-max of the tile whose product is running
   // per-column constants of the tile in the epilogue, 8 floats per column: noise scale, bound,
   // ADC step, its reciprocal, abs-max for the noise, abs-max for the bound
@@ -299,16 +300,22 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
         if (!(EPI && CLAMP)) return;
         const int pbi = pu >> 2, pbj = (pu >> 1) & 1, pgp = pu & 1;
         // rare: an output of that unit left the range; its sums are redone with the clamped values
+        // (not rare at all with wide weight distributions: kept to a compare, two lane writes and a
+        // median per element; the compare's scalar result IS the wave's mask bits of two rows)
         if (__builtin_expect(__any(overp), 0)) {
+          if (a.keep != nullptr) {
+            uint64_t cols = ~0ull;   // columns of this block that exist
+            if (__builtin_expect(ncheck, 0)) cols = __builtin_amdgcn_ballot_w64(nbase + 32 * pbj < a.N);
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            const bool cl = fabsf(yp[e]) > Bp[e];
-            const int g = 2 * pgp + (e >> 2);
-            if (a.keep != nullptr)
-              clamp_record(cl && nbase + 32 * pbj < a.N, 32 * (pbi & 1) + 8 * g + (e & 3), cwords[pbi >> 1][pbj]);
-            yp[e] = fminf(fmaxf(yp[e], -Bp[e]), Bp[e]);
+            for (int e = 0; e < 8; ++e) {
+              const int g = 2 * pgp + (e >> 2);
+              const uint64_t bits = __builtin_amdgcn_ballot_w64(fabsf(yp[e]) > Bp[e]) & cols;
+              clamp_record_bits(bits, 32 * (pbi & 1) + 8 * g + (e & 3), cwords[pbi >> 1][pbj]);
+            }
           }
-          any_clamp |= overp ? 1u : 0u;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) yp[e] = __builtin_amdgcn_fmed3f(yp[e], -Bp[e], Bp[e]);
+          any_clamp = 1u;   // wave-uniform here; only "any lane" is read at the end
         }
         // total = rd(total + y), bf16 pairs
 #pragma unroll
