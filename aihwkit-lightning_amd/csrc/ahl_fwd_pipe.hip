@@ -304,13 +304,25 @@ __global__ __launch_bounds__(1024 / NBI, NBI == 4 ? 1 : 2) void k_fwd_pipe(FastF
         // median per element; the compare's scalar result IS the wave's mask bits of two rows)
         if (__builtin_expect(__any(overp), 0)) {
           if (a.keep != nullptr) {
-            uint64_t cols = ~0ull;   // columns of this block that exist
-            if (__builtin_expect(ncheck, 0)) cols = __builtin_amdgcn_ballot_w64(nbase + 32 * pbj < a.N);
+            if (__builtin_expect(ncheck, 0)) {
+              const uint64_t cols = __builtin_amdgcn_ballot_w64(nbase + 32 * pbj < a.N);   // columns that exist
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-              const int g = 2 * pgp + (e >> 2);
-              const uint64_t bits = __builtin_amdgcn_ballot_w64(fabsf(yp[e]) > Bp[e]) & cols;
-              clamp_record_bits(bits, 32 * (pbi & 1) + 8 * g + (e & 3), cwords[pbi >> 1][pbj]);
+              for (int e = 0; e < 8; ++e)
+                clamp_record_bits(__builtin_amdgcn_ballot_w64(fabsf(yp[e]) > Bp[e]) & cols,
+                                  32 * (pbi & 1) + 8 * (2 * pgp + (e >> 2)) + (e & 3), cwords[pbi >> 1][pbj]);
+            } else {
+              // four compares, then their eight lane writes: a lane write right behind the compare
+              // whose scalar result it takes waits out the distance
+#pragma unroll
+              for (int e0 = 0; e0 < 8; e0 += 4) {
+                uint64_t bits[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) bits[e] = __builtin_amdgcn_ballot_w64(fabsf(yp[e0 + e]) > Bp[e0 + e]);
+                asm volatile("" : "+s"(bits[0]), "+s"(bits[1]), "+s"(bits[2]), "+s"(bits[3]));
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  clamp_record_bits(bits[e], 32 * (pbi & 1) + 8 * (2 * pgp + (e0 >> 2)) + e, cwords[pbi >> 1][pbj]);
+              }
             }
           }
 #pragma unroll
