@@ -364,3 +364,57 @@ def test_calibration_max_sees_patches():
             .reshape(-1, 27) for b in batches]
     assert torch.equal(layer.input_range.data.cpu(), om.calibrate_max(rows, layer.in_sizes))
     assert layer(batches[0].cuda()).shape == (2, 4, 5, 4)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_weight_layouts_through_the_c_abi(dtype):
+    """ahl_conv_weight_layout modes 0, 1, 2 against index arithmetic on the host, mode 1 with tiles
+    that start every `stride` columns, and ahl_conv_weight_layouts (modes 0 and 2 in one launch)
+    against the two single launches, bit for bit."""
+    from ctypes import byref
+    from aihwkit_lightning.nn.modules.hip_utils import library as L, ops
+
+    lib = L.load()
+    n_out, chan, kern, ct = 64, 128, (3, 2), 64
+    kvol, n_tiles = kern[0] * kern[1], chan // ct
+    k_in = chan * kvol
+    geom = [2, chan, 7, 6, 1, kern[0], kern[1], 1, 1, 1, 1, 1, 1, 1, 1, 1, 1]
+    cgeom = ops.conv_geom(geom)
+    ends = L.tile_ends_array([ct * kvol] * n_tiles)
+    dt = L.AHL_BF16 if dtype == torch.bfloat16 else L.AHL_F16
+    stream = ops.current_stream()
+    gen = torch.Generator().manual_seed(5)
+    w = torch.randn(n_out, k_in, generator=gen).to(dtype).cuda()
+
+    def layout(src, ld_src, mode, stride, shape):
+        dst = torch.zeros(shape, dtype=dtype, device="cuda")
+        rc = lib.ahl_conv_weight_layout(ops.ptr(src), ld_src, dt, n_out, byref(cgeom), ends, n_tiles, mode, stride,
+                                        ops.ptr(dst), dst.size(1), stream)
+        assert rc == 0
+        return dst
+
+    # the layer's order: column (channel, tap); the forward's: per tile (tap, channel in the tile)
+    w4 = w.view(n_out, n_tiles, ct, kvol)
+    want_taps = w4.permute(0, 1, 3, 2).reshape(n_out, k_in)
+    want_dx = w.view(n_out, chan, kvol).permute(1, 2, 0).reshape(chan, kvol * n_out)
+    taps = layout(w, k_in, 0, 0, (n_out, k_in))
+    w_dx = layout(w, k_in, 2, 0, (chan, kvol * n_out))
+    assert torch.equal(taps, want_taps) and torch.equal(w_dx, want_dx)
+    # mode 1 from tiles that start every 448 columns (384 of them data)
+    stride = 448
+    spaced = torch.full((n_out, n_tiles * stride), float("nan"), dtype=dtype, device="cuda")
+    for t in range(n_tiles):
+        spaced[:, t * stride:t * stride + ct * kvol] = taps[:, t * ct * kvol:(t + 1) * ct * kvol]
+    assert torch.equal(layout(spaced, spaced.size(1), 1, stride, (n_out, k_in)), w)
+    both_taps = torch.zeros_like(taps)
+    both_dx = torch.zeros_like(w_dx)
+    rc = lib.ahl_conv_weight_layouts(ops.ptr(w), k_in, dt, n_out, byref(cgeom), ends, n_tiles, ops.ptr(both_taps), k_in,
+                                     ops.ptr(both_dx), both_dx.size(1), stream)
+    assert rc == 0
+    assert torch.equal(both_taps, taps) and torch.equal(both_dx, w_dx)
+    # refusals: a missing destination, tiles that split a channel's taps
+    assert lib.ahl_conv_weight_layouts(ops.ptr(w), k_in, dt, n_out, byref(cgeom), ends, n_tiles, ops.ptr(both_taps), k_in,
+                                       None, 0, stream) == 1   # AHL_ERR_ARG
+    odd = L.tile_ends_array([100, k_in - 100])
+    assert lib.ahl_conv_weight_layouts(ops.ptr(w), k_in, dt, n_out, byref(cgeom), odd, 2, ops.ptr(both_taps), k_in,
+                                       ops.ptr(both_dx), both_dx.size(1), stream) != 0
