@@ -179,7 +179,10 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
       const int64_t m = m0 + tid;
       const float irm = m < a.M ? D::load(a.ir, (int64_t)tt * a.M + m) : 0.0f;
       float* rc = rowc + (tt & 1) * 384;
-      rc[tid] = D::rd(a.noise_scale * irm);
+      // a noise scale that is the same for every channel of the tile (the tile's abs-max) is folded
+      // in here, once per row, instead of once per element in the epilogue
+      const float nrow = D::rd(a.noise_scale * irm);
+      rc[tid] = (!NOISE || a.noise_per_channel) ? nrow : D::rd(a.tile_max[tt] * nrow);
       rc[128 + tid] = D::rd(irm * a.out_bound);
     }
     __syncthreads();
@@ -288,15 +291,20 @@ __global__ __launch_bounds__(256, NBJ == 1 ? 3 : 2) void k_fwd_fast(FastFwdArgs 
               const int rl0 = rbase + 8 * g;
               if (NOISE) {
                 const f32x4 nr = *(const f32x4*)(rc_t + rl0);
+                if (a.noise_per_channel) {   // uniform over the launch
 #pragma unroll
-                for (int c = 0; c < 4; ++c) ns[c] = wr * nr[c];
+                  for (int c = 0; c < 4; ++c) ns[c] = wr * nr[c];
+                  round2<D>(ns[0], ns[1]); round2<D>(ns[2], ns[3]);
+                } else {
+#pragma unroll
+                  for (int c = 0; c < 4; ++c) ns[c] = nr[c];   // the row's scale, tile abs-max included
+                }
               }
               if (bound_on) {
                 const f32x4 br = *(const f32x4*)(rc_t + 128 + rl0);
 #pragma unroll
                 for (int c = 0; c < 4; ++c) Bv[c] = br[c] * wb;
               }
-              if (NOISE) { round2<D>(ns[0], ns[1]); round2<D>(ns[2], ns[3]); }
               if (bound_on) {
                 round2<D>(Bv[0], Bv[1]); round2<D>(Bv[2], Bv[3]);
                 if (ADC) {
