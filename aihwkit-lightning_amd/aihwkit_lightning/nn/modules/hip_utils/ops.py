@@ -79,11 +79,15 @@ def _aligned16(tensor: Tensor) -> bool:
     return bool(_SHAPES_ONLY.depth) or tensor.data_ptr() % 16 == 0
 
 
+_raw_stream = torch._C._cuda_getCurrentRawStream  # pylint: disable=protected-access
+_current_device = torch._C._cuda_getDevice if hasattr(torch._C, "_cuda_getDevice") else torch.cuda.current_device  # pylint: disable=protected-access
+
+
 def _stream():
     if _SHAPES_ONLY.depth:
         return None
     # the raw handle of torch's current stream, without building a Stream object per launch
-    return c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device()))  # pylint: disable=protected-access
+    return c_void_p(_raw_stream(_current_device()))
 
 
 def _rows2d(tensor: Tensor, name: str) -> Tensor:
@@ -434,12 +438,19 @@ def ir_init_update(ir: Tensor, idx: Tensor, std: Tensor, init_from_data: float, 
 def running_absmax(x: Tensor, in_sizes: List[int], cache: Tensor) -> None:
     """``cache[t] = max(cache[t], max |x[:, tile t]|)``; cache is float32 ``[T]`` on the device."""
     lib = _lib()
-    x = _rows2d(x, "x")
     if cache.dtype != torch.float32 or not cache.is_contiguous() or cache.numel() != len(in_sizes):
         raise HipBackendError("cache must be a contiguous float32 tensor with one entry per tile")
+    # a calibration pass calls this once per layer and batch, and the launch is short: the usual
+    # case (a contiguous 2-D batch) skips the general stride handling
+    if x.dim() == 2 and x.is_contiguous():
+        rows, cols = x.shape
+        ld = cols
+    else:
+        x = _rows2d(x, "x")
+        rows, cols, ld = x.size(0), x.size(1), _ld(x)
     L.check(
         lib.ahl_running_absmax(
-            _ptr(x), dtype_id(x.dtype), x.size(0), x.size(1), _ld(x), L.tile_ends_array(in_sizes),
+            _ptr(x), dtype_id(x.dtype), rows, cols, ld, L.tile_ends_array(in_sizes),
             len(in_sizes), _ptr(cache), _stream(),
         ),
         "ahl_running_absmax",

@@ -268,23 +268,25 @@ __global__ __launch_bounds__(256) void k_quantize_rows(ModArgs a, void* __restri
 // After k_quantize_rows, one block per tile: the tile's largest and smallest segment abs-max
 // (what k_tile_minmax computes), and the segments that kernel deferred, if any: with no such
 // segment (the usual case) the block is done after the reduction. With some, every wave walks a
-// quarter of the channels, 64 at a time, and quantises the deferred ones among them.
+// sixteenth of the channels, 64 at a time, and quantises the deferred ones among them. 1024
+// threads: the kernel's duration is a thread's chain of dependent loads, one pass of eight for up
+// to 8192 channels.
 template <class D>
-__global__ __launch_bounds__(256) void k_quantize_finish(ModArgs a, const void* __restrict__ wmax,
-                                                         float* __restrict__ tile_max,
-                                                         float* __restrict__ tile_min) {
-  __shared__ float smax[4], smin[4];
+__global__ __launch_bounds__(1024) void k_quantize_finish(ModArgs a, const void* __restrict__ wmax,
+                                                          float* __restrict__ tile_max,
+                                                          float* __restrict__ tile_min) {
+  __shared__ float smax[16], smin[16];
   __shared__ int s_any;
   const int32_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   float mx = 0.0f, mn = __builtin_inff();
   bool mine = false;
   if (threadIdx.x == 0) s_any = 0;
-  for (int64_t r0 = threadIdx.x; r0 < a.N; r0 += 256 * 8) {
+  for (int64_t r0 = threadIdx.x; r0 < a.N; r0 += 1024 * 8) {
     float v[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      const int64_t r = r0 + 256 * u;
+      const int64_t r = r0 + 1024 * u;
       v[u] = D::load(wmax, (int64_t)t * a.N + (r < a.N ? r : r0));  // r0 again: no effect
     }
 #pragma unroll
@@ -300,12 +302,13 @@ __global__ __launch_bounds__(256) void k_quantize_finish(ModArgs a, const void* 
   __syncthreads();
   if (mine) s_any = 1;
   __syncthreads();
-  const float tmax = fmaxf(fmaxf(smax[0], smax[1]), fmaxf(smax[2], smax[3]));
-  const float tmin = fminf(fminf(smin[0], smin[1]), fminf(smin[2], smin[3]));
+  float tmax = smax[0], tmin = smin[0];
+#pragma unroll
+  for (int w = 1; w < 16; ++w) { tmax = fmaxf(tmax, smax[w]); tmin = fminf(tmin, smin[w]); }
   if (threadIdx.x == 0) { tile_max[t] = tmax; tile_min[t] = tmin; }
   if (s_any == 0) return;
   const bool all_gt1 = quantize_deferred<D>(tmin, a.n_states);
-  for (int64_t base = (int64_t)wv * 64; base < a.N; base += 256) {
+  for (int64_t base = (int64_t)wv * 64; base < a.N; base += 1024) {
     const int64_t nl = base + lane;
     const float m = nl < a.N ? D::load(wmax, (int64_t)t * a.N + nl) : 0.0f;
     uint64_t todo = __ballot(nl < a.N && quantize_deferred<D>(m, a.n_states));
@@ -409,7 +412,7 @@ static int launch_prep(const void* w, int64_t N, int64_t K, int64_t ld, const Ti
       a.maxq = host_round_dtype(D::kId, a.n_states / 2.0f);
       a.std_dev = 0.0f; a.seed = 0; a.offset = 0; a.seed_state = nullptr;
       hipLaunchKernelGGL((k_quantize_rows<D>), grid, dim3(256), 0, s, a, wmax);
-      hipLaunchKernelGGL((k_quantize_finish<D>), dim3(tl.n_tiles), dim3(256), 0, s, a, (const void*)wmax, tile_max,
+      hipLaunchKernelGGL((k_quantize_finish<D>), dim3(tl.n_tiles), dim3(1024), 0, s, a, (const void*)wmax, tile_max,
                          tile_min);
       return check_launch("ahl_weight_prep(one-pass quantiser)");
     }
