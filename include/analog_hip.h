@@ -496,12 +496,14 @@ int ahl_conv_image_rows(const void* x, const AhlConvGeom* geom, int32_t dtype, c
 /* Weight layouts for the three products, from / to the layer's [N, C * kvol] matrix
  * (weight.view(out_channels, -1)): mode 0 reorders every tile's columns to (tap, channel) -- the
  * forward's operand; mode 1 is its inverse from a matrix whose tiles start every `stride` columns
- * (what ahl_conv_bwd_dw leaves) ; mode 2 writes [C, kvol * N] for the input gradient.          */
+ * (what ahl_conv_bwd_dw leaves) ; mode 2 writes [C, kvol * N] for the input gradient. The
+ * layer's matrix is nn/modules/conv.py:324 (modified_weights.view(out_channels, -1)), whose column
+ * order (channel, tap) is that of unfold's patch entries (:325-352).                            */
 int ahl_conv_weight_layout(const void* src, int64_t ld_src, int32_t dtype, int64_t N, const AhlConvGeom* geom,
                            const int32_t* tile_ends_host, int32_t n_tiles, int32_t mode, int64_t stride, void* dst,
                            int64_t ld_dst, void* stream);
 /* Modes 0 and 2 of ahl_conv_weight_layout in one launch: a training step's forward leaves the
- * input gradient's operand beside its own.                                                      */
+ * input gradient's operand beside its own (same source matrix, nn/modules/conv.py:324).         */
 int ahl_conv_weight_layouts(const void* src, int64_t ld_src, int32_t dtype, int64_t N, const AhlConvGeom* geom,
                             const int32_t* tile_ends_host, int32_t n_tiles, void* w_taps, int64_t ld_taps, void* w_dx,
                             int64_t ld_dx, void* stream);
