@@ -16,7 +16,8 @@
 // Block: 512 threads = 8 waves as 2 (rows) x 4 (columns); block tile 256 x 256, wave tile
 // 128 x 64 (4 x 2 MFMA blocks, 128 fp32 accumulators), 64 contraction steps per chunk,
 // double-buffered LDS (2 x 72 KB), one barrier per chunk, next chunk's global loads in flight
-// during the MFMAs of the current one.
+// during the MFMAs of the current one. The weight gradient also exists with a block tile of
+// 256 x 192 (4 x 2 waves of 64 x 96), for K-tiles that 192 divides and 256 does not.
 #include "ahl_host.h"
 #include <type_traits>
 
@@ -46,7 +47,7 @@ struct BwdArgs {
   float* partial;                      // DX static range: [blocks][4]
   float* bias_partial;                 // DW: [K / 256][N] partial column sums of g, or null
   int64_t M, N, K;
-  int32_t tile;                        // K-tile width (multiple of 256)
+  int32_t tile;                        // K-tile width (a multiple of the block width: 256, or 192)
   int32_t ir_static;                   // 0: no range gradient; 1 + AHL_IR_GRAD_* otherwise
   int32_t dense_tile;                  // DX: 0, or the true tile width when x and dx are dense
                                        // while W_eff is in the padded tile layout (K, tile then
